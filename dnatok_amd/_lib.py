@@ -1,0 +1,77 @@
+"""ctypes binding of libdnatok_hip.so (the C ABI declared in include/dnatok_hip.h).
+
+The library is the only compute path: there is no CPU or torch fallback.  If the
+shared object is missing, :func:`lib` raises with the build command.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, c_char_p, c_int, c_int32, c_int64, c_size_t, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libdnatok_hip.so")
+
+# every symbol include/dnatok_hip.h declares
+EXPORTS = [
+    "dnatok_version", "dnatok_last_error",
+    "dnatok_char_table_create", "dnatok_char_table_destroy",
+    "dnatok_char_encode_padded", "dnatok_char_encode_packed",
+    "dnatok_kmer_table_create", "dnatok_kmer_table_destroy", "dnatok_kmer_encode_padded",
+    "dnatok_bpe_table_create", "dnatok_bpe_table_destroy", "dnatok_bpe_scratch_bytes",
+    "dnatok_bpe_encode", "dnatok_pack_ragged", "dnatok_pad_rows",
+]
+
+_lib = None
+
+
+class DnatokError(RuntimeError):
+    pass
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise DnatokError(
+            f"{LIB_PATH} is missing: build it with `python -m dnatok_amd.build` "
+            "(hipcc --offload-arch=gfx950). There is no fallback path.")
+    L = ctypes.CDLL(LIB_PATH)
+    L.dnatok_version.restype = c_int
+    L.dnatok_last_error.restype = c_char_p
+    L.dnatok_char_table_create.argtypes = [c_void_p, c_void_p, c_int32, POINTER(c_void_p)]
+    L.dnatok_char_table_destroy.argtypes = [c_void_p]
+    L.dnatok_char_table_destroy.restype = None
+    L.dnatok_char_encode_padded.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int,
+                                            c_void_p, c_void_p, c_void_p]
+    L.dnatok_char_encode_packed.argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_void_p,
+                                            c_void_p, c_void_p]
+    L.dnatok_kmer_table_create.argtypes = [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                           c_int64, c_void_p, c_int32, c_int32, POINTER(c_void_p)]
+    L.dnatok_kmer_table_destroy.argtypes = [c_void_p]
+    L.dnatok_kmer_table_destroy.restype = None
+    L.dnatok_kmer_encode_padded.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                                            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    L.dnatok_bpe_table_create.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32,
+                                          c_void_p, POINTER(c_void_p)]
+    L.dnatok_bpe_table_destroy.argtypes = [c_void_p]
+    L.dnatok_bpe_table_destroy.restype = None
+    L.dnatok_bpe_scratch_bytes.argtypes = [c_void_p, c_int64, c_int64, c_int64]
+    L.dnatok_bpe_scratch_bytes.restype = c_size_t
+    L.dnatok_bpe_encode.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                                    c_void_p, c_size_t, c_void_p, c_void_p, c_void_p]
+    L.dnatok_pack_ragged.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p,
+                                     c_void_p, c_void_p, c_void_p]
+    L.dnatok_pad_rows.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int32, c_int64,
+                                  c_int64, c_void_p, c_void_p, c_void_p, c_void_p]
+    for name in EXPORTS:
+        getattr(L, name)          # AttributeError here means the library is stale
+    _lib = L
+    return L
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = lib().dnatok_last_error()
+        raise DnatokError(f"{what} failed ({rc}): {msg.decode(errors='replace') if msg else ''}")

@@ -1,0 +1,519 @@
+// BPE merge engine: reproduces the Hugging Face word-merge order exactly.
+//
+// HF pops adjacent pairs from a heap keyed (rank, position), skips stale entries, merges, and
+// pushes the two new neighbour pairs.  That is "always merge the pair with the smallest
+// (rank, position) key".  The engine below gets the same result in rounds:
+//
+//   * every live position i keeps the rank R[i] of the pair it starts; a team of threads
+//     (one wave, or one workgroup) finds rmin = min R and the gate G = min over current
+//     pairs of minchild[R[i]], where minchild[r] is the lowest rank of any rule that uses the
+//     symbol rule r creates.  No pair born in this round can have a rank below G, so all
+//     current pairs with rank in [rmin, G) can be settled together;
+//   * among those candidates a pair merges unless an overlapping candidate with a smaller
+//     key merges.  Overlaps form chains of strictly decreasing key, along which the decision
+//     alternates, so each candidate walks its left and right chain and merges iff both have
+//     even length (for a run x x x x this is "every other one from the left", HF's tie rule);
+//   * merges are applied in a doubly linked list over the original positions (a merge keeps
+//     the left position), the two neighbour pairs of each new symbol are re-ranked through
+//     the hashed merge table, and only the threads whose positions changed refresh their
+//     cached minima.
+//
+// A table in which some rule's product is used by a LOWER-ranked rule (possible when two
+// rules produce the same string) makes G <= rmin; such a round merges only the single
+// smallest-key pair, which is exactly HF's next step.
+//
+// State lives in LDS for rows up to the LDS capacity (symbols, ranks and links as uint16),
+// and in a global scratch area (L2-resident) for longer rows.
+#include "common.hpp"
+
+#include <stdlib.h>
+#include <string.h>
+#include <vector>
+
+struct dnatok_bpe_table {
+    int32_t n_merges, n_symbols;
+    uint32_t slots, shift;       // hash table size (power of two) and 32 - log2(slots)
+    int monotone;                // no rule's product is used by a lower-ranked rule
+    void *blob;
+    uint2 *tab;                  // [slots]  {key = a << 16 | b, val = rank}
+    uint16_t *newsym;            // [n_merges]
+    uint16_t *minchild;          // [n_merges]
+    uint16_t *byte_to_sym;       // [256]
+    int32_t *out_remap;          // [n_symbols] or nullptr
+};
+
+namespace dnatok {
+
+constexpr uint32_t kNone = 0xFFFFu;          // "no rule" rank / dead symbol
+constexpr uint32_t kEmptyKey = 0xFFFFFFFFu;
+
+struct BpeArgs {
+    const uint2 *tab;
+    const uint16_t *newsym, *minchild, *byte_to_sym;
+    const int32_t *out_remap;
+    uint32_t slots, shift;
+    int32_t n_merges;
+};
+
+__host__ __device__ __forceinline__ uint32_t pair_hash(uint32_t key, uint32_t shift)
+{
+    return (key * 0x9E3779B1u) >> shift;
+}
+
+// rank of the rule for (a, b), or kNone
+__device__ __forceinline__ uint32_t pair_rank(const uint2 *tab, uint32_t mask, uint32_t shift,
+                                              uint32_t a, uint32_t b)
+{
+    const uint32_t key = (a << 16) | b;
+    uint32_t h = pair_hash(key, shift);
+    for (;;) {
+        const uint2 e = tab[h];
+        if (e.x == key) return e.y;
+        if (e.x == kEmptyKey) return kNone;
+        h = (h + 1) & mask;
+    }
+}
+
+template <int NT>
+__device__ __forceinline__ void team_sync()
+{
+    if (NT == 64) {
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    } else {
+        __syncthreads();
+    }
+}
+
+// Minimum of two values over the team; includes exactly one team_sync.
+template <int NT>
+__device__ __forceinline__ void team_min2(uint32_t a, uint32_t b, uint32_t *red, int wv,
+                                          uint32_t &ra, uint32_t &rb)
+{
+    a = wave_min_u32(a);
+    b = wave_min_u32(b);
+    if (NT == 64) {
+        team_sync<NT>();
+        ra = a; rb = b;
+        return;
+    }
+    constexpr int NW = NT / 64;
+    if ((threadIdx.x & 63) == 0) { red[wv * 2] = a; red[wv * 2 + 1] = b; }
+    __syncthreads();
+    uint32_t x = kEmptyKey, y = kEmptyKey;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) { x = umin(x, red[w * 2]); y = umin(y, red[w * 2 + 1]); }
+    ra = x; rb = y;
+}
+
+// Exclusive prefix sum over the team (one value per thread) and the team total.
+template <int NT>
+__device__ __forceinline__ uint32_t team_exclusive_sum(uint32_t v, uint32_t *red, int wv, uint32_t &total)
+{
+    const uint32_t inc = wave_inclusive_sum_u32(v);
+    if (NT == 64) {
+        total = __builtin_amdgcn_readlane(inc, 63);
+        return inc - v;
+    }
+    constexpr int NW = NT / 64;
+    if ((threadIdx.x & 63) == 63) red[wv] = inc;
+    __syncthreads();
+    uint32_t carry = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) { const uint32_t t = red[w]; if (w < wv) carry += t; tot += t; }
+    __syncthreads();
+    total = tot;
+    return carry + inc - v;
+}
+
+// One row.  tid = index in the team; S/R/NX/PV/F hold n0 entries; D holds NT bytes;
+// red holds 4 * (NT / 64) words.  Tokens go to out[0 .. *out_len).
+template <int NT, typename IT>
+__device__ __forceinline__ void bpe_row(
+    const uint2 *tab, uint32_t tab_mask, uint32_t tab_shift, const uint16_t *newsym,
+    const uint16_t *minchild, const uint16_t *byte_to_sym, const int32_t *out_remap,
+    const uint8_t *__restrict__ src, const int n0, uint16_t *S, uint16_t *R, IT *NX, IT *PV,
+    uint8_t *F, uint8_t *D, uint32_t *red, const int tid, int32_t *__restrict__ out,
+    int32_t *__restrict__ out_len)
+{
+    constexpr IT NIL = (IT)~(IT)0;
+    const int wv = (NT == 64) ? 0 : (tid >> 6);
+    const int c = (n0 + NT - 1) / NT;
+    const int lo = (tid * c < n0) ? tid * c : n0;
+    const int hi = (lo + c < n0) ? lo + c : n0;
+
+    for (int i = lo; i < hi; ++i) {
+        S[i] = byte_to_sym[src[i]];
+        NX[i] = (i + 1 < n0) ? (IT)(i + 1) : NIL;
+        PV[i] = (i > 0) ? (IT)(i - 1) : NIL;
+        F[i] = 0;
+    }
+    D[tid] = 0;
+    team_sync<NT>();
+
+    uint32_t cmin = kEmptyKey, cgate = kEmptyKey;
+    for (int i = lo; i < hi; ++i) {
+        uint32_t r = kNone;
+        if (i + 1 < n0) r = pair_rank(tab, tab_mask, tab_shift, S[i], S[i + 1]);
+        R[i] = (uint16_t)r;
+        if (r != kNone) { cmin = umin(cmin, r); cgate = umin(cgate, minchild[r]); }
+    }
+
+    int flip = 0;
+    for (;;) {
+        uint32_t rmin, gate;
+        team_min2<NT>(cmin, cgate, red + flip * (NT / 64) * 2, wv, rmin, gate);
+        flip ^= 1;
+        if (rmin >= kNone) break;
+        const bool single = gate <= rmin;          // non-monotone table: one merge this round
+        uint32_t leftmost = 0;
+        if (single) {
+            uint32_t mypos = kEmptyKey;
+            if (cmin == rmin)
+                for (int i = lo; i < hi; ++i)
+                    if (R[i] == rmin) { mypos = (uint32_t)i; break; }
+            uint32_t dummy;
+            team_min2<NT>(mypos, mypos, red + flip * (NT / 64) * 2, wv, leftmost, dummy);
+            flip ^= 1;
+        }
+        const uint32_t limit = single ? rmin + 1 : gate;
+
+        // decide (reads only, except the owner's own flags)
+        bool mine = false;
+        if (cmin < limit) {
+            for (int i = lo; i < hi; ++i) {
+                const uint32_t r = R[i];
+                if (r >= limit) continue;
+                bool m;
+                if (single) {
+                    m = ((uint32_t)i == leftmost);
+                } else {
+                    uint32_t chain = 0;
+                    IT p = (IT)i;
+                    uint32_t rp = r;
+                    for (;;) {                       // candidates to the left with key <= ours
+                        const IT q = PV[p];
+                        if (q == NIL) break;
+                        const uint32_t rq = R[q];
+                        if (rq > rp) break;
+                        ++chain; p = q; rp = rq;
+                    }
+                    uint32_t chain_r = 0;
+                    p = (IT)i; rp = r;
+                    for (;;) {                       // candidates to the right with key < ours
+                        const IT q = NX[p];
+                        if (q == NIL) break;
+                        const uint32_t rq = R[q];
+                        if (rq >= rp) break;
+                        ++chain_r; p = q; rp = rq;
+                    }
+                    m = ((chain | chain_r) & 1u) == 0;
+                }
+                if (m) { F[i] = 1; mine = true; }
+            }
+        }
+        team_sync<NT>();
+
+        // apply: position i absorbs its right neighbour j
+        if (mine) {
+            for (int i = lo; i < hi; ++i) {
+                if (!F[i]) continue;
+                const IT j = NX[i];
+                const IT k = NX[j];
+                S[i] = newsym[R[i]];
+                S[j] = (uint16_t)kNone;
+                R[j] = (uint16_t)kNone;
+                NX[i] = k;
+                if (k != NIL) PV[k] = (IT)i;
+                if ((int)j >= hi) D[(int)j / c] = 1;
+            }
+        }
+        team_sync<NT>();
+
+        // re-rank the two pairs around every new symbol
+        if (mine) {
+            for (int i = lo; i < hi; ++i) {
+                if (!F[i]) continue;
+                F[i] = 0;
+                const IT k = NX[i];
+                const uint32_t s = S[i];
+                R[i] = (uint16_t)((k != NIL) ? pair_rank(tab, tab_mask, tab_shift, s, S[k]) : kNone);
+                const IT p = PV[i];
+                if (p != NIL) {
+                    R[p] = (uint16_t)pair_rank(tab, tab_mask, tab_shift, S[p], s);
+                    if ((int)p < lo) D[(int)p / c] = 1;
+                }
+            }
+        }
+        team_sync<NT>();
+
+        if (mine || D[tid]) {
+            D[tid] = 0;
+            cmin = kEmptyKey; cgate = kEmptyKey;
+            for (int i = lo; i < hi; ++i) {
+                const uint32_t r = R[i];
+                if (r != kNone) { cmin = umin(cmin, r); cgate = umin(cgate, minchild[r]); }
+            }
+        }
+    }
+
+    // compact the live symbols to the output
+    uint32_t live = 0;
+    for (int i = lo; i < hi; ++i) live += (S[i] != kNone);
+    uint32_t total;
+    uint32_t off = team_exclusive_sum<NT>(live, red, wv, total);
+    for (int i = lo; i < hi; ++i) {
+        const uint32_t s = S[i];
+        if (s != kNone) out[off++] = out_remap ? out_remap[s] : (int32_t)s;
+    }
+    if (tid == 0) *out_len = (int32_t)total;
+}
+
+// Rows of at most CAP bytes, state in LDS.  NT = 64: every wave of the workgroup takes its
+// own row (no workgroup barrier after the set-up); NT = blockDim.x: the workgroup shares a row.
+template <int NT, int TEAMS, int CAP, bool TAB_LDS>
+__global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
+    BpeArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
+    int64_t n_rows, int32_t *__restrict__ tok_tmp, int32_t *__restrict__ lengths)
+{
+    extern __shared__ __align__(16) uint8_t smem[];
+    uint8_t *sp = smem;
+    const uint2 *tab = a.tab;
+    const uint16_t *newsym = a.newsym, *minchild = a.minchild;
+    if (TAB_LDS) {
+        uint2 *t = reinterpret_cast<uint2 *>(sp); sp += (size_t)a.slots * sizeof(uint2);
+        uint16_t *ns = reinterpret_cast<uint16_t *>(sp); sp += (((size_t)a.n_merges * 2 + 15) & ~(size_t)15);
+        uint16_t *mc = reinterpret_cast<uint16_t *>(sp); sp += (((size_t)a.n_merges * 2 + 15) & ~(size_t)15);
+        for (uint32_t i = threadIdx.x; i < a.slots; i += NT * TEAMS) t[i] = a.tab[i];
+        for (int i = threadIdx.x; i < a.n_merges; i += NT * TEAMS) { ns[i] = a.newsym[i]; mc[i] = a.minchild[i]; }
+        tab = t; newsym = ns; minchild = mc;
+    }
+    uint16_t *b2s = reinterpret_cast<uint16_t *>(sp); sp += 512;
+    for (int i = threadIdx.x; i < 256; i += NT * TEAMS) b2s[i] = a.byte_to_sym[i];
+    const int team = threadIdx.x / NT, tid = threadIdx.x % NT;
+    uint32_t *red = reinterpret_cast<uint32_t *>(sp) + team * (4 * (NT / 64)); sp += TEAMS * 4 * (NT / 64) * 4;
+    uint16_t *S = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
+    uint16_t *R = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
+    uint16_t *NX = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
+    uint16_t *PV = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
+    uint8_t *F = sp + (size_t)team * CAP; sp += (size_t)TEAMS * CAP;
+    uint8_t *D = sp + (size_t)team * NT;
+    __syncthreads();
+
+    const uint32_t mask = a.slots - 1;
+    for (int64_t row = (int64_t)blockIdx.x * TEAMS + team; row < n_rows; row += (int64_t)gridDim.x * TEAMS) {
+        const int64_t start = offsets[row];
+        const int64_t len = offsets[row + 1] - start;
+        if (len > CAP) continue;                 // handled by the long-row kernel
+        if (len <= 0) { if (tid == 0) lengths[row] = 0; continue; }
+        bpe_row<NT, uint16_t>(tab, mask, a.shift, newsym, minchild, b2s, a.out_remap, bytes + start,
+                              (int)len, S, R, NX, PV, F, D, red, tid, tok_tmp + start, lengths + row);
+        team_sync<NT>();
+    }
+}
+
+// Rows longer than min_len: one workgroup per row, state in global scratch (13 bytes / base).
+template <int NT>
+__global__ __launch_bounds__(NT) void bpe_long_kernel(
+    BpeArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
+    int64_t n_rows, int64_t min_len, uint8_t *__restrict__ scratch, int64_t scratch_stride,
+    int32_t *__restrict__ tok_tmp, int32_t *__restrict__ lengths)
+{
+    __shared__ uint32_t red[4 * (NT / 64)];
+    __shared__ uint8_t D[NT];
+    __shared__ uint16_t b2s[256];
+    for (int i = threadIdx.x; i < 256; i += NT) b2s[i] = a.byte_to_sym[i];
+    __syncthreads();
+    // each workgroup owns one slab of scratch, sized for the longest row
+    uint8_t *slab = scratch + (size_t)blockIdx.x * (size_t)scratch_stride;
+    const uint32_t mask = a.slots - 1;
+    for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
+        const int64_t start = offsets[row];
+        const int64_t len = offsets[row + 1] - start;
+        if (len <= min_len) continue;
+        const size_t n = ((size_t)len + 7) & ~(size_t)7;
+        uint32_t *NX = reinterpret_cast<uint32_t *>(slab);
+        uint32_t *PV = NX + n;
+        uint16_t *S = reinterpret_cast<uint16_t *>(PV + n);
+        uint16_t *R = S + n;
+        uint8_t *F = reinterpret_cast<uint8_t *>(R + n);
+        bpe_row<NT, uint32_t>(a.tab, mask, a.shift, a.newsym, a.minchild, b2s, a.out_remap,
+                              bytes + start, (int)len, S, R, NX, PV, F, D, red, threadIdx.x,
+                              tok_tmp + start, lengths + row);
+        __syncthreads();
+    }
+}
+
+constexpr int kLdsCap = 4096;            // longest row the LDS kernels take
+constexpr int kLongThreads = 1024;
+constexpr int kLongGrid = 512;           // slabs of scratch for the long-row kernel
+
+static size_t long_slab_bytes(int64_t max_len)
+{
+    const size_t n = ((size_t)max_len + 7) & ~(size_t)7;
+    return ((n * 13) + 255) & ~(size_t)255;
+}
+
+}  // namespace dnatok
+
+using namespace dnatok;
+
+extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_t *pair_a_h,
+                                       const int32_t *pair_b_h, const int32_t *new_id_h,
+                                       int32_t n_merges, int32_t n_symbols,
+                                       const int32_t *out_remap_h, dnatok_bpe_t **out)
+{
+    DNATOK_REQUIRE(byte_to_id_h && out && (n_merges == 0 || (pair_a_h && pair_b_h && new_id_h)),
+                   DNATOK_E_INVALID, "dnatok_bpe_table_create: null argument");
+    DNATOK_REQUIRE(n_merges >= 0 && n_symbols > 0, DNATOK_E_INVALID,
+                   "dnatok_bpe_table_create: bad sizes");
+    DNATOK_REQUIRE(n_symbols <= 65535 && n_merges <= 65534, DNATOK_E_TOO_LARGE,
+                   "dnatok_bpe_table_create: %d symbols / %d merges exceed the 16-bit state",
+                   n_symbols, n_merges);
+    for (int i = 0; i < 256; ++i)
+        DNATOK_REQUIRE(byte_to_id_h[i] >= 0 && byte_to_id_h[i] < n_symbols, DNATOK_E_INVALID,
+                       "dnatok_bpe_table_create: byte_to_id[%d] out of range", i);
+    uint32_t slots = 64, shift = 26;
+    while (slots < (uint32_t)n_merges * 2u + 2u) { slots <<= 1; --shift; }
+    std::vector<uint2> tab(slots, uint2{kEmptyKey, kNone});
+    std::vector<uint16_t> newsym(n_merges > 0 ? n_merges : 1), minchild(n_merges > 0 ? n_merges : 1, (uint16_t)kNone);
+    std::vector<uint32_t> first_use(n_symbols, 0xFFFFFFFFu);   // lowest rank using a symbol
+    for (int32_t i = 0; i < n_merges; ++i) {
+        const int32_t pa = pair_a_h[i], pb = pair_b_h[i], nid = new_id_h[i];
+        DNATOK_REQUIRE(pa >= 0 && pa < n_symbols && pb >= 0 && pb < n_symbols && nid >= 0 && nid < n_symbols,
+                       DNATOK_E_INVALID, "dnatok_bpe_table_create: merge %d has an id out of range", i);
+        newsym[i] = (uint16_t)nid;
+        const uint32_t key = ((uint32_t)pa << 16) | (uint32_t)pb;
+        uint32_t h = pair_hash(key, shift);
+        bool dup = false;
+        while (tab[h].x != kEmptyKey) {
+            if (tab[h].x == key) { dup = true; break; }
+            h = (h + 1) & (slots - 1);
+        }
+        if (dup) continue;                      // a repeated pair keeps its first rank
+        tab[h] = uint2{key, (uint32_t)i};
+        if (first_use[pa] == 0xFFFFFFFFu) first_use[pa] = (uint32_t)i;
+        if (first_use[pb] == 0xFFFFFFFFu) first_use[pb] = (uint32_t)i;
+    }
+    int monotone = 1;
+    for (int32_t i = 0; i < n_merges; ++i) {
+        const uint32_t fu = first_use[new_id_h[i]];
+        minchild[i] = (uint16_t)(fu == 0xFFFFFFFFu ? kNone : fu);
+        if (fu <= (uint32_t)i) monotone = 0;
+    }
+    std::vector<uint16_t> b2s(256);
+    for (int i = 0; i < 256; ++i) b2s[i] = (uint16_t)byte_to_id_h[i];
+
+    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    const size_t o_tab = 0;
+    const size_t o_new = up(o_tab + (size_t)slots * sizeof(uint2));
+    const size_t o_mc = up(o_new + newsym.size() * 2);
+    const size_t o_b2s = up(o_mc + minchild.size() * 2);
+    const size_t o_remap = up(o_b2s + 512);
+    const size_t total = up(o_remap + (out_remap_h ? (size_t)n_symbols * 4 : 0)) + 256;
+    std::vector<uint8_t> host(total, 0);
+    memcpy(&host[o_tab], tab.data(), (size_t)slots * sizeof(uint2));
+    memcpy(&host[o_new], newsym.data(), newsym.size() * 2);
+    memcpy(&host[o_mc], minchild.data(), minchild.size() * 2);
+    memcpy(&host[o_b2s], b2s.data(), 512);
+    if (out_remap_h) memcpy(&host[o_remap], out_remap_h, (size_t)n_symbols * 4);
+    void *blob = nullptr;
+    hipError_t e = hipMalloc(&blob, total);
+    if (e == hipSuccess) e = hipMemcpy(blob, host.data(), total, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        set_error("dnatok_bpe_table_create: %s", hipGetErrorString(e));
+        if (blob) (void)hipFree(blob);
+        return DNATOK_E_HIP;
+    }
+    dnatok_bpe_table *t = new dnatok_bpe_table();
+    uint8_t *b = (uint8_t *)blob;
+    t->n_merges = n_merges; t->n_symbols = n_symbols; t->slots = slots; t->shift = shift;
+    t->monotone = monotone; t->blob = blob;
+    t->tab = (uint2 *)(b + o_tab);
+    t->newsym = (uint16_t *)(b + o_new);
+    t->minchild = (uint16_t *)(b + o_mc);
+    t->byte_to_sym = (uint16_t *)(b + o_b2s);
+    t->out_remap = out_remap_h ? (int32_t *)(b + o_remap) : nullptr;
+    *out = t;
+    return DNATOK_OK;
+}
+
+extern "C" void dnatok_bpe_table_destroy(dnatok_bpe_t *t)
+{
+    if (!t) return;
+    if (t->blob) (void)hipFree(t->blob);
+    delete t;
+}
+
+extern "C" size_t dnatok_bpe_scratch_bytes(const dnatok_bpe_t *t, int64_t n_rows, int64_t max_len,
+                                           int64_t total)
+{
+    (void)t; (void)total;
+    if (max_len <= kLdsCap || n_rows <= 0) return 256;
+    const int64_t slabs = n_rows < kLongGrid ? n_rows : kLongGrid;
+    return (size_t)slabs * long_slab_bytes(max_len);
+}
+
+namespace {
+
+template <int NT, int TEAMS, int CAP, bool TAB_LDS>
+int launch_lds(const dnatok_bpe_t *t, const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets,
+               int64_t n_rows, int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
+{
+    size_t lds = 512 + (size_t)TEAMS * 4 * (NT / 64) * 4 + (size_t)TEAMS * CAP * 9 + (size_t)TEAMS * NT + 64;
+    if (TAB_LDS)
+        lds += (size_t)t->slots * sizeof(uint2) + 2 * ((((size_t)t->n_merges * 2) + 15) & ~(size_t)15);
+    auto kern = bpe_lds_kernel<NT, TEAMS, CAP, TAB_LDS>;
+    DNATOK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    int64_t grid = (n_rows + TEAMS - 1) / TEAMS;
+    const int64_t cap = TAB_LDS ? 256 * 2 : 256 * 8;   // persistent workgroups when the table is staged
+    if (grid > cap) grid = cap;
+    kern<<<(int)grid, NT * TEAMS, lds, s>>>(a, bytes, offsets, n_rows, tok_tmp, lengths);
+    DNATOK_HIP_TRY(hipGetLastError());
+    return DNATOK_OK;
+}
+
+}  // namespace
+
+extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets,
+                                 int64_t n_rows, int64_t max_len, int64_t total, void *scratch,
+                                 size_t scratch_bytes, int32_t *tok_tmp, int32_t *lengths, void *stream)
+{
+    DNATOK_REQUIRE(t && offsets && lengths, DNATOK_E_INVALID, "dnatok_bpe_encode: null argument");
+    DNATOK_REQUIRE(n_rows >= 0 && max_len >= 0 && total >= 0, DNATOK_E_INVALID,
+                   "dnatok_bpe_encode: negative size");
+    DNATOK_REQUIRE(max_len < (int64_t)1 << 31, DNATOK_E_TOO_LARGE,
+                   "dnatok_bpe_encode: rows of 2^31 bytes or more are not supported");
+    if (n_rows == 0) return DNATOK_OK;
+    DNATOK_REQUIRE(total == 0 || (bytes && tok_tmp), DNATOK_E_INVALID, "dnatok_bpe_encode: null buffer");
+    hipStream_t s = (hipStream_t)stream;
+    BpeArgs a{t->tab, t->newsym, t->minchild, t->byte_to_sym, t->out_remap, t->slots, t->shift, t->n_merges};
+
+    static const char *variant_env = getenv("DNATOK_BPE_VARIANT");
+    const int variant = variant_env ? atoi(variant_env) : 0;
+    const size_t tab_lds_bytes = (size_t)t->slots * sizeof(uint2) + 4 * (size_t)t->n_merges;
+    const bool tab_fits = tab_lds_bytes <= 96 * 1024;
+    int rc;
+    switch (variant) {
+        case 1:  rc = launch_lds<256, 1, kLdsCap, false>(t, a, bytes, offsets, n_rows, tok_tmp, lengths, s); break;
+        case 2:  rc = tab_fits ? launch_lds<256, 1, kLdsCap, true>(t, a, bytes, offsets, n_rows, tok_tmp, lengths, s)
+                               : launch_lds<256, 1, kLdsCap, false>(t, a, bytes, offsets, n_rows, tok_tmp, lengths, s);
+                 break;
+        case 3:  rc = launch_lds<64, 4, kLdsCap, false>(t, a, bytes, offsets, n_rows, tok_tmp, lengths, s); break;
+        case 4:  rc = launch_lds<1024, 1, kLdsCap, false>(t, a, bytes, offsets, n_rows, tok_tmp, lengths, s); break;
+        default: rc = launch_lds<256, 1, kLdsCap, false>(t, a, bytes, offsets, n_rows, tok_tmp, lengths, s); break;
+    }
+    if (rc) return rc;
+    if (max_len > kLdsCap) {
+        const int64_t slabs = n_rows < kLongGrid ? n_rows : kLongGrid;
+        const size_t slab = long_slab_bytes(max_len);
+        DNATOK_REQUIRE(scratch && scratch_bytes >= (size_t)slabs * slab, DNATOK_E_SCRATCH,
+                       "dnatok_bpe_encode: scratch holds %zu bytes, %zu needed", scratch_bytes,
+                       (size_t)slabs * slab);
+        bpe_long_kernel<kLongThreads><<<(int)slabs, kLongThreads, 0, s>>>(
+            a, bytes, offsets, n_rows, (int64_t)kLdsCap, (uint8_t *)scratch, (int64_t)slab, tok_tmp, lengths);
+        DNATOK_HIP_TRY(hipGetLastError());
+    }
+    return DNATOK_OK;
+}

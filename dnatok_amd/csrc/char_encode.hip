@@ -1,0 +1,263 @@
+// Single-nucleotide encoder: ids = table[byte], with padding and attention mask.
+//
+// HBM-bound streaming map: 1 byte read and 5 bytes written per base (int32 id + uint8 mask).
+// The 256-entry table (and the optional first-column table) sit in LDS; DNA input touches
+// five entries, so lanes either broadcast or hit distinct banks.  Each lane reads 4 bytes
+// per step as one dword (a wave covers 256 contiguous bytes) and writes its 4 ids as one
+// 16-byte store (a wave covers 1 KiB contiguous) and its 4 mask bytes as one dword.
+#include "common.hpp"
+
+#include <string.h>
+
+namespace dnatok {
+
+struct CharTableDev {
+    int32_t lut[256];
+    int32_t start[256];
+};
+
+}  // namespace dnatok
+
+struct dnatok_char_table {
+    dnatok::CharTableDev *dev;   // device copy
+    int32_t pad_id;
+    int has_start;
+};
+
+namespace dnatok {
+
+constexpr int kCharThreads = 256;
+constexpr int kCharSteps = 4;                                   // dwords per lane per tile
+constexpr int kCharTile = kCharThreads * 4 * kCharSteps;        // 4096 bases per tile
+
+typedef int32_t int4v __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int4v lookup4(const int32_t *lut, uint32_t w)
+{
+    int4v v;
+    v.x = lut[w & 255u];
+    v.y = lut[(w >> 8) & 255u];
+    v.z = lut[(w >> 16) & 255u];
+    v.w = lut[w >> 24];
+    return v;
+}
+
+// Flat stream; requires bytes 4-byte aligned, ids 16-byte aligned, mask 4-byte aligned.
+template <bool HAS_MASK, bool HAS_START>
+__global__ __launch_bounds__(kCharThreads) void char_packed_kernel(
+    const uint8_t *__restrict__ bytes, int64_t total, int64_t row_len,
+    const CharTableDev *__restrict__ tab, int32_t *__restrict__ ids, uint8_t *__restrict__ mask)
+{
+    __shared__ int32_t lut[256];
+    __shared__ int32_t start[256];
+    lut[threadIdx.x] = tab->lut[threadIdx.x];
+    if (HAS_START) start[threadIdx.x] = tab->start[threadIdx.x];
+    __syncthreads();
+
+    const int64_t n_tiles = (total + kCharTile - 1) / kCharTile;
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int64_t base = tile * kCharTile + (int64_t)threadIdx.x * 4;
+        uint32_t w[kCharSteps];
+        if (tile * kCharTile + kCharTile <= total) {
+#pragma unroll
+            for (int s = 0; s < kCharSteps; ++s)
+                w[s] = __builtin_nontemporal_load(
+                    reinterpret_cast<const uint32_t *>(bytes + base + s * (kCharThreads * 4)));
+#pragma unroll
+            for (int s = 0; s < kCharSteps; ++s) {
+                const int64_t i = base + s * (kCharThreads * 4);
+                int4v v = lookup4(lut, w[s]);
+                if (HAS_START) {
+                    // rare path (separate first-column table): test each position exactly
+                    const int64_t r = i % row_len;
+                    if (r == 0) v.x = start[w[s] & 255u];
+                    if ((r + 1) % row_len == 0) v.y = start[(w[s] >> 8) & 255u];
+                    if ((r + 2) % row_len == 0) v.z = start[(w[s] >> 16) & 255u];
+                    if ((r + 3) % row_len == 0) v.w = start[w[s] >> 24];
+                }
+                __builtin_nontemporal_store(v, reinterpret_cast<int4v *>(ids + i));
+                if (HAS_MASK)
+                    __builtin_nontemporal_store(0x01010101u, reinterpret_cast<uint32_t *>(mask + i));
+            }
+        } else {
+            // last, partial tile: position by position
+            for (int s = 0; s < kCharSteps; ++s) {
+                for (int k = 0; k < 4; ++k) {
+                    const int64_t i = base + s * (kCharThreads * 4) + k;
+                    if (i < total) {
+                        const uint8_t c = bytes[i];
+                        const bool first = HAS_START && (i % row_len == 0);
+                        ids[i] = first ? start[c] : lut[c];
+                        if (HAS_MASK) mask[i] = 1;
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Ragged rows to a padded [n_rows, t_out] matrix.  One tile = 1024 output columns of one row.
+// ALIGNED: t_out % 4 == 0 and ids / mask bases are 16- / 4-byte aligned, so each lane stores
+// its 4 columns with one 16-byte and one 4-byte store.
+template <bool HAS_MASK, bool HAS_START, bool ALIGNED>
+__global__ __launch_bounds__(kCharThreads) void char_padded_kernel(
+    const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets, int64_t n_rows,
+    int64_t t_out, int64_t tiles_per_row, int pad_left, int32_t pad_id,
+    const CharTableDev *__restrict__ tab, int32_t *__restrict__ ids, uint8_t *__restrict__ mask)
+{
+    __shared__ int32_t lut[256];
+    __shared__ int32_t start[256];
+    lut[threadIdx.x] = tab->lut[threadIdx.x];
+    if (HAS_START) start[threadIdx.x] = tab->start[threadIdx.x];
+    __syncthreads();
+
+    const int64_t n_tiles = n_rows * tiles_per_row;
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int64_t b = tile / tiles_per_row;
+        const int64_t col0 = (tile - b * tiles_per_row) * (kCharThreads * 4) + (int64_t)threadIdx.x * 4;
+        if (col0 >= t_out) continue;
+        const int64_t row_start = offsets[b];
+        int64_t len = offsets[b + 1] - row_start;
+        if (len > t_out) len = t_out;
+        const int64_t shift = pad_left ? (t_out - len) : 0;   // first real column
+        const uint8_t *src = bytes + row_start - shift;       // src[col] for shift <= col < shift+len
+        int32_t v[4];
+        uint32_t m = 0;
+        if (col0 >= shift && col0 + 4 <= shift + len) {
+            uint32_t w;
+            memcpy(&w, src + col0, 4);                        // row starts are not aligned
+            v[0] = lut[w & 255u]; v[1] = lut[(w >> 8) & 255u];
+            v[2] = lut[(w >> 16) & 255u]; v[3] = lut[w >> 24];
+            if (HAS_START && col0 == shift) v[0] = start[w & 255u];
+            m = 0x01010101u;
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int64_t c = col0 + k;
+                if (c >= shift && c < shift + len) {
+                    const uint8_t ch = src[c];
+                    v[k] = (HAS_START && c == shift) ? start[ch] : lut[ch];
+                    m |= 1u << (8 * k);
+                } else {
+                    v[k] = pad_id;
+                }
+            }
+        }
+        int32_t *o = ids + b * t_out + col0;
+        if (ALIGNED) {
+            int4v vv = {v[0], v[1], v[2], v[3]};
+            __builtin_nontemporal_store(vv, reinterpret_cast<int4v *>(o));
+            if (HAS_MASK)
+                __builtin_nontemporal_store(m, reinterpret_cast<uint32_t *>(mask + b * t_out + col0));
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                if (col0 + k < t_out) {
+                    o[k] = v[k];
+                    if (HAS_MASK) mask[b * t_out + col0 + k] = (uint8_t)((m >> (8 * k)) & 1u);
+                }
+            }
+        }
+    }
+}
+
+static int grid_for(int64_t n_tiles)
+{
+    // enough workgroups to fill 256 CUs several times over; tiles beyond that are grid-strided
+    const int64_t cap = 256 * 32;
+    return (int)(n_tiles < cap ? (n_tiles > 0 ? n_tiles : 1) : cap);
+}
+
+}  // namespace dnatok
+
+using namespace dnatok;
+
+extern "C" int dnatok_char_table_create(const int32_t *lut_h, const int32_t *start_lut_h,
+                                        int32_t pad_id, dnatok_char_t **out)
+{
+    DNATOK_REQUIRE(lut_h && out, DNATOK_E_INVALID, "dnatok_char_table_create: null argument");
+    CharTableDev h;
+    memcpy(h.lut, lut_h, sizeof(h.lut));
+    memcpy(h.start, start_lut_h ? start_lut_h : lut_h, sizeof(h.start));
+    dnatok_char_table *t = new dnatok_char_table();
+    t->pad_id = pad_id;
+    t->has_start = start_lut_h != nullptr;
+    t->dev = nullptr;
+    hipError_t e = hipMalloc((void **)&t->dev, sizeof(CharTableDev));
+    if (e == hipSuccess) e = hipMemcpy(t->dev, &h, sizeof(h), hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        set_error("dnatok_char_table_create: %s", hipGetErrorString(e));
+        if (t->dev) (void)hipFree(t->dev);
+        delete t;
+        return DNATOK_E_HIP;
+    }
+    *out = t;
+    return DNATOK_OK;
+}
+
+extern "C" void dnatok_char_table_destroy(dnatok_char_t *t)
+{
+    if (!t) return;
+    if (t->dev) (void)hipFree(t->dev);
+    delete t;
+}
+
+extern "C" int dnatok_char_encode_packed(const dnatok_char_t *t, const uint8_t *bytes, int64_t total,
+                                         int64_t row_len, int32_t *ids, uint8_t *mask, void *stream)
+{
+    DNATOK_REQUIRE(t && ids, DNATOK_E_INVALID, "dnatok_char_encode_packed: null argument");
+    DNATOK_REQUIRE(total >= 0 && row_len >= 0, DNATOK_E_INVALID,
+                   "dnatok_char_encode_packed: negative size");
+    if (total == 0) return DNATOK_OK;
+    DNATOK_REQUIRE(bytes, DNATOK_E_INVALID, "dnatok_char_encode_packed: null input");
+    DNATOK_REQUIRE(((uintptr_t)bytes & 3) == 0 && ((uintptr_t)ids & 15) == 0 &&
+                       ((uintptr_t)mask & 3) == 0,
+                   DNATOK_E_INVALID,
+                   "dnatok_char_encode_packed: bytes/mask must be 4-byte and ids 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t n_tiles = (total + kCharTile - 1) / kCharTile;
+    const int grid = grid_for(n_tiles);
+    const bool use_start = t->has_start && row_len > 0;
+    if (mask) {
+        if (use_start)
+            char_packed_kernel<true, true><<<grid, kCharThreads, 0, s>>>(bytes, total, row_len, t->dev, ids, mask);
+        else
+            char_packed_kernel<true, false><<<grid, kCharThreads, 0, s>>>(bytes, total, 1, t->dev, ids, mask);
+    } else {
+        if (use_start)
+            char_packed_kernel<false, true><<<grid, kCharThreads, 0, s>>>(bytes, total, row_len, t->dev, ids, mask);
+        else
+            char_packed_kernel<false, false><<<grid, kCharThreads, 0, s>>>(bytes, total, 1, t->dev, ids, mask);
+    }
+    DNATOK_HIP_TRY(hipGetLastError());
+    return DNATOK_OK;
+}
+
+extern "C" int dnatok_char_encode_padded(const dnatok_char_t *t, const uint8_t *bytes,
+                                         const int64_t *offsets, int64_t n_rows, int64_t t_out,
+                                         int pad_left, int32_t *ids, uint8_t *mask, void *stream)
+{
+    DNATOK_REQUIRE(t && offsets && ids, DNATOK_E_INVALID, "dnatok_char_encode_padded: null argument");
+    DNATOK_REQUIRE(n_rows >= 0 && t_out >= 0, DNATOK_E_INVALID,
+                   "dnatok_char_encode_padded: negative size");
+    if (n_rows == 0 || t_out == 0) return DNATOK_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t tiles_per_row = (t_out + kCharThreads * 4 - 1) / (kCharThreads * 4);
+    const int grid = grid_for(n_rows * tiles_per_row);
+    const bool aligned = (t_out % 4 == 0) && ((uintptr_t)ids & 15) == 0 && ((uintptr_t)mask & 3) == 0;
+    const bool hs = t->has_start;
+#define LAUNCH(M, S, A)                                                                          \
+    char_padded_kernel<M, S, A><<<grid, kCharThreads, 0, s>>>(bytes, offsets, n_rows, t_out,      \
+                                                              tiles_per_row, pad_left, t->pad_id, \
+                                                              t->dev, ids, mask)
+    if (mask) {
+        if (hs) { if (aligned) LAUNCH(true, true, true); else LAUNCH(true, true, false); }
+        else    { if (aligned) LAUNCH(true, false, true); else LAUNCH(true, false, false); }
+    } else {
+        if (hs) { if (aligned) LAUNCH(false, true, true); else LAUNCH(false, true, false); }
+        else    { if (aligned) LAUNCH(false, false, true); else LAUNCH(false, false, false); }
+    }
+#undef LAUNCH
+    DNATOK_HIP_TRY(hipGetLastError());
+    return DNATOK_OK;
+}

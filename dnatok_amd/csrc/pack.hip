@@ -1,0 +1,148 @@
+// Ragged-batch packer: per-row token runs -> packed ids + offsets (+mask), or a padded
+// [rows, stride] matrix + mask, entirely on the device.  The id remap (kernel id -> tokenizer
+// id) is fused into the copy.  One wave copies one row, 64 tokens per step.
+#include "common.hpp"
+
+namespace dnatok {
+
+int launch_pad_to_max(int32_t *ids, uint8_t *mask, const int32_t *lengths, int64_t n_rows,
+                      int64_t t_cap, const int32_t *max_len, int32_t pad_id, hipStream_t s);
+int launch_zero_i32(int32_t *p, hipStream_t s);
+
+constexpr int kScanThreads = 1024;
+
+// out_offsets[b] = sum of max(lengths[0..b), 0); single workgroup, 1024 rows per step.
+__global__ __launch_bounds__(kScanThreads) void scan_lengths_kernel(
+    const int32_t *__restrict__ lengths, int64_t n_rows, int64_t *__restrict__ out_offsets)
+{
+    __shared__ uint32_t wave_tot[kScanThreads / 64];
+    __shared__ int64_t carry;
+    if (threadIdx.x == 0) carry = 0;
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    for (int64_t base = 0; base < n_rows; base += kScanThreads) {
+        const int64_t i = base + threadIdx.x;
+        int32_t v = (i < n_rows) ? lengths[i] : 0;
+        if (v < 0) v = 0;
+        const uint32_t inc = wave_inclusive_sum_u32((uint32_t)v);
+        if (lane == 63) wave_tot[wv] = inc;
+        __syncthreads();
+        uint32_t before = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < kScanThreads / 64; ++w) {
+            const uint32_t t = wave_tot[w];
+            if (w < wv) before += t;
+            total += t;
+        }
+        const int64_t c = carry;
+        if (i < n_rows) out_offsets[i] = c + before + inc - (uint32_t)v;
+        __syncthreads();
+        if (threadIdx.x == 0) carry = c + total;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out_offsets[n_rows] = carry;
+}
+
+__global__ __launch_bounds__(256) void pack_copy_kernel(
+    const int32_t *__restrict__ tok_tmp, const int64_t *__restrict__ in_offsets,
+    const int32_t *__restrict__ lengths, int64_t n_rows, const int32_t *__restrict__ remap,
+    const int64_t *__restrict__ out_offsets, int32_t *__restrict__ ids_out,
+    uint8_t *__restrict__ mask_out)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t n_waves = (int64_t)gridDim.x * 4;
+    for (int64_t row = wave; row < n_rows; row += n_waves) {
+        const int64_t len = lengths[row];
+        const int32_t *src = tok_tmp + in_offsets[row];
+        const int64_t o = out_offsets[row];
+        for (int64_t j = lane; j < len; j += 64) {
+            int32_t v = src[j];
+            if (remap) v = remap[v];
+            ids_out[o + j] = v;
+            if (mask_out) mask_out[o + j] = 1;
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void pad_rows_kernel(
+    const int32_t *__restrict__ tok_tmp, const int64_t *__restrict__ in_offsets,
+    const int32_t *__restrict__ lengths, int64_t n_rows, const int32_t *__restrict__ remap,
+    int32_t pad_id, int64_t t_cap, int64_t fill_to, int32_t *__restrict__ ids,
+    uint8_t *__restrict__ mask, int32_t *__restrict__ max_len)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t n_waves = (int64_t)gridDim.x * 4;
+    for (int64_t row = wave; row < n_rows; row += n_waves) {
+        int64_t len = lengths[row];
+        if (len < 0) len = 0;
+        if (len > t_cap) len = t_cap;
+        const int32_t *src = tok_tmp + in_offsets[row];
+        int32_t *o = ids + row * t_cap;
+        uint8_t *m = mask ? mask + row * t_cap : nullptr;
+        for (int64_t j = lane; j < len; j += 64) {
+            int32_t v = src[j];
+            if (remap) v = remap[v];
+            o[j] = v;
+            if (m) m[j] = 1;
+        }
+        for (int64_t j = len + lane; j < fill_to; j += 64) {
+            o[j] = pad_id;
+            if (m) m[j] = 0;
+        }
+        if (max_len && lane == 0) atomicMax(max_len, (int32_t)len);
+    }
+}
+
+static int wave_grid(int64_t n_rows)
+{
+    int64_t g = (n_rows + 3) / 4;
+    if (g > 256 * 16) g = 256 * 16;
+    return (int)(g < 1 ? 1 : g);
+}
+
+}  // namespace dnatok
+
+using namespace dnatok;
+
+extern "C" int dnatok_pack_ragged(const int32_t *tok_tmp, const int64_t *in_offsets,
+                                  const int32_t *lengths, int64_t n_rows, const int32_t *remap,
+                                  int32_t *ids_out, int64_t *out_offsets, uint8_t *mask_out,
+                                  void *stream)
+{
+    DNATOK_REQUIRE(in_offsets && lengths && out_offsets, DNATOK_E_INVALID,
+                   "dnatok_pack_ragged: null argument");
+    DNATOK_REQUIRE(n_rows >= 0, DNATOK_E_INVALID, "dnatok_pack_ragged: negative row count");
+    hipStream_t s = (hipStream_t)stream;
+    scan_lengths_kernel<<<1, kScanThreads, 0, s>>>(lengths, n_rows, out_offsets);
+    DNATOK_HIP_TRY(hipGetLastError());
+    if (n_rows == 0) return DNATOK_OK;
+    DNATOK_REQUIRE(tok_tmp && ids_out, DNATOK_E_INVALID, "dnatok_pack_ragged: null buffer");
+    pack_copy_kernel<<<wave_grid(n_rows), 256, 0, s>>>(tok_tmp, in_offsets, lengths, n_rows, remap,
+                                                       out_offsets, ids_out, mask_out);
+    DNATOK_HIP_TRY(hipGetLastError());
+    return DNATOK_OK;
+}
+
+extern "C" int dnatok_pad_rows(const int32_t *tok_tmp, const int64_t *in_offsets,
+                               const int32_t *lengths, int64_t n_rows, const int32_t *remap,
+                               int32_t pad_id, int64_t t_cap, int64_t fill_to, int32_t *ids,
+                               uint8_t *mask, int32_t *max_len, void *stream)
+{
+    DNATOK_REQUIRE(in_offsets && lengths && ids, DNATOK_E_INVALID, "dnatok_pad_rows: null argument");
+    DNATOK_REQUIRE(n_rows >= 0 && t_cap >= 0 && fill_to >= 0 && fill_to <= t_cap, DNATOK_E_INVALID,
+                   "dnatok_pad_rows: need 0 <= fill_to <= t_cap");
+    DNATOK_REQUIRE(fill_to > 0 || max_len, DNATOK_E_INVALID, "dnatok_pad_rows: fill_to = 0 needs max_len");
+    if (n_rows == 0) return DNATOK_OK;
+    hipStream_t s = (hipStream_t)stream;
+    if (max_len) {
+        int rc = launch_zero_i32(max_len, s);
+        if (rc) return rc;
+    }
+    pad_rows_kernel<<<wave_grid(n_rows), 256, 0, s>>>(tok_tmp, in_offsets, lengths, n_rows, remap,
+                                                      pad_id, t_cap, fill_to, ids, mask, max_len);
+    DNATOK_HIP_TRY(hipGetLastError());
+    if (fill_to == 0) return launch_pad_to_max(ids, mask, lengths, n_rows, t_cap, max_len, pad_id, s);
+    return DNATOK_OK;
+}

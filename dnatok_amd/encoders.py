@@ -1,0 +1,241 @@
+"""Device-side encoders: thin torch-tensor wrappers over the C ABI.
+
+torch is used for device memory and the current stream only; every encode is a
+call into libdnatok_hip.so on ``torch.cuda.current_stream()``.  Inputs are
+device uint8 buffers plus int64 row offsets (the layout
+``workloads.Batch`` / ``bytes_from_strings`` produce); outputs are int32 ids
+and uint8 masks that stay on the device.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from . import _lib
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _np_ptr(a: Optional[np.ndarray]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if a is None else a.ctypes.data)
+
+
+def _require_cuda(t: torch.Tensor, dtype: torch.dtype, name: str) -> None:
+    if not t.is_cuda or t.dtype != dtype or not t.is_contiguous():
+        raise ValueError(f"{name} must be a contiguous {dtype} tensor on the GPU")
+
+
+def bytes_from_strings(seqs: Sequence[str], device="cuda") -> Tuple[torch.Tensor, torch.Tensor, np.ndarray]:
+    """Concatenate ASCII strings into one device uint8 buffer + device int64 offsets.
+
+    Returns (data, offsets, host_lengths).  One join and one H2D copy per call
+    (reference: DNATokBPE::tokenize_batch, src/dnatok_bpe_kernel/dnatok_bpe.cu:872-887).
+    """
+    lens = np.fromiter((len(s) for s in seqs), dtype=np.int64, count=len(seqs))
+    offsets = np.zeros(len(seqs) + 1, dtype=np.int64)
+    np.cumsum(lens, out=offsets[1:])
+    buf = "".join(seqs).encode("ascii", errors="replace")
+    host = torch.frombuffer(bytearray(buf), dtype=torch.uint8) if buf else torch.empty(0, dtype=torch.uint8)
+    data = host.to(device)
+    return data, torch.from_numpy(offsets).to(device), lens
+
+
+class CharEncoder:
+    """ids = table[byte] with padding and mask (C ABI: dnatok_char_*)."""
+
+    def __init__(self, lut, pad_id: int, start_lut=None):
+        self.lut = np.ascontiguousarray(lut, dtype=np.int32)
+        if self.lut.shape != (256,):
+            raise ValueError("lut must have 256 entries")
+        self.start_lut = None if start_lut is None else np.ascontiguousarray(start_lut, dtype=np.int32)
+        self.pad_id = int(pad_id)
+        h = ctypes.c_void_p()
+        _lib.check(_lib.lib().dnatok_char_table_create(_np_ptr(self.lut), _np_ptr(self.start_lut),
+                                                       self.pad_id, ctypes.byref(h)),
+                   "dnatok_char_table_create")
+        self._h = h
+
+    def __del__(self):
+        h = getattr(self, "_h", None)
+        if h:
+            try:
+                _lib.lib().dnatok_char_table_destroy(h)
+            except Exception:
+                pass
+
+    def encode_padded(self, data: torch.Tensor, offsets: torch.Tensor, t_out: int, *,
+                      pad_left: bool = False, want_mask: bool = True,
+                      ids: Optional[torch.Tensor] = None, mask: Optional[torch.Tensor] = None):
+        _require_cuda(data, torch.uint8, "data")
+        _require_cuda(offsets, torch.int64, "offsets")
+        n_rows = offsets.numel() - 1
+        if ids is None:
+            ids = torch.empty((n_rows, t_out), dtype=torch.int32, device=data.device)
+        if want_mask and mask is None:
+            mask = torch.empty((n_rows, t_out), dtype=torch.uint8, device=data.device)
+        _lib.check(_lib.lib().dnatok_char_encode_padded(self._h, _ptr(data), _ptr(offsets), n_rows,
+                                                        int(t_out), int(pad_left), _ptr(ids),
+                                                        _ptr(mask if want_mask else None), _stream()),
+                   "dnatok_char_encode_padded")
+        return ids, (mask if want_mask else None)
+
+    def encode_packed(self, data: torch.Tensor, *, row_len: int = 0, want_mask: bool = False,
+                      ids: Optional[torch.Tensor] = None, mask: Optional[torch.Tensor] = None):
+        _require_cuda(data, torch.uint8, "data")
+        total = data.numel()
+        if ids is None:
+            ids = torch.empty(total, dtype=torch.int32, device=data.device)
+        if want_mask and mask is None:
+            mask = torch.empty(total, dtype=torch.uint8, device=data.device)
+        _lib.check(_lib.lib().dnatok_char_encode_packed(self._h, _ptr(data), total, int(row_len),
+                                                        _ptr(ids), _ptr(mask if want_mask else None),
+                                                        _stream()),
+                   "dnatok_char_encode_packed")
+        return ids, (mask if want_mask else None)
+
+
+class KmerEncoder:
+    """Grid-aligned k-mer windows with per-window fallback (C ABI: dnatok_kmer_*)."""
+
+    def __init__(self, k: int, digit, kmer_lut, single, pad_id: int, missing_id: int,
+                 exp_off=None, exp_len=None, exp_flat=None):
+        self.k = int(k)
+        self.digit = np.ascontiguousarray(digit, dtype=np.int8)
+        self.kmer_lut = np.ascontiguousarray(kmer_lut, dtype=np.int32)
+        self.single = np.ascontiguousarray(single, dtype=np.int32)
+        if self.kmer_lut.size != 5 ** self.k:
+            raise ValueError("kmer_lut must have 5**k entries")
+        self.pad_id = int(pad_id)
+        self.exp_off = None if exp_off is None else np.ascontiguousarray(exp_off, dtype=np.int32)
+        self.exp_len = None if exp_len is None else np.ascontiguousarray(exp_len, dtype=np.int32)
+        self.exp_flat = None if exp_flat is None else np.ascontiguousarray(exp_flat, dtype=np.int32)
+        n_flat = 0 if self.exp_flat is None else int(self.exp_flat.size)
+        h = ctypes.c_void_p()
+        _lib.check(_lib.lib().dnatok_kmer_table_create(
+            self.k, _np_ptr(self.digit), _np_ptr(self.kmer_lut), _np_ptr(self.exp_off),
+            _np_ptr(self.exp_len), _np_ptr(self.exp_flat), n_flat, _np_ptr(self.single),
+            self.pad_id, int(missing_id), ctypes.byref(h)), "dnatok_kmer_table_create")
+        self._h = h
+
+    def __del__(self):
+        h = getattr(self, "_h", None)
+        if h:
+            try:
+                _lib.lib().dnatok_kmer_table_destroy(h)
+            except Exception:
+                pass
+
+    def encode_padded(self, data: torch.Tensor, offsets: torch.Tensor, t_cap: int, *,
+                      fill_to: int = 0, want_mask: bool = True, out=None):
+        """Returns (ids[B, t_cap], mask, lengths[B], status[B], max_len[1]); with fill_to = 0 the
+        rows are padded to the device-side maximum, view ``ids[:, :max_len]``."""
+        _require_cuda(data, torch.uint8, "data")
+        _require_cuda(offsets, torch.int64, "offsets")
+        n_rows = offsets.numel() - 1
+        dev = data.device
+        if out is None:
+            ids = torch.empty((n_rows, t_cap), dtype=torch.int32, device=dev)
+            mask = torch.empty((n_rows, t_cap), dtype=torch.uint8, device=dev) if want_mask else None
+            lengths = torch.empty(n_rows, dtype=torch.int32, device=dev)
+            status = torch.empty(n_rows, dtype=torch.int32, device=dev)
+            max_len = torch.empty(1, dtype=torch.int32, device=dev)
+        else:
+            ids, mask, lengths, status, max_len = out
+        _lib.check(_lib.lib().dnatok_kmer_encode_padded(
+            self._h, _ptr(data), _ptr(offsets), n_rows, int(t_cap), int(fill_to), _ptr(ids),
+            _ptr(mask), _ptr(lengths), _ptr(status), _ptr(max_len), _stream()),
+            "dnatok_kmer_encode_padded")
+        return ids, mask, lengths, status, max_len
+
+
+class BpeEncoder:
+    """BPE merge engine + packer (C ABI: dnatok_bpe_*, dnatok_pack_ragged, dnatok_pad_rows)."""
+
+    def __init__(self, pair_a, pair_b, new_id, n_symbols: int, byte_to_id=None, out_remap=None):
+        self.pair_a = np.ascontiguousarray(pair_a, dtype=np.int32)
+        self.pair_b = np.ascontiguousarray(pair_b, dtype=np.int32)
+        self.new_id = np.ascontiguousarray(new_id, dtype=np.int32)
+        self.n_symbols = int(n_symbols)
+        self.byte_to_id = (np.arange(256, dtype=np.int32) if byte_to_id is None
+                           else np.ascontiguousarray(byte_to_id, dtype=np.int32))
+        self.out_remap = None if out_remap is None else np.ascontiguousarray(out_remap, dtype=np.int32)
+        h = ctypes.c_void_p()
+        _lib.check(_lib.lib().dnatok_bpe_table_create(
+            _np_ptr(self.byte_to_id), _np_ptr(self.pair_a), _np_ptr(self.pair_b),
+            _np_ptr(self.new_id), int(self.pair_a.size), self.n_symbols, _np_ptr(self.out_remap),
+            ctypes.byref(h)), "dnatok_bpe_table_create")
+        self._h = h
+        self._scratch: Optional[torch.Tensor] = None
+
+    def __del__(self):
+        h = getattr(self, "_h", None)
+        if h:
+            try:
+                _lib.lib().dnatok_bpe_table_destroy(h)
+            except Exception:
+                pass
+
+    def _get_scratch(self, n_rows: int, max_len: int, total: int, device) -> torch.Tensor:
+        need = int(_lib.lib().dnatok_bpe_scratch_bytes(self._h, n_rows, max_len, total))
+        if self._scratch is None or self._scratch.numel() < need or self._scratch.device != device:
+            self._scratch = torch.empty(need, dtype=torch.uint8, device=device)   # grow-only
+        return self._scratch
+
+    def encode(self, data: torch.Tensor, offsets: torch.Tensor, max_len: int, *,
+               tok_tmp: Optional[torch.Tensor] = None, lengths: Optional[torch.Tensor] = None):
+        """Row b's tokens land in tok_tmp[offsets[b] : offsets[b] + lengths[b]]."""
+        _require_cuda(data, torch.uint8, "data")
+        _require_cuda(offsets, torch.int64, "offsets")
+        n_rows = offsets.numel() - 1
+        total = data.numel()
+        if tok_tmp is None:
+            tok_tmp = torch.empty(max(total, 1), dtype=torch.int32, device=data.device)
+        if lengths is None:
+            lengths = torch.empty(n_rows, dtype=torch.int32, device=data.device)
+        scratch = self._get_scratch(n_rows, int(max_len), total, data.device)
+        _lib.check(_lib.lib().dnatok_bpe_encode(self._h, _ptr(data), _ptr(offsets), n_rows,
+                                                int(max_len), total, _ptr(scratch), scratch.numel(),
+                                                _ptr(tok_tmp), _ptr(lengths), _stream()),
+                   "dnatok_bpe_encode")
+        return tok_tmp, lengths
+
+
+def pack_ragged(tok_tmp: torch.Tensor, in_offsets: torch.Tensor, lengths: torch.Tensor, *,
+                remap: Optional[torch.Tensor] = None, want_mask: bool = True,
+                ids_out: Optional[torch.Tensor] = None):
+    """Packed ids (capacity = tok_tmp.numel()), int64 offsets[B+1], mask; all on the device."""
+    n_rows = lengths.numel()
+    dev = tok_tmp.device
+    if ids_out is None:
+        ids_out = torch.empty(tok_tmp.numel(), dtype=torch.int32, device=dev)
+    out_offsets = torch.empty(n_rows + 1, dtype=torch.int64, device=dev)
+    mask = torch.empty(tok_tmp.numel(), dtype=torch.uint8, device=dev) if want_mask else None
+    _lib.check(_lib.lib().dnatok_pack_ragged(_ptr(tok_tmp), _ptr(in_offsets), _ptr(lengths), n_rows,
+                                             _ptr(remap), _ptr(ids_out), _ptr(out_offsets),
+                                             _ptr(mask), _stream()), "dnatok_pack_ragged")
+    return ids_out, out_offsets, mask
+
+
+def pad_rows(tok_tmp: torch.Tensor, in_offsets: torch.Tensor, lengths: torch.Tensor, pad_id: int,
+             t_cap: int, *, fill_to: int = 0, remap: Optional[torch.Tensor] = None,
+             want_mask: bool = True):
+    """Padded ids[B, t_cap] + mask + max_len[1]; with fill_to = 0 view ``ids[:, :max_len]``."""
+    n_rows = lengths.numel()
+    dev = tok_tmp.device
+    ids = torch.empty((n_rows, t_cap), dtype=torch.int32, device=dev)
+    mask = torch.empty((n_rows, t_cap), dtype=torch.uint8, device=dev) if want_mask else None
+    max_len = torch.empty(1, dtype=torch.int32, device=dev)
+    _lib.check(_lib.lib().dnatok_pad_rows(_ptr(tok_tmp), _ptr(in_offsets), _ptr(lengths), n_rows,
+                                          _ptr(remap), int(pad_id), int(t_cap), int(fill_to),
+                                          _ptr(ids), _ptr(mask), _ptr(max_len), _stream()),
+               "dnatok_pad_rows")
+    return ids, mask, max_len

@@ -1,0 +1,157 @@
+/*
+ * dnatok_hip.h -- C ABI of libdnatok_hip.so, the MI355X (gfx950) DNA tokenization backend.
+ *
+ * Plain pointers and sizes only; no torch / pybind types.  Unless marked "host", every
+ * pointer is a DEVICE pointer the caller owns.  `stream` is a hipStream_t passed as void*
+ * (NULL = the default stream).  Every launch is asynchronous on that stream and nothing
+ * here synchronises the device.  Functions return 0 on success or a negative DNATOK_E_*
+ * code; dnatok_last_error() gives the message of the calling thread's last failure.
+ *
+ * Each entry point names the interface of the reference (eniktab/DNAtok, paths relative
+ * to its root) that it stands in for.
+ */
+#ifndef DNATOK_HIP_H
+#define DNATOK_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DNATOK_VERSION 100
+
+#define DNATOK_OK            0
+#define DNATOK_E_INVALID    -1   /* bad argument */
+#define DNATOK_E_HIP        -2   /* a HIP runtime call failed */
+#define DNATOK_E_TOO_LARGE  -3   /* vocabulary / merge table / input beyond what the kernels index */
+#define DNATOK_E_SCRATCH    -4   /* scratch buffer too small */
+
+/* per-row status bits written by the k-mer encoder */
+#define DNATOK_ROW_INVALID_BYTE  1   /* a byte outside the digit table (encoded as N) */
+#define DNATOK_ROW_MISSING_KMER  2   /* a window with neither an id nor an expansion */
+#define DNATOK_ROW_TRUNCATED     4   /* more tokens than the row stride holds */
+
+typedef struct dnatok_char_table dnatok_char_t;
+typedef struct dnatok_kmer_table dnatok_kmer_t;
+typedef struct dnatok_bpe_table  dnatok_bpe_t;
+
+int         dnatok_version(void);
+const char *dnatok_last_error(void);
+
+/* ---------------------------------------------------------------------------------------
+ * Single-nucleotide (char) encoder.
+ * Replaces DNATok._encode_batch_ascii_lut_numpy / _variable_length
+ * (src/dna_tokenizer.py:1779-1858), DNATok._encode_batch_numpy's first-column fix-up
+ * (1582-1589) and DNATok._map_ascii_bytes_to_ids_cuda (2653-2723).
+ * ------------------------------------------------------------------------------------- */
+
+/* lut_h / start_lut_h: host int32[256]; start_lut_h may be NULL (no separate table for the
+ * first character of a row). */
+int  dnatok_char_table_create(const int32_t *lut_h, const int32_t *start_lut_h, int32_t pad_id,
+                              dnatok_char_t **out);
+void dnatok_char_table_destroy(dnatok_char_t *t);
+
+/* Ragged rows -> ids int32[n_rows, t_out] and mask uint8[n_rows, t_out] (mask may be NULL).
+ * Row b is bytes[offsets[b] .. offsets[b+1]); rows longer than t_out are cut, shorter ones
+ * padded with pad_id on the right (pad_left = 0) or on the left (pad_left = 1). */
+int dnatok_char_encode_padded(const dnatok_char_t *t, const uint8_t *bytes, const int64_t *offsets,
+                              int64_t n_rows, int64_t t_out, int pad_left,
+                              int32_t *ids, uint8_t *mask, void *stream);
+
+/* Flat stream: ids[i] = lut[bytes[i]], i < total; mask (may be NULL) is set to 1.
+ * row_len > 0 declares equal-length rows, so that positions i % row_len == 0 use the start
+ * table; row_len = 0 means no row structure.  This is also the dense [B, T] -> [B, T] case. */
+int dnatok_char_encode_packed(const dnatok_char_t *t, const uint8_t *bytes, int64_t total,
+                              int64_t row_len, int32_t *ids, uint8_t *mask, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Non-overlapping k-mer encoder (grid-aligned windows, per-window fallback, tail as single
+ * characters).  Replaces DNATok._encode_batch_kmer_numpy_partial (src/dna_tokenizer.py:
+ * 1369-1474), _encode_kmer_fallback_from_lut / _merge_kmer_fallback (1896-2047) and
+ * _map_kmer_bytes_to_ids_cuda / _expand_kmer_packed_cuda (2736-2940); the tables are the
+ * ones DNATok._build_kmer_lut (743-822) produces.
+ * ------------------------------------------------------------------------------------- */
+
+/* All table arguments are host pointers.
+ *   digit_h[256]     base-5 digit of a byte (A0 C1 G2 T3 N4), -1 = not in the alphabet
+ *   kmer_lut_h[5^k]  token id of a window (digits most significant first), or -1
+ *   exp_off_h/exp_len_h[5^k], exp_flat_h[n_flat]  token list of a window whose id is -1
+ *                    (may all be NULL / 0: then such windows emit missing_id)
+ *   single_h[256]    token id of one character (used for the trailing len % k bases)
+ * 2 <= k <= 8. */
+int  dnatok_kmer_table_create(int k, const int8_t *digit_h, const int32_t *kmer_lut_h,
+                              const int32_t *exp_off_h, const int32_t *exp_len_h,
+                              const int32_t *exp_flat_h, int64_t n_flat,
+                              const int32_t *single_h, int32_t pad_id, int32_t missing_id,
+                              dnatok_kmer_t **out);
+void dnatok_kmer_table_destroy(dnatok_kmer_t *t);
+
+/* ids int32[n_rows, t_cap], mask uint8[n_rows, t_cap] (NULL allowed): t_cap is the row stride.
+ * lengths int32[n_rows] receives each row's token count (also when it exceeds t_cap),
+ * status int32[n_rows] the DNATOK_ROW_* bits (NULL allowed), max_len int32[1] the largest
+ * stored row length (NULL allowed).
+ * fill_to > 0: every row is padded to column fill_to (<= t_cap).
+ * fill_to = 0: rows are padded to the longest row of the batch, found on the device, so the
+ *              caller may view ids[:, :max_len] without a second pass over the data. */
+int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *bytes, const int64_t *offsets,
+                              int64_t n_rows, int64_t t_cap, int64_t fill_to,
+                              int32_t *ids, uint8_t *mask, int32_t *lengths, int32_t *status,
+                              int32_t *max_len, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * BPE merge engine.  Replaces the pybind class DNATokBPE and its kernel
+ * (src/dnatok_bpe_kernel/dnatok_bpe.cu:237-740 bpe_kernel, 761-791 build_vocab_from_merges,
+ * 797-838 constructor, 865-947 tokenize_batch, 956-1015 ensure_workspace).
+ * ------------------------------------------------------------------------------------- */
+
+/* Host arrays.  Merge rule i (its rank) is (pair_a_h[i], pair_b_h[i]) -> new_id_h[i]; ids are
+ * symbol indices < n_symbols (the reference's kernel id space: 0..255 bytes, then merge
+ * results in first-seen order).  byte_to_id_h[256] gives the initial symbol of a byte.
+ * out_remap_h[n_symbols] (may be NULL) translates a symbol to the id that is written out,
+ * which is what GPUTokBPEBackend's remap table does after the kernel
+ * (src/gputok_bpe_backend.py:451-466, 581).  n_symbols <= 65535, n_merges <= 65534. */
+int  dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_t *pair_a_h,
+                             const int32_t *pair_b_h, const int32_t *new_id_h, int32_t n_merges,
+                             int32_t n_symbols, const int32_t *out_remap_h, dnatok_bpe_t **out);
+void dnatok_bpe_table_destroy(dnatok_bpe_t *t);
+
+/* Bytes of device scratch dnatok_bpe_encode needs for a batch whose longest row has max_len
+ * bytes and whose rows sum to total bytes. */
+size_t dnatok_bpe_scratch_bytes(const dnatok_bpe_t *t, int64_t n_rows, int64_t max_len,
+                                int64_t total);
+
+/* Row b's tokens are written to tok_tmp[offsets[b] .. offsets[b] + lengths[b]) (a row never has
+ * more tokens than bytes), tok_tmp is int32[total].  max_len is a host-known upper bound of the
+ * row lengths (it selects the kernel variant); scratch is device memory of at least
+ * dnatok_bpe_scratch_bytes() bytes, reusable across calls on the same stream. */
+int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets,
+                      int64_t n_rows, int64_t max_len, int64_t total,
+                      void *scratch, size_t scratch_bytes,
+                      int32_t *tok_tmp, int32_t *lengths, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Ragged-batch packer: turns per-row token runs (tok_tmp + in_offsets + lengths, as the BPE
+ * engine leaves them) into the tensors a model consumes, without a host round trip.
+ * Replaces the torch op chain of GPUTokBPEBackend.encode_batch
+ * (src/gputok_bpe_backend.py:578-601: remap gather, lens.max().item(), arange mask, where).
+ * ------------------------------------------------------------------------------------- */
+
+/* Packed layout: ids_out int32[sum lengths] holds the rows back to back, out_offsets
+ * int64[n_rows + 1] their boundaries, mask_out uint8[sum lengths] (NULL allowed) is all ones.
+ * remap (device int32, NULL allowed) translates every id. */
+int dnatok_pack_ragged(const int32_t *tok_tmp, const int64_t *in_offsets, const int32_t *lengths,
+                       int64_t n_rows, const int32_t *remap, int32_t *ids_out,
+                       int64_t *out_offsets, uint8_t *mask_out, void *stream);
+
+/* Padded layout: ids int32[n_rows, t_cap] / mask uint8[n_rows, t_cap]; fill_to and max_len as
+ * for dnatok_kmer_encode_padded. */
+int dnatok_pad_rows(const int32_t *tok_tmp, const int64_t *in_offsets, const int32_t *lengths,
+                    int64_t n_rows, const int32_t *remap, int32_t pad_id, int64_t t_cap,
+                    int64_t fill_to, int32_t *ids, uint8_t *mask, int32_t *max_len, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DNATOK_HIP_H */

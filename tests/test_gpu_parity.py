@@ -1,0 +1,323 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle and the golden vectors.
+Bit-exact: everything here is integer / index work."""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from dnatok_amd import bpe_vocab, encoders, hf_tokenizers as hf, kmer_tables
+from dnatok_amd import workloads as wl
+from oracle import oracle as O
+from tests import util
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def to_dev(b: wl.Batch):
+    return torch.from_numpy(b.data).to(DEV), torch.from_numpy(b.offsets).to(DEV)
+
+
+def say(msg):
+    print(msg, flush=True)
+
+
+# ------------------------------------------------------------------ char
+
+@pytest.fixture(scope="module")
+def char_enc():
+    return encoders.CharEncoder(util.char_lut(), pad_id=1)
+
+
+def test_char_c1_dense(char_enc):
+    say("char C1 64x8192 packed/dense")
+    b = wl.config1_char()
+    data, off = to_dev(b)
+    ids, mask = char_enc.encode_packed(data, row_len=8192, want_mask=True)
+    torch.cuda.synchronize()
+    rows = list(ids.cpu().numpy().reshape(64, 8192))
+    util.check_against_golden("C1_char", rows)
+    assert bool((mask == 1).all())
+    ids2, mask2 = char_enc.encode_padded(data, off, 8192)
+    torch.cuda.synchronize()
+    assert torch.equal(ids2.reshape(-1), ids) and bool((mask2 == 1).all())
+
+
+@pytest.mark.parametrize("t_out,pad_left", [(0, False), (37, False), (64, False), (1031, True), (4100, False), (50, True)])
+def test_char_ragged_padded(t_out, pad_left):
+    say(f"char ragged padded t_out={t_out} left={pad_left}")
+    rng = np.random.default_rng(t_out + 1)
+    lens = rng.integers(0, 3000, size=97)
+    lens[:4] = [0, 1, 3, 4099]
+    strings = ["".join(rng.choice(list("ACGTNacgtX"), size=n)) for n in lens]
+    b = util.batch_from_strings(strings)
+    lut = util.char_lut(fold_case=True)
+    start = lut + 50
+    for st in (None, start):
+        enc = encoders.CharEncoder(lut, pad_id=1, start_lut=st)
+        data, off = to_dev(b)
+        ids, mask = enc.encode_padded(data, off, t_out, pad_left=pad_left)
+        torch.cuda.synchronize()
+        eids, emask = O.char_encode_padded(lut, b.data, b.offsets, t_out, 1, start_lut=st, pad_left=pad_left)
+        np.testing.assert_array_equal(ids.cpu().numpy(), eids)
+        np.testing.assert_array_equal(mask.cpu().numpy(), emask)
+
+
+@pytest.mark.parametrize("total", [0, 1, 5, 4095, 4096, 4097, 123457])
+def test_char_packed_sizes(char_enc, total):
+    say(f"char packed total={total}")
+    rng = np.random.default_rng(total)
+    data_h = rng.integers(0, 256, size=total, dtype=np.uint8)
+    data = torch.from_numpy(data_h).to(DEV)
+    ids, mask = char_enc.encode_packed(data, want_mask=True)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(ids.cpu().numpy(), O.char_encode_packed(util.char_lut(), data_h))
+    assert bool((mask == 1).all())
+
+
+def test_char_packed_start_table():
+    lut = util.char_lut()
+    enc = encoders.CharEncoder(lut, pad_id=1, start_lut=lut + 7)
+    for row_len in (1, 2, 3, 5, 512, 4096):
+        say(f"char packed start table row_len={row_len}")
+        b = wl.config1_char(9, row_len, seed=row_len)
+        data, off = to_dev(b)
+        ids, _ = enc.encode_packed(data, row_len=row_len)
+        torch.cuda.synchronize()
+        eids, _ = O.char_encode_padded(lut, b.data, b.offsets, row_len, 1, start_lut=lut + 7)
+        np.testing.assert_array_equal(ids.cpu().numpy().reshape(9, row_len), eids)
+
+
+def test_char_c5_packed(char_enc):
+    say("char C5 packed")
+    b = wl.config5_ragged()
+    data, off = to_dev(b)
+    ids, _ = char_enc.encode_packed(data)
+    torch.cuda.synchronize()
+    flat = ids.cpu().numpy()
+    util.check_against_golden("C5_char", [flat[b.offsets[i]:b.offsets[i + 1]] for i in range(b.n_seqs)])
+
+
+# ----------------------------------------------------------------- k-mer
+
+@pytest.fixture(scope="module")
+def kmer_enc():
+    t = kmer_tables.tables_from_vocab(hf.kmer_vocab(6), 6, 0)
+    return encoders.KmerEncoder(6, t.digit, t.kmer_lut, t.single, pad_id=1, missing_id=0,
+                                exp_off=t.exp_off, exp_len=t.exp_len, exp_flat=t.exp_flat)
+
+
+def rows_from_padded(ids, lengths):
+    ids, lengths = ids.cpu().numpy(), lengths.cpu().numpy()
+    return [ids[r, :lengths[r]] for r in range(ids.shape[0])]
+
+
+def test_kmer_c2(kmer_enc):
+    say("kmer C2 256x6000")
+    b = wl.config2_kmer()
+    data, off = to_dev(b)
+    ids, mask, lengths, status, max_len = kmer_enc.encode_padded(data, off, 6000)
+    torch.cuda.synchronize()
+    rows = rows_from_padded(ids, lengths)
+    util.check_against_golden("C2_kmer", rows)
+    m = int(max_len.item())
+    assert m == int(lengths.max().item())
+    eids, emask = O.pad_rows(rows, 1, m)
+    np.testing.assert_array_equal(ids[:, :m].cpu().numpy(), eids)
+    np.testing.assert_array_equal(mask[:, :m].cpu().numpy(), emask)
+    assert int(status.abs().sum().item()) == 0
+
+
+@pytest.mark.parametrize("k", [2, 3, 4, 5, 6, 7, 8])
+def test_kmer_ragged_all_k(k):
+    say(f"kmer ragged k={k}")
+    vocab = hf.kmer_vocab(k)
+    t = kmer_tables.tables_from_vocab(vocab, k, 0)
+    enc = encoders.KmerEncoder(k, t.digit, t.kmer_lut, t.single, pad_id=1, missing_id=0,
+                               exp_off=t.exp_off, exp_len=t.exp_len, exp_flat=t.exp_flat)
+    ot = O.kmer_tables_from_vocab(vocab, k, 0)
+    rng = np.random.default_rng(k)
+    lens = rng.integers(0, 9000, size=61)
+    lens[:6] = [0, 1, k - 1, k, k + 1, 5000 * k + 3]
+    strings = ["".join(rng.choice(list("ACGTN"), p=[.24, .24, .24, .24, .04], size=n)) for n in lens]
+    strings[7] = "N" * 3000
+    strings[8] = "ACGTx" * 300
+    b = util.batch_from_strings(strings)
+    data, off = to_dev(b)
+    t_cap = int(max(len(s) for s in strings)) + 3
+    t_cap += (-t_cap) % 4
+    for fill_to, cap in ((0, t_cap), (t_cap, t_cap), (0, 1000), (0, 1001)):
+        ids, mask, lengths, status, max_len = enc.encode_padded(data, off, cap, fill_to=fill_to)
+        torch.cuda.synchronize()
+        erows, estatus = O.kmer_encode(ot, b.data, b.offsets)
+        np.testing.assert_array_equal(lengths.cpu().numpy(), [r.size for r in erows])
+        st = status.cpu().numpy()
+        np.testing.assert_array_equal(st & 3, estatus)
+        np.testing.assert_array_equal((st & 4) != 0, np.array([r.size > cap for r in erows]))
+        width = fill_to if fill_to else min(cap, max(r.size for r in erows))
+        assert int(max_len.item()) == min(cap, max(r.size for r in erows))
+        eids, emask = O.pad_rows(erows, 1, width)
+        np.testing.assert_array_equal(ids[:, :width].cpu().numpy(), eids)
+        np.testing.assert_array_equal(mask[:, :width].cpu().numpy(), emask)
+
+
+def test_kmer_missing_windows_without_expansion():
+    say("kmer missing windows")
+    t = kmer_tables.tables_from_vocab(hf.kmer_vocab(4), 4, 0)
+    enc = encoders.KmerEncoder(4, t.digit, t.kmer_lut, t.single, pad_id=1, missing_id=3)
+    b = util.batch_from_strings(["ACGTACNTACGTAC", "ACGTACGT"])
+    data, off = to_dev(b)
+    ids, mask, lengths, status, _ = enc.encode_padded(data, off, 16)
+    torch.cuda.synchronize()
+    assert lengths.tolist() == [3 + 2, 2]
+    assert status.tolist() == [2, 0]
+    assert ids[0, 1].item() == 3
+
+
+# ------------------------------------------------------------------- BPE
+
+@pytest.fixture(scope="module", params=["4096", "32000"])
+def bpe(request):
+    which = request.param
+    cfg = util.tokenizer_json(which)
+    kv = bpe_vocab.KernelVocab(bpe_vocab.split_merges(cfg["model"]["merges"]))
+    remap = kv.remap_to(cfg["model"]["vocab"], cfg["model"]["vocab"]["[UNK]"])
+    enc = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv), out_remap=remap)
+    return which, enc, util.bpe_oracle(which)
+
+
+def bpe_rows(enc, b: wl.Batch):
+    data, off = to_dev(b)
+    max_len = int(b.lengths().max()) if b.n_seqs else 0
+    tok, lengths = enc.encode(data, off, max_len)
+    torch.cuda.synchronize()
+    tok, lengths = tok.cpu().numpy(), lengths.cpu().numpy()
+    return [tok[b.offsets[i]:b.offsets[i] + lengths[i]] for i in range(b.n_seqs)]
+
+
+def test_bpe_small_and_edge_cases(bpe):
+    which, enc, bo = bpe
+    say(f"bpe{which} small cases")
+    cases = util.small_cases()
+    rows = bpe_rows(enc, util.batch_from_strings(cases))
+    for s, r, g in zip(cases, rows, util.split_small("bpe" + which)):
+        np.testing.assert_array_equal(r, g, err_msg=repr(s))
+
+
+def test_bpe_random_lengths_and_homopolymers(bpe):
+    which, enc, bo = bpe
+    say(f"bpe{which} random lengths / homopolymers")
+    random.seed(0)
+    seqs = ["".join(random.choices("ACGT", k=random.choice([4, 8, 16, 32, 64, 128, 256, 512, 1024, 2048])))
+            for _ in range(256)]
+    seqs += [c * n for c in "ACGTN" for n in (32, 64, 128, 256, 512, 1024, 4096)]
+    seqs += ["AC" * 700, "ACG" * 500, "AAAT" * 300 + "A" * 100, "N" * 10 + "ACGT" * 100 + "NN"]
+    b = util.batch_from_strings(seqs)
+    rows = bpe_rows(enc, b)
+    ref = bo.encode_batch(b.data, b.offsets)
+    for s, r, e in zip(seqs, rows, ref):
+        np.testing.assert_array_equal(r, e, err_msg=s[:40])
+
+
+def test_bpe_c3_golden():
+    say("bpe4096 C3 1024x1024")
+    cfg = util.tokenizer_json("4096")
+    kv = bpe_vocab.KernelVocab(bpe_vocab.split_merges(cfg["model"]["merges"]))
+    enc = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv),
+                              out_remap=kv.remap_to(cfg["model"]["vocab"], 0))
+    util.check_against_golden("C3_bpe4096", bpe_rows(enc, wl.config3_bpe4096()))
+
+
+def test_bpe_long_rows(bpe):
+    which, enc, bo = bpe
+    say(f"bpe{which} long rows (global-state path)")
+    b = wl.config4_bpe32000(3, 20_000, seed=77)
+    rows = bpe_rows(enc, b)
+    for r, e in zip(rows, bo.encode_batch(b.data, b.offsets)):
+        np.testing.assert_array_equal(r, e)
+    # mixed short and long rows in one batch, with N
+    strings = wl.config5_ragged(40, seed=9).strings() + ["A" * 9000, "ACGT" * 3000 + "N" + "TG" * 2000]
+    b2 = util.batch_from_strings(strings)
+    for r, e in zip(bpe_rows(enc, b2), bo.encode_batch(b2.data, b2.offsets)):
+        np.testing.assert_array_equal(r, e)
+
+
+def test_bpe_c4_golden():
+    say("bpe32000 C4 32x100k")
+    cfg = util.tokenizer_json("32000")
+    kv = bpe_vocab.KernelVocab(bpe_vocab.split_merges(cfg["model"]["merges"]))
+    enc = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv),
+                              out_remap=kv.remap_to(cfg["model"]["vocab"], 0))
+    util.check_against_golden("C4_bpe32000", bpe_rows(enc, wl.config4_bpe32000()))
+
+
+def test_bpe_nonmonotone_random_tables():
+    """Random small merge tables, including ones where two rules give the same string."""
+    say("bpe random tables")
+    rng = random.Random(11)
+    for trial in range(40):
+        alpha = "ACGT"[:rng.choice([2, 3, 4])]
+        toks, merges, seen, strings = list(alpha), [], set(), set(alpha)
+        for _ in range(rng.randint(1, 50)):
+            a, b2 = rng.choice(toks), rng.choice(toks)
+            if (a, b2) in seen or len(a + b2) > 10:
+                continue
+            seen.add((a, b2))
+            merges.append((a, b2))
+            if a + b2 not in strings:
+                strings.add(a + b2)
+                toks.append(a + b2)
+        kv = bpe_vocab.KernelVocab(merges)
+        enc = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv))
+        bo = O.BpeOracle(merges)
+        seqs = ["".join(rng.choice(alpha) for _ in range(rng.randint(1, 300))) for _ in range(30)]
+        seqs += [rng.choice(alpha) * rng.randint(1, 200) for _ in range(6)]
+        b = util.batch_from_strings(seqs)
+        for s, r, e in zip(seqs, bpe_rows(enc, b), bo.encode_batch(b.data, b.offsets, remap=False)):
+            np.testing.assert_array_equal(r, e, err_msg=f"trial {trial} {s} {merges}")
+
+
+# ---------------------------------------------------------------- packer
+
+def test_c5_ragged_bpe_and_char_packed(char_enc):
+    say("C5 ragged: BPE-4096 + char, packed on device")
+    cfg = util.tokenizer_json("4096")
+    kv = bpe_vocab.KernelVocab(bpe_vocab.split_merges(cfg["model"]["merges"]))
+    enc = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv))        # kernel ids out
+    remap = torch.from_numpy(kv.remap_to(cfg["model"]["vocab"], 0)).to(DEV)
+    b = wl.config5_ragged()
+    data, off = to_dev(b)
+    tok, lengths = enc.encode(data, off, int(b.lengths().max()))
+    ids, out_off, mask = encoders.pack_ragged(tok, off, lengths, remap=remap)
+    cids, _ = char_enc.encode_packed(data)
+    torch.cuda.synchronize()
+    oo = out_off.cpu().numpy()
+    flat = ids.cpu().numpy()
+    rows = [flat[oo[i]:oo[i + 1]] for i in range(b.n_seqs)]
+    util.check_against_golden("C5_bpe4096", rows)
+    assert bool((mask[:oo[-1]] == 1).all())
+    cf = cids.cpu().numpy()
+    util.check_against_golden("C5_char", [cf[b.offsets[i]:b.offsets[i + 1]] for i in range(b.n_seqs)])
+
+
+def test_pad_rows_matches_reference_semantics():
+    say("pad_rows")
+    cfg = util.tokenizer_json("4096")
+    kv = bpe_vocab.KernelVocab(bpe_vocab.split_merges(cfg["model"]["merges"]))
+    enc = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv))
+    remap_h = kv.remap_to(cfg["model"]["vocab"], 0)
+    remap = torch.from_numpy(remap_h).to(DEV)
+    b = wl.config5_ragged(50, seed=3)
+    data, off = to_dev(b)
+    tok, lengths = enc.encode(data, off, int(b.lengths().max()))
+    erows = util.bpe_oracle("4096").encode_batch(b.data, b.offsets)
+    cap = max(r.size for r in erows) + 5
+    for fill_to in (0, cap):
+        ids, mask, max_len = encoders.pad_rows(tok, off, lengths, 3, cap, fill_to=fill_to, remap=remap)
+        torch.cuda.synchronize()
+        width = fill_to or int(max_len.item())
+        assert int(max_len.item()) == max(r.size for r in erows)
+        eids, emask = O.pad_rows(erows, 3, width)
+        np.testing.assert_array_equal(ids[:, :width].cpu().numpy(), eids)
+        np.testing.assert_array_equal(mask[:, :width].cpu().numpy(), emask)

@@ -1,0 +1,183 @@
+"""Pins the CPU oracle: against the committed golden vectors (written by the Hugging Face
+`tokenizers` library), against the live HF library when it is importable, against closed
+forms, and heap form vs. the textbook O(n^2) form of BPE."""
+import random
+
+import numpy as np
+import pytest
+
+from dnatok_amd import hf_tokenizers as hf
+from dnatok_amd import workloads as wl
+from oracle import oracle as O
+from tests import util
+
+
+def hf_rows(tk, strings):
+    return [np.asarray(e.ids, dtype=np.int32) for e in tk.encode_batch(strings, add_special_tokens=False)]
+
+
+# ------------------------------------------------------------------ char
+
+def test_char_closed_form_and_golden():
+    b = wl.config1_char()
+    lut = util.char_lut()
+    ids, mask = O.char_encode_padded(lut, b.data, b.offsets, 8192, pad_id=1)
+    # closed form: ids = lut[byte]
+    np.testing.assert_array_equal(ids, lut[b.data].reshape(64, 8192))
+    assert mask.all()
+    util.check_against_golden("C1_char", list(ids))
+    np.testing.assert_array_equal(O.char_encode_packed(lut, b.data), ids.reshape(-1))
+
+
+def test_char_ragged_padding_sides_and_start_table():
+    strings = ["ACGT", "", "NNA", "ACGTACGTAC"]
+    b = util.batch_from_strings(strings)
+    lut = util.char_lut()
+    start = lut + 100
+    ids, mask = O.char_encode_padded(lut, b.data, b.offsets, 6, pad_id=1, start_lut=start)
+    exp = np.full((4, 6), 1, np.int32)
+    expm = np.zeros((4, 6), np.uint8)
+    for r, s in enumerate(strings):
+        row = [lut[ord(c)] for c in s][:6]
+        if row:
+            row[0] += 100
+        exp[r, :len(row)] = row
+        expm[r, :len(row)] = 1
+    np.testing.assert_array_equal(ids, exp)
+    np.testing.assert_array_equal(mask, expm)
+    ids_l, mask_l = O.char_encode_padded(lut, b.data, b.offsets, 6, pad_id=1, pad_left=True)
+    for r, s in enumerate(strings):
+        n = min(len(s), 6)
+        np.testing.assert_array_equal(ids_l[r, 6 - n:], [lut[ord(c)] for c in s[:n]])
+        assert (ids_l[r, :6 - n] == 1).all() and mask_l[r].sum() == n
+
+
+def test_char_matches_hf_live():
+    tk = hf.build_char_tokenizer()
+    b = wl.config1_char(8, 1000, seed=5)
+    rows = hf_rows(tk, b.strings())
+    ids, _ = O.char_encode_padded(util.char_lut(), b.data, b.offsets, 1000, pad_id=1)
+    for r in range(8):
+        np.testing.assert_array_equal(ids[r], rows[r])
+
+
+# ----------------------------------------------------------------- k-mer
+
+def test_kmer_golden_and_brute_force():
+    t = util.kmer_oracle_tables()
+    b = wl.config2_kmer()
+    rows, status = O.kmer_encode(t, b.data, b.offsets)
+    assert (status == 0).all()
+    util.check_against_golden("C2_kmer", rows)
+    # brute force over every ACGT 6-mer: id = 5 + base-4 value
+    vocab = hf.kmer_vocab(6)
+    import itertools
+    allk = ["".join(p) for p in itertools.product("ACGT", repeat=6)]
+    bb = util.batch_from_strings(["".join(allk)])
+    got, _ = O.kmer_encode(t, bb.data, bb.offsets)
+    np.testing.assert_array_equal(got[0], np.arange(5, 5 + 4096))
+    assert [vocab[k] for k in allk] == list(range(5, 5 + 4096))
+
+
+def test_kmer_small_cases_and_hf_live():
+    t = util.kmer_oracle_tables()
+    cases = [c for c in util.small_cases()]
+    b = util.batch_from_strings([c.upper().replace("X", "N") for c in cases])
+    rows, _ = O.kmer_encode(t, b.data, b.offsets)
+    tk = hf.build_kmer_tokenizer(6)
+    ref = hf_rows(tk, b.strings())
+    for r, e in zip(rows, ref):
+        np.testing.assert_array_equal(r, e)
+    # golden small cases were written from the raw strings; compare those without lower case / X
+    gold = util.split_small("kmer")
+    for c, g, r in zip(cases, gold, rows):
+        if c == c.upper() and "X" not in c:
+            np.testing.assert_array_equal(r, g)
+
+
+def test_kmer_status_bits():
+    t = util.kmer_oracle_tables()
+    b = util.batch_from_strings(["ACGTAxACGTAC"])
+    rows, status = O.kmer_encode(t, b.data, b.offsets)
+    assert status[0] == 1                      # byte outside the alphabet, encoded as N
+    assert rows[0].size == 6 + 1
+
+
+# ------------------------------------------------------------------- BPE
+
+@pytest.mark.parametrize("which,name,maker", [
+    ("4096", "C3_bpe4096", wl.config3_bpe4096),
+    ("32000", "C4_bpe32000", wl.config4_bpe32000),
+])
+def test_bpe_golden(which, name, maker):
+    bo = util.bpe_oracle(which)
+    b = maker()
+    util.check_against_golden(name, bo.encode_batch(b.data, b.offsets))
+
+
+def test_c5_golden_char_and_bpe():
+    b = wl.config5_ragged()
+    lut = util.char_lut()
+    flat = O.char_encode_packed(lut, b.data)
+    util.check_against_golden("C5_char", [flat[b.offsets[i]:b.offsets[i + 1]] for i in range(b.n_seqs)])
+    util.check_against_golden("C5_bpe4096", util.bpe_oracle("4096").encode_batch(b.data, b.offsets))
+
+
+@pytest.mark.parametrize("which", ["4096", "32000"])
+def test_bpe_small_cases_golden(which):
+    bo = util.bpe_oracle(which)
+    for s, g in zip(util.small_cases(), util.split_small("bpe" + which)):
+        row = np.frombuffer(s.encode(), dtype=np.uint8)
+        np.testing.assert_array_equal(bo.encode_row(row), g, err_msg=repr(s))
+        np.testing.assert_array_equal(bo.encode_row(row, naive=True), g, err_msg=repr(s))
+
+
+@pytest.mark.parametrize("which", ["4096", "32000"])
+def test_bpe_invariants_and_hf_live(which):
+    """Replay of the reference's random generator (tests/test_gputok_bpe_backend.py:100-105):
+    random.seed(0), lengths from a fixed menu; plus homopolymers 32..1024 (293-308)."""
+    bo = util.bpe_oracle(which)
+    tk = hf.load_bpe_tokenizer(which)
+    random.seed(0)
+    seqs = ["".join(random.choices("ACGT", k=random.choice([4, 8, 16, 32, 64, 128, 256, 512, 1024, 2048])))
+            for _ in range(64)]
+    seqs += [c * n for c in "ACGT" for n in (32, 64, 128, 256, 512, 1024)]
+    b = util.batch_from_strings(seqs)
+    rows = bo.encode_batch(b.data, b.offsets)
+    ref = hf_rows(tk, seqs)
+    id_to_tok = {v: k for k, v in util.tokenizer_json(which)["model"]["vocab"].items()}
+    merges = set(O.merges_from_tokenizer_json(util.tokenizer_json(which)))
+    for s, r, e in zip(seqs, rows, ref):
+        np.testing.assert_array_equal(r, e)
+        toks = [id_to_tok[int(i)] for i in r]
+        assert "".join(toks) == s                                  # decode round trip
+        assert not any((a, b2) in merges for a, b2 in zip(toks, toks[1:]))   # nothing left to merge
+
+
+def test_bpe_heap_equals_naive_on_random_tables():
+    rng = random.Random(7)
+    for trial in range(300):
+        alpha = "ACGT"[:rng.choice([2, 3, 4])]
+        toks, merges, seen, strings = list(alpha), [], set(), set(alpha)
+        for _ in range(rng.randint(1, 40)):
+            a, b2 = rng.choice(toks), rng.choice(toks)
+            if (a, b2) in seen or len(a + b2) > 10:
+                continue
+            seen.add((a, b2))
+            merges.append((a, b2))
+            if a + b2 not in strings:
+                strings.add(a + b2)
+                toks.append(a + b2)
+        bo = O.BpeOracle(merges)
+        for _ in range(4):
+            s = "".join(rng.choice(alpha) for _ in range(rng.randint(1, 80)))
+            row = np.frombuffer(s.encode(), dtype=np.uint8)
+            np.testing.assert_array_equal(bo.encode_row(row, remap=False),
+                                          bo.encode_row(row, naive=True, remap=False))
+
+
+def test_kernel_vocab_first_seen_order():
+    vocab, a, b2, n = O.kernel_vocab_from_merges([("A", "C"), ("AC", "G"), ("G", "T"), ("A", "CG")])
+    assert vocab[256:] == ["AC", "ACG", "GT", "CG"]       # 'CG' is interned before 'A'+'CG' reuses 'ACG'
+    assert a.tolist() == [65, 256, 71, 65] and b2.tolist() == [67, 71, 84, 259]
+    assert n.tolist() == [256, 257, 258, 257]

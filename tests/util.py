@@ -1,0 +1,85 @@
+"""Shared helpers of the test suite: golden fixtures, oracle tables, HF tokenizers."""
+from __future__ import annotations
+
+import hashlib
+import json
+import os
+from functools import lru_cache
+
+import numpy as np
+
+from dnatok_amd import hf_tokenizers as hf
+from dnatok_amd import workloads as wl
+from oracle import oracle as O
+
+GOLDEN_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+@lru_cache(maxsize=None)
+def golden():
+    return dict(np.load(os.path.join(GOLDEN_DIR, "golden_vectors.npz"), allow_pickle=False))
+
+
+@lru_cache(maxsize=None)
+def tokenizer_json(which: str) -> dict:
+    with open(hf.bpe_tokenizer_path(which)) as fh:
+        return json.load(fh)
+
+
+@lru_cache(maxsize=None)
+def bpe_oracle(which: str):
+    return O.bpe_oracle_from_tokenizer_json(tokenizer_json(which))
+
+
+@lru_cache(maxsize=None)
+def kmer_oracle_tables():
+    return O.kmer_tables_from_vocab(hf.kmer_vocab(6), 6, 0)
+
+
+def char_lut(fold_case: bool = False) -> np.ndarray:
+    """NTv3 rule: A T C G N keep their ids, everything else is <unk> (id 0)."""
+    vocab = hf.char_vocab()
+    lut = np.zeros(256, dtype=np.int32)
+    for ch in "ACGTN":
+        lut[ord(ch)] = vocab[ch]
+        if fold_case:
+            lut[ord(ch.lower())] = vocab[ch]
+    return lut
+
+
+def sha_of_rows(rows) -> np.ndarray:
+    flat = np.concatenate([np.asarray(r, dtype=np.int32) for r in rows]) if len(rows) else np.zeros(0, np.int32)
+    return np.frombuffer(hashlib.sha256(flat.astype("<i4").tobytes()).digest(), dtype=np.uint8)
+
+
+def check_against_golden(name: str, rows) -> None:
+    g = golden()
+    lengths = np.array([len(r) for r in rows], dtype=np.int32)
+    np.testing.assert_array_equal(lengths, g[name + "_lengths"], err_msg=name + " lengths")
+    np.testing.assert_array_equal(np.asarray(rows[0][:2048], dtype=np.int32), g[name + "_row0"],
+                                  err_msg=name + " row 0")
+    np.testing.assert_array_equal(sha_of_rows(rows), g[name + "_sha256"], err_msg=name + " sha256")
+
+
+def small_cases():
+    from tests.golden.make_golden import SMALL_CASES
+    return SMALL_CASES
+
+
+def batch_from_strings(strings) -> wl.Batch:
+    lens = np.array([len(s) for s in strings], dtype=np.int64)
+    off = np.zeros(len(strings) + 1, dtype=np.int64)
+    np.cumsum(lens, out=off[1:])
+    data = np.frombuffer("".join(strings).encode("ascii"), dtype=np.uint8).copy()
+    return wl.Batch(data, off)
+
+
+def split_small(name: str):
+    g = golden()
+    lens = g[f"small_{name}_lengths"]
+    ids = g[f"small_{name}_ids"]
+    out, p = [], 0
+    for n in lens:
+        out.append(ids[p:p + n])
+        p += n
+    return out
