@@ -160,7 +160,10 @@ __device__ __forceinline__ void bpe_row(
     }
 
     int flip = 0;
+    int budget = n0 + 8;                       // every round merges at least one pair
+    bool stuck = false;
     for (;;) {
+        if (--budget < 0) { stuck = true; break; }   // cannot happen; keeps the loop bounded
         uint32_t rmin, gate;
         team_min2<NT>(cmin, cgate, red + flip * (NT / 64) * 2, wv, rmin, gate);
         flip ^= 1;
@@ -266,7 +269,7 @@ __device__ __forceinline__ void bpe_row(
         const uint32_t s = S[i];
         if (s != kNone) out[off++] = out_remap ? out_remap[s] : (int32_t)s;
     }
-    if (tid == 0) *out_len = (int32_t)total;
+    if (tid == 0) *out_len = stuck ? -2 : (int32_t)total;
 }
 
 // Rows of at most CAP bytes, state in LDS.  NT = 64: every wave of the workgroup takes its
@@ -304,7 +307,10 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     for (int64_t row = (int64_t)blockIdx.x * TEAMS + team; row < n_rows; row += (int64_t)gridDim.x * TEAMS) {
         const int64_t start = offsets[row];
         const int64_t len = offsets[row + 1] - start;
-        if (len > CAP) continue;                 // handled by the long-row kernel
+        if (len > CAP) {                         // left to the long-row kernel, which overwrites this
+            if (tid == 0) lengths[row] = -1;
+            continue;
+        }
         if (len <= 0) { if (tid == 0) lengths[row] = 0; continue; }
         bpe_row<NT, uint16_t>(tab, mask, a.shift, newsym, minchild, b2s, a.out_remap, bytes + start,
                               (int)len, S, R, NX, PV, F, D, red, tid, tok_tmp + start, lengths + row);
@@ -316,7 +322,8 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
 template <int NT>
 __global__ __launch_bounds__(NT) void bpe_long_kernel(
     BpeArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
-    int64_t n_rows, int64_t min_len, uint8_t *__restrict__ scratch, int64_t scratch_stride,
+    int64_t n_rows, int64_t min_len, int64_t max_len, uint8_t *__restrict__ scratch,
+    int64_t scratch_stride,
     int32_t *__restrict__ tok_tmp, int32_t *__restrict__ lengths)
 {
     __shared__ uint32_t red[4 * (NT / 64)];
@@ -331,6 +338,10 @@ __global__ __launch_bounds__(NT) void bpe_long_kernel(
         const int64_t start = offsets[row];
         const int64_t len = offsets[row + 1] - start;
         if (len <= min_len) continue;
+        if (len > max_len) {                     // longer than the caller declared: no room in the slab
+            if (threadIdx.x == 0) lengths[row] = -1;
+            continue;
+        }
         const size_t n = ((size_t)len + 7) & ~(size_t)7;
         uint32_t *NX = reinterpret_cast<uint32_t *>(slab);
         uint32_t *PV = NX + n;
@@ -512,7 +523,8 @@ extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, co
                        "dnatok_bpe_encode: scratch holds %zu bytes, %zu needed", scratch_bytes,
                        (size_t)slabs * slab);
         bpe_long_kernel<kLongThreads><<<(int)slabs, kLongThreads, 0, s>>>(
-            a, bytes, offsets, n_rows, (int64_t)kLdsCap, (uint8_t *)scratch, (int64_t)slab, tok_tmp, lengths);
+            a, bytes, offsets, n_rows, (int64_t)kLdsCap, max_len, (uint8_t *)scratch, (int64_t)slab,
+            tok_tmp, lengths);
         DNATOK_HIP_TRY(hipGetLastError());
     }
     return DNATOK_OK;

@@ -205,11 +205,11 @@ extern "C" void dnatok_char_table_destroy(dnatok_char_t *t)
 extern "C" int dnatok_char_encode_packed(const dnatok_char_t *t, const uint8_t *bytes, int64_t total,
                                          int64_t row_len, int32_t *ids, uint8_t *mask, void *stream)
 {
-    DNATOK_REQUIRE(t && ids, DNATOK_E_INVALID, "dnatok_char_encode_packed: null argument");
+    DNATOK_REQUIRE(t, DNATOK_E_INVALID, "dnatok_char_encode_packed: null argument");
     DNATOK_REQUIRE(total >= 0 && row_len >= 0, DNATOK_E_INVALID,
                    "dnatok_char_encode_packed: negative size");
     if (total == 0) return DNATOK_OK;
-    DNATOK_REQUIRE(bytes, DNATOK_E_INVALID, "dnatok_char_encode_packed: null input");
+    DNATOK_REQUIRE(bytes && ids, DNATOK_E_INVALID, "dnatok_char_encode_packed: null buffer");
     DNATOK_REQUIRE(((uintptr_t)bytes & 3) == 0 && ((uintptr_t)ids & 15) == 0 &&
                        ((uintptr_t)mask & 3) == 0,
                    DNATOK_E_INVALID,
@@ -237,10 +237,11 @@ extern "C" int dnatok_char_encode_padded(const dnatok_char_t *t, const uint8_t *
                                          const int64_t *offsets, int64_t n_rows, int64_t t_out,
                                          int pad_left, int32_t *ids, uint8_t *mask, void *stream)
 {
-    DNATOK_REQUIRE(t && offsets && ids, DNATOK_E_INVALID, "dnatok_char_encode_padded: null argument");
+    DNATOK_REQUIRE(t && offsets, DNATOK_E_INVALID, "dnatok_char_encode_padded: null argument");
     DNATOK_REQUIRE(n_rows >= 0 && t_out >= 0, DNATOK_E_INVALID,
                    "dnatok_char_encode_padded: negative size");
     if (n_rows == 0 || t_out == 0) return DNATOK_OK;
+    DNATOK_REQUIRE(ids, DNATOK_E_INVALID, "dnatok_char_encode_padded: null output");
     hipStream_t s = (hipStream_t)stream;
     const int64_t tiles_per_row = (t_out + kCharThreads * 4 - 1) / (kCharThreads * 4);
     const int grid = grid_for(n_rows * tiles_per_row);
