@@ -1,0 +1,470 @@
+#!/usr/bin/env python3
+"""Encode-throughput benchmark of the MI355X DNA tokenization backend.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config C2] [--no-extras] [--no-cpu]
+
+A step is one pass of the encode path over one batch of seeded synthetic input that is
+already resident in HBM.  The headline workload (default C2, the non-overlapping 6-mer
+tokenizer) is timed in its sustained form: many distinct 256 x 6000 bp batches laid out
+back to back and encoded by one call, because a single 1.5 Mbp batch (2.8 MB of traffic)
+is launch-bound and says nothing about the HBM roofline; the per-call latency of the
+exact configurations is reported under "per_call".  One JSON line is printed.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import subprocess
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+# ------------------------------------------------------------------------------ inputs
+
+def many_batches_uniform(n_rows: int, length: int, seed: int, n_rate: float = 0.0,
+                         n_run_fraction: float = 0.0) -> np.ndarray:
+    """Fast generator for the sustained runs: same distributions as workloads.config1_char /
+    config2_kmer, vectorised for hundreds of Mbp."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    total = n_rows * length
+    codes = rng.integers(0, 4, size=total, dtype=np.uint8)
+    arr = np.frombuffer(b"ACGT", dtype=np.uint8)[codes]
+    del codes
+    if n_rate > 0:
+        n = rng.binomial(total, n_rate)
+        arr[rng.integers(0, total, size=n)] = ord("N")
+    if n_run_fraction > 0:
+        n = rng.binomial(total, n_run_fraction / 25.5)
+        starts = rng.integers(0, total, size=n)
+        runs = rng.integers(1, 51, size=n)
+        for s, r in zip(starts.tolist(), runs.tolist()):
+            e = min(s + r, (s // length + 1) * length)       # runs do not cross rows
+            arr[s:e] = ord("N")
+    return arr
+
+
+class Workload:
+    name = ""
+    dtype = "u8"
+
+    def step(self):
+        raise NotImplementedError
+
+
+def _dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).to("cuda")
+
+
+class CharDense(Workload):
+    """C1: 64 x 8192 bp char tokenizer; ids int32 + mask uint8, dense [B, T]."""
+
+    def __init__(self, n_batches: int):
+        from dnatok_amd import encoders, hf_tokenizers as hf, workloads as wl
+        vocab = hf.char_vocab()
+        lut = np.zeros(256, dtype=np.int32)
+        for ch in "ACGTN":
+            lut[ord(ch)] = vocab[ch]
+        self.lut = lut
+        self.enc = encoders.CharEncoder(lut, pad_id=vocab["<pad>"])
+        first = wl.config1_char()
+        parts = [first.data]
+        if n_batches > 1:
+            parts.append(many_batches_uniform(64 * (n_batches - 1), 8192, 7001, n_rate=0.001))
+        host = np.concatenate(parts)
+        self.host = host
+        self.data = _dev(host)
+        import torch
+        self.ids = torch.empty(host.size, dtype=torch.int32, device="cuda")
+        self.mask = torch.empty(host.size, dtype=torch.uint8, device="cuda")
+        self.bases = host.size
+        self.algorithmic_bytes = 6 * host.size
+        self.kernel = "char_packed_kernel"
+        self.name = f"C1 char vocab-11, 64x8192 bp batches, {n_batches} distinct batch(es) per call"
+
+    def step(self):
+        self.enc.encode_packed(self.data, row_len=8192, want_mask=True, ids=self.ids, mask=self.mask)
+
+    def check(self):
+        from tests.golden import check as util
+        ids = self.ids[:64 * 8192].cpu().numpy().reshape(64, 8192)
+        util.check_against_golden("C1_char", list(ids))
+        tail = self.ids[-8192:].cpu().numpy()
+        assert np.array_equal(tail, self.lut[self.host[-8192:]])
+        assert bool((self.mask == 1).all())
+
+    def cpu_baseline(self, budget_s: float):
+        from oracle import oracle as O
+        n = min(self.host.size, 64 * 8192 * 64)
+        sample = self.host[:n]
+        off = np.arange(n // 8192 + 1, dtype=np.int64) * 8192
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            O.char_encode_padded(self.lut, sample, off, 8192, 1)
+            reps += 1
+            if time.perf_counter() - t0 > budget_s:
+                break
+        dt = time.perf_counter() - t0
+        return n * reps / dt / 1e6, f"{n // (64 * 8192)} batches of 64x8192 bp, {reps} passes"
+
+
+class KmerPadded(Workload):
+    """C2: 256 x 6000 bp 6-mer tokenizer; padded int32 ids + uint8 mask + lengths."""
+
+    def __init__(self, n_batches: int, t_cap: int = 6000):
+        from dnatok_amd import encoders, hf_tokenizers as hf, kmer_tables, workloads as wl
+        import torch
+        vocab = hf.kmer_vocab(6)
+        self.vocab = vocab
+        t = kmer_tables.tables_from_vocab(vocab, 6, vocab["<unk>"])
+        self.enc = encoders.KmerEncoder(6, t.digit, t.kmer_lut, t.single, vocab["<pad>"], vocab["<unk>"],
+                                        t.exp_off, t.exp_len, t.exp_flat)
+        first = wl.config2_kmer()
+        parts = [first.data]
+        if n_batches > 1:
+            parts.append(many_batches_uniform(256 * (n_batches - 1), 6000, 7002, n_run_fraction=0.005))
+        host = np.concatenate(parts)
+        self.host = host
+        self.n_rows = 256 * n_batches
+        self.t_cap = t_cap
+        self.data = _dev(host)
+        self.off = _dev(np.arange(self.n_rows + 1, dtype=np.int64) * 6000)
+        dev = "cuda"
+        self.out = (torch.empty((self.n_rows, t_cap), dtype=torch.int32, device=dev),
+                    torch.empty((self.n_rows, t_cap), dtype=torch.uint8, device=dev),
+                    torch.empty(self.n_rows, dtype=torch.int32, device=dev),
+                    torch.empty(self.n_rows, dtype=torch.int32, device=dev),
+                    torch.empty(1, dtype=torch.int32, device=dev))
+        self.bases = host.size
+        self.kernel = "kmer_rows_kernel"
+        self.name = (f"C2 non-overlapping 6-mer vocab-4106, 256x6000 bp batches, "
+                     f"{n_batches} distinct batch(es) per call, pad to longest row")
+        self.step()
+        torch.cuda.synchronize()
+        lengths = self.out[2].cpu().numpy()
+        t_max = int(self.out[4].item())
+        assert t_max == int(lengths.max())
+        # 1 B/base read; int32 id + uint8 mask for every cell of [rows, T_max]; int32 length per row
+        self.algorithmic_bytes = host.size + 5 * self.n_rows * t_max + 4 * self.n_rows
+        self.t_max = t_max
+
+    def step(self):
+        self.enc.encode_padded(self.data, self.off, self.t_cap, fill_to=0, out=self.out)
+
+    def check(self):
+        from tests.golden import check as util
+        ids, mask, lengths, status, max_len = self.out
+        ln = lengths.cpu().numpy()
+        assert int(status.abs().sum().item()) == 0
+        rows = [ids[r, :ln[r]].cpu().numpy() for r in range(256)]
+        util.check_against_golden("C2_kmer", rows)
+        # every cell outside the tokens is pad with mask 0, inside mask 1
+        import torch
+        m = self.t_max
+        col = torch.arange(m, device="cuda")[None, :]
+        inside = col < lengths[:, None]
+        assert bool((mask[:, :m].bool() == inside).all())
+        assert bool((ids[:, :m][~inside] == self.vocab["<pad>"]).all())
+        # token-count closed form: windows + 5 per N-window
+        assert int(ln.sum()) >= self.n_rows * 1000
+
+    def cpu_baseline(self, budget_s: float):
+        from oracle import oracle as O
+        ot = O.kmer_tables_from_vocab(self.vocab, 6, self.vocab["<unk>"])
+        rows = min(self.n_rows, 256 * 16)
+        sample = self.host[:rows * 6000]
+        off = np.arange(rows + 1, dtype=np.int64) * 6000
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            O.kmer_encode_batch(ot, sample, off, self.t_max, self.vocab["<pad>"])
+            reps += 1
+            if time.perf_counter() - t0 > budget_s:
+                break
+        dt = time.perf_counter() - t0
+        return rows * 6000 * reps / dt / 1e6, f"{rows // 256} batches of 256x6000 bp, {reps} passes"
+
+
+class BpePadded(Workload):
+    """C3 / C4: BPE encode, then fused remap + pad-to-longest + mask."""
+
+    def __init__(self, which: str, n_batches: int):
+        from dnatok_amd import bpe_vocab, encoders, hf_tokenizers as hf, workloads as wl
+        import torch
+        with open(hf.bpe_tokenizer_path(which)) as fh:
+            cfg = json.load(fh)
+        self.cfg = cfg
+        self.which = which
+        kv = bpe_vocab.KernelVocab(bpe_vocab.split_merges(cfg["model"]["merges"]))
+        vocab = cfg["model"]["vocab"]
+        self.pad_id = vocab["[PAD]"]
+        self.enc = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv),
+                                       out_remap=kv.remap_to(vocab, vocab["[UNK]"]))
+        if which == "4096":
+            rows, length, golden, seed0 = 1024, 1024, "C3_bpe4096", wl.SEEDS["C3"]
+            mk = wl.config3_bpe4096
+        else:
+            rows, length, golden, seed0 = 32, 100_000, "C4_bpe32000", wl.SEEDS["C4"]
+            mk = wl.config4_bpe32000
+        self.golden = golden
+        self.rows_per_batch, self.length = rows, length
+        parts = [mk().data] + [mk(rows, length, seed=seed0 + 100 + i).data for i in range(n_batches - 1)]
+        host = np.concatenate(parts)
+        self.host = host
+        self.n_rows = rows * n_batches
+        self.data = _dev(host)
+        self.off = _dev(np.arange(self.n_rows + 1, dtype=np.int64) * length)
+        self.tok = torch.empty(host.size, dtype=torch.int32, device="cuda")
+        self.lengths = torch.empty(self.n_rows, dtype=torch.int32, device="cuda")
+        self.t_cap = length
+        self.pad_out = (torch.empty((self.n_rows, length), dtype=torch.int32, device="cuda"),
+                        torch.empty((self.n_rows, length), dtype=torch.uint8, device="cuda"),
+                        torch.empty(1, dtype=torch.int32, device="cuda"))
+        self.bases = host.size
+        self.kernel = "bpe_lds_kernel" if length <= 4096 else "bpe_long_kernel"
+        self.name = (f"{'C3' if which == '4096' else 'C4'} BPE vocab-{which}, {rows}x{length} bp batches, "
+                     f"{n_batches} distinct batch(es) per call, pad to longest row")
+        self.step()
+        torch.cuda.synchronize()
+        t_max = int(self.max_len.item())
+        self.t_max = t_max
+        self.algorithmic_bytes = host.size + 5 * self.n_rows * t_max + 4 * self.n_rows
+
+    def step(self):
+        from dnatok_amd import encoders
+        self.enc.encode(self.data, self.off, self.length, tok_tmp=self.tok, lengths=self.lengths)
+        self.ids, self.mask, self.max_len = encoders.pad_rows(self.tok, self.off, self.lengths, self.pad_id,
+                                                              self.t_cap, fill_to=0, out=self.pad_out)
+
+    def check(self):
+        from tests.golden import check as util
+        ln = self.lengths.cpu().numpy()
+        rows = [self.ids[r, :ln[r]].cpu().numpy() for r in range(self.rows_per_batch)]
+        util.check_against_golden(self.golden, rows)
+        assert (ln > 0).all()
+
+    def cpu_baseline(self, budget_s: float):
+        from oracle import oracle as O
+        bo = O.bpe_oracle_from_tokenizer_json(self.cfg)
+        rows = min(self.n_rows, self.rows_per_batch)
+        sample = self.host[:rows * self.length]
+        off = np.arange(rows + 1, dtype=np.int64) * self.length
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            bo.encode_batch(sample, off)
+            reps += 1
+            if time.perf_counter() - t0 > budget_s:
+                break
+        dt = time.perf_counter() - t0
+        return rows * self.length * reps / dt / 1e6, f"1 batch of {rows}x{self.length} bp, {reps} passes"
+
+
+class RaggedBoth(Workload):
+    """C5: 4096 ragged sequences through the vocab-4096 BPE and the char tokenizer in one
+    pass over the same device buffer; packed ids + offsets + masks stay on the device."""
+
+    def __init__(self, n_batches: int = 1):
+        from dnatok_amd import bpe_vocab, encoders, hf_tokenizers as hf, workloads as wl
+        import torch
+        with open(hf.bpe_tokenizer_path("4096")) as fh:
+            cfg = json.load(fh)
+        self.cfg = cfg
+        kv = bpe_vocab.KernelVocab(bpe_vocab.split_merges(cfg["model"]["merges"]))
+        vocab = cfg["model"]["vocab"]
+        self.bpe = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv),
+                                       out_remap=kv.remap_to(vocab, vocab["[UNK]"]))
+        cv = hf.char_vocab()
+        lut = np.zeros(256, dtype=np.int32)
+        for ch in "ACGTN":
+            lut[ord(ch)] = cv[ch]
+        self.lut = lut
+        self.char = encoders.CharEncoder(lut, pad_id=cv["<pad>"])
+        b = wl.config5_ragged()
+        self.batch = b
+        self.data, self.off = _dev(b.data), _dev(b.offsets)
+        self.max_len = int(b.lengths().max())
+        self.tok = torch.empty(b.total, dtype=torch.int32, device="cuda")
+        self.lengths = torch.empty(b.n_seqs, dtype=torch.int32, device="cuda")
+        self.pack_out = (torch.empty(b.total, dtype=torch.int32, device="cuda"),
+                         torch.empty(b.n_seqs + 1, dtype=torch.int64, device="cuda"),
+                         torch.empty(b.total, dtype=torch.uint8, device="cuda"))
+        self.cids = torch.empty(b.total, dtype=torch.int32, device="cuda")
+        self.cmask = torch.empty(b.total, dtype=torch.uint8, device="cuda")
+        self.bases = b.total
+        self.kernel = "bpe_lds_kernel"
+        self.name = "C5 ragged 4096 sequences (~12 Mbp): BPE vocab-4096 + char, packed ids/offsets/masks"
+        self.step()
+        torch.cuda.synchronize()
+        n_tok = int(self.out_off[-1].item())
+        # input once; char: 4+1 B/base; BPE: 4+1 B/token; two offset arrays
+        self.algorithmic_bytes = b.total + 5 * b.total + 5 * n_tok + 2 * 8 * (b.n_seqs + 1)
+
+    def step(self):
+        from dnatok_amd import encoders
+        self.bpe.encode(self.data, self.off, self.max_len, tok_tmp=self.tok, lengths=self.lengths)
+        self.pids, self.out_off, self.pmask = encoders.pack_ragged(self.tok, self.off, self.lengths,
+                                                                   out=self.pack_out)
+        self.char.encode_packed(self.data, want_mask=True, ids=self.cids, mask=self.cmask)
+
+    def check(self):
+        from tests.golden import check as util
+        b = self.batch
+        oo, flat = self.out_off.cpu().numpy(), self.pids.cpu().numpy()
+        util.check_against_golden("C5_bpe4096", [flat[oo[i]:oo[i + 1]] for i in range(b.n_seqs)])
+        cf = self.cids.cpu().numpy()
+        util.check_against_golden("C5_char", [cf[b.offsets[i]:b.offsets[i + 1]] for i in range(b.n_seqs)])
+
+    def cpu_baseline(self, budget_s: float):
+        from oracle import oracle as O
+        bo = O.bpe_oracle_from_tokenizer_json(self.cfg)
+        b = self.batch
+        rows = 1024
+        data, off = b.data[:b.offsets[rows]], b.offsets[:rows + 1]
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            bo.encode_batch(data, off)
+            O.char_encode_packed(self.lut, data)
+            reps += 1
+            if time.perf_counter() - t0 > budget_s:
+                break
+        dt = time.perf_counter() - t0
+        return int(off[-1]) * reps / dt / 1e6, f"first {rows} sequences ({int(off[-1])} bp), {reps} passes"
+
+
+def make_workload(config: str, sustained: bool) -> Workload:
+    if config == "C1":
+        return CharDense(340 if sustained else 1)
+    if config == "C2":
+        return KmerPadded(128 if sustained else 1)
+    if config == "C3":
+        return BpePadded("4096", 16 if sustained else 1)
+    if config == "C4":
+        return BpePadded("32000", 1)
+    if config == "C5":
+        return RaggedBoth(1)
+    raise SystemExit(f"unknown config {config}")
+
+
+# ------------------------------------------------------------------------------ timing
+
+def time_steps(w: Workload, steps: int, warmup: int):
+    import torch
+    for _ in range(warmup):
+        w.step()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        w.step()
+    end.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    dev_ms = start.elapsed_time(end) / steps
+    return wall_ms, dev_ms
+
+
+def hf_cpu(config: str, threads: int, max_bases: int) -> dict | None:
+    env = dict(os.environ, RAYON_NUM_THREADS=str(threads), TOKENIZERS_PARALLELISM="true")
+    cmd = [sys.executable, "-m", "dnatok_amd.hf_baseline", "--config", config, "--budget", "12"]
+    if max_bases:
+        cmd += ["--max-bases", str(max_bases)]
+    try:
+        out = subprocess.run(cmd, env=env, cwd=ROOT, capture_output=True, text=True, timeout=240)
+        line = [l for l in out.stdout.splitlines() if l.startswith("{")][-1]
+        return json.loads(line)
+    except Exception as e:          # tokenizers missing or too slow: report that, invent nothing
+        return {"error": f"{type(e).__name__}: {e}"}
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="C2", choices=["C1", "C2", "C3", "C4", "C5"])
+    ap.add_argument("--per-call", action="store_true", help="time one exact batch instead of the sustained form")
+    ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this backend and this benchmark are single-GPU (rows are independent; "
+              "see DESIGN.md for how the path would shard). Run with --gpus 1.", file=sys.stderr)
+        raise SystemExit(2)
+
+    import torch
+    from dnatok_amd import _lib
+    _lib.lib()                                   # fail loudly if the HIP library is missing
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+
+    w = make_workload(args.config, sustained=not args.per_call)
+    w.step()
+    torch.cuda.synchronize()
+    w.check()                                    # bit-exact against the HF-written golden vectors
+    wall_ms, dev_ms = time_steps(w, args.steps, args.warmup)
+    value = w.bases / (wall_ms * 1e-3) / 1e6
+    achieved = w.algorithmic_bytes / (dev_ms * 1e-3) / 1e9
+
+    result = {
+        "metric": "encode Mbp/s on 1 MI355X (bit-exact vs HF) + % of HBM BW roofline",
+        "value": value, "unit": "Mbp/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8", "data": "synthetic",
+        "config": {"workload": w.name, "bases_per_step": int(w.bases),
+                   "algorithmic_bytes_per_step": int(w.algorithmic_bytes)},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": w.kernel,
+                     "device_ms_per_step": dev_ms},
+        "bit_exact_vs_golden": True,
+    }
+
+    if not args.no_cpu:
+        cores = os.cpu_count() or 1
+        v, sample = w.cpu_baseline(10.0)
+        result["cpu_baseline"] = {"value": v, "unit": "Mbp/s", "cores": 1, "kind": "port",
+                                  "sample": sample + " (C oracle, one thread)"}
+        cap = {"C1": 0, "C2": 0, "C3": 0, "C4": 400_000, "C5": 1_500_000}[args.config]
+        result["hf_tokenizers_cpu"] = {
+            "threads_1": hf_cpu(args.config, 1, cap), f"threads_{cores}": hf_cpu(args.config, cores, cap),
+            "host_cores": cores, "note": "Hugging Face tokenizers encode_batch on this host, own subprocess per thread count"}
+
+    if not args.no_extras:
+        per_call = {}
+        for cfg in ["C1", "C2", "C3", "C4", "C5"]:
+            ww = make_workload(cfg, sustained=False)
+            ww.step()
+            torch.cuda.synchronize()
+            ww.check()
+            wm, dm = time_steps(ww, 20, 3)
+            per_call[cfg] = {"workload": ww.name, "ms_per_call": wm, "device_ms_per_call": dm,
+                             "mbp_per_s": ww.bases / (wm * 1e-3) / 1e6,
+                             "hbm_frac": ww.algorithmic_bytes / (dm * 1e-3) / 1e9 / HBM_PEAK_GBS}
+            del ww
+            torch.cuda.empty_cache()
+        result["per_call"] = per_call
+        sustained = {}
+        for cfg in ["C1", "C3"]:
+            if cfg == args.config and not args.per_call:
+                continue
+            ww = make_workload(cfg, sustained=True)
+            wm, dm = time_steps(ww, 10, 2)
+            sustained[cfg] = {"workload": ww.name, "ms_per_step": wm, "mbp_per_s": ww.bases / (wm * 1e-3) / 1e6,
+                              "hbm_frac": ww.algorithmic_bytes / (dm * 1e-3) / 1e9 / HBM_PEAK_GBS}
+            del ww
+            torch.cuda.empty_cache()
+        result["sustained"] = sustained
+
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -210,15 +210,17 @@ class BpeEncoder:
 
 
 def pack_ragged(tok_tmp: torch.Tensor, in_offsets: torch.Tensor, lengths: torch.Tensor, *,
-                remap: Optional[torch.Tensor] = None, want_mask: bool = True,
-                ids_out: Optional[torch.Tensor] = None):
-    """Packed ids (capacity = tok_tmp.numel()), int64 offsets[B+1], mask; all on the device."""
+                remap: Optional[torch.Tensor] = None, want_mask: bool = True, out=None):
+    """Packed ids (capacity = tok_tmp.numel()), int64 offsets[B+1], mask; all on the device.
+    ``out`` = (ids_out, out_offsets, mask) reuses caller buffers."""
     n_rows = lengths.numel()
     dev = tok_tmp.device
-    if ids_out is None:
+    if out is not None:
+        ids_out, out_offsets, mask = out
+    else:
         ids_out = torch.empty(tok_tmp.numel(), dtype=torch.int32, device=dev)
-    out_offsets = torch.empty(n_rows + 1, dtype=torch.int64, device=dev)
-    mask = torch.empty(tok_tmp.numel(), dtype=torch.uint8, device=dev) if want_mask else None
+        out_offsets = torch.empty(n_rows + 1, dtype=torch.int64, device=dev)
+        mask = torch.empty(tok_tmp.numel(), dtype=torch.uint8, device=dev) if want_mask else None
     _lib.check(_lib.lib().dnatok_pack_ragged(_ptr(tok_tmp), _ptr(in_offsets), _ptr(lengths), n_rows,
                                              _ptr(remap), _ptr(ids_out), _ptr(out_offsets),
                                              _ptr(mask), _stream()), "dnatok_pack_ragged")
@@ -227,13 +229,17 @@ def pack_ragged(tok_tmp: torch.Tensor, in_offsets: torch.Tensor, lengths: torch.
 
 def pad_rows(tok_tmp: torch.Tensor, in_offsets: torch.Tensor, lengths: torch.Tensor, pad_id: int,
              t_cap: int, *, fill_to: int = 0, remap: Optional[torch.Tensor] = None,
-             want_mask: bool = True):
-    """Padded ids[B, t_cap] + mask + max_len[1]; with fill_to = 0 view ``ids[:, :max_len]``."""
+             want_mask: bool = True, out=None):
+    """Padded ids[B, t_cap] + mask + max_len[1]; with fill_to = 0 view ``ids[:, :max_len]``.
+    ``out`` = (ids, mask, max_len) reuses caller buffers."""
     n_rows = lengths.numel()
     dev = tok_tmp.device
-    ids = torch.empty((n_rows, t_cap), dtype=torch.int32, device=dev)
-    mask = torch.empty((n_rows, t_cap), dtype=torch.uint8, device=dev) if want_mask else None
-    max_len = torch.empty(1, dtype=torch.int32, device=dev)
+    if out is not None:
+        ids, mask, max_len = out
+    else:
+        ids = torch.empty((n_rows, t_cap), dtype=torch.int32, device=dev)
+        mask = torch.empty((n_rows, t_cap), dtype=torch.uint8, device=dev) if want_mask else None
+        max_len = torch.empty(1, dtype=torch.int32, device=dev)
     _lib.check(_lib.lib().dnatok_pad_rows(_ptr(tok_tmp), _ptr(in_offsets), _ptr(lengths), n_rows,
                                           _ptr(remap), int(pad_id), int(t_cap), int(fill_to),
                                           _ptr(ids), _ptr(mask), _ptr(max_len), _stream()),

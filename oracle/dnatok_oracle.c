@@ -121,6 +121,29 @@ int64_t oracle_kmer_encode_row(int k, const int8_t *digit, const int32_t *kmer_l
     return n;
 }
 
+/* Whole batch into a padded [n_rows, t_cap] matrix (ids + mask), rows padded to t_cap. */
+void oracle_kmer_encode_batch(int k, const int8_t *digit, const int32_t *kmer_lut,
+                              const int32_t *exp_off, const int32_t *exp_len,
+                              const int32_t *exp_flat, const int32_t *single,
+                              int32_t missing_id, int32_t pad_id, const uint8_t *bytes,
+                              const int64_t *offsets, int64_t n_rows, int64_t t_cap,
+                              int32_t *ids, uint8_t *mask, int32_t *lengths)
+{
+    for (int64_t b = 0; b < n_rows; ++b) {
+        int32_t st;
+        int32_t *o = ids + b * t_cap;
+        int64_t n = oracle_kmer_encode_row(k, digit, kmer_lut, exp_off, exp_len, exp_flat, single,
+                                           missing_id, bytes + offsets[b],
+                                           offsets[b + 1] - offsets[b], o, t_cap, &st);
+        lengths[b] = (int32_t)n;
+        if (n > t_cap) n = t_cap;
+        for (int64_t j = 0; j < t_cap; ++j) {
+            if (j >= n) o[j] = pad_id;
+            if (mask) mask[b * t_cap + j] = j < n;
+        }
+    }
+}
+
 /* ------------------------------------------------------------------- BPE */
 
 typedef struct {

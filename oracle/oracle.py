@@ -147,6 +147,22 @@ def kmer_encode(t: KmerTables, data: np.ndarray, offsets: np.ndarray
     return rows, status
 
 
+def kmer_encode_batch(t: KmerTables, data: np.ndarray, offsets: np.ndarray, t_cap: int,
+                      pad_id: int) -> Tuple[np.ndarray, np.ndarray, np.ndarray]:
+    """Whole batch in one C call: padded ids [B, t_cap], mask, lengths."""
+    offsets = np.ascontiguousarray(offsets, dtype=np.int64)
+    b = offsets.size - 1
+    ids = np.empty((b, t_cap), dtype=np.int32)
+    mask = np.empty((b, t_cap), dtype=np.uint8)
+    lengths = np.empty(b, dtype=np.int32)
+    lib().oracle_kmer_encode_batch(
+        ctypes.c_int(t.k), _p(t.digit), _p(t.kmer_lut), _p(t.exp_off), _p(t.exp_len),
+        _p(t.exp_flat), _p(t.single), ctypes.c_int32(t.missing_id), ctypes.c_int32(pad_id),
+        _p(data), _p(offsets), ctypes.c_int64(b), ctypes.c_int64(t_cap), _p(ids), _p(mask),
+        _p(lengths))
+    return ids, mask, lengths
+
+
 def pad_rows(rows: Sequence[np.ndarray], pad_id: int, t_out: int | None = None
              ) -> Tuple[np.ndarray, np.ndarray]:
     """Right-pad to the longest row: ids int32 [B,T], mask uint8 [B,T]

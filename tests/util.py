@@ -1,7 +1,6 @@
 """Shared helpers of the test suite: golden fixtures, oracle tables, HF tokenizers."""
 from __future__ import annotations
 
-import hashlib
 import json
 import os
 from functools import lru_cache
@@ -12,12 +11,7 @@ from dnatok_amd import hf_tokenizers as hf
 from dnatok_amd import workloads as wl
 from oracle import oracle as O
 
-GOLDEN_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
-
-
-@lru_cache(maxsize=None)
-def golden():
-    return dict(np.load(os.path.join(GOLDEN_DIR, "golden_vectors.npz"), allow_pickle=False))
+from tests.golden.check import GOLDEN_DIR, check_against_golden, golden, sha_of_rows  # noqa: F401
 
 
 @lru_cache(maxsize=None)
@@ -45,20 +39,6 @@ def char_lut(fold_case: bool = False) -> np.ndarray:
         if fold_case:
             lut[ord(ch.lower())] = vocab[ch]
     return lut
-
-
-def sha_of_rows(rows) -> np.ndarray:
-    flat = np.concatenate([np.asarray(r, dtype=np.int32) for r in rows]) if len(rows) else np.zeros(0, np.int32)
-    return np.frombuffer(hashlib.sha256(flat.astype("<i4").tobytes()).digest(), dtype=np.uint8)
-
-
-def check_against_golden(name: str, rows) -> None:
-    g = golden()
-    lengths = np.array([len(r) for r in rows], dtype=np.int32)
-    np.testing.assert_array_equal(lengths, g[name + "_lengths"], err_msg=name + " lengths")
-    np.testing.assert_array_equal(np.asarray(rows[0][:2048], dtype=np.int32), g[name + "_row0"],
-                                  err_msg=name + " row 0")
-    np.testing.assert_array_equal(sha_of_rows(rows), g[name + "_sha256"], err_msg=name + " sha256")
 
 
 def small_cases():
