@@ -30,6 +30,24 @@ void set_error(const char *fmt, ...);
 
 constexpr int kWave = 64;
 
+// Workgroups of `kernel` that are resident at once on the current device (all CUs), for
+// persistent launches: a grid of exactly this size runs as one wave of workgroups.
+template <typename Kernel>
+inline int resident_workgroups(Kernel kernel, int block_threads, size_t dynamic_lds, int fallback_per_cu)
+{
+    int dev = 0, cus = 256, per_cu = 0;
+    if (hipGetDevice(&dev) == hipSuccess) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
+    }
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, block_threads, dynamic_lds) != hipSuccess ||
+        per_cu <= 0) {
+        (void)hipGetLastError();
+        per_cu = fallback_per_cu;
+    }
+    return cus * per_cu;
+}
+
 // ---- wave64 cross-lane primitives (DPP within rows of 16 lanes, readlane across rows) ----
 
 template <int CTRL>
@@ -55,16 +73,30 @@ __device__ __forceinline__ uint32_t wave_min_u32(uint32_t v)
     return umin(umin(r0, r1), umin(r2, r3));
 }
 
-// Inclusive prefix sum over the 64 lanes.
+// row_shr:N within each row of 16 lanes; lanes without a source read 0.
+template <int N>
+__device__ __forceinline__ uint32_t dpp_row_shr_zero(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x110 + N, 0xF, 0xF, true);
+}
+
+// Inclusive prefix sum over the 64 lanes: DPP scan inside each row of 16, then the three
+// row totals are carried across with readlane.
 __device__ __forceinline__ uint32_t wave_inclusive_sum_u32(uint32_t v)
 {
-    const int lane = threadIdx.x & 63;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        uint32_t o = __shfl_up(v, d, 64);
-        if (lane >= d) v += o;
-    }
-    return v;
+    v += dpp_row_shr_zero<1>(v);
+    v += dpp_row_shr_zero<2>(v);
+    v += dpp_row_shr_zero<4>(v);
+    v += dpp_row_shr_zero<8>(v);
+    const uint32_t t0 = __builtin_amdgcn_readlane(v, 15);
+    const uint32_t t1 = __builtin_amdgcn_readlane(v, 31);
+    const uint32_t t2 = __builtin_amdgcn_readlane(v, 47);
+    const uint32_t row = (threadIdx.x & 63) >> 4;
+    uint32_t carry = 0;
+    if (row >= 1) carry += t0;
+    if (row >= 2) carry += t1;
+    if (row >= 3) carry += t2;
+    return v + carry;
 }
 
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v)

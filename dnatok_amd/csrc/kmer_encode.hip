@@ -1,16 +1,25 @@
 // Non-overlapping k-mer encoder with per-window fallback, tail handling, padding and mask.
 //
-// One workgroup walks one row in tiles of 1024 units (a unit is a k-base window, or one of
+// Persistent workgroups stage the tables in LDS once; after that every wave works alone:
+// it takes a row and walks it in steps of 256 units (a unit is a k-base window, or one of
 // the trailing len % k characters).  Each lane owns 4 consecutive units: it loads its 4k
-// bytes, turns them into base-5 digits through an LDS digit table, and looks the window up
-// in an LDS table of the 4^k N-free windows; a window holding N (or a byte outside the
-// alphabet) goes through the global 5^k table and, when that entry is -1, is spelled out
-// from the expansion lists.  Unit token counts are prefix-summed across the workgroup
-// (wave64 scan + LDS carry), so every lane knows where its tokens land and a lane whose 4
-// windows are plain writes one aligned 16-byte store.  Traffic: 1 byte read per base,
-// 5 bytes written per token.
+// bytes, turns them into base-5 digits through the LDS digit table, and looks the window up
+// in the LDS table of the 4^k N-free windows.
+//
+//   * Step without exceptions (the common case): every lane holds 4 plain windows, so token
+//     positions are known without a scan and each lane issues one 16-byte id store and one
+//     4-byte mask store (a wave covers 1 KiB + 256 B contiguous).
+//   * Step with exceptions (a window holding N or a byte outside the alphabet, a window
+//     without an id, the ragged end of a row): unit token counts are prefix-summed across
+//     the wave with a DPP scan (no barrier) and every lane writes at its own offset.  When
+//     the table spells every non-plain window character by character (the usual grid-aligned
+//     tokenizer), the spelled tokens come from 5 LDS entries; otherwise from the global
+//     5^k entry table and its expansion lists.
+//
+// Traffic: 1 byte read per base, 5 bytes written per token.
 #include "common.hpp"
 
+#include <limits.h>
 #include <string.h>
 #include <vector>
 
@@ -18,75 +27,86 @@ struct dnatok_kmer_table {
     int k;
     int64_t pow4, pow5;
     int32_t pad_id, missing_id;
-    int has_exp;
+    int chars_mode;          // every non-plain window expands to its own characters
     void *blob;              // one device allocation holding all tables
     int8_t *digit;           // [256]
     int32_t *single;         // [256]
     int32_t *lut4;           // [4^k]  id of an ACGT-only window, or -1
-    int32_t *lut5;           // [5^k]
-    int32_t *exp_off, *exp_len, *exp_flat;
+    int2 *entry;             // [5^k]  {id, 0} | {-len, offset into flat} | {INT_MIN, 0} = nothing known
+    int32_t *flat;           // expansion lists
 };
 
 namespace dnatok {
 
 struct KmerArgs {
     const int8_t *digit;
-    const int32_t *single, *lut4, *lut5, *exp_off, *exp_len, *exp_flat;
+    const int32_t *single, *lut4;
+    const int2 *entry;
+    const int32_t *flat;
     int32_t pad_id, missing_id;
 };
 
 constexpr int kKmerThreads = 256;
 constexpr int kUnitsPerLane = 4;
-constexpr int kTileUnits = kKmerThreads * kUnitsPerLane;
+constexpr int kWaveUnits = 64 * kUnitsPerLane;          // units one wave handles per step
+
+// LDS digit entries: 0..3 for A C G T; flags above every window code (4^8 = 1 << 16) for N and
+// for a byte outside the alphabet, so that "window code < 4^k" means "k plain bases".
+constexpr uint32_t kDigN = 1u << 16;
+constexpr uint32_t kDigBad = 1u << 17;
 
 typedef int32_t int4v __attribute__((ext_vector_type(4)));
+// the same vectors at element alignment: a row's token position is not a multiple of 4 once a
+// window has expanded, and global stores only need the element alignment
+typedef int32_t int4v_a4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t u32_a1 __attribute__((aligned(1)));
 
 __global__ void zero_i32_kernel(int32_t *p) { *p = 0; }
 
-// Exclusive prefix sum of one value per thread over the workgroup; total in *total_out.
-__device__ __forceinline__ uint32_t block_exclusive_sum(uint32_t v, uint32_t *wave_tot, uint32_t *total_out)
+__device__ __forceinline__ void store4(int32_t *out, uint8_t *mout, int64_t p, const int32_t *t)
 {
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    const uint32_t inc = wave_inclusive_sum_u32(v);
-    if (lane == 63) wave_tot[wv] = inc;
-    __syncthreads();
-    uint32_t carry = 0, total = 0;
-#pragma unroll
-    for (int i = 0; i < kKmerThreads / 64; ++i) {
-        const uint32_t t = wave_tot[i];
-        if (i < wv) carry += t;
-        total += t;
-    }
-    __syncthreads();   // wave_tot is reused by the next tile
-    *total_out = total;
-    return carry + inc - v;
+    int4v_a4 v = {t[0], t[1], t[2], t[3]};
+    __builtin_nontemporal_store(v, reinterpret_cast<int4v_a4 *>(out + p));
+    if (mout) __builtin_nontemporal_store((u32_a1)0x01010101u, reinterpret_cast<u32_a1 *>(mout + p));
 }
 
-template <int K, bool LUT4_LDS>
+__device__ __forceinline__ void store1(int32_t *out, uint8_t *mout, int64_t p, int64_t t_cap, int32_t v)
+{
+    if (p < t_cap) {
+        out[p] = v;
+        if (mout) mout[p] = 1;
+    }
+}
+
+template <int K, bool LUT4_LDS, bool CHARS>
 __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
     KmerArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
     int64_t n_rows, int64_t t_cap, int64_t fill_to, int32_t *__restrict__ ids,
     uint8_t *__restrict__ mask, int32_t *__restrict__ lengths, int32_t *__restrict__ status,
     int32_t *__restrict__ max_len)
 {
-    constexpr int POW4 = 1 << (2 * K);
-    __shared__ int8_t s_digit[256];
+    constexpr uint32_t POW4 = 1u << (2 * K);
+    __shared__ uint32_t s_dig[256];
     __shared__ int32_t s_single[256];
     __shared__ int32_t s_lut4[LUT4_LDS ? POW4 : 1];
-    __shared__ uint32_t s_wave_tot[kKmerThreads / 64];
-    __shared__ int32_t s_status;
+    __shared__ int32_t s_spell[8];       // token of the characters A C G T N
 
-    s_digit[threadIdx.x] = a.digit[threadIdx.x];
-    s_single[threadIdx.x] = a.single[threadIdx.x];
+    for (int i = threadIdx.x; i < 256; i += kKmerThreads) {
+        const int d = a.digit[i];
+        s_dig[i] = d < 0 ? kDigBad : (d >= 4 ? kDigN : (uint32_t)d);
+        s_single[i] = a.single[i];
+    }
+    if (threadIdx.x < 5) s_spell[threadIdx.x] = a.single[(int)"ACGTN"[threadIdx.x]];
     if (LUT4_LDS)
-        for (int i = threadIdx.x; i < POW4; i += kKmerThreads) s_lut4[i] = a.lut4[i];
-    if (threadIdx.x == 0) s_status = 0;
-    __syncthreads();
+        for (uint32_t i = threadIdx.x; i < POW4; i += kKmerThreads) s_lut4[i] = a.lut4[i];
+    __syncthreads();          // the only workgroup barrier: from here on every wave runs alone
 
-    const bool ids_aligned = (((uintptr_t)ids & 15) == 0) && (t_cap % 4 == 0);
-    const bool mask_aligned = mask && (((uintptr_t)mask & 3) == 0) && (t_cap % 4 == 0);
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * (kKmerThreads / 64) + (threadIdx.x >> 6);
+    const int64_t n_waves = (int64_t)gridDim.x * (kKmerThreads / 64);
+    int64_t wave_max = 0;
 
-    for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
+    for (int64_t row = wave; row < n_rows; row += n_waves) {
         const int64_t row_start = offsets[row];
         const int64_t len = offsets[row + 1] - row_start;
         const int64_t full = len / K;
@@ -97,110 +117,211 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
         int64_t running = 0;
         int32_t my_status = 0;
 
-        for (int64_t u0 = 0; u0 < n_units; u0 += kTileUnits) {
-            const int64_t ub = u0 + (int64_t)threadIdx.x * kUnitsPerLane;
-            int32_t tok[kUnitsPerLane];     // the unit's token when cnt == 1
-            int32_t cnt[kUnitsPerLane];     // tokens the unit produces
-            int32_t code5[kUnitsPerLane];   // window code for units that expand
-            uint32_t lane_cnt = 0;
-
-            uint8_t ch[kUnitsPerLane * K];
-            if (ub + kUnitsPerLane <= full) {
-                uint32_t w[K];
-                memcpy(w, src + ub * K, 4 * K);           // 4 windows = 4K bytes, unaligned
+        for (int64_t u0 = 0; u0 < n_units; u0 += kWaveUnits) {
+            const int64_t ub = u0 + (int64_t)lane * kUnitsPerLane;
+            const bool lane_full = ub + kUnitsPerLane <= full;     // 4 whole windows
+            const bool empty = ub >= n_units;
+            uint32_t w[K];
 #pragma unroll
-                for (int i = 0; i < kUnitsPerLane * K; ++i)
-                    ch[i] = (uint8_t)((w[i >> 2] >> (8 * (i & 3))) & 255u);
-            } else {
-#pragma unroll
-                for (int j = 0; j < kUnitsPerLane; ++j) {
-                    const int64_t u = ub + j;
-#pragma unroll
-                    for (int i = 0; i < K; ++i)
-                        ch[j * K + i] = (u < full) ? src[u * K + i] : (uint8_t)0;
-                }
-            }
+            for (int i = 0; i < K; ++i) w[i] = 0;          // byte 0 is never a base
+            if (lane_full) memcpy(w, src + ub * K, 4 * K);  // 4 windows = 4K bytes, unaligned
+            uint32_t dig[kUnitsPerLane * K];
+            uint32_t code[kUnitsPerLane];
 #pragma unroll
             for (int j = 0; j < kUnitsPerLane; ++j) {
-                const int64_t u = ub + j;
-                tok[j] = 0; cnt[j] = 0; code5[j] = -1;
-                if (u < full) {
-                    int c4 = 0, c5 = 0;
-                    bool plain = true;
+                uint32_t c = 0;
 #pragma unroll
-                    for (int i = 0; i < K; ++i) {
-                        int d = s_digit[ch[j * K + i]];
-                        if (d < 0) { d = 4; my_status |= DNATOK_ROW_INVALID_BYTE; }
-                        plain = plain && (d < 4);
-                        c4 = (c4 << 2) | (d & 3);
-                        c5 = c5 * 5 + d;
-                    }
-                    int32_t id = -1;
-                    if (plain) id = LUT4_LDS ? s_lut4[c4] : a.lut4[c4];
-                    if (id < 0) id = a.lut5[c5];
-                    if (id >= 0) {
-                        tok[j] = id; cnt[j] = 1;
-                    } else if (a.exp_len && a.exp_len[c5] > 0) {
-                        cnt[j] = a.exp_len[c5]; code5[j] = c5;
-                    } else {
-                        tok[j] = a.missing_id; cnt[j] = 1; my_status |= DNATOK_ROW_MISSING_KMER;
-                    }
-                } else if (u < n_units) {
-                    tok[j] = s_single[src[full * K + (u - full)]];
-                    cnt[j] = 1;
+                for (int i = 0; i < K; ++i) {
+                    const int bi = j * K + i;
+                    dig[bi] = s_dig[(w[bi >> 2] >> (8 * (bi & 3))) & 255u];
+                    c = (c << 2) + dig[bi];
                 }
-                lane_cnt += (uint32_t)cnt[j];
+                code[j] = c;
+            }
+            int32_t t[kUnitsPerLane];
+#pragma unroll
+            for (int j = 0; j < kUnitsPerLane; ++j) {
+                const uint32_t idx = code[j] & (POW4 - 1);
+                t[j] = LUT4_LDS ? s_lut4[idx] : a.lut4[idx];
+            }
+            const uint32_t any_flag = code[0] | code[1] | code[2] | code[3];
+            const bool fast = lane_full && any_flag < POW4 && (t[0] | t[1] | t[2] | t[3]) >= 0;
+            const uint64_t fast_mask = __ballot(fast);
+            const uint64_t rest_mask = __ballot(!fast && !empty);
+
+            if (rest_mask == 0) {
+                // every lane is plain or past the end: positions are known without a scan
+                const int64_t p = running + (int64_t)lane * kUnitsPerLane;
+                if (fast) {
+                    if (p + 4 <= t_cap) {
+                        store4(out, mout, p, t);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < kUnitsPerLane; ++j) store1(out, mout, p + j, t_cap, t[j]);
+                    }
+                }
+                running += (int64_t)kUnitsPerLane * __popcll(fast_mask);
+                continue;
             }
 
-            uint32_t tile_total;
-            const uint32_t off = block_exclusive_sum(lane_cnt, s_wave_tot, &tile_total);
-            int64_t p = running + off;
-            if (lane_cnt == kUnitsPerLane && code5[0] < 0 && code5[1] < 0 && code5[2] < 0 &&
-                code5[3] < 0 && (p & 3) == 0 && p + 4 <= t_cap && ids_aligned) {
-                int4v v = {tok[0], tok[1], tok[2], tok[3]};
-                __builtin_nontemporal_store(v, reinterpret_cast<int4v *>(out + p));
-                if (mask_aligned)
-                    __builtin_nontemporal_store(0x01010101u, reinterpret_cast<uint32_t *>(mout + p));
-                else if (mout) { mout[p] = 1; mout[p + 1] = 1; mout[p + 2] = 1; mout[p + 3] = 1; }
-            } else {
+            // ---- step with exceptions ----
+            // per unit: cnt = number of tokens; ex/ey = entry of a window that is not plain
+            int32_t cnt[kUnitsPerLane], ex[kUnitsPerLane], ey[kUnitsPerLane];
+            uint32_t lane_cnt = 0;
+            if (lane_full) {
 #pragma unroll
                 for (int j = 0; j < kUnitsPerLane; ++j) {
-                    if (code5[j] < 0) {
-                        if (cnt[j] == 1) {
-                            if (p < t_cap) { out[p] = tok[j]; if (mout) mout[p] = 1; }
-                            ++p;
-                        }
+                    ex[j] = 0; ey[j] = 0;
+                    if (code[j] < POW4 && t[j] >= 0) {
+                        cnt[j] = 1;
+                    } else if (CHARS) {
+                        cnt[j] = K;
                     } else {
-                        const int32_t eo = a.exp_off[code5[j]];
-                        for (int e = 0; e < cnt[j]; ++e) {
-                            if (p < t_cap) { out[p] = a.exp_flat[eo + e]; if (mout) mout[p] = 1; }
-                            ++p;
+                        int c5 = 0;
+#pragma unroll
+                        for (int i = 0; i < K; ++i) {
+                            const uint32_t v = dig[j * K + i];
+                            c5 = c5 * 5 + ((v & (kDigN | kDigBad)) ? 4 : (int)v);
                         }
+                        const int2 e = a.entry[c5];
+                        ex[j] = e.x; ey[j] = e.y;
+                        cnt[j] = e.x >= 0 ? 1 : (e.x == INT_MIN ? 1 : -e.x);
+                        if (e.x == INT_MIN) my_status |= DNATOK_ROW_MISSING_KMER;
+                    }
+                    if ((code[j] >> 17) != 0) {
+                        // some digit may carry the foreign-byte flag (bit 17, shifted left by 0..2(K-1))
+                        bool bad = false;
+#pragma unroll
+                        for (int i = 0; i < K; ++i) bad = bad || (dig[j * K + i] & kDigBad);
+                        if (bad) my_status |= DNATOK_ROW_INVALID_BYTE;
+                    }
+                    lane_cnt += (uint32_t)cnt[j];
+                }
+            } else if (!empty) {
+                // the ragged end of the row: whole windows first, then single characters
+#pragma unroll 1
+                for (int j = 0; j < kUnitsPerLane; ++j) {
+                    const int64_t u = ub + j;
+                    int n = 0;
+                    if (u < full) {
+                        uint32_t c = 0;
+                        int c5 = 0;
+#pragma unroll
+                        for (int i = 0; i < K; ++i) {
+                            const uint32_t v = s_dig[src[u * K + i]];
+                            c = (c << 2) + v;
+                            if (v & kDigBad) my_status |= DNATOK_ROW_INVALID_BYTE;
+                            c5 = c5 * 5 + ((v & (kDigN | kDigBad)) ? 4 : (int)v);
+                        }
+                        int32_t id = -1;
+                        if (c < POW4) id = LUT4_LDS ? s_lut4[c] : a.lut4[c];
+                        if (id >= 0) {
+                            n = 1;
+                        } else {
+                            const int2 e = a.entry[c5];
+                            n = e.x >= 0 ? 1 : (e.x == INT_MIN ? 1 : -e.x);
+                            if (e.x == INT_MIN) my_status |= DNATOK_ROW_MISSING_KMER;
+                        }
+                    } else if (u < n_units) {
+                        n = 1;
+                    }
+                    lane_cnt += (uint32_t)n;
+                }
+            }
+
+            const uint32_t inc = wave_inclusive_sum_u32(lane_cnt);
+            const uint32_t step_total = __builtin_amdgcn_readlane(inc, 63);
+            int64_t p = running + (inc - lane_cnt);
+
+            if (fast) {
+                if (p + 4 <= t_cap) {
+                    store4(out, mout, p, t);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < kUnitsPerLane; ++j) store1(out, mout, p + j, t_cap, t[j]);
+                }
+            } else if (lane_full) {
+#pragma unroll
+                for (int j = 0; j < kUnitsPerLane; ++j) {
+                    if (code[j] < POW4 && t[j] >= 0) {
+                        store1(out, mout, p, t_cap, t[j]);
+                        ++p;
+                    } else if (CHARS) {
+#pragma unroll
+                        for (int i = 0; i < K; ++i) {
+                            const uint32_t v = dig[j * K + i];
+                            store1(out, mout, p + i, t_cap, s_spell[(v & (kDigN | kDigBad)) ? 4 : v]);
+                        }
+                        p += K;
+                    } else if (ex[j] >= 0) {
+                        store1(out, mout, p, t_cap, ex[j]);
+                        ++p;
+                    } else if (ex[j] == INT_MIN) {
+                        store1(out, mout, p, t_cap, a.missing_id);
+                        ++p;
+                    } else {
+                        for (int e = 0; e < -ex[j]; ++e) store1(out, mout, p + e, t_cap, a.flat[ey[j] + e]);
+                        p += -ex[j];
+                    }
+                }
+            } else if (!empty) {
+#pragma unroll 1
+                for (int j = 0; j < kUnitsPerLane; ++j) {
+                    const int64_t u = ub + j;
+                    if (u < full) {
+                        uint32_t c = 0;
+                        int c5 = 0;
+#pragma unroll
+                        for (int i = 0; i < K; ++i) {
+                            const uint32_t v = s_dig[src[u * K + i]];
+                            c = (c << 2) + v;
+                            c5 = c5 * 5 + ((v & (kDigN | kDigBad)) ? 4 : (int)v);
+                        }
+                        int32_t id = -1;
+                        if (c < POW4) id = LUT4_LDS ? s_lut4[c] : a.lut4[c];
+                        if (id >= 0) {
+                            store1(out, mout, p, t_cap, id);
+                            ++p;
+                        } else {
+                            const int2 e = a.entry[c5];
+                            if (e.x >= 0 || e.x == INT_MIN) {
+                                store1(out, mout, p, t_cap, e.x >= 0 ? e.x : a.missing_id);
+                                ++p;
+                            } else {
+                                for (int q = 0; q < -e.x; ++q) store1(out, mout, p + q, t_cap, a.flat[e.y + q]);
+                                p += -e.x;
+                            }
+                        }
+                    } else if (u < n_units) {
+                        store1(out, mout, p, t_cap, s_single[src[full * K + (u - full)]]);
+                        ++p;
                     }
                 }
             }
-            running += tile_total;
+            running += step_total;
         }
 
-        if (my_status) atomicOr(&s_status, my_status);
-        __syncthreads();
         const int64_t stored = running < t_cap ? running : t_cap;
-        if (threadIdx.x == 0) {
-            int32_t st = s_status;
-            if (running > t_cap) st |= DNATOK_ROW_TRUNCATED;
+        int32_t st = 0;
+        if (__ballot(my_status & DNATOK_ROW_INVALID_BYTE)) st |= DNATOK_ROW_INVALID_BYTE;
+        if (__ballot(my_status & DNATOK_ROW_MISSING_KMER)) st |= DNATOK_ROW_MISSING_KMER;
+        if (running > t_cap) st |= DNATOK_ROW_TRUNCATED;
+        if (lane == 0) {
             lengths[row] = (int32_t)running;
             if (status) status[row] = st;
-            if (max_len) atomicMax(max_len, (int32_t)stored);
-            s_status = 0;
         }
+        if (stored > wave_max) wave_max = stored;
         if (fill_to > 0) {
-            for (int64_t p = stored + threadIdx.x; p < fill_to; p += kKmerThreads) {
+            for (int64_t p = stored + lane; p < fill_to; p += 64) {
                 out[p] = a.pad_id;
                 if (mout) mout[p] = 0;
             }
         }
-        __syncthreads();
     }
+    // one atomic per wave at most, skipped when another wave already published a larger value
+    if (max_len && lane == 0 && wave_max > 0 &&
+        (int64_t)__builtin_nontemporal_load(max_len) < wave_max)
+        atomicMax(max_len, (int32_t)wave_max);
 }
 
 // Pads every row from its stored length up to the batch maximum found on the device.
@@ -273,25 +394,43 @@ extern "C" int dnatok_kmer_table_create(int k, const int8_t *digit_h, const int3
         for (int i = k - 1; i >= 0; --i) c5 = c5 * 5 + ((c4 >> (2 * i)) & 3);
         lut4[c4] = kmer_lut_h[c5];
     }
+    // entry[c5]: one 8-byte record per window, and whether every window without an id is
+    // spelled by its own characters (then the kernel never reads entry / flat)
+    std::vector<int2> entry(pow5);
+    const char alphabet[6] = "ACGTN";
+    bool chars_mode = true;
+    for (int64_t c = 0; c < pow5; ++c) {
+        if (kmer_lut_h[c] >= 0) {
+            entry[c] = int2{kmer_lut_h[c], 0};
+            bool has_n = false;
+            int64_t v = c;
+            for (int i = 0; i < k; ++i, v /= 5) has_n = has_n || (v % 5 == 4);
+            if (has_n) chars_mode = false;             // an N window with an id of its own
+        } else if (has_exp && exp_len_h[c] > 0) {
+            entry[c] = int2{-exp_len_h[c], exp_off_h[c]};
+            bool spelled = exp_len_h[c] == k;
+            int64_t v = c;
+            for (int i = k - 1; i >= 0 && spelled; --i, v /= 5)
+                spelled = exp_flat_h[exp_off_h[c] + i] == single_h[(int)alphabet[v % 5]];
+            if (!spelled) chars_mode = false;
+        } else {
+            entry[c] = int2{INT_MIN, 0};
+            chars_mode = false;
+        }
+    }
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
     const size_t o_digit = 0;
     const size_t o_single = up(o_digit + 256);
     const size_t o_lut4 = up(o_single + 256 * 4);
-    const size_t o_lut5 = up(o_lut4 + pow4 * 4);
-    const size_t o_eoff = up(o_lut5 + pow5 * 4);
-    const size_t o_elen = up(o_eoff + (has_exp ? pow5 * 4 : 0));
-    const size_t o_flat = up(o_elen + (has_exp ? pow5 * 4 : 0));
+    const size_t o_entry = up(o_lut4 + pow4 * 4);
+    const size_t o_flat = up(o_entry + pow5 * sizeof(int2));
     const size_t bytes = up(o_flat + (has_exp ? n_flat * 4 : 0)) + 256;
     std::vector<uint8_t> host(bytes, 0);
     memcpy(&host[o_digit], digit_h, 256);
     memcpy(&host[o_single], single_h, 256 * 4);
     memcpy(&host[o_lut4], lut4.data(), pow4 * 4);
-    memcpy(&host[o_lut5], kmer_lut_h, pow5 * 4);
-    if (has_exp) {
-        memcpy(&host[o_eoff], exp_off_h, pow5 * 4);
-        memcpy(&host[o_elen], exp_len_h, pow5 * 4);
-        memcpy(&host[o_flat], exp_flat_h, n_flat * 4);
-    }
+    memcpy(&host[o_entry], entry.data(), pow5 * sizeof(int2));
+    if (has_exp) memcpy(&host[o_flat], exp_flat_h, n_flat * 4);
     void *blob = nullptr;
     hipError_t e = hipMalloc(&blob, bytes);
     if (e == hipSuccess) e = hipMemcpy(blob, host.data(), bytes, hipMemcpyHostToDevice);
@@ -303,14 +442,12 @@ extern "C" int dnatok_kmer_table_create(int k, const int8_t *digit_h, const int3
     dnatok_kmer_table *t = new dnatok_kmer_table();
     uint8_t *b = (uint8_t *)blob;
     t->k = k; t->pow4 = pow4; t->pow5 = pow5; t->pad_id = pad_id; t->missing_id = missing_id;
-    t->has_exp = has_exp; t->blob = blob;
+    t->chars_mode = chars_mode; t->blob = blob;
     t->digit = (int8_t *)(b + o_digit);
     t->single = (int32_t *)(b + o_single);
     t->lut4 = (int32_t *)(b + o_lut4);
-    t->lut5 = (int32_t *)(b + o_lut5);
-    t->exp_off = has_exp ? (int32_t *)(b + o_eoff) : nullptr;
-    t->exp_len = has_exp ? (int32_t *)(b + o_elen) : nullptr;
-    t->exp_flat = has_exp ? (int32_t *)(b + o_flat) : nullptr;
+    t->entry = (int2 *)(b + o_entry);
+    t->flat = (int32_t *)(b + o_flat);
     *out = t;
     return DNATOK_OK;
 }
@@ -340,12 +477,21 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
         int rc = launch_zero_i32(max_len, s);
         if (rc) return rc;
     }
-    KmerArgs a{t->digit, t->single, t->lut4, t->lut5, t->exp_off, t->exp_len, t->exp_flat,
-               t->pad_id, t->missing_id};
-    int64_t grid = n_rows < 256 * 64 ? n_rows : 256 * 64;
-#define LAUNCH(KK, L)                                                                            \
-    kmer_rows_kernel<KK, L><<<(int)grid, kKmerThreads, 0, s>>>(a, bytes, offsets, n_rows, t_cap, \
-                                                               fill_to, ids, mask, lengths, status, max_len)
+    KmerArgs a{t->digit, t->single, t->lut4, t->entry, t->flat, t->pad_id, t->missing_id};
+    // persistent waves: the tables are staged into LDS once per workgroup, rows are dealt
+    // round-robin to waves
+    const int64_t want = (n_rows + kKmerThreads / 64 - 1) / (kKmerThreads / 64);
+#define LAUNCH2(KK, L, C)                                                                         \
+    do {                                                                                          \
+        static const int resident = resident_workgroups(kmer_rows_kernel<KK, L, C>, kKmerThreads, 0, 4); \
+        const int64_t grid = want < resident ? want : resident;                                   \
+        kmer_rows_kernel<KK, L, C><<<(int)grid, kKmerThreads, 0, s>>>(                            \
+            a, bytes, offsets, n_rows, t_cap, fill_to, ids, mask, lengths, status, max_len);      \
+    } while (0)
+#define LAUNCH(KK, L)                                                                             \
+    do {                                                                                          \
+        if (t->chars_mode) LAUNCH2(KK, L, true); else LAUNCH2(KK, L, false);                      \
+    } while (0)
     switch (t->k) {
         case 2: LAUNCH(2, true); break;
         case 3: LAUNCH(3, true); break;
@@ -356,6 +502,7 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
         default: LAUNCH(8, false); break;
     }
 #undef LAUNCH
+#undef LAUNCH2
     DNATOK_HIP_TRY(hipGetLastError());
     if (fill_to == 0) return launch_pad_to_max(ids, mask, lengths, n_rows, t_cap, max_len, t->pad_id, s);
     return DNATOK_OK;

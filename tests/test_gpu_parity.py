@@ -162,6 +162,47 @@ def test_kmer_ragged_all_k(k):
         np.testing.assert_array_equal(mask[:, :width].cpu().numpy(), emask)
 
 
+def test_kmer_general_tables_not_spelled():
+    """Tables whose N windows are not spelled character by character: N windows that have an
+    id of their own, expansions of other lengths, and windows with nothing at all."""
+    say("kmer general (non-spelled) tables")
+    k = 4
+    vocab = hf.kmer_vocab(k)
+
+    def tok(batch):
+        out = []
+        for s in batch:
+            if len(s) == k and "N" not in s:
+                out.append([vocab[s]])
+            elif len(s) == k and s.count("N") == 1:
+                out.append([2])                                   # one token for the whole window
+            elif len(s) == k and s.count("N") == 2:
+                out.append([vocab[c] for c in s if c != "N"] + [3])   # 3 tokens
+            elif len(s) == k and s.count("N") == 3:
+                out.append([])                                    # nothing known
+            else:
+                out.append([vocab.get(c, 0) for c in s])
+        return out
+    t = kmer_tables.tables_from_tokenize(tok, k, 0)
+    enc = encoders.KmerEncoder(k, t.digit, t.kmer_lut, t.single, pad_id=1, missing_id=4,
+                               exp_off=t.exp_off, exp_len=t.exp_len, exp_flat=t.exp_flat)
+    ot = O.KmerTables(k, t.digit, t.kmer_lut, t.exp_off, t.exp_len, t.exp_flat, t.single, 4)
+    rng = np.random.default_rng(5)
+    strings = ["".join(rng.choice(list("ACGTN"), p=[.2, .2, .2, .2, .2], size=n))
+               for n in rng.integers(0, 5000, size=40)]
+    b = util.batch_from_strings(strings)
+    data, off = to_dev(b)
+    ids, mask, lengths, status, max_len = enc.encode_padded(data, off, 5000)
+    torch.cuda.synchronize()
+    erows, estatus = O.kmer_encode(ot, b.data, b.offsets)
+    np.testing.assert_array_equal(lengths.cpu().numpy(), [r.size for r in erows])
+    np.testing.assert_array_equal(status.cpu().numpy() & 3, estatus)
+    m = int(max_len.item())
+    eids, emask = O.pad_rows(erows, 1, m)
+    np.testing.assert_array_equal(ids[:, :m].cpu().numpy(), eids)
+    np.testing.assert_array_equal(mask[:, :m].cpu().numpy(), emask)
+
+
 def test_kmer_missing_windows_without_expansion():
     say("kmer missing windows")
     t = kmer_tables.tables_from_vocab(hf.kmer_vocab(4), 4, 0)
