@@ -343,7 +343,7 @@ def make_workload(config: str, sustained: bool) -> Workload:
     if config == "C1":
         return CharDense(340 if sustained else 1)
     if config == "C2":
-        return KmerPadded(128 if sustained else 1)
+        return KmerPadded(256 if sustained else 1)
     if config == "C3":
         return BpePadded("4096", 16 if sustained else 1)
     if config == "C4":

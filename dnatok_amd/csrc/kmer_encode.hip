@@ -63,18 +63,49 @@ typedef uint32_t u32_a1 __attribute__((aligned(1)));
 
 __global__ void zero_i32_kernel(int32_t *p) { *p = 0; }
 
-__device__ __forceinline__ void store4(int32_t *out, uint8_t *mout, int64_t p, const int32_t *t)
+__device__ __forceinline__ void store4(int32_t *out, uint8_t *mout, int p, const int32_t *t)
 {
     int4v_a4 v = {t[0], t[1], t[2], t[3]};
     __builtin_nontemporal_store(v, reinterpret_cast<int4v_a4 *>(out + p));
     if (mout) __builtin_nontemporal_store((u32_a1)0x01010101u, reinterpret_cast<u32_a1 *>(mout + p));
 }
 
-__device__ __forceinline__ void store1(int32_t *out, uint8_t *mout, int64_t p, int64_t t_cap, int32_t v)
+__device__ __forceinline__ void store1(int32_t *out, uint8_t *mout, int p, int t_cap, int32_t v)
 {
     if (p < t_cap) {
         out[p] = v;
         if (mout) mout[p] = 1;
+    }
+}
+
+typedef int32_t int2v_a4 __attribute__((ext_vector_type(2), aligned(4)));
+typedef uint16_t u16_a1 __attribute__((aligned(1)));
+
+// N consecutive tokens (a spelled window) with as few stores as possible.
+template <int N>
+__device__ __forceinline__ void storeN(int32_t *out, uint8_t *mout, int p, int t_cap, const int32_t *t)
+{
+    if (p + N <= t_cap) {
+        int i = 0;
+#pragma unroll
+        for (; i + 4 <= N; i += 4) {
+            int4v_a4 v = {t[i], t[i + 1], t[i + 2], t[i + 3]};
+            *reinterpret_cast<int4v_a4 *>(out + p + i) = v;
+            if (mout) *reinterpret_cast<u32_a1 *>(mout + p + i) = 0x01010101u;
+        }
+        if (i + 2 <= N) {
+            int2v_a4 v = {t[i], t[i + 1]};
+            *reinterpret_cast<int2v_a4 *>(out + p + i) = v;
+            if (mout) *reinterpret_cast<u16_a1 *>(mout + p + i) = (uint16_t)0x0101u;
+            i += 2;
+        }
+        if (i < N) {
+            out[p + i] = t[i];
+            if (mout) mout[p + i] = 1;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) store1(out, mout, p + i, t_cap, t[i]);
     }
 }
 
@@ -89,14 +120,15 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
     __shared__ uint32_t s_dig[256];
     __shared__ int32_t s_single[256];
     __shared__ int32_t s_lut4[LUT4_LDS ? POW4 : 1];
-    __shared__ int32_t s_spell[8];       // token of the characters A C G T N
+    __shared__ int32_t s_spell[256];     // token a byte is spelled with inside a non-plain window
 
     for (int i = threadIdx.x; i < 256; i += kKmerThreads) {
         const int d = a.digit[i];
         s_dig[i] = d < 0 ? kDigBad : (d >= 4 ? kDigN : (uint32_t)d);
         s_single[i] = a.single[i];
+        // a byte outside the alphabet counts as N inside a window
+        s_spell[i] = a.single[(int)"ACGTN"[d < 0 || d > 4 ? 4 : d]];
     }
-    if (threadIdx.x < 5) s_spell[threadIdx.x] = a.single[(int)"ACGTN"[threadIdx.x]];
     if (LUT4_LDS)
         for (uint32_t i = threadIdx.x; i < POW4; i += kKmerThreads) s_lut4[i] = a.lut4[i];
     __syncthreads();          // the only workgroup barrier: from here on every wave runs alone
@@ -108,34 +140,40 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
 
     for (int64_t row = wave; row < n_rows; row += n_waves) {
         const int64_t row_start = offsets[row];
-        const int64_t len = offsets[row + 1] - row_start;
-        const int64_t full = len / K;
-        const int64_t n_units = full + (len - full * K);
+        // positions inside a row are 32-bit: a row is shorter than 2^31 bytes
+        const int len = (int)(offsets[row + 1] - row_start);
+        const int full = len / K;
+        const int n_units = full + (len - full * K);
         const uint8_t *src = bytes + row_start;
         int32_t *out = ids + row * t_cap;
         uint8_t *mout = mask ? mask + row * t_cap : nullptr;
-        int64_t running = 0;
+        const int cap = t_cap > INT_MAX ? INT_MAX : (int)t_cap;
+        int running = 0;
         int32_t my_status = 0;
 
-        for (int64_t u0 = 0; u0 < n_units; u0 += kWaveUnits) {
-            const int64_t ub = u0 + (int64_t)lane * kUnitsPerLane;
+        // software pipeline: the bytes of the next step are requested before this step is decoded
+        uint32_t wn[K];
+#pragma unroll
+        for (int i = 0; i < K; ++i) wn[i] = 0;             // byte 0 is never a base
+        if (lane * kUnitsPerLane + kUnitsPerLane <= full) memcpy(wn, src + lane * kUnitsPerLane * K, 4 * K);
+
+        for (int u0 = 0; u0 < n_units; u0 += kWaveUnits) {
+            const int ub = u0 + lane * kUnitsPerLane;
             const bool lane_full = ub + kUnitsPerLane <= full;     // 4 whole windows
             const bool empty = ub >= n_units;
             uint32_t w[K];
 #pragma unroll
-            for (int i = 0; i < K; ++i) w[i] = 0;          // byte 0 is never a base
-            if (lane_full) memcpy(w, src + ub * K, 4 * K);  // 4 windows = 4K bytes, unaligned
-            uint32_t dig[kUnitsPerLane * K];
+            for (int i = 0; i < K; ++i) { w[i] = wn[i]; wn[i] = 0; }
+            if (ub + kWaveUnits + kUnitsPerLane <= full)            // 4 windows = 4K bytes, unaligned
+                memcpy(wn, src + (ub + kWaveUnits) * K, 4 * K);
+            // digit of byte bi of this lane (LDS lookup)
+            auto digit_of = [&](int bi) -> uint32_t { return s_dig[(w[bi >> 2] >> (8 * (bi & 3))) & 255u]; };
             uint32_t code[kUnitsPerLane];
 #pragma unroll
             for (int j = 0; j < kUnitsPerLane; ++j) {
                 uint32_t c = 0;
 #pragma unroll
-                for (int i = 0; i < K; ++i) {
-                    const int bi = j * K + i;
-                    dig[bi] = s_dig[(w[bi >> 2] >> (8 * (bi & 3))) & 255u];
-                    c = (c << 2) + dig[bi];
-                }
+                for (int i = 0; i < K; ++i) c = (c << 2) + digit_of(j * K + i);
                 code[j] = c;
             }
             int32_t t[kUnitsPerLane];
@@ -151,16 +189,16 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
 
             if (rest_mask == 0) {
                 // every lane is plain or past the end: positions are known without a scan
-                const int64_t p = running + (int64_t)lane * kUnitsPerLane;
+                const int p = running + lane * kUnitsPerLane;
                 if (fast) {
-                    if (p + 4 <= t_cap) {
+                    if (p + 4 <= cap) {
                         store4(out, mout, p, t);
                     } else {
 #pragma unroll
-                        for (int j = 0; j < kUnitsPerLane; ++j) store1(out, mout, p + j, t_cap, t[j]);
+                        for (int j = 0; j < kUnitsPerLane; ++j) store1(out, mout, p + j, cap, t[j]);
                     }
                 }
-                running += (int64_t)kUnitsPerLane * __popcll(fast_mask);
+                running += kUnitsPerLane * (int)__popcll(fast_mask);
                 continue;
             }
 
@@ -180,7 +218,7 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
                         int c5 = 0;
 #pragma unroll
                         for (int i = 0; i < K; ++i) {
-                            const uint32_t v = dig[j * K + i];
+                            const uint32_t v = digit_of(j * K + i);
                             c5 = c5 * 5 + ((v & (kDigN | kDigBad)) ? 4 : (int)v);
                         }
                         const int2 e = a.entry[c5];
@@ -192,7 +230,7 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
                         // some digit may carry the foreign-byte flag (bit 17, shifted left by 0..2(K-1))
                         bool bad = false;
 #pragma unroll
-                        for (int i = 0; i < K; ++i) bad = bad || (dig[j * K + i] & kDigBad);
+                        for (int i = 0; i < K; ++i) bad = bad || (digit_of(j * K + i) & kDigBad);
                         if (bad) my_status |= DNATOK_ROW_INVALID_BYTE;
                     }
                     lane_cnt += (uint32_t)cnt[j];
@@ -201,7 +239,7 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
                 // the ragged end of the row: whole windows first, then single characters
 #pragma unroll 1
                 for (int j = 0; j < kUnitsPerLane; ++j) {
-                    const int64_t u = ub + j;
+                    const int u = ub + j;
                     int n = 0;
                     if (u < full) {
                         uint32_t c = 0;
@@ -231,43 +269,45 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
 
             const uint32_t inc = wave_inclusive_sum_u32(lane_cnt);
             const uint32_t step_total = __builtin_amdgcn_readlane(inc, 63);
-            int64_t p = running + (inc - lane_cnt);
+            int p = running + (int)(inc - lane_cnt);
 
             if (fast) {
-                if (p + 4 <= t_cap) {
+                if (p + 4 <= cap) {
                     store4(out, mout, p, t);
                 } else {
 #pragma unroll
-                    for (int j = 0; j < kUnitsPerLane; ++j) store1(out, mout, p + j, t_cap, t[j]);
+                    for (int j = 0; j < kUnitsPerLane; ++j) store1(out, mout, p + j, cap, t[j]);
                 }
             } else if (lane_full) {
 #pragma unroll
                 for (int j = 0; j < kUnitsPerLane; ++j) {
                     if (code[j] < POW4 && t[j] >= 0) {
-                        store1(out, mout, p, t_cap, t[j]);
+                        store1(out, mout, p, cap, t[j]);
                         ++p;
                     } else if (CHARS) {
+                        int32_t sp[K];
 #pragma unroll
                         for (int i = 0; i < K; ++i) {
-                            const uint32_t v = dig[j * K + i];
-                            store1(out, mout, p + i, t_cap, s_spell[(v & (kDigN | kDigBad)) ? 4 : v]);
+                            const int bi = j * K + i;
+                            sp[i] = s_spell[(w[bi >> 2] >> (8 * (bi & 3))) & 255u];
                         }
+                        storeN<K>(out, mout, p, cap, sp);
                         p += K;
                     } else if (ex[j] >= 0) {
-                        store1(out, mout, p, t_cap, ex[j]);
+                        store1(out, mout, p, cap, ex[j]);
                         ++p;
                     } else if (ex[j] == INT_MIN) {
-                        store1(out, mout, p, t_cap, a.missing_id);
+                        store1(out, mout, p, cap, a.missing_id);
                         ++p;
                     } else {
-                        for (int e = 0; e < -ex[j]; ++e) store1(out, mout, p + e, t_cap, a.flat[ey[j] + e]);
+                        for (int e = 0; e < -ex[j]; ++e) store1(out, mout, p + e, cap, a.flat[ey[j] + e]);
                         p += -ex[j];
                     }
                 }
             } else if (!empty) {
 #pragma unroll 1
                 for (int j = 0; j < kUnitsPerLane; ++j) {
-                    const int64_t u = ub + j;
+                    const int u = ub + j;
                     if (u < full) {
                         uint32_t c = 0;
                         int c5 = 0;
@@ -280,28 +320,28 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
                         int32_t id = -1;
                         if (c < POW4) id = LUT4_LDS ? s_lut4[c] : a.lut4[c];
                         if (id >= 0) {
-                            store1(out, mout, p, t_cap, id);
+                            store1(out, mout, p, cap, id);
                             ++p;
                         } else {
                             const int2 e = a.entry[c5];
                             if (e.x >= 0 || e.x == INT_MIN) {
-                                store1(out, mout, p, t_cap, e.x >= 0 ? e.x : a.missing_id);
+                                store1(out, mout, p, cap, e.x >= 0 ? e.x : a.missing_id);
                                 ++p;
                             } else {
-                                for (int q = 0; q < -e.x; ++q) store1(out, mout, p + q, t_cap, a.flat[e.y + q]);
+                                for (int q = 0; q < -e.x; ++q) store1(out, mout, p + q, cap, a.flat[e.y + q]);
                                 p += -e.x;
                             }
                         }
                     } else if (u < n_units) {
-                        store1(out, mout, p, t_cap, s_single[src[full * K + (u - full)]]);
+                        store1(out, mout, p, cap, s_single[src[full * K + (u - full)]]);
                         ++p;
                     }
                 }
             }
-            running += step_total;
+            running += (int)step_total;
         }
 
-        const int64_t stored = running < t_cap ? running : t_cap;
+        const int64_t stored = running < cap ? running : cap;
         int32_t st = 0;
         if (__ballot(my_status & DNATOK_ROW_INVALID_BYTE)) st |= DNATOK_ROW_INVALID_BYTE;
         if (__ballot(my_status & DNATOK_ROW_MISSING_KMER)) st |= DNATOK_ROW_MISSING_KMER;
