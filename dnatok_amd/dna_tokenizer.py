@@ -1,0 +1,504 @@
+"""``DNATok``: the reference's drop-in wrapper API over the MI355X encode kernels.
+
+Same constructor, ``discover()`` and ``encode_*`` surface as the reference's
+``dna_tokenizer.DNATok`` (src/dna_tokenizer.py:85-133, 864-1110, 2049-2338, 2594-3110).
+``discover()`` probes the embedder's tokenizer with short strings and selects one of
+three paths; all three run on the GPU through libdnatok_hip.so:
+
+* single-nucleotide tokenizers -> 256-entry byte table  (char kernel)
+* non-overlapping k-mer tokenizers (2 <= k <= 6) -> 5**k window table with per-window
+  expansion lists (k-mer kernel)
+* BPE tokenizers -> ``GPUTokBPEBackend`` (merge engine + packer)
+
+There is no numpy / torch fallback for the encode itself; a missing library raises.
+Rows the tables cannot express (a k-mer window with no known tokenization) are
+re-tokenized by the tokenizer object itself, as the reference does
+(src/dna_tokenizer.py:1955-2047).
+"""
+from __future__ import annotations
+
+import logging
+import os
+from typing import Any, Iterator, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from . import encoders, kmer_tables
+
+_DNA_UPPER = "ACGTN"
+
+
+def _smallest_dtype(max_id: int) -> torch.dtype:
+    if max_id <= 255:
+        return torch.uint8
+    if max_id <= 32_767:
+        return torch.int16
+    if max_id <= 2_147_483_647:
+        return torch.int32
+    return torch.int64
+
+
+class DNATok:
+    DEFAULT_IDS_MAX_TOKENS_PER_CALL = 1_048_576
+
+    def __init__(self, embedder: object, ids_max_tokens_per_call: int = DEFAULT_IDS_MAX_TOKENS_PER_CALL,
+                 logger: Optional[logging.Logger] = None, *,
+                 prefer_int32_h2d: bool = True, overlap_h2d_compute: bool = True,
+                 force_fp32_outputs: bool = True, strict_lut_check: bool = True,
+                 normalize_case: bool = False, handle_invalid_chars: bool = False,
+                 require_valid_chars: bool = False, allow_incomplete_kmer_lut: bool = False,
+                 padding_side: str = "left", pack_2bit_h2d: bool = False, use_uint8_ids: bool = False,
+                 use_cuda_graph: bool = False, use_fused_kernel: bool = False) -> None:
+        self.embedder = embedder
+        self.log = logger or logging.getLogger("DNATok")
+        if not self.log.handlers:
+            h = logging.StreamHandler()
+            h.setFormatter(logging.Formatter("[%(name)s] %(message)s"))
+            self.log.addHandler(h)
+            level = os.environ.get("DNATOK_LOG_LEVEL", "WARNING").upper()
+            self.log.setLevel(getattr(logging, level, logging.WARNING))
+        if padding_side not in ("left", "right"):
+            raise ValueError("padding_side must be 'left' or 'right'")
+        self.ids_max_tokens_per_call = int(ids_max_tokens_per_call)
+        self.prefer_int32_h2d = bool(prefer_int32_h2d)
+        self.overlap_h2d_compute = bool(overlap_h2d_compute)
+        self.force_fp32_outputs = bool(force_fp32_outputs)
+        self.strict_lut_check = bool(strict_lut_check)
+        self.normalize_case = bool(normalize_case)
+        self.handle_invalid_chars = bool(handle_invalid_chars)
+        self.require_valid_chars = bool(require_valid_chars)
+        env_allow = os.environ.get("DNATOK_ALLOW_INCOMPLETE_KMER_LUT")
+        self.allow_incomplete_kmer_lut = (env_allow.strip().lower() in ("1", "true", "yes", "y")
+                                          if env_allow is not None else bool(allow_incomplete_kmer_lut))
+        self.padding_side = padding_side
+        # accepted for interface compatibility; the device kernels make them moot
+        self.pack_2bit_h2d, self.use_uint8_ids = bool(pack_2bit_h2d), bool(use_uint8_ids)
+        self.use_cuda_graph, self.use_fused_kernel = bool(use_cuda_graph), bool(use_fused_kernel)
+        self._reset()
+
+    # ------------------------------------------------------------------ state
+
+    def _reset(self) -> None:
+        self.use_ids_path = False
+        self.ascii_lut: Optional[np.ndarray] = None         # int64 [256]
+        self.ascii_start_lut: Optional[np.ndarray] = None
+        self.id_pad = 0
+        self.id_N = 0
+        self.id_unk: Optional[int] = None
+        self.invalid_char_id: Optional[int] = None
+        self.token_len: Optional[int] = None
+        self.vocab_size = 0
+        self.kmer_k: Optional[int] = None
+        self.kmer_lut: Optional[np.ndarray] = None
+        self.kmer_single_char_lut: Optional[np.ndarray] = None
+        self.bpe_backend: Optional[Any] = None
+        self.lmm_bpe: Optional[Any] = None
+        self._char_enc: Optional[encoders.CharEncoder] = None
+        self._kmer_enc: Optional[encoders.KmerEncoder] = None
+        self._kmer_tables: Optional[kmer_tables.KmerTables] = None
+        self._staging_bytes_cpu: Optional[torch.Tensor] = None
+
+    def free_buffers(self) -> None:
+        self._staging_bytes_cpu = None
+
+    # ------------------------------------------------------------- tokenizer access
+
+    def _tok_ids(self, texts: Sequence[str]) -> List[List[int]]:
+        """Token ids of each text, no special tokens, through whatever call style the
+        tokenizer object offers."""
+        tok = self.embedder.tokenizer
+        texts = list(texts)
+        try:
+            out = tok(texts, add_special_tokens=False)
+            ids = out["input_ids"] if isinstance(out, dict) or hasattr(out, "__getitem__") else out.input_ids
+            if torch.is_tensor(ids):
+                ids = ids.tolist()
+            return [list(map(int, r)) for r in ids]
+        except TypeError:
+            pass
+        if hasattr(tok, "encode_batch"):
+            return [list(e.ids) for e in tok.encode_batch(texts, add_special_tokens=False)]
+        return [list(map(int, tok.encode(t))) for t in texts]
+
+    def _tokenize_batch_cpu(self, seqs: Sequence[str], dtype: torch.dtype = torch.long,
+                            pin: bool = False) -> torch.Tensor:
+        """The tokenizer itself, padded like the fast paths pad (reference: 1591-1777)."""
+        rows = self._tok_ids(seqs)
+        width = max((len(r) for r in rows), default=0)
+        if self.token_len is not None and self.token_len > width:
+            width = int(self.token_len)
+        out = torch.full((len(rows), width), int(self.id_pad), dtype=dtype)
+        for i, r in enumerate(rows):
+            if r:
+                cur = torch.as_tensor(r, dtype=dtype)
+                if self.padding_side == "left":
+                    out[i, width - len(r):] = cur
+                else:
+                    out[i, :len(r)] = cur
+        return out.pin_memory() if pin and torch.cuda.is_available() else out
+
+    # ---------------------------------------------------------------- discovery
+
+    def discover(self) -> None:
+        self._reset()
+        emb = self.embedder
+        if not callable(getattr(emb, "embed_tokens", None)):
+            self.log.info("embedder has no embed_tokens(); ids path disabled")
+            return
+        tok = getattr(emb, "tokenizer", None)
+        self.id_pad = self._first_int((emb, "pad_id"), (emb, "pad_token_id"), (tok, "pad_token_id"), default=0)
+        self.id_unk = self._first_int((tok, "unk_token_id"), (emb, "unk_id"), default=None)
+        side = getattr(tok, "padding_side", None)
+        if side in ("left", "right"):
+            self.padding_side = side
+        if tok is None:
+            # fixed map when no tokenizer is attached (reference: 907-932)
+            lut = np.zeros(256, dtype=np.int64)
+            for ch, v in zip("ACGTN", (1, 2, 3, 4, 0)):
+                lut[ord(ch)] = v
+                lut[ord(ch.lower())] = v
+            self._install_char(lut, None, id_n=0, vocab_size=5)
+            return
+        self.vocab_size = self._discover_vocab_size(tok)
+        # a probe can be fooled (a BPE vocabulary may split homopolymers evenly); a table that
+        # does not reproduce the tokenizer on random input is dropped and the next path is tried
+        k = self._probe_kmer()
+        if k is not None:
+            try:
+                self._install_kmer(k)
+                return
+            except RuntimeError as e:
+                self.log.info("k-mer probe (k=%d) rejected: %s", k, e)
+                keep = (self.id_pad, self.id_unk, self.padding_side, self.vocab_size)
+                self._reset()
+                self.id_pad, self.id_unk, self.padding_side, self.vocab_size = keep
+        try:
+            if self._probe_char():
+                return
+        except RuntimeError as e:
+            self.log.info("single-nucleotide probe rejected: %s", e)
+            keep = (self.id_pad, self.id_unk, self.padding_side, self.vocab_size)
+            self._reset()
+            self.id_pad, self.id_unk, self.padding_side, self.vocab_size = keep
+        from .gputok_bpe_backend import GPUTokBPEBackend
+        if GPUTokBPEBackend.is_supported(tok):
+            self.bpe_backend = GPUTokBPEBackend(tok, engine="dnatok")
+            self.id_pad = self.bpe_backend.pad_id
+            self.use_ids_path = True
+            return
+        self.log.warning("tokenizer is neither single-nucleotide, k-mer nor a supported BPE; ids path disabled")
+
+    @staticmethod
+    def _first_int(*candidates, default):
+        for obj, name in candidates:
+            v = getattr(obj, name, None) if obj is not None else None
+            if isinstance(v, (int, np.integer)) and not isinstance(v, bool):
+                return int(v)
+        return default
+
+    def _discover_vocab_size(self, tok) -> int:
+        for name in ("vocab_size",):
+            v = getattr(tok, name, None)
+            if isinstance(v, (int, np.integer)):
+                return int(v)
+        for name in ("get_vocab_size",):
+            f = getattr(tok, name, None)
+            if callable(f):
+                try:
+                    return int(f())
+                except Exception:
+                    pass
+        try:
+            return int(len(tok))
+        except Exception:
+            pass
+        gv = getattr(tok, "get_vocab", None)
+        if callable(gv):
+            try:
+                return int(max(gv().values())) + 1
+            except Exception:
+                pass
+        return 0
+
+    def _probe_kmer(self) -> Optional[int]:
+        """k = 24 / tokens("A" * 24), accepted when it divides, 2 <= k <= 6, and the other
+        homopolymers and a mixed probe give the same count (reference: 655-741)."""
+        try:
+            n = len(self._tok_ids(["A" * 24])[0])
+            if n == 0 or 24 % n != 0:
+                return None
+            k = 24 // n
+            if not 2 <= k <= 6:
+                return None
+            probes = ["C" * 24, "G" * 24, "T" * 24, ("ACGT" * 6)]
+            if any(len(r) != n for r in self._tok_ids(probes)):
+                return None
+            rng = np.random.default_rng(1)
+            mixed = ["".join(rng.choice(list("ACGT"), size=m * k)) for m in (1, 2, 3, 5, 8)]
+            if [len(r) for r in self._tok_ids(mixed)] != [1, 2, 3, 5, 8]:
+                return None
+            return k
+        except Exception:
+            return None
+
+    def _install_kmer(self, k: int) -> None:
+        unk = self.id_unk if self.id_unk is not None else self.id_pad
+        t = kmer_tables.tables_from_tokenize(self._tok_ids, k, int(unk))
+        t.digit = kmer_tables.digit_table(fold_case=self.normalize_case)
+        if self.normalize_case:
+            for ch in _DNA_UPPER:
+                t.single[ord(ch.lower())] = t.single[ord(ch)]
+        n_missing = int(((t.kmer_lut < 0) & (t.exp_len == 0)).sum())
+        if n_missing and not self.allow_incomplete_kmer_lut:
+            self.log.info("%d of %d windows have no tokenization of their own; such rows are "
+                          "re-tokenized by the tokenizer", n_missing, t.kmer_lut.size)
+        self._kmer_tables = t
+        self.kmer_k = k
+        self.kmer_lut = t.kmer_lut.astype(np.int64)
+        self.kmer_single_char_lut = t.single.astype(np.int64)
+        self.id_N = int(t.single[ord("N")])
+        missing = int(unk)
+        self._kmer_enc = encoders.KmerEncoder(k, t.digit, t.kmer_lut, t.single, int(self.id_pad), missing,
+                                              t.exp_off, t.exp_len, t.exp_flat)
+        if self.vocab_size <= 0:
+            self.vocab_size = int(max(t.kmer_lut.max(), t.single.max())) + 1
+        self.use_ids_path = True
+        self._self_check()            # always: a mis-probed k must not survive
+
+    def _probe_char(self) -> bool:
+        """One token per character on fixed probes, then a byte table from probing every
+        printable byte (reference: 447-653, 1139-1218)."""
+        probes = ["ACGTACGT", "NNNNACGT", "TTTTGGGG", "CAGTNACG"]
+        try:
+            if any(len(r) != 8 for r in self._tok_ids(probes)):
+                return False
+            chars = [chr(b) if 32 < b < 127 else "N" for b in range(256)]
+            singles = self._tok_ids(chars)
+        except Exception:
+            return False
+        id_n_row = singles[ord("N")]
+        if len(id_n_row) != 1:
+            return False
+        id_n = int(id_n_row[0])
+        fallback = self.id_unk if self.id_unk is not None else id_n
+        lut = np.full(256, int(fallback), dtype=np.int64)
+        for b in range(256):
+            if 32 < b < 127 and len(singles[b]) == 1:
+                lut[b] = int(singles[b][0])
+        # a separate first-position table only if the tokenizer treats position 0 differently
+        start = None
+        try:
+            firsts = self._tok_ids([c + "A" for c in _DNA_UPPER])
+            if all(len(r) == 2 for r in firsts) and any(int(r[0]) != lut[ord(c)] for r, c in zip(firsts, _DNA_UPPER)):
+                start = lut.copy()
+                for r, c in zip(firsts, _DNA_UPPER):
+                    start[ord(c)] = int(r[0])
+        except Exception:
+            start = None
+        self._install_char(lut, start, id_n=id_n, vocab_size=self.vocab_size or int(lut.max()) + 1)
+        if self.strict_lut_check:
+            self._self_check()
+        return True
+
+    def _install_char(self, lut: np.ndarray, start: Optional[np.ndarray], *, id_n: int, vocab_size: int) -> None:
+        lut = lut.copy()
+        self.id_N = int(id_n)
+        if self.normalize_case:
+            for ch in _DNA_UPPER:
+                lut[ord(ch.lower())] = lut[ord(ch)]
+                if start is not None:
+                    start[ord(ch.lower())] = start[ord(ch)]
+        if self.handle_invalid_chars:
+            valid = set(map(ord, _DNA_UPPER)) | set(map(ord, _DNA_UPPER.lower()))
+            inv = self.invalid_char_id if self.invalid_char_id is not None else self.id_N
+            for b in range(256):
+                if b not in valid:
+                    lut[b] = inv
+                    if start is not None:
+                        start[b] = inv
+        self.ascii_lut = lut
+        self.ascii_start_lut = start
+        self.vocab_size = int(vocab_size)
+        self._char_enc = encoders.CharEncoder(lut.astype(np.int32), int(self.id_pad),
+                                              None if start is None else start.astype(np.int32))
+        self.use_ids_path = True
+
+    def _self_check(self) -> None:
+        """32 random ACGTN strings must encode exactly as the tokenizer does
+        (reference: 1220-1273)."""
+        if not torch.cuda.is_available():
+            return
+        rng = np.random.default_rng(0)
+        k = self.kmer_k or 1
+        seqs = ["".join(rng.choice(list(_DNA_UPPER), size=8 * k)) for _ in range(32)]
+        got = self.encode_batch_to_ids(seqs)
+        want = self._tokenize_batch_cpu(seqs)
+        if got.shape != want.shape or not torch.equal(got.cpu(), want):
+            raise RuntimeError("DNATok.discover(): table encode disagrees with the tokenizer")
+
+    # ------------------------------------------------------------------- encode
+
+    def _require_ready(self) -> None:
+        if not self.use_ids_path:
+            raise RuntimeError("DNATok.discover() must be called before encoding.")
+
+    def encode_batch_device(self, seqs: Sequence[str], device="cuda") -> Tuple[torch.Tensor, torch.Tensor]:
+        """Device-resident encode: (ids int32 [B, T], mask uint8 [B, T]) on the GPU, padded on
+        ``padding_side`` (char) or on the right (k-mer, BPE) to the longest row."""
+        self._require_ready()
+        if not seqs:
+            raise ValueError("No sequences provided for encoding.")
+        if self.bpe_backend is not None:
+            ids, mask = self.bpe_backend.encode_batch(list(seqs), device=device)
+            return ids.to(torch.int32), mask
+        data, offsets, lens = encoders.bytes_from_strings(seqs, device)
+        if self._kmer_enc is not None:
+            return self._encode_kmer_device(seqs, data, offsets, lens)
+        width = int(lens.max())
+        if self.token_len is not None and self.token_len > width:
+            width = int(self.token_len)
+        return self._char_enc.encode_padded(data, offsets, width, pad_left=(self.padding_side == "left"))
+
+    def _encode_kmer_device(self, seqs, data, offsets, lens) -> Tuple[torch.Tensor, torch.Tensor]:
+        from ._lib import lib  # noqa: F401  (fail early if the library is missing)
+        k = int(self.kmer_k)
+        t_cap = int(lens.max()) + 4
+        t_cap += (-t_cap) % 4
+        ids, mask, lengths, status, longest = self._kmer_enc.encode_padded(data, offsets, t_cap, fill_to=0)
+        width = int(longest.item())                      # one scalar: the output shape
+        if self.token_len is not None and self.token_len > width:
+            extra = int(self.token_len)
+            ids, mask, lengths, status, longest = self._kmer_enc.encode_padded(
+                data, offsets, max(t_cap, extra + (-extra) % 4), fill_to=extra)
+            width = extra
+        ids, mask = ids[:, :width], mask[:, :width]
+        bad = status.cpu().numpy()
+        need = (bad & 2) != 0
+        if self.require_valid_chars or not self.handle_invalid_chars:
+            need |= (bad & 1) != 0
+        if need.any() and not self.allow_incomplete_kmer_lut:
+            # rows the tables cannot express: the tokenizer's own answer, spliced in
+            rows = np.nonzero(need)[0].tolist()
+            fixed = self._tok_ids([seqs[i] for i in rows])
+            new_w = max(width, max(len(r) for r in fixed))
+            if new_w > width:
+                pad_i = torch.full((ids.shape[0], new_w - width), int(self.id_pad), dtype=ids.dtype, device=ids.device)
+                ids = torch.cat([ids, pad_i], dim=1)
+                mask = torch.cat([mask, torch.zeros_like(pad_i, dtype=torch.uint8)], dim=1)
+            else:
+                ids, mask = ids.clone(), mask.clone()
+            for i, r in zip(rows, fixed):
+                ids[i] = int(self.id_pad)
+                mask[i] = 0
+                if r:
+                    ids[i, :len(r)] = torch.as_tensor(r, dtype=ids.dtype, device=ids.device)
+                    mask[i, :len(r)] = 1
+        return ids, mask
+
+    def encode_batch_to_ids(self, seqs: List[str]) -> torch.Tensor:
+        """CPU pinned int64 [B, T] (reference: 2049-2148)."""
+        ids, _ = self.encode_batch_device(seqs)
+        out = torch.empty(ids.shape, dtype=torch.int64, pin_memory=True)
+        out.copy_(ids)                                   # int32 -> int64 on the way down
+        return out
+
+    def encode_batch_to_ids_staging(self, seqs: List[str], *, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        ids = self.encode_batch_to_ids(seqs)
+        want = dtype or (torch.int32 if self.prefer_int32_h2d else torch.int64)
+        return ids.to(want).pin_memory() if want != ids.dtype else ids
+
+    def encode_batch_with_padding(self, seqs: List[str], max_tokens: int, pad_to_max: bool = False,
+                                  pad_multiple: int = 16) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Truncate to max_tokens, pad to a multiple of pad_multiple tokens, smallest integer
+        dtype that holds the vocabulary (reference: 2150-2236).  Returned on the GPU."""
+        self._require_ready()
+        if not seqs:
+            raise ValueError("Empty batch")
+        k = int(self.kmer_k) if self.kmer_k else 1
+        max_chars = int(max_tokens) * k
+        seqs = [s[:max_chars] for s in seqs]
+        old = self.token_len
+        self.token_len = None
+        try:
+            ids, mask = self.encode_batch_device(seqs)
+        finally:
+            self.token_len = old
+        target = ids.shape[1]
+        if pad_to_max:
+            target = max(target, int(max_tokens))
+        if pad_multiple > 1 and target % pad_multiple:
+            target += pad_multiple - target % pad_multiple
+        if target > ids.shape[1]:
+            extra = target - ids.shape[1]
+            pad_i = torch.full((ids.shape[0], extra), int(self.id_pad), dtype=ids.dtype, device=ids.device)
+            pad_m = torch.zeros((ids.shape[0], extra), dtype=torch.uint8, device=ids.device)
+            left = self.padding_side == "left" and self._char_enc is not None
+            ids = torch.cat([pad_i, ids] if left else [ids, pad_i], dim=1)
+            mask = torch.cat([pad_m, mask] if left else [mask, pad_m], dim=1)
+        max_id = max(int(self.vocab_size) - 1, int(self.id_pad))
+        return ids.to(_smallest_dtype(max_id)), mask
+
+    # ------------------------------------------------------------------ bytes path
+
+    def encode_batch_to_ascii_bytes(self, seqs: List[str]) -> torch.Tensor:
+        """Equal-length strings -> persistent pinned uint8 [B, T] (reference: 2594-2651)."""
+        if not seqs:
+            raise ValueError("No sequences provided for encoding.")
+        t = len(seqs[0])
+        if any(len(s) != t for s in seqs):
+            raise ValueError("All sequences in a batch must have equal length.")
+        buf = "".join(seqs).encode("ascii", errors="replace")
+        need = len(seqs) * t
+        if self._staging_bytes_cpu is None or self._staging_bytes_cpu.numel() < need:
+            self._staging_bytes_cpu = torch.empty(max(need, 1), dtype=torch.uint8,
+                                                  pin_memory=torch.cuda.is_available())
+        out = self._staging_bytes_cpu[:need].view(len(seqs), t)
+        out.copy_(torch.frombuffer(bytearray(buf), dtype=torch.uint8).view(len(seqs), t))
+        return out
+
+    def ids_from_ascii_bytes_cuda(self, u8_cpu: torch.Tensor, device="cuda") -> torch.Tensor:
+        """uint8 [B, T] on the host -> int64 ids on the GPU (reference: 2653-2723, 2826-2940)."""
+        self._require_ready()
+        if self.bpe_backend is not None:
+            raise RuntimeError("the bytes path serves table tokenizers; BPE goes through encode_batch_device")
+        b, t = u8_cpu.shape
+        data = u8_cpu.to(device, non_blocking=True).reshape(-1)
+        offsets = torch.arange(b + 1, dtype=torch.int64, device=device) * t
+        if self._kmer_enc is not None:
+            t_cap = t + 4 + (-(t + 4)) % 4
+            ids, mask, lengths, status, longest = self._kmer_enc.encode_padded(data, offsets, t_cap, fill_to=0)
+            if int(status.abs().max().item()) & 3:
+                raise RuntimeError("k-mer bytes path: a row needs the tokenizer's own answer")
+            return ids[:, :int(longest.item())].to(torch.int64)
+        ids, _ = self._char_enc.encode_packed(data, row_len=t)
+        return ids.view(b, t).to(torch.int64)
+
+    # ------------------------------------------------------------------ embedding
+
+    def iter_embed_tokens_in_slices(self, ids: torch.Tensor, emb_batch: int, device) -> Iterator[torch.Tensor]:
+        dev = torch.device(device)
+        for s in range(0, ids.shape[0], max(1, int(emb_batch))):
+            chunk = ids[s:s + emb_batch].to(dev, dtype=torch.long, non_blocking=True)
+            out = self.embedder.embed_tokens(chunk)
+            yield out.float() if self.force_fp32_outputs and out.is_floating_point() else out
+
+    iter_embed_tokens_pipelined = iter_embed_tokens_in_slices
+
+    def embed_from_strings(self, seqs: List[str], emb_batch: int, device, *, path: str = "ids"
+                           ) -> Iterator[torch.Tensor]:
+        """Tokenize on the GPU, then feed ``embedder.embed_tokens`` in slices of emb_batch rows
+        on ``device`` (reference: 2962-3110).  ``path`` = "ids" | "bytes" select the same
+        kernels; "bytes" falls back to "ids" when a row needs the tokenizer's own answer."""
+        self._require_ready()
+        if path == "bytes" and self.bpe_backend is None and len({len(s) for s in seqs}) == 1:
+            try:
+                ids = self.ids_from_ascii_bytes_cuda(self.encode_batch_to_ascii_bytes(seqs))
+                if self.token_len is not None and self.token_len > ids.shape[1]:
+                    raise RuntimeError("needs padding")
+                yield from self.iter_embed_tokens_in_slices(ids, emb_batch, device)
+                return
+            except RuntimeError:
+                pass
+        ids, _ = self.encode_batch_device(seqs)
+        yield from self.iter_embed_tokens_in_slices(ids, emb_batch, device)

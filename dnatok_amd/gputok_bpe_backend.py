@@ -1,0 +1,276 @@
+"""``GPUTokBPEBackend``: HF-compatible BPE encode on the MI355X engine.
+
+Same surface as the reference's ``gputok_bpe_backend`` module
+(src/gputok_bpe_backend.py): the constructor takes a Hugging Face tokenizer,
+reads its ``tokenizer.json``, compiles the normalizer, materialises merges.txt
+and builds the kernel-id -> HF-id remap; ``encode_batch`` returns
+``(input_ids int64 [B, L], attention_mask uint8 [B, L])`` on the device, padded
+with the tokenizer's pad id to the longest row, with ids identical to
+``hf_tokenizer(seqs, add_special_tokens=False)``.
+
+What differs from the reference underneath: remap, padding and mask are fused
+into one packer kernel, nothing is routed to the CPU tokenizer by length (the
+engine has no length pathology), and negative per-row lengths raise instead of
+silently becoming all-pad rows.
+"""
+from __future__ import annotations
+
+import hashlib
+import json
+import os
+import re as _re
+from pathlib import Path
+from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from . import bpe_vocab, encoders
+
+
+# ------------------------------------------------------------------ tokenizer.json
+
+def _read_tokenizer_json(hf_tokenizer: Any) -> Optional[Dict[str, Any]]:
+    """tokenizer.json of an HF tokenizer: a local path in ``name_or_path`` / ``vocab_file``,
+    else the in-memory spec of a ``tokenizers`` object (``to_str``), directly or through
+    ``backend_tokenizer`` (reference: src/gputok_bpe_backend.py:132-176; the hub-cache
+    lookup is left out: there is no network path in this backend)."""
+    for attr in ("name_or_path", "vocab_file"):
+        base = getattr(hf_tokenizer, attr, None)
+        if isinstance(base, str) and base:
+            for cand in (os.path.join(base, "tokenizer.json"), base):
+                if os.path.isfile(cand) and cand.endswith("tokenizer.json"):
+                    with open(cand) as fh:
+                        return json.load(fh)
+    for obj in (getattr(hf_tokenizer, "backend_tokenizer", None), hf_tokenizer):
+        to_str = getattr(obj, "to_str", None)
+        if callable(to_str):
+            try:
+                return json.loads(to_str())
+            except Exception:
+                continue
+    return None
+
+
+def _compile_normalizer_step(step: Dict[str, Any]) -> Optional[Callable[[str], str]]:
+    """One HF normalizer step as a str -> str callable, or None when it cannot be reproduced
+    (reference: src/gputok_bpe_backend.py:179-236)."""
+    if not isinstance(step, dict):
+        return None
+    kind = step.get("type")
+    if kind == "Strip":
+        left = bool(step.get("strip_left", True))
+        right = bool(step.get("strip_right", True))
+        if left and right:
+            return lambda s: s.strip()
+        if left:
+            return lambda s: s.lstrip()
+        if right:
+            return lambda s: s.rstrip()
+        return lambda s: s
+    if kind == "Replace":
+        pattern = step.get("pattern")
+        content = str(step.get("content", ""))
+        if isinstance(pattern, dict) and "String" in pattern:
+            literal = pattern["String"]
+            return lambda s: s.replace(literal, content)
+        if isinstance(pattern, dict) and "Regex" in pattern:
+            rx = _re.compile(pattern["Regex"])
+            return lambda s: rx.sub(content, s)
+        return None
+    if kind == "Prepend":
+        prefix = str(step.get("prepend", ""))
+        return lambda s: prefix + s
+    if kind == "Lowercase":
+        return lambda s: s.lower()
+    if kind in (None, "NFC", "NFKC", "NFD", "NFKD", "StripAccents"):
+        return lambda s: s            # identity on ASCII DNA
+    if kind == "Sequence":
+        parts = [_compile_normalizer_step(sub) for sub in step.get("normalizers", [])]
+        if any(p is None for p in parts):
+            return None
+
+        def run(s: str) -> str:
+            for p in parts:
+                s = p(s)
+            return s
+        return run
+    return None
+
+
+def _compile_normalizer(cfg: Dict[str, Any]) -> Optional[Callable[[str], str]]:
+    norm = cfg.get("normalizer")
+    if norm is None:
+        return None
+    fn = _compile_normalizer_step(norm)
+    if fn is None:
+        raise ValueError(f"Unsupported normalizer config: {norm.get('type')!r}")
+    return fn
+
+
+def _extract_merges(cfg: Dict[str, Any]) -> List[str]:
+    """Merges as ``"a b"`` strings in rank order (reference: 251-262)."""
+    out: List[str] = []
+    for m in cfg.get("model", {}).get("merges", []):
+        if isinstance(m, str):
+            out.append(m)
+        elif isinstance(m, (list, tuple)) and len(m) == 2:
+            out.append(f"{m[0]} {m[1]}")
+        else:
+            raise ValueError(f"Unrecognised merge entry: {m!r}")
+    return out
+
+
+def _supported_tokenizer(cfg: Optional[Dict[str, Any]]) -> Tuple[bool, str]:
+    """(ok, reason): BPE model, whitespace-type or no pre-tokenizer, reproducible normalizer
+    (reference: 265-295)."""
+    if cfg is None:
+        return False, "tokenizer.json not found"
+    model = cfg.get("model") or {}
+    if model.get("type") != "BPE":
+        return False, f"model.type={model.get('type')!r} (only BPE supported)"
+    pre = cfg.get("pre_tokenizer")
+    if pre is not None:
+        kind = pre.get("type") if isinstance(pre, dict) else None
+        if kind not in (None, "Whitespace", "Split", "WhitespaceSplit"):
+            return False, f"pre_tokenizer={kind!r}"
+    norm = cfg.get("normalizer")
+    if norm is not None and _compile_normalizer_step(norm) is None:
+        return False, f"unsupported normalizer={norm.get('type')!r}"
+    return True, "ok"
+
+
+def _cache_dir() -> Path:
+    p = Path(os.environ.get("DNATOK_GPUTOK_CACHE", str(Path.home() / ".cache" / "dnatok-gputok")))
+    p.mkdir(parents=True, exist_ok=True)
+    return p
+
+
+def _merges_cache_path(merges: Sequence[str]) -> Path:
+    h = hashlib.sha256()
+    for m in merges:
+        h.update(m.encode("utf-8"))
+        h.update(b"\n")
+    return _cache_dir() / f"merges_{h.hexdigest()[:16]}.txt"
+
+
+def _reconstruct_gputok_vocab(merges: Sequence[str]) -> List[str]:
+    """Kernel id -> token string (reference: 358-393)."""
+    return list(bpe_vocab.KernelVocab(bpe_vocab.split_merges(merges)).id_to_token)
+
+
+# ------------------------------------------------------------------------- backend
+
+class GPUTokBPEBackend:
+    """HF-compatible GPU BPE encoder (reference: src/gputok_bpe_backend.py:396-679)."""
+
+    def __init__(self, hf_tokenizer: Any, *, engine: str = "dnatok") -> None:
+        if engine not in ("gputok", "dnatok"):
+            raise ValueError(f"engine must be 'gputok' or 'dnatok', got {engine!r}")
+        if engine == "gputok":
+            raise RuntimeError("engine='gputok' is the reference's third-party comparison kernel; "
+                               "this backend ships the 'dnatok' engine only")
+        self.tokenizer = hf_tokenizer
+        self.engine = engine
+        cfg = _read_tokenizer_json(hf_tokenizer)
+        ok, reason = _supported_tokenizer(cfg)
+        if not ok:
+            raise RuntimeError(f"GPUTokBPEBackend cannot accelerate this tokenizer: {reason}")
+        self._normalize = _compile_normalizer(cfg)
+        self._merges: List[str] = _extract_merges(cfg)
+        if not self._merges:
+            raise RuntimeError("Tokenizer has no merges; nothing to accelerate.")
+        path = _merges_cache_path(self._merges)
+        if not path.exists():
+            with open(path, "w") as fh:
+                fh.write("#version: 0.2\n")
+                for m in self._merges:
+                    fh.write(m + "\n")
+        self._merges_path = str(path)
+
+        from .dnatok_bpe_kernel import DnatokBpeKernel
+        self._dnatok = DnatokBpeKernel(self._merges_path, max_iters=1024)
+
+        model = cfg.get("model", {})
+        get_vocab = getattr(hf_tokenizer, "get_vocab", None)
+        hf_vocab = get_vocab() if callable(get_vocab) else dict(model.get("vocab", {}))
+        unk_id = getattr(hf_tokenizer, "unk_token_id", None)
+        if unk_id is None:
+            unk_tok = model.get("unk_token")
+            unk_id = hf_vocab.get(unk_tok, 0) if unk_tok is not None else 0
+        self.unk_id = int(unk_id or 0)
+        pad_id = getattr(hf_tokenizer, "pad_token_id", None)
+        if pad_id is None:
+            pad = (cfg.get("padding") or {})
+            pad_id = pad.get("pad_id", hf_vocab.get("[PAD]", hf_vocab.get("<pad>", 0)))
+        self.pad_id = int(pad_id or 0)
+        kvocab = self._dnatok._impl.vocab
+        remap = kvocab.remap_to(hf_vocab, self.unk_id)
+        self._n_unmapped = int(sum(1 for t in kvocab.id_to_token if t not in hf_vocab))
+        self._remap_cpu = torch.from_numpy(remap.astype("int64"))          # int64 [V_kernel]
+        self._remap_i32 = torch.from_numpy(remap)                          # int32, what the packer reads
+        self._remap_cuda: Optional[torch.Tensor] = None
+        size = getattr(hf_tokenizer, "vocab_size", None)
+        if callable(size):
+            size = None
+        if size is None:
+            gvs = getattr(hf_tokenizer, "get_vocab_size", None)
+            size = gvs() if callable(gvs) else len(hf_vocab)
+        self.vocab_size = int(size or len(hf_vocab))
+
+    @staticmethod
+    def is_supported(hf_tokenizer: Any) -> bool:
+        try:
+            ok, _ = _supported_tokenizer(_read_tokenizer_json(hf_tokenizer))
+            return ok
+        except Exception:
+            return False
+
+    # -------------------------------------------------------------- device-resident path
+
+    def _remap_on(self, dev: torch.device) -> torch.Tensor:
+        if self._remap_cuda is None or self._remap_cuda.device != dev:
+            self._remap_cuda = self._remap_i32.to(dev)
+        return self._remap_cuda
+
+    def encode_device(self, data: torch.Tensor, offsets: torch.Tensor, max_len: int, *,
+                      packed: bool = False):
+        """Bytes already on the device (uint8 [total] + int64 offsets [B+1]).
+
+        padded (default): ``(ids int32 [B, max_len], mask uint8 [B, max_len], lengths int32 [B],
+        longest int32 [1])`` -- rows are padded to the longest row found on the device, view
+        ``ids[:, :longest]``.  packed: ``(ids int32 [cap], out_offsets int64 [B+1], mask)``.
+        No host synchronisation either way.
+        """
+        tok, lengths = self._dnatok.tokenize_device(data, offsets, max_len)
+        remap = self._remap_on(data.device)
+        if packed:
+            return encoders.pack_ragged(tok, offsets, lengths, remap=remap)
+        ids, mask, longest = encoders.pad_rows(tok, offsets, lengths, self.pad_id, max(int(max_len), 1),
+                                               fill_to=0, remap=remap)
+        return ids, mask, lengths, longest
+
+    # ------------------------------------------------------------------- reference API
+
+    def encode_batch(self, seqs: List[str], *, device: object = "cuda"
+                     ) -> Tuple[torch.Tensor, torch.Tensor]:
+        if not seqs:
+            raise ValueError("No sequences provided.")
+        norm = [self._normalize(s) for s in seqs] if self._normalize is not None else list(seqs)
+        dev = torch.device(device) if not isinstance(device, torch.device) else device
+        if dev.type != "cuda":
+            raise RuntimeError("GPUTokBPEBackend.encode_batch runs on the GPU only (device='cuda')")
+        data, offsets, lens = encoders.bytes_from_strings(norm, dev)
+        b = len(seqs)
+        t_cap = max(int(lens.max()), 1)
+        ids32, mask, lengths, longest = self.encode_device(data, offsets, t_cap)
+        width = int(longest.item())                       # the one host sync: the output shape
+        if int(lengths.min().item()) < 0:
+            raise RuntimeError("BPE engine reported a failed row (negative length)")
+        if width == 0:
+            return (torch.empty((b, 0), dtype=torch.long, device=dev),
+                    torch.empty((b, 0), dtype=torch.uint8, device=dev))
+        return ids32[:, :width].to(torch.long), mask[:, :width].contiguous()
+
+    def encode_batch_ids_only(self, seqs: List[str], *, device: object = "cuda") -> torch.Tensor:
+        ids, _ = self.encode_batch(seqs, device=device)
+        return ids

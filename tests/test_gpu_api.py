@@ -1,0 +1,265 @@
+"""The drop-in Python surface on a GPU: DNATok / GPUTokBPEBackend / DnatokBpeKernel against the
+tokenizers they wrap.  The fake tokenizers follow the reference's own test doubles
+(tests/test_benchmark_correctness.py:22-57, tests/test_ids_path_equivalence.py:310-345,
+tests/test_kmer_bytes_fallback.py:8-59)."""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from dnatok_amd import dnatok_compat, hf_tokenizers as hf
+from dnatok_amd.dna_tokenizer import DNATok
+from dnatok_amd.dnatok_bpe_kernel import DnatokBpeKernel
+from dnatok_amd.gputok_bpe_backend import GPUTokBPEBackend
+from tests import util
+
+pytestmark = pytest.mark.gpu
+
+
+class SimpleCharTokenizer(dnatok_compat._SimpleTokenizer):
+    def __init__(self):
+        self.pad_token_id = 0
+        self.padding_side = "left"
+        self.vocab = {"<pad>": 0, "A": 1, "C": 2, "G": 3, "T": 4, "N": 5}
+        for k, v in list(self.vocab.items()):
+            if len(k) == 1:
+                self.vocab[k.lower()] = v
+
+    def _encode_one(self, text):
+        return [self.vocab.get(ch, self.vocab["N"]) for ch in text]
+
+
+class MockKmerTokenizer(dnatok_compat._SimpleTokenizer):
+    """Non-overlapping k-mers over ACGT; a window holding anything else is spelled out."""
+
+    def __init__(self, k=4):
+        self.k, self.pad_token_id, self.unk_token_id, self.padding_side = k, 0, 1, "right"
+        import itertools
+        self.vocab = {"".join(p): i + 10 for i, p in enumerate(itertools.product("ACGT", repeat=k))}
+        self.single = {c: 2 + i for i, c in enumerate("ACGTN")}
+
+    def __len__(self):
+        return 10 + 4 ** self.k
+
+    def _encode_one(self, text):
+        out = []
+        for i in range(0, len(text), self.k):
+            w = text[i:i + self.k]
+            if len(w) == self.k and w in self.vocab:
+                out.append(self.vocab[w])
+            else:
+                out.extend(self.single.get(c, self.unk_token_id) for c in w)
+        return out
+
+
+class FakeKmerTokenizer(dnatok_compat._SimpleTokenizer):
+    """k = 3; a window holding N gives two tokens (97, 98), so its table entry stays -1."""
+
+    def __init__(self, k=3):
+        self.k, self.pad_token_id, self.padding_side, self._ids = k, 0, "right", {}
+
+    def __len__(self):
+        return 256
+
+    def _encode_one(self, text):
+        ids = []
+        for i in range(0, len(text), self.k):
+            chunk = text[i:i + self.k]
+            if len(chunk) < self.k:
+                continue
+            if "N" in chunk:
+                ids.extend([97, 98])
+            else:
+                ids.append(self._ids.setdefault(chunk, len(self._ids) + 1))
+        return ids
+
+
+class RecordingEmbedder(torch.nn.Module):
+    def __init__(self, tokenizer, vocab=8192):
+        super().__init__()
+        self.tokenizer = tokenizer
+        self.pad_id = tokenizer.pad_token_id if tokenizer is not None else 0
+        self._embed = torch.nn.Embedding(vocab, 4)
+        self.last_ids = None
+
+    def embed_tokens(self, input_ids, rc_invariant=False):
+        self.last_ids = input_ids.detach().clone()
+        return self._embed(input_ids)
+
+
+def random_seqs(b, t, alphabet="ACGTN", seed=0):
+    random.seed(seed)
+    return ["".join(random.choice(alphabet) for _ in range(t)) for _ in range(b)]
+
+
+def test_char_discover_and_encode_matches_tokenizer():
+    tok = SimpleCharTokenizer()
+    helper = DNATok(RecordingEmbedder(tok))
+    helper.discover()
+    assert helper.use_ids_path and helper.kmer_k is None and helper.bpe_backend is None
+    assert helper.id_pad == 0 and helper.id_N == 5 and helper.padding_side == "left"
+    seqs = random_seqs(100, 64, seed=42)
+    want = tok(seqs, padding=True, return_tensors="pt")["input_ids"]
+    got = helper.encode_batch_to_ids(seqs)
+    assert got.dtype == torch.int64 and got.is_pinned() and torch.equal(got, want)
+    for base in "ACGTN":
+        assert bool((helper.encode_batch_to_ids([base * 16]) == tok.vocab[base]).all())
+    with pytest.raises(ValueError, match="No sequences"):
+        helper.encode_batch_to_ids([])
+    # ragged input is padded on the tokenizer's side
+    ragged = ["ACGT", "ACGTACGTAC", "N"]
+    assert torch.equal(helper.encode_batch_to_ids(ragged), tok(ragged, padding=True, return_tensors="pt")["input_ids"])
+
+
+def test_char_case_and_invalid_handling():
+    tok = SimpleCharTokenizer()
+    h = DNATok(RecordingEmbedder(tok), normalize_case=True)
+    h.discover()
+    ids = h.encode_batch_to_ids(["AcGt", "acgt", "ACGT"])
+    assert torch.equal(ids[0], ids[1]) and torch.equal(ids[0], ids[2])
+    h2 = DNATok(RecordingEmbedder(tok), handle_invalid_chars=True)
+    h2.discover()
+    assert torch.equal(h2.encode_batch_to_ids(["ACXGT", "AC$GT"]), h2.encode_batch_to_ids(["ACNGT", "ACNGT"]))
+
+
+def test_no_tokenizer_uses_fixed_map():
+    h = DNATok(RecordingEmbedder(None))
+    h.discover()
+    assert h.encode_batch_to_ids(["ACGTN"]).tolist() == [[1, 2, 3, 4, 0]]
+
+
+def test_ids_and_bytes_paths_feed_the_same_ids():
+    tok = SimpleCharTokenizer()
+    emb = RecordingEmbedder(tok)
+    h = DNATok(emb)
+    h.discover()
+    seqs = random_seqs(4, 16)
+    out_ids = list(h.embed_from_strings(seqs, emb_batch=4, device="cpu", path="ids"))
+    a = emb.last_ids.clone()
+    out_bytes = list(h.embed_from_strings(seqs, emb_batch=4, device="cpu", path="bytes"))
+    assert torch.equal(a, emb.last_ids)
+    assert torch.equal(a, tok(seqs, padding=True, return_tensors="pt")["input_ids"])
+    assert all(torch.equal(x, y) for x, y in zip(out_ids, out_bytes))
+
+
+def test_kmer_discover_and_encode():
+    tok = MockKmerTokenizer(4)
+    h = DNATok(RecordingEmbedder(tok))
+    h.discover()
+    assert h.kmer_k == 4 and h.use_ids_path
+    seqs = random_seqs(64, 130, alphabet="ACGTACGTACGTN", seed=3)     # tail of 2, some N windows
+    want = tok(seqs, padding=True, return_tensors="pt")["input_ids"]
+    assert torch.equal(h.encode_batch_to_ids(seqs), want)
+    ids, mask = h.encode_batch_with_padding(seqs, max_tokens=20, pad_multiple=16)
+    assert ids.shape[1] % 16 == 0 and ids.dtype == torch.int16 and mask.dtype == torch.uint8
+    short = tok([s[:80] for s in seqs], padding=True, return_tensors="pt")["input_ids"]
+    assert torch.equal(ids[:, :short.shape[1]].cpu().long(), short)
+    assert bool((ids[:, short.shape[1]:] == 0).all()) and bool((mask[:, short.shape[1]:] == 0).all())
+
+
+def test_kmer_multi_token_windows_follow_the_tokenizer():
+    tok = FakeKmerTokenizer(3)
+    emb = RecordingEmbedder(tok, 256)
+    h = DNATok(emb)
+    h.discover()
+    assert h.kmer_k == 3
+    seqs = ["AAANNN", "ACGTAC", "NNNACG"]
+    want = h._tokenize_batch_cpu(seqs)
+    list(h.embed_from_strings(seqs, emb_batch=2, device="cpu", path="bytes"))
+    assert torch.equal(h.encode_batch_to_ids(seqs), want)
+
+
+@pytest.mark.parametrize("which", ["4096", "32000"])
+def test_bpe_backend_matches_hf(which):
+    tk = hf.load_bpe_tokenizer(which)
+    assert GPUTokBPEBackend.is_supported(tk)
+    be = GPUTokBPEBackend(tk, engine="dnatok")
+    assert be.pad_id == 3 and be.unk_id == 0 and be.vocab_size == int(which)
+    random.seed(0)
+    seqs = ["".join(random.choices("ACGT", k=random.choice([4, 8, 16, 32, 64, 128, 256, 512, 1024, 2048])))
+            for _ in range(256)]
+    seqs[3] = "ACGTNNNNNNACGTacgtXACGT"          # N, lower case and a byte outside the vocabulary
+    ids, mask = be.encode_batch(seqs, device="cuda")
+    assert ids.dtype == torch.int64 and mask.dtype == torch.uint8 and ids.is_cuda
+    ref = [e.ids for e in tk.encode_batch(seqs, add_special_tokens=False)]
+    assert ids.shape[1] == max(len(r) for r in ref)
+    ids_h, mask_h = ids.cpu(), mask.cpu()
+    for i, r in enumerate(ref):
+        assert ids_h[i, :len(r)].tolist() == r
+        assert bool((ids_h[i, len(r):] == be.pad_id).all())
+        assert int(mask_h[i].sum()) == len(r) and bool(mask_h[i, :len(r)].all())
+    # determinism and B = 1
+    ids2, _ = be.encode_batch(seqs, device="cuda")
+    assert torch.equal(ids, ids2)
+    one, m1 = be.encode_batch([seqs[7]], device="cuda")
+    assert one[0].tolist() == ref[7] and bool(m1.all())
+    with pytest.raises(ValueError):
+        be.encode_batch([], device="cuda")
+    with pytest.raises(RuntimeError):
+        GPUTokBPEBackend(tk, engine="gputok")
+
+
+def test_bpe_backend_with_normalizer():
+    import json
+    from tokenizers import Tokenizer
+    cfg = dict(util.tokenizer_json("4096"))
+    cfg["normalizer"] = {"type": "Sequence", "normalizers": [
+        {"type": "Strip", "strip_left": True, "strip_right": True},
+        {"type": "Replace", "pattern": {"Regex": "N{10,}"}, "content": "N"}]}
+    tk = Tokenizer.from_str(json.dumps(cfg))
+    be = GPUTokBPEBackend(tk)
+    seqs = ["  ACGTACGTTTGA  ", "ACGT" + "N" * 14 + "GGCATTA", "ACGTNNNACGT"]
+    ids, mask = be.encode_batch(seqs)
+    for i, e in enumerate(tk.encode_batch(seqs, add_special_tokens=False)):
+        assert ids[i, :len(e.ids)].tolist() == e.ids and int(mask[i].sum()) == len(e.ids)
+
+
+def test_dnatok_routes_bpe_tokenizers_to_the_backend():
+    tk = hf.load_bpe_tokenizer("4096")
+
+    class Wrapped:                       # the attributes DNATok reads from an HF tokenizer
+        pad_token_id, unk_token_id, padding_side = 3, 0, "right"
+        backend_tokenizer = tk
+
+        def __call__(self, texts, add_special_tokens=False, **kw):
+            return {"input_ids": [e.ids for e in tk.encode_batch(list(texts), add_special_tokens=False)]}
+
+        def get_vocab(self):
+            return tk.get_vocab()
+
+    h = DNATok(RecordingEmbedder(Wrapped()))
+    h.discover()
+    assert h.bpe_backend is not None and h.kmer_k is None and h.ascii_lut is None
+    seqs = random_seqs(20, 300, alphabet="ACGT", seed=5) + ["ACGTACGTACGT"]
+    got = h.encode_batch_to_ids(seqs)
+    ref = [e.ids for e in tk.encode_batch(seqs, add_special_tokens=False)]
+    for i, r in enumerate(ref):
+        assert got[i, :len(r)].tolist() == r and bool((got[i, len(r):] == 3).all())
+
+
+def test_bpe_kernel_wrapper_contract(tmp_path):
+    cfg = util.tokenizer_json("4096")
+    p = tmp_path / "merges.txt"
+    p.write_text("#version: 0.2\n" + "\n".join(m if isinstance(m, str) else " ".join(m) for m in cfg["model"]["merges"]) + "\n")
+    k = DnatokBpeKernel(str(p))
+    bo = util.bpe_oracle("4096")
+    assert k.vocab_size() == len(bo.vocab) and k.id_to_token(65) == "A" and k.id_to_token(300) == bo.vocab[300]
+    with pytest.raises(IndexError):
+        k.id_to_token(10 ** 6)
+    seqs = random_seqs(9, 200, alphabet="ACGT", seed=1) + ["A", "ACGTACGTAC" * 90]
+    ids, lens = k.tokenize_batch(seqs)
+    assert ids.dtype == torch.int32 and ids.shape == (11, 900) and lens.dtype == torch.int32
+    ids_h, lens_h = ids.cpu().numpy(), lens.cpu().numpy()
+    for i, s in enumerate(seqs):
+        want = bo.encode_row(np.frombuffer(s.encode(), dtype=np.uint8), remap=False)
+        assert lens_h[i] == want.size and np.array_equal(ids_h[i, :want.size], want)
+        assert (ids_h[i, want.size:] == 0).all()                 # zero-filled tail
+    # views into a workspace: the next call overwrites them unless clone=True
+    kept, kept_l = k.tokenize_batch(seqs, clone=True)
+    view, _ = k.tokenize_batch(seqs)
+    k.tokenize_batch(["T" * 900] * 11)
+    torch.cuda.synchronize()
+    assert torch.equal(kept.cpu(), torch.from_numpy(ids_h)) and not torch.equal(view.cpu(), kept.cpu())
+    e_ids, e_len = k.tokenize_batch([])
+    assert e_ids.shape == (0, 0) and e_len.shape == (0,)

@@ -1,0 +1,82 @@
+"""Host-side logic of the drop-in API that needs no GPU: normalizer compiler truth tables
+(the reference's own CPU unit tests, tests/test_gputok_bpe_backend.py:319-425), tokenizer.json
+handling, and the compat tokenizer classes."""
+import numpy as np
+
+from dnatok_amd import dnatok_compat, hf_tokenizers as hf
+from dnatok_amd.gputok_bpe_backend import (_compile_normalizer, _compile_normalizer_step, _extract_merges,
+                                           _read_tokenizer_json, _reconstruct_gputok_vocab,
+                                           _supported_tokenizer)
+
+
+def test_normalizer_strip():
+    fn = _compile_normalizer_step({"type": "Strip", "strip_left": True, "strip_right": True})
+    assert fn("  ACGT  ") == "ACGT" and fn("ACGT") == "ACGT"
+    assert _compile_normalizer_step({"type": "Strip", "strip_left": True, "strip_right": False})("  ACGT  ") == "ACGT  "
+    assert _compile_normalizer_step({"type": "Strip", "strip_left": False, "strip_right": True})("  ACGT  ") == "  ACGT"
+
+
+def test_normalizer_replace_string_and_regex():
+    fn = _compile_normalizer_step({"type": "Replace", "pattern": {"String": "N"}, "content": "-"})
+    assert fn("ACGTNNACGT") == "ACGT--ACGT"
+    rx = _compile_normalizer_step({"type": "Replace", "pattern": {"Regex": "N{10,}"}, "content": "-"})
+    assert rx("ACGT" + "N" * 9 + "ACGT") == "ACGT" + "N" * 9 + "ACGT"
+    assert rx("ACGT" + "N" * 10 + "ACGT") == "ACGT-ACGT"
+
+
+def test_normalizer_prepend_lowercase_identity():
+    assert _compile_normalizer_step({"type": "Prepend", "prepend": "_"})("ACGT") == "_ACGT"
+    assert _compile_normalizer_step({"type": "Prepend", "prepend": "_"})("") == "_"
+    assert _compile_normalizer_step({"type": "Lowercase"})("ACGTACGT") == "acgtacgt"
+    for typ in ("NFC", "NFKC", "NFD", "NFKD", "StripAccents"):
+        assert _compile_normalizer_step({"type": typ})("ACGT") == "ACGT"
+
+
+def test_normalizer_sequence_and_rejections():
+    fn = _compile_normalizer_step({"type": "Sequence", "normalizers": [
+        {"type": "Strip", "strip_left": True, "strip_right": True},
+        {"type": "Replace", "pattern": {"Regex": "N{10,}"}, "content": "-"}]})
+    assert fn("   " + "N" * 12 + "ACGT  ") == "-ACGT"
+    for typ in ("BertNormalizer", "Nmt", "Precompiled", "SomeNewThingHFAdds"):
+        assert _compile_normalizer_step({"type": typ}) is None
+    assert _compile_normalizer_step({"type": "Sequence", "normalizers": [
+        {"type": "Strip"}, {"type": "BertNormalizer"}]}) is None
+    ok, reason = _supported_tokenizer({"model": {"type": "BPE", "merges": ["A A"]},
+                                       "pre_tokenizer": {"type": "Whitespace"},
+                                       "normalizer": {"type": "BertNormalizer"}})
+    assert not ok and "normalizer" in reason.lower()
+    assert _compile_normalizer({"normalizer": None}) is None
+
+
+def test_supported_tokenizer_gate():
+    assert _supported_tokenizer(None) == (False, "tokenizer.json not found")
+    assert not _supported_tokenizer({"model": {"type": "WordLevel"}})[0]
+    assert not _supported_tokenizer({"model": {"type": "BPE"}, "pre_tokenizer": {"type": "ByteLevel"}})[0]
+    assert _supported_tokenizer({"model": {"type": "BPE"}, "pre_tokenizer": None})[0]
+
+
+def test_tokenizer_json_from_live_object_and_merges():
+    tk = hf.load_bpe_tokenizer("4096")
+    cfg = _read_tokenizer_json(tk)
+    assert cfg["model"]["type"] == "BPE"
+    merges = _extract_merges(cfg)
+    assert len(merges) == len(cfg["model"]["merges"]) and all(len(m.split(" ")) == 2 for m in merges)
+    assert _extract_merges({"model": {"merges": [["A", "C"], "AC G"]}}) == ["A C", "AC G"]
+    vocab = _reconstruct_gputok_vocab(["A C", "AC G", "G T", "A CG"])
+    assert vocab[:256] == [chr(b) for b in range(256)] and vocab[256:] == ["AC", "ACG", "GT", "CG"]
+
+
+def test_compat_tokenizers():
+    nt = dnatok_compat.NTv3Tokenizer()
+    assert nt.vocab_size == 11 and nt.pad_token_id == 1 and nt.unk_token_id == 0
+    assert nt.encode("ATCGNxa") == [6, 7, 8, 9, 10, 0, 6]
+    out = nt(["AC", "ACGT"], padding=True, return_tensors="pt")["input_ids"]
+    assert out.tolist() == [[6, 8, 1, 1], [6, 8, 9, 7]]
+    evo = dnatok_compat.Evo2ByteTokenizer()
+    assert evo.encode("ACGT") == [65, 67, 71, 84] and evo.vocab_size == 512
+    ch = dnatok_compat.CharTokenizer()
+    assert ch.encode("acgtnX") == [7, 8, 9, 10, 11, 11] and ch.pad_token_id == 0
+    # the HF WordLevel tokenizer of the benchmark and NTv3Tokenizer agree on upper-case DNA
+    tk = hf.build_char_tokenizer()
+    s = "ACGTNNACGTTTGACN"
+    assert tk.encode(s, add_special_tokens=False).ids == nt.encode(s)
