@@ -134,7 +134,7 @@ __device__ __forceinline__ void bpe_row(
     const uint16_t *minchild, const uint16_t *byte_to_sym, const int32_t *out_remap,
     const uint8_t *__restrict__ src, const int n0, uint16_t *S, uint16_t *R, IT *NX, IT *PV,
     uint8_t *F, uint8_t *D, uint32_t *red, const int tid, int32_t *__restrict__ out,
-    int32_t *__restrict__ out_len)
+    int32_t *__restrict__ out_len, uint16_t *__restrict__ raw_out = nullptr)
 {
     constexpr IT NIL = (IT)~(IT)0;
     const int wv = (NT == 64) ? 0 : (tid >> 6);
@@ -260,6 +260,12 @@ __device__ __forceinline__ void bpe_row(
         }
     }
 
+    if (raw_out) {
+        // chunk of a long row: hand back the symbol at every start position (kNone elsewhere);
+        // the seam and gather kernels assemble the row
+        for (int i = lo; i < hi; ++i) raw_out[i] = stuck ? (uint16_t)kNone : S[i];
+        return;
+    }
     // compact the live symbols to the output
     uint32_t live = 0;
     for (int i = lo; i < hi; ++i) live += (S[i] != kNone);
@@ -272,12 +278,135 @@ __device__ __forceinline__ void bpe_row(
     if (tid == 0) *out_len = stuck ? -2 : (int32_t)total;
 }
 
-// Rows of at most CAP bytes, state in LDS.  NT = 64: every wave of the workgroup takes its
-// own row (no workgroup barrier after the set-up); NT = blockDim.x: the workgroup shares a row.
+// ---- long rows in chunks -------------------------------------------------------------------
+//
+// A row longer than the LDS capacity is cut into chunks of kChunkCore bytes, each extended by
+// kChunkOverlap bytes on both sides, and every extended chunk is merged on its own.  Two
+// neighbouring chunks A and B are then joined at a seam: a position p inside their overlap
+// where both runs end with a token boundary, the token ending at p is the same token in both,
+// and the token starting at p is the same token in both.  A token's own merge history depends
+// only on its string, so at such a p the two boundary symbols evolve identically in A and B;
+// taking A's merges left of p and B's merges right of p therefore is a legal run of the
+// (rank, position) order on the whole row, hence THE run (with a merge table in which every
+// rule's product is only used by higher-ranked rules, so that merges happen in key order).
+// If an overlap holds no such p (e.g. a tandem repeat longer than the overlap), the row is
+// redone by the whole-row kernel.
+constexpr int kLdsCap = 4096;            // longest row / extended chunk the LDS kernel takes
+constexpr int kChunkOverlap = 512;
+constexpr int kChunkCore = kLdsCap - 2 * kChunkOverlap;
+constexpr int kLongThreads = 1024;
+constexpr int kLongGrid = 64;            // slabs of scratch for the whole-row fallback kernel
+
+struct BpePlan {                          // device arrays inside the scratch buffer
+    int32_t *counts;      // [0] items, [1] chunk items of multi-chunk rows, [2] work counter
+    int32_t *item_off;    // [n_rows + 1] first item of a row
+    int32_t *mc_off;      // [n_rows + 1] first chunk slot of a row (multi-chunk rows only)
+    int32_t *item_row;    // [max_items]
+    int32_t *mc_row;      // [max_mc]
+    int32_t *seam;        // [max_mc] seam to the right of a chunk (row position), -1 = none found
+    int32_t *row_fail;    // [n_rows] 1 = redo the row with the whole-row kernel
+    uint16_t *chunk_sym;  // [max_mc][kLdsCap]
+    uint8_t *slabs;       // whole-row fallback state
+    size_t slab_bytes, total_bytes;
+    int64_t max_items, max_mc;
+};
+
+static size_t long_slab_bytes(int64_t max_len)
+{
+    const size_t n = ((size_t)max_len + 7) & ~(size_t)7;
+    return ((n * 13) + 255) & ~(size_t)255;
+}
+
+static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t total)
+{
+    BpePlan p{};
+    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    const bool chunks = max_len > kLdsCap;
+    p.max_items = n_rows + (chunks ? total / kChunkCore + 1 : 0);
+    p.max_mc = chunks ? 2 * (total / kChunkCore) + 2 : 0;
+    size_t o = 0;
+    auto take = [&](size_t bytes) { size_t at = o; o = up(o + bytes); return at; };
+    const size_t o_counts = take(64);
+    const size_t o_item_off = take(4 * (size_t)(n_rows + 1));
+    const size_t o_mc_off = take(4 * (size_t)(n_rows + 1));
+    const size_t o_item_row = take(4 * (size_t)p.max_items);
+    const size_t o_mc_row = take(4 * (size_t)p.max_mc);
+    const size_t o_seam = take(4 * (size_t)p.max_mc);
+    const size_t o_fail = take(4 * (size_t)n_rows);
+    const size_t o_sym = take(2 * (size_t)kLdsCap * (size_t)p.max_mc);
+    p.slab_bytes = chunks ? long_slab_bytes(max_len) : 0;
+    const int64_t slabs = n_rows < kLongGrid ? n_rows : kLongGrid;
+    const size_t o_slabs = take(chunks ? p.slab_bytes * (size_t)slabs : 0);
+    p.total_bytes = o + 256;
+    if (base) {
+        p.counts = (int32_t *)(base + o_counts);
+        p.item_off = (int32_t *)(base + o_item_off);
+        p.mc_off = (int32_t *)(base + o_mc_off);
+        p.item_row = (int32_t *)(base + o_item_row);
+        p.mc_row = (int32_t *)(base + o_mc_row);
+        p.seam = (int32_t *)(base + o_seam);
+        p.row_fail = (int32_t *)(base + o_fail);
+        p.chunk_sym = (uint16_t *)(base + o_sym);
+        p.slabs = base + o_slabs;
+    }
+    return p;
+}
+
+// Work list: one item per short row, ceil(len / core) items per long row.  Single workgroup.
+__global__ __launch_bounds__(1024) void bpe_plan_kernel(
+    const int64_t *__restrict__ offsets, int64_t n_rows, int chunking, BpePlan p)
+{
+    __shared__ uint32_t wt[2][16];
+    __shared__ int32_t carry[2];
+    if (threadIdx.x == 0) { carry[0] = 0; carry[1] = 0; }
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    for (int64_t base = 0; base < n_rows; base += 1024) {
+        const int64_t row = base + threadIdx.x;
+        uint32_t nc = 0, mc = 0;
+        if (row < n_rows) {
+            const int64_t len = offsets[row + 1] - offsets[row];
+            nc = 1;
+            if (len > kLdsCap && chunking) { nc = (uint32_t)((len + kChunkCore - 1) / kChunkCore); mc = nc; }
+            p.row_fail[row] = (len > kLdsCap && !chunking) ? 1 : 0;
+        }
+        const uint32_t inc0 = wave_inclusive_sum_u32(nc), inc1 = wave_inclusive_sum_u32(mc);
+        if (lane == 63) { wt[0][wv] = inc0; wt[1][wv] = inc1; }
+        __syncthreads();
+        uint32_t b0 = 0, b1 = 0, t0 = 0, t1 = 0;
+#pragma unroll
+        for (int w = 0; w < 16; ++w) {
+            if (w < wv) { b0 += wt[0][w]; b1 += wt[1][w]; }
+            t0 += wt[0][w]; t1 += wt[1][w];
+        }
+        const int32_t c0 = carry[0], c1 = carry[1];
+        if (row < n_rows) {
+            const int32_t io = c0 + (int32_t)(b0 + inc0 - nc), mo = c1 + (int32_t)(b1 + inc1 - mc);
+            p.item_off[row] = io;
+            p.mc_off[row] = mo;
+            for (uint32_t k = 0; k < nc; ++k) p.item_row[io + k] = (int32_t)row;
+            for (uint32_t k = 0; k < mc; ++k) { p.mc_row[mo + k] = (int32_t)row; p.seam[mo + k] = -1; }
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) { carry[0] = c0 + (int32_t)t0; carry[1] = c1 + (int32_t)t1; }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        p.item_off[n_rows] = carry[0];
+        p.mc_off[n_rows] = carry[1];
+        p.counts[0] = carry[0];
+        p.counts[1] = carry[1];
+        p.counts[2] = 0;
+    }
+}
+
+// Rows and chunks of at most CAP bytes, state in LDS.  NT = 64: every wave of the workgroup
+// takes its own item (no workgroup barrier after the set-up); NT = blockDim.x: the workgroup
+// shares an item.  Items are handed out through an atomic counter.
 template <int NT, int TEAMS, int CAP, bool TAB_LDS>
 __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     BpeArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
-    int64_t n_rows, int32_t *__restrict__ tok_tmp, int32_t *__restrict__ lengths)
+    BpePlan p, int32_t *__restrict__ tok_tmp, int32_t *__restrict__ lengths)
 {
     extern __shared__ __align__(16) uint8_t smem[];
     uint8_t *sp = smem;
@@ -294,6 +423,7 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     uint16_t *b2s = reinterpret_cast<uint16_t *>(sp); sp += 512;
     for (int i = threadIdx.x; i < 256; i += NT * TEAMS) b2s[i] = a.byte_to_sym[i];
     const int team = threadIdx.x / NT, tid = threadIdx.x % NT;
+    int32_t *next_item = reinterpret_cast<int32_t *>(sp) + team; sp += 16 * sizeof(int32_t);
     uint32_t *red = reinterpret_cast<uint32_t *>(sp) + team * (4 * (NT / 64)); sp += TEAMS * 4 * (NT / 64) * 4;
     uint16_t *S = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
     uint16_t *R = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
@@ -304,27 +434,119 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     __syncthreads();
 
     const uint32_t mask = a.slots - 1;
-    for (int64_t row = (int64_t)blockIdx.x * TEAMS + team; row < n_rows; row += (int64_t)gridDim.x * TEAMS) {
+    const int32_t n_items = p.counts[0];
+    for (;;) {
+        if (tid == 0) *next_item = atomicAdd(&p.counts[2], 1);
+        team_sync<NT>();
+        const int32_t item = *next_item;
+        team_sync<NT>();
+        if (item >= n_items) break;
+        const int32_t row = p.item_row[item];
+        const int32_t k = item - p.item_off[row];
+        const int32_t nc = p.item_off[row + 1] - p.item_off[row];
         const int64_t start = offsets[row];
         const int64_t len = offsets[row + 1] - start;
-        if (len > CAP) {                         // left to the long-row kernel, which overwrites this
-            if (tid == 0) lengths[row] = -1;
-            continue;
+        // one straight path per iteration (no `continue`): every lane of the team must come
+        // back to the fetch above together, or lanes that skipped ahead would re-read the
+        // old item while lane 0 has not fetched the next one yet
+        if (nc == 1 && (len > CAP || len <= 0)) {
+            // too long: left to the whole-row kernel (row_fail is set); empty: no tokens
+            if (tid == 0) lengths[row] = len > CAP ? -1 : 0;
+        } else if (nc == 1) {
+            bpe_row<NT, uint16_t>(tab, mask, a.shift, newsym, minchild, b2s, a.out_remap, bytes + start,
+                                  (int)len, S, R, NX, PV, F, D, red, tid, tok_tmp + start, lengths + row);
+        } else {
+            const int64_t e0 = (int64_t)k * kChunkCore - kChunkOverlap < 0 ? 0 : (int64_t)k * kChunkCore - kChunkOverlap;
+            int64_t e1 = (int64_t)(k + 1) * kChunkCore + kChunkOverlap;
+            if (e1 > len) e1 = len;
+            uint16_t *raw = p.chunk_sym + (size_t)(p.mc_off[row] + k) * kLdsCap;
+            bpe_row<NT, uint16_t>(tab, mask, a.shift, newsym, minchild, b2s, a.out_remap, bytes + start + e0,
+                                  (int)(e1 - e0), S, R, NX, PV, F, D, red, tid, nullptr, nullptr, raw);
         }
-        if (len <= 0) { if (tid == 0) lengths[row] = 0; continue; }
-        bpe_row<NT, uint16_t>(tab, mask, a.shift, newsym, minchild, b2s, a.out_remap, bytes + start,
-                              (int)len, S, R, NX, PV, F, D, red, tid, tok_tmp + start, lengths + row);
         team_sync<NT>();
     }
 }
 
-// Rows longer than min_len: one workgroup per row, state in global scratch (13 bytes / base).
+// One workgroup per chunk of a multi-chunk row: the seam with the chunk to its right.
+__global__ __launch_bounds__(256) void bpe_seam_kernel(const int64_t *__restrict__ offsets, BpePlan p)
+{
+    __shared__ uint32_t best[4];
+    const int32_t n_mc = p.counts[1];
+    for (int32_t m = blockIdx.x; m < n_mc; m += gridDim.x) {
+        const int32_t row = p.mc_row[m];
+        const int32_t k = m - p.mc_off[row];
+        const int32_t nc = p.mc_off[row + 1] - p.mc_off[row];
+        if (k + 1 >= nc) continue;                                   // last chunk: no seam to the right
+        const int64_t len = offsets[row + 1] - offsets[row];
+        const int64_t ea0 = (int64_t)k * kChunkCore - kChunkOverlap < 0 ? 0 : (int64_t)k * kChunkCore - kChunkOverlap;
+        int64_t ea1 = (int64_t)(k + 1) * kChunkCore + kChunkOverlap;
+        if (ea1 > len) ea1 = len;
+        const int64_t eb0 = (int64_t)(k + 1) * kChunkCore - kChunkOverlap;
+        const uint16_t *A = p.chunk_sym + (size_t)m * kLdsCap;       // A[i - ea0]
+        const uint16_t *B = p.chunk_sym + (size_t)(m + 1) * kLdsCap; // B[i - eb0]
+        uint32_t mine = 0xFFFFFFFFu;
+        for (int64_t i = eb0 + threadIdx.x; i < ea1; i += 256) {
+            const uint32_t sa = A[i - ea0];
+            if (sa == kNone || sa != B[i - eb0]) continue;
+            int64_t j = i + 1;                                       // next token start in A
+            while (j < ea1 && A[j - ea0] == kNone) ++j;
+            if (j < ea1 && A[j - ea0] == B[j - eb0]) { mine = (uint32_t)j; break; }
+        }
+        mine = wave_min_u32(mine);
+        if ((threadIdx.x & 63) == 0) best[threadIdx.x >> 6] = mine;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            const uint32_t b = umin(umin(best[0], best[1]), umin(best[2], best[3]));
+            if (b == 0xFFFFFFFFu) { p.seam[m] = -1; p.row_fail[row] = 1; }
+            else p.seam[m] = (int32_t)b;
+        }
+        __syncthreads();
+    }
+}
+
+// One workgroup per multi-chunk row: tokens of chunk k between seam k-1 and seam k, compacted.
+__global__ __launch_bounds__(1024) void bpe_gather_kernel(
+    BpeArgs a, const int64_t *__restrict__ offsets, int64_t n_rows, BpePlan p,
+    int32_t *__restrict__ tok_tmp, int32_t *__restrict__ lengths)
+{
+    __shared__ uint32_t red[16];
+    const int wv = threadIdx.x >> 6;
+    for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
+        const int32_t nc = p.mc_off[row + 1] - p.mc_off[row];
+        if (nc <= 1 || p.row_fail[row]) continue;
+        const int32_t m0 = p.mc_off[row];
+        const int64_t start = offsets[row];
+        const int64_t len = offsets[row + 1] - start;
+        int32_t *out = tok_tmp + start;
+        int64_t written = 0;
+        for (int64_t base = 0; base < len; base += 1024) {
+            const int64_t i = base + threadIdx.x;
+            uint32_t sym = kNone;
+            if (i < len) {
+                int32_t k = (int32_t)(i / kChunkCore);
+                if (k >= nc) k = nc - 1;
+                if (k > 0 && i < p.seam[m0 + k - 1]) --k;            // still left of the seam before chunk k
+                else if (k + 1 < nc && i >= p.seam[m0 + k]) ++k;     // already right of the seam after chunk k
+                const int64_t e0 = (int64_t)k * kChunkCore - kChunkOverlap < 0 ? 0 : (int64_t)k * kChunkCore - kChunkOverlap;
+                sym = p.chunk_sym[(size_t)(m0 + k) * kLdsCap + (i - e0)];
+            }
+            const uint32_t live = sym != kNone;
+            uint32_t total;
+            const uint32_t off = team_exclusive_sum<1024>(live, red, wv, total);
+            if (live) out[written + off] = a.out_remap ? a.out_remap[sym] : (int32_t)sym;
+            written += total;
+        }
+        if (threadIdx.x == 0) lengths[row] = (int32_t)written;
+    }
+}
+
+// Whole-row kernel for rows above the LDS capacity that could not be chunked: one workgroup per
+// row, state in global scratch (13 bytes / base).
 template <int NT>
 __global__ __launch_bounds__(NT) void bpe_long_kernel(
     BpeArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
-    int64_t n_rows, int64_t min_len, int64_t max_len, uint8_t *__restrict__ scratch,
-    int64_t scratch_stride,
-    int32_t *__restrict__ tok_tmp, int32_t *__restrict__ lengths)
+    int64_t n_rows, int64_t max_len, BpePlan p, int32_t *__restrict__ tok_tmp,
+    int32_t *__restrict__ lengths)
 {
     __shared__ uint32_t red[4 * (NT / 64)];
     __shared__ uint8_t D[NT];
@@ -332,12 +554,12 @@ __global__ __launch_bounds__(NT) void bpe_long_kernel(
     for (int i = threadIdx.x; i < 256; i += NT) b2s[i] = a.byte_to_sym[i];
     __syncthreads();
     // each workgroup owns one slab of scratch, sized for the longest row
-    uint8_t *slab = scratch + (size_t)blockIdx.x * (size_t)scratch_stride;
+    uint8_t *slab = p.slabs + (size_t)blockIdx.x * p.slab_bytes;
     const uint32_t mask = a.slots - 1;
     for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
+        if (!p.row_fail[row]) continue;
         const int64_t start = offsets[row];
         const int64_t len = offsets[row + 1] - start;
-        if (len <= min_len) continue;
         if (len > max_len) {                     // longer than the caller declared: no room in the slab
             if (threadIdx.x == 0) lengths[row] = -1;
             continue;
@@ -353,16 +575,6 @@ __global__ __launch_bounds__(NT) void bpe_long_kernel(
                               tok_tmp + start, lengths + row);
         __syncthreads();
     }
-}
-
-constexpr int kLdsCap = 4096;            // longest row the LDS kernels take
-constexpr int kLongThreads = 1024;
-constexpr int kLongGrid = 512;           // slabs of scratch for the long-row kernel
-
-static size_t long_slab_bytes(int64_t max_len)
-{
-    const size_t n = ((size_t)max_len + 7) & ~(size_t)7;
-    return ((n * 13) + 255) & ~(size_t)255;
 }
 
 }  // namespace dnatok
@@ -459,28 +671,28 @@ extern "C" void dnatok_bpe_table_destroy(dnatok_bpe_t *t)
 extern "C" size_t dnatok_bpe_scratch_bytes(const dnatok_bpe_t *t, int64_t n_rows, int64_t max_len,
                                            int64_t total)
 {
-    (void)t; (void)total;
-    if (max_len <= kLdsCap || n_rows <= 0) return 256;
-    const int64_t slabs = n_rows < kLongGrid ? n_rows : kLongGrid;
-    return (size_t)slabs * long_slab_bytes(max_len);
+    (void)t;
+    if (n_rows <= 0) return 256;
+    return make_plan(nullptr, n_rows, max_len, total).total_bytes;
 }
 
 namespace {
 
 template <int NT, int TEAMS, int CAP, bool TAB_LDS>
 int launch_lds(const dnatok_bpe_t *t, const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets,
-               int64_t n_rows, int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
+               const BpePlan &p, int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
 {
-    size_t lds = 512 + (size_t)TEAMS * 4 * (NT / 64) * 4 + (size_t)TEAMS * CAP * 9 + (size_t)TEAMS * NT + 64;
+    size_t lds = 512 + 64 + (size_t)TEAMS * 4 * (NT / 64) * 4 + (size_t)TEAMS * CAP * 9 + (size_t)TEAMS * NT + 64;
     if (TAB_LDS)
         lds += (size_t)t->slots * sizeof(uint2) + 2 * ((((size_t)t->n_merges * 2) + 15) & ~(size_t)15);
     auto kern = bpe_lds_kernel<NT, TEAMS, CAP, TAB_LDS>;
     DNATOK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    int64_t grid = (n_rows + TEAMS - 1) / TEAMS;
-    const int64_t cap = TAB_LDS ? 256 * 2 : 256 * 8;   // persistent workgroups when the table is staged
-    if (grid > cap) grid = cap;
-    kern<<<(int)grid, NT * TEAMS, lds, s>>>(a, bytes, offsets, n_rows, tok_tmp, lengths);
+    const int resident = resident_workgroups(kern, NT * TEAMS, lds, 2);
+    int64_t grid = (p.max_items + TEAMS - 1) / TEAMS;
+    if (grid > resident) grid = resident;
+    if (grid < 1) grid = 1;
+    kern<<<(int)grid, NT * TEAMS, lds, s>>>(a, bytes, offsets, p, tok_tmp, lengths);
     DNATOK_HIP_TRY(hipGetLastError());
     return DNATOK_OK;
 }
@@ -494,37 +706,50 @@ extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, co
     DNATOK_REQUIRE(t && offsets && lengths, DNATOK_E_INVALID, "dnatok_bpe_encode: null argument");
     DNATOK_REQUIRE(n_rows >= 0 && max_len >= 0 && total >= 0, DNATOK_E_INVALID,
                    "dnatok_bpe_encode: negative size");
-    DNATOK_REQUIRE(max_len < (int64_t)1 << 31, DNATOK_E_TOO_LARGE,
-                   "dnatok_bpe_encode: rows of 2^31 bytes or more are not supported");
+    DNATOK_REQUIRE(max_len < (int64_t)1 << 31 && total / kChunkCore + n_rows < (int64_t)1 << 30, DNATOK_E_TOO_LARGE,
+                   "dnatok_bpe_encode: batch too large for 32-bit work indices");
     if (n_rows == 0) return DNATOK_OK;
     DNATOK_REQUIRE(total == 0 || (bytes && tok_tmp), DNATOK_E_INVALID, "dnatok_bpe_encode: null buffer");
+    const BpePlan need = make_plan(nullptr, n_rows, max_len, total);
+    DNATOK_REQUIRE(scratch && scratch_bytes >= need.total_bytes, DNATOK_E_SCRATCH,
+                   "dnatok_bpe_encode: scratch holds %zu bytes, %zu needed", scratch_bytes, need.total_bytes);
+    DNATOK_REQUIRE(((uintptr_t)scratch & 255) == 0, DNATOK_E_INVALID, "dnatok_bpe_encode: scratch must be 256-byte aligned");
+    const BpePlan p = make_plan((uint8_t *)scratch, n_rows, max_len, total);
     hipStream_t s = (hipStream_t)stream;
     BpeArgs a{t->tab, t->newsym, t->minchild, t->byte_to_sym, t->out_remap, t->slots, t->shift, t->n_merges};
 
     static const char *variant_env = getenv("DNATOK_BPE_VARIANT");
+    static const char *chunk_env = getenv("DNATOK_BPE_NO_CHUNKS");
     const int variant = variant_env ? atoi(variant_env) : 0;
+    const bool long_rows = max_len > kLdsCap;
+    const int chunking = (long_rows && t->monotone && !chunk_env) ? 1 : 0;
+    bpe_plan_kernel<<<1, 1024, 0, s>>>(offsets, n_rows, chunking, p);
+    DNATOK_HIP_TRY(hipGetLastError());
+
     const size_t tab_lds_bytes = (size_t)t->slots * sizeof(uint2) + 4 * (size_t)t->n_merges;
     const bool tab_fits = tab_lds_bytes <= 96 * 1024;
     int rc;
     switch (variant) {
-        case 1:  rc = launch_lds<256, 1, kLdsCap, false>(t, a, bytes, offsets, n_rows, tok_tmp, lengths, s); break;
-        case 2:  rc = tab_fits ? launch_lds<256, 1, kLdsCap, true>(t, a, bytes, offsets, n_rows, tok_tmp, lengths, s)
-                               : launch_lds<256, 1, kLdsCap, false>(t, a, bytes, offsets, n_rows, tok_tmp, lengths, s);
+        case 2:  rc = tab_fits ? launch_lds<256, 1, kLdsCap, true>(t, a, bytes, offsets, p, tok_tmp, lengths, s)
+                               : launch_lds<256, 1, kLdsCap, false>(t, a, bytes, offsets, p, tok_tmp, lengths, s);
                  break;
-        case 3:  rc = launch_lds<64, 4, kLdsCap, false>(t, a, bytes, offsets, n_rows, tok_tmp, lengths, s); break;
-        case 4:  rc = launch_lds<1024, 1, kLdsCap, false>(t, a, bytes, offsets, n_rows, tok_tmp, lengths, s); break;
-        default: rc = launch_lds<256, 1, kLdsCap, false>(t, a, bytes, offsets, n_rows, tok_tmp, lengths, s); break;
+        case 3:  rc = launch_lds<64, 4, kLdsCap, false>(t, a, bytes, offsets, p, tok_tmp, lengths, s); break;
+        case 4:  rc = launch_lds<1024, 1, kLdsCap, false>(t, a, bytes, offsets, p, tok_tmp, lengths, s); break;
+        default: rc = launch_lds<256, 1, kLdsCap, false>(t, a, bytes, offsets, p, tok_tmp, lengths, s); break;
     }
     if (rc) return rc;
-    if (max_len > kLdsCap) {
+    if (long_rows) {
+        if (chunking) {
+            int64_t g = p.max_mc < 4096 ? p.max_mc : 4096;
+            bpe_seam_kernel<<<(int)(g < 1 ? 1 : g), 256, 0, s>>>(offsets, p);
+            DNATOK_HIP_TRY(hipGetLastError());
+            int64_t gr = n_rows < 1024 ? n_rows : 1024;
+            bpe_gather_kernel<<<(int)gr, 1024, 0, s>>>(a, offsets, n_rows, p, tok_tmp, lengths);
+            DNATOK_HIP_TRY(hipGetLastError());
+        }
         const int64_t slabs = n_rows < kLongGrid ? n_rows : kLongGrid;
-        const size_t slab = long_slab_bytes(max_len);
-        DNATOK_REQUIRE(scratch && scratch_bytes >= (size_t)slabs * slab, DNATOK_E_SCRATCH,
-                       "dnatok_bpe_encode: scratch holds %zu bytes, %zu needed", scratch_bytes,
-                       (size_t)slabs * slab);
-        bpe_long_kernel<kLongThreads><<<(int)slabs, kLongThreads, 0, s>>>(
-            a, bytes, offsets, n_rows, (int64_t)kLdsCap, max_len, (uint8_t *)scratch, (int64_t)slab,
-            tok_tmp, lengths);
+        bpe_long_kernel<kLongThreads><<<(int)slabs, kLongThreads, 0, s>>>(a, bytes, offsets, n_rows, max_len, p,
+                                                                         tok_tmp, lengths);
         DNATOK_HIP_TRY(hipGetLastError());
     }
     return DNATOK_OK;
