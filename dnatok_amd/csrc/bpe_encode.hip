@@ -6,7 +6,7 @@
 //
 //   * every live position i keeps the rank R[i] of the pair it starts; a team of threads
 //     (one wave, or one workgroup) finds rmin = min R and the gate G = min over current
-//     pairs of minchild[R[i]], where minchild[r] is the lowest rank of any rule that uses the
+//     pairs of gate(R[i]), where gate(r) is the lowest rank of any rule that uses the
 //     symbol rule r creates.  No pair born in this round can have a rank below G, so all
 //     current pairs with rank in [rmin, G) can be settled together;
 //   * among those candidates a pair merges unless an overlapping candidate with a smaller
@@ -35,9 +35,7 @@ struct dnatok_bpe_table {
     uint32_t slots, shift;       // hash table size (power of two) and 32 - log2(slots)
     int monotone;                // no rule's product is used by a lower-ranked rule
     void *blob;
-    uint2 *tab;                  // [slots]  {key = a << 16 | b, val = rank}
-    uint16_t *newsym;            // [n_merges]
-    uint16_t *minchild;          // [n_merges]
+    uint4 *tab;                  // [slots]  {key = a << 16 | b, rank, product | gate << 16, 0}
     uint16_t *byte_to_sym;       // [256]
     int32_t *out_remap;          // [n_symbols] or nullptr
 };
@@ -48,11 +46,17 @@ constexpr uint32_t kNone = 0xFFFFu;          // "no rule" rank / dead symbol
 constexpr uint32_t kEmptyKey = 0xFFFFFFFFu;
 
 struct BpeArgs {
-    const uint2 *tab;
-    const uint16_t *newsym, *minchild, *byte_to_sym;
+    const uint4 *tab;
+    const uint16_t *byte_to_sym;
     const int32_t *out_remap;
     uint32_t slots, shift;
     int32_t n_merges;
+};
+
+// What a position keeps about the pair it starts: the rule's rank (kNone = no rule), the
+// symbol the rule produces, and the rule's gate (lowest rank of any rule using that product).
+struct PairInfo {
+    uint32_t rank, product, gate;
 };
 
 __host__ __device__ __forceinline__ uint32_t pair_hash(uint32_t key, uint32_t shift)
@@ -60,17 +64,25 @@ __host__ __device__ __forceinline__ uint32_t pair_hash(uint32_t key, uint32_t sh
     return (key * 0x9E3779B1u) >> shift;
 }
 
-// rank of the rule for (a, b), or kNone
-__device__ __forceinline__ uint32_t pair_rank(const uint2 *tab, uint32_t mask, uint32_t shift,
-                                              uint32_t a, uint32_t b)
+// First probe of the rule for (a, b): issued for several pairs back to back, so that their
+// memory latencies overlap; pair_finish resolves the (rare) collisions afterwards.
+__device__ __forceinline__ uint4 pair_probe(const uint4 *tab, uint32_t shift, uint32_t a, uint32_t b,
+                                            uint32_t *slot)
+{
+    const uint32_t h = pair_hash((a << 16) | b, shift);
+    *slot = h;
+    return tab[h];
+}
+
+__device__ __forceinline__ PairInfo pair_finish(const uint4 *tab, uint32_t mask, uint32_t a, uint32_t b,
+                                                uint4 e, uint32_t h)
 {
     const uint32_t key = (a << 16) | b;
-    uint32_t h = pair_hash(key, shift);
     for (;;) {
-        const uint2 e = tab[h];
-        if (e.x == key) return e.y;
-        if (e.x == kEmptyKey) return kNone;
+        if (e.x == key) return PairInfo{e.y, e.z & 0xFFFFu, e.z >> 16};
+        if (e.x == kEmptyKey) return PairInfo{kNone, kNone, kNone};
         h = (h + 1) & mask;
+        e = tab[h];
     }
 }
 
@@ -126,15 +138,14 @@ __device__ __forceinline__ uint32_t team_exclusive_sum(uint32_t v, uint32_t *red
     return carry + inc - v;
 }
 
-// One row.  tid = index in the team; S/R/NX/PV/F hold n0 entries; D holds NT bytes;
+// One row.  tid = index in the team; S/R/NS/MC/NX/PV/F hold n0 entries; D holds NT bytes;
 // red holds 4 * (NT / 64) words.  Tokens go to out[0 .. *out_len).
 template <int NT, typename IT>
 __device__ __forceinline__ void bpe_row(
-    const uint2 *tab, uint32_t tab_mask, uint32_t tab_shift, const uint16_t *newsym,
-    const uint16_t *minchild, const uint16_t *byte_to_sym, const int32_t *out_remap,
-    const uint8_t *__restrict__ src, const int n0, uint16_t *S, uint16_t *R, IT *NX, IT *PV,
-    uint8_t *F, uint8_t *D, uint32_t *red, const int tid, int32_t *__restrict__ out,
-    int32_t *__restrict__ out_len, uint16_t *__restrict__ raw_out = nullptr)
+    const uint4 *tab, uint32_t tab_mask, uint32_t tab_shift, const uint16_t *byte_to_sym,
+    const int32_t *out_remap, const uint8_t *__restrict__ src, const int n0, uint16_t *S, uint16_t *R,
+    uint16_t *NS, uint16_t *MC, IT *NX, IT *PV, uint8_t *F, uint8_t *D, uint32_t *red, const int tid,
+    int32_t *__restrict__ out, int32_t *__restrict__ out_len, uint16_t *__restrict__ raw_out = nullptr)
 {
     constexpr IT NIL = (IT)~(IT)0;
     const int wv = (NT == 64) ? 0 : (tid >> 6);
@@ -151,12 +162,28 @@ __device__ __forceinline__ void bpe_row(
     D[tid] = 0;
     team_sync<NT>();
 
+    // initial pair of every position, four table probes in flight at a time
     uint32_t cmin = kEmptyKey, cgate = kEmptyKey;
-    for (int i = lo; i < hi; ++i) {
-        uint32_t r = kNone;
-        if (i + 1 < n0) r = pair_rank(tab, tab_mask, tab_shift, S[i], S[i + 1]);
-        R[i] = (uint16_t)r;
-        if (r != kNone) { cmin = umin(cmin, r); cgate = umin(cgate, minchild[r]); }
+    for (int i0 = lo; i0 < hi; i0 += 4) {
+        uint4 e[4];
+        uint32_t h[4], sa[4], sb[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = i0 + j;
+            const bool ok = i < hi && i + 1 < n0;
+            sa[j] = ok ? S[i] : 0u;
+            sb[j] = ok ? S[i + 1] : 0u;
+            e[j] = pair_probe(tab, tab_shift, sa[j], sb[j], &h[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = i0 + j;
+            if (i >= hi) continue;
+            PairInfo pi{kNone, kNone, kNone};
+            if (i + 1 < n0) pi = pair_finish(tab, tab_mask, sa[j], sb[j], e[j], h[j]);
+            R[i] = (uint16_t)pi.rank; NS[i] = (uint16_t)pi.product; MC[i] = (uint16_t)pi.gate;
+            if (pi.rank != kNone) { cmin = umin(cmin, pi.rank); cgate = umin(cgate, pi.gate); }
+        }
     }
 
     int flip = 0;
@@ -223,7 +250,7 @@ __device__ __forceinline__ void bpe_row(
                 if (!F[i]) continue;
                 const IT j = NX[i];
                 const IT k = NX[j];
-                S[i] = newsym[R[i]];
+                S[i] = NS[i];
                 S[j] = (uint16_t)kNone;
                 R[j] = (uint16_t)kNone;
                 NX[i] = k;
@@ -233,17 +260,25 @@ __device__ __forceinline__ void bpe_row(
         }
         team_sync<NT>();
 
-        // re-rank the two pairs around every new symbol
+        // re-rank the two pairs around every new symbol (both probes in flight together)
         if (mine) {
             for (int i = lo; i < hi; ++i) {
                 if (!F[i]) continue;
                 F[i] = 0;
                 const IT k = NX[i];
-                const uint32_t s = S[i];
-                R[i] = (uint16_t)((k != NIL) ? pair_rank(tab, tab_mask, tab_shift, s, S[k]) : kNone);
                 const IT p = PV[i];
+                const uint32_t s = S[i];
+                const uint32_t sk = (k != NIL) ? S[k] : 0u;
+                const uint32_t sp = (p != NIL) ? S[p] : 0u;
+                uint32_t h0, h1;
+                const uint4 e0 = pair_probe(tab, tab_shift, s, sk, &h0);
+                const uint4 e1 = pair_probe(tab, tab_shift, sp, s, &h1);
+                PairInfo right{kNone, kNone, kNone};
+                if (k != NIL) right = pair_finish(tab, tab_mask, s, sk, e0, h0);
+                R[i] = (uint16_t)right.rank; NS[i] = (uint16_t)right.product; MC[i] = (uint16_t)right.gate;
                 if (p != NIL) {
-                    R[p] = (uint16_t)pair_rank(tab, tab_mask, tab_shift, S[p], s);
+                    const PairInfo left = pair_finish(tab, tab_mask, sp, s, e1, h1);
+                    R[p] = (uint16_t)left.rank; NS[p] = (uint16_t)left.product; MC[p] = (uint16_t)left.gate;
                     if ((int)p < lo) D[(int)p / c] = 1;
                 }
             }
@@ -255,7 +290,7 @@ __device__ __forceinline__ void bpe_row(
             cmin = kEmptyKey; cgate = kEmptyKey;
             for (int i = lo; i < hi; ++i) {
                 const uint32_t r = R[i];
-                if (r != kNone) { cmin = umin(cmin, r); cgate = umin(cgate, minchild[r]); }
+                if (r != kNone) { cmin = umin(cmin, r); cgate = umin(cgate, MC[i]); }
             }
         }
     }
@@ -314,7 +349,7 @@ struct BpePlan {                          // device arrays inside the scratch bu
 static size_t long_slab_bytes(int64_t max_len)
 {
     const size_t n = ((size_t)max_len + 7) & ~(size_t)7;
-    return ((n * 13) + 255) & ~(size_t)255;
+    return ((n * 17) + 255) & ~(size_t)255;
 }
 
 static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t total)
@@ -400,26 +435,18 @@ __global__ __launch_bounds__(1024) void bpe_plan_kernel(
     }
 }
 
-// Rows and chunks of at most CAP bytes, state in LDS.  NT = 64: every wave of the workgroup
-// takes its own item (no workgroup barrier after the set-up); NT = blockDim.x: the workgroup
-// shares an item.  Items are handed out through an atomic counter.
-template <int NT, int TEAMS, int CAP, bool TAB_LDS>
+// Rows and chunks of at most CAP bytes, state in LDS (13 bytes per position); the merge table
+// stays in global memory (L2-resident) and is probed in batches.  NT = 64: every wave of the
+// workgroup takes its own item (no workgroup barrier after the set-up); NT = blockDim.x: the
+// workgroup shares an item.  Items are handed out through an atomic counter.
+template <int NT, int TEAMS, int CAP>
 __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     BpeArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
     BpePlan p, int32_t *__restrict__ tok_tmp, int32_t *__restrict__ lengths)
 {
     extern __shared__ __align__(16) uint8_t smem[];
     uint8_t *sp = smem;
-    const uint2 *tab = a.tab;
-    const uint16_t *newsym = a.newsym, *minchild = a.minchild;
-    if (TAB_LDS) {
-        uint2 *t = reinterpret_cast<uint2 *>(sp); sp += (size_t)a.slots * sizeof(uint2);
-        uint16_t *ns = reinterpret_cast<uint16_t *>(sp); sp += (((size_t)a.n_merges * 2 + 15) & ~(size_t)15);
-        uint16_t *mc = reinterpret_cast<uint16_t *>(sp); sp += (((size_t)a.n_merges * 2 + 15) & ~(size_t)15);
-        for (uint32_t i = threadIdx.x; i < a.slots; i += NT * TEAMS) t[i] = a.tab[i];
-        for (int i = threadIdx.x; i < a.n_merges; i += NT * TEAMS) { ns[i] = a.newsym[i]; mc[i] = a.minchild[i]; }
-        tab = t; newsym = ns; minchild = mc;
-    }
+    const uint4 *tab = a.tab;
     uint16_t *b2s = reinterpret_cast<uint16_t *>(sp); sp += 512;
     for (int i = threadIdx.x; i < 256; i += NT * TEAMS) b2s[i] = a.byte_to_sym[i];
     const int team = threadIdx.x / NT, tid = threadIdx.x % NT;
@@ -427,6 +454,8 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     uint32_t *red = reinterpret_cast<uint32_t *>(sp) + team * (4 * (NT / 64)); sp += TEAMS * 4 * (NT / 64) * 4;
     uint16_t *S = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
     uint16_t *R = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
+    uint16_t *NS = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
+    uint16_t *MC = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
     uint16_t *NX = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
     uint16_t *PV = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
     uint8_t *F = sp + (size_t)team * CAP; sp += (size_t)TEAMS * CAP;
@@ -453,15 +482,15 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
             // too long: left to the whole-row kernel (row_fail is set); empty: no tokens
             if (tid == 0) lengths[row] = len > CAP ? -1 : 0;
         } else if (nc == 1) {
-            bpe_row<NT, uint16_t>(tab, mask, a.shift, newsym, minchild, b2s, a.out_remap, bytes + start,
-                                  (int)len, S, R, NX, PV, F, D, red, tid, tok_tmp + start, lengths + row);
+            bpe_row<NT, uint16_t>(tab, mask, a.shift, b2s, a.out_remap, bytes + start, (int)len, S, R, NS, MC,
+                                  NX, PV, F, D, red, tid, tok_tmp + start, lengths + row);
         } else {
             const int64_t e0 = (int64_t)k * kChunkCore - kChunkOverlap < 0 ? 0 : (int64_t)k * kChunkCore - kChunkOverlap;
             int64_t e1 = (int64_t)(k + 1) * kChunkCore + kChunkOverlap;
             if (e1 > len) e1 = len;
             uint16_t *raw = p.chunk_sym + (size_t)(p.mc_off[row] + k) * kLdsCap;
-            bpe_row<NT, uint16_t>(tab, mask, a.shift, newsym, minchild, b2s, a.out_remap, bytes + start + e0,
-                                  (int)(e1 - e0), S, R, NX, PV, F, D, red, tid, nullptr, nullptr, raw);
+            bpe_row<NT, uint16_t>(tab, mask, a.shift, b2s, a.out_remap, bytes + start + e0, (int)(e1 - e0),
+                                  S, R, NS, MC, NX, PV, F, D, red, tid, nullptr, nullptr, raw);
         }
         team_sync<NT>();
     }
@@ -541,7 +570,7 @@ __global__ __launch_bounds__(1024) void bpe_gather_kernel(
 }
 
 // Whole-row kernel for rows above the LDS capacity that could not be chunked: one workgroup per
-// row, state in global scratch (13 bytes / base).
+// row, state in global scratch (17 bytes / base).
 template <int NT>
 __global__ __launch_bounds__(NT) void bpe_long_kernel(
     BpeArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
@@ -569,10 +598,11 @@ __global__ __launch_bounds__(NT) void bpe_long_kernel(
         uint32_t *PV = NX + n;
         uint16_t *S = reinterpret_cast<uint16_t *>(PV + n);
         uint16_t *R = S + n;
-        uint8_t *F = reinterpret_cast<uint8_t *>(R + n);
-        bpe_row<NT, uint32_t>(a.tab, mask, a.shift, a.newsym, a.minchild, b2s, a.out_remap,
-                              bytes + start, (int)len, S, R, NX, PV, F, D, red, threadIdx.x,
-                              tok_tmp + start, lengths + row);
+        uint16_t *NS = R + n;
+        uint16_t *MC = NS + n;
+        uint8_t *F = reinterpret_cast<uint8_t *>(MC + n);
+        bpe_row<NT, uint32_t>(a.tab, mask, a.shift, b2s, a.out_remap, bytes + start, (int)len, S, R, NS, MC,
+                              NX, PV, F, D, red, threadIdx.x, tok_tmp + start, lengths + row);
         __syncthreads();
     }
 }
@@ -598,14 +628,13 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
                        "dnatok_bpe_table_create: byte_to_id[%d] out of range", i);
     uint32_t slots = 64, shift = 26;
     while (slots < (uint32_t)n_merges * 2u + 2u) { slots <<= 1; --shift; }
-    std::vector<uint2> tab(slots, uint2{kEmptyKey, kNone});
-    std::vector<uint16_t> newsym(n_merges > 0 ? n_merges : 1), minchild(n_merges > 0 ? n_merges : 1, (uint16_t)kNone);
+    std::vector<uint4> tab(slots, uint4{kEmptyKey, kNone, 0, 0});
+    std::vector<uint32_t> slot_of(n_merges > 0 ? n_merges : 1, 0xFFFFFFFFu);
     std::vector<uint32_t> first_use(n_symbols, 0xFFFFFFFFu);   // lowest rank using a symbol
     for (int32_t i = 0; i < n_merges; ++i) {
         const int32_t pa = pair_a_h[i], pb = pair_b_h[i], nid = new_id_h[i];
         DNATOK_REQUIRE(pa >= 0 && pa < n_symbols && pb >= 0 && pb < n_symbols && nid >= 0 && nid < n_symbols,
                        DNATOK_E_INVALID, "dnatok_bpe_table_create: merge %d has an id out of range", i);
-        newsym[i] = (uint16_t)nid;
         const uint32_t key = ((uint32_t)pa << 16) | (uint32_t)pb;
         uint32_t h = pair_hash(key, shift);
         bool dup = false;
@@ -614,14 +643,15 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
             h = (h + 1) & (slots - 1);
         }
         if (dup) continue;                      // a repeated pair keeps its first rank
-        tab[h] = uint2{key, (uint32_t)i};
+        tab[h] = uint4{key, (uint32_t)i, (uint32_t)nid, 0};
+        slot_of[i] = h;
         if (first_use[pa] == 0xFFFFFFFFu) first_use[pa] = (uint32_t)i;
         if (first_use[pb] == 0xFFFFFFFFu) first_use[pb] = (uint32_t)i;
     }
     int monotone = 1;
     for (int32_t i = 0; i < n_merges; ++i) {
         const uint32_t fu = first_use[new_id_h[i]];
-        minchild[i] = (uint16_t)(fu == 0xFFFFFFFFu ? kNone : fu);
+        if (slot_of[i] != 0xFFFFFFFFu) tab[slot_of[i]].z |= (fu == 0xFFFFFFFFu ? kNone : fu) << 16;
         if (fu <= (uint32_t)i) monotone = 0;
     }
     std::vector<uint16_t> b2s(256);
@@ -629,15 +659,11 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
 
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
     const size_t o_tab = 0;
-    const size_t o_new = up(o_tab + (size_t)slots * sizeof(uint2));
-    const size_t o_mc = up(o_new + newsym.size() * 2);
-    const size_t o_b2s = up(o_mc + minchild.size() * 2);
+    const size_t o_b2s = up(o_tab + (size_t)slots * sizeof(uint4));
     const size_t o_remap = up(o_b2s + 512);
     const size_t total = up(o_remap + (out_remap_h ? (size_t)n_symbols * 4 : 0)) + 256;
     std::vector<uint8_t> host(total, 0);
-    memcpy(&host[o_tab], tab.data(), (size_t)slots * sizeof(uint2));
-    memcpy(&host[o_new], newsym.data(), newsym.size() * 2);
-    memcpy(&host[o_mc], minchild.data(), minchild.size() * 2);
+    memcpy(&host[o_tab], tab.data(), (size_t)slots * sizeof(uint4));
     memcpy(&host[o_b2s], b2s.data(), 512);
     if (out_remap_h) memcpy(&host[o_remap], out_remap_h, (size_t)n_symbols * 4);
     void *blob = nullptr;
@@ -652,9 +678,7 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
     uint8_t *b = (uint8_t *)blob;
     t->n_merges = n_merges; t->n_symbols = n_symbols; t->slots = slots; t->shift = shift;
     t->monotone = monotone; t->blob = blob;
-    t->tab = (uint2 *)(b + o_tab);
-    t->newsym = (uint16_t *)(b + o_new);
-    t->minchild = (uint16_t *)(b + o_mc);
+    t->tab = (uint4 *)(b + o_tab);
     t->byte_to_sym = (uint16_t *)(b + o_b2s);
     t->out_remap = out_remap_h ? (int32_t *)(b + o_remap) : nullptr;
     *out = t;
@@ -678,17 +702,19 @@ extern "C" size_t dnatok_bpe_scratch_bytes(const dnatok_bpe_t *t, int64_t n_rows
 
 namespace {
 
-template <int NT, int TEAMS, int CAP, bool TAB_LDS>
-int launch_lds(const dnatok_bpe_t *t, const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets,
-               const BpePlan &p, int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
+template <int NT, int TEAMS, int CAP>
+int launch_lds(const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets, const BpePlan &p,
+               int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
 {
-    size_t lds = 512 + 64 + (size_t)TEAMS * 4 * (NT / 64) * 4 + (size_t)TEAMS * CAP * 9 + (size_t)TEAMS * NT + 64;
-    if (TAB_LDS)
-        lds += (size_t)t->slots * sizeof(uint2) + 2 * ((((size_t)t->n_merges * 2) + 15) & ~(size_t)15);
-    auto kern = bpe_lds_kernel<NT, TEAMS, CAP, TAB_LDS>;
-    DNATOK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    const int resident = resident_workgroups(kern, NT * TEAMS, lds, 2);
+    const size_t lds = 512 + 64 + (size_t)TEAMS * 4 * (NT / 64) * 4 + (size_t)TEAMS * CAP * 13 + (size_t)TEAMS * NT + 64;
+    auto kern = bpe_lds_kernel<NT, TEAMS, CAP>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        DNATOK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_set = true;
+    }
+    static const int resident = resident_workgroups(kern, NT * TEAMS, lds, 2);
     int64_t grid = (p.max_items + TEAMS - 1) / TEAMS;
     if (grid > resident) grid = resident;
     if (grid < 1) grid = 1;
@@ -716,7 +742,7 @@ extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, co
     DNATOK_REQUIRE(((uintptr_t)scratch & 255) == 0, DNATOK_E_INVALID, "dnatok_bpe_encode: scratch must be 256-byte aligned");
     const BpePlan p = make_plan((uint8_t *)scratch, n_rows, max_len, total);
     hipStream_t s = (hipStream_t)stream;
-    BpeArgs a{t->tab, t->newsym, t->minchild, t->byte_to_sym, t->out_remap, t->slots, t->shift, t->n_merges};
+    BpeArgs a{t->tab, t->byte_to_sym, t->out_remap, t->slots, t->shift, t->n_merges};
 
     static const char *variant_env = getenv("DNATOK_BPE_VARIANT");
     static const char *chunk_env = getenv("DNATOK_BPE_NO_CHUNKS");
@@ -726,17 +752,13 @@ extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, co
     bpe_plan_kernel<<<1, 1024, 0, s>>>(offsets, n_rows, chunking, p);
     DNATOK_HIP_TRY(hipGetLastError());
 
-    const size_t tab_lds_bytes = (size_t)t->slots * sizeof(uint2) + 4 * (size_t)t->n_merges;
-    const bool tab_fits = tab_lds_bytes <= 96 * 1024;
+    // the LDS capacity variant follows the longest row (or the chunk size for longer rows):
+    // less LDS per workgroup means more workgroups per CU
     int rc;
-    switch (variant) {
-        case 2:  rc = tab_fits ? launch_lds<256, 1, kLdsCap, true>(t, a, bytes, offsets, p, tok_tmp, lengths, s)
-                               : launch_lds<256, 1, kLdsCap, false>(t, a, bytes, offsets, p, tok_tmp, lengths, s);
-                 break;
-        case 3:  rc = launch_lds<64, 4, kLdsCap, false>(t, a, bytes, offsets, p, tok_tmp, lengths, s); break;
-        case 4:  rc = launch_lds<1024, 1, kLdsCap, false>(t, a, bytes, offsets, p, tok_tmp, lengths, s); break;
-        default: rc = launch_lds<256, 1, kLdsCap, false>(t, a, bytes, offsets, p, tok_tmp, lengths, s); break;
-    }
+    if (variant == 3)            rc = launch_lds<64, 4, kLdsCap>(a, bytes, offsets, p, tok_tmp, lengths, s);
+    else if (max_len <= 1024)    rc = launch_lds<256, 1, 1024>(a, bytes, offsets, p, tok_tmp, lengths, s);
+    else if (max_len <= 2048)    rc = launch_lds<256, 1, 2048>(a, bytes, offsets, p, tok_tmp, lengths, s);
+    else                         rc = launch_lds<256, 1, kLdsCap>(a, bytes, offsets, p, tok_tmp, lengths, s);
     if (rc) return rc;
     if (long_rows) {
         if (chunking) {
