@@ -149,11 +149,10 @@ __device__ __forceinline__ void bpe_row(
 {
     constexpr IT NIL = (IT)~(IT)0;
     const int wv = (NT == 64) ? 0 : (tid >> 6);
-    const int c = (n0 + NT - 1) / NT;
-    const int lo = (tid * c < n0) ? tid * c : n0;
-    const int hi = (lo + c < n0) ? lo + c : n0;
+    // position i belongs to thread i % NT: in every pass the lanes of a wave touch consecutive
+    // positions, so the LDS state arrays are read and written without bank conflicts
 
-    for (int i = lo; i < hi; ++i) {
+    for (int i = tid; i < n0; i += NT) {
         S[i] = byte_to_sym[src[i]];
         NX[i] = (i + 1 < n0) ? (IT)(i + 1) : NIL;
         PV[i] = (i > 0) ? (IT)(i - 1) : NIL;
@@ -164,21 +163,21 @@ __device__ __forceinline__ void bpe_row(
 
     // initial pair of every position, four table probes in flight at a time
     uint32_t cmin = kEmptyKey, cgate = kEmptyKey;
-    for (int i0 = lo; i0 < hi; i0 += 4) {
+    for (int i0 = tid; i0 < n0; i0 += 4 * NT) {
         uint4 e[4];
         uint32_t h[4], sa[4], sb[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int i = i0 + j;
-            const bool ok = i < hi && i + 1 < n0;
+            const int i = i0 + j * NT;
+            const bool ok = i + 1 < n0;
             sa[j] = ok ? S[i] : 0u;
             sb[j] = ok ? S[i + 1] : 0u;
             e[j] = pair_probe(tab, tab_shift, sa[j], sb[j], &h[j]);
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int i = i0 + j;
-            if (i >= hi) continue;
+            const int i = i0 + j * NT;
+            if (i >= n0) continue;
             PairInfo pi{kNone, kNone, kNone};
             if (i + 1 < n0) pi = pair_finish(tab, tab_mask, sa[j], sb[j], e[j], h[j]);
             R[i] = (uint16_t)pi.rank; NS[i] = (uint16_t)pi.product; MC[i] = (uint16_t)pi.gate;
@@ -200,7 +199,7 @@ __device__ __forceinline__ void bpe_row(
         if (single) {
             uint32_t mypos = kEmptyKey;
             if (cmin == rmin)
-                for (int i = lo; i < hi; ++i)
+                for (int i = tid; i < n0; i += NT)
                     if (R[i] == rmin) { mypos = (uint32_t)i; break; }
             uint32_t dummy;
             team_min2<NT>(mypos, mypos, red + flip * (NT / 64) * 2, wv, leftmost, dummy);
@@ -211,7 +210,7 @@ __device__ __forceinline__ void bpe_row(
         // decide (reads only, except the owner's own flags)
         bool mine = false;
         if (cmin < limit) {
-            for (int i = lo; i < hi; ++i) {
+            for (int i = tid; i < n0; i += NT) {
                 const uint32_t r = R[i];
                 if (r >= limit) continue;
                 bool m;
@@ -246,7 +245,7 @@ __device__ __forceinline__ void bpe_row(
 
         // apply: position i absorbs its right neighbour j
         if (mine) {
-            for (int i = lo; i < hi; ++i) {
+            for (int i = tid; i < n0; i += NT) {
                 if (!F[i]) continue;
                 const IT j = NX[i];
                 const IT k = NX[j];
@@ -255,31 +254,48 @@ __device__ __forceinline__ void bpe_row(
                 R[j] = (uint16_t)kNone;
                 NX[i] = k;
                 if (k != NIL) PV[k] = (IT)i;
-                if ((int)j >= hi) D[(int)j / c] = 1;
+                D[(int)j % NT] = 1;           // j's owner must refresh its cached minimum
             }
         }
         team_sync<NT>();
 
-        // re-rank the two pairs around every new symbol (both probes in flight together)
+        // re-rank the two pairs around every new symbol; the probes of four positions (eight
+        // table reads) are in flight together
         if (mine) {
-            for (int i = lo; i < hi; ++i) {
-                if (!F[i]) continue;
-                F[i] = 0;
-                const IT k = NX[i];
-                const IT p = PV[i];
-                const uint32_t s = S[i];
-                const uint32_t sk = (k != NIL) ? S[k] : 0u;
-                const uint32_t sp = (p != NIL) ? S[p] : 0u;
-                uint32_t h0, h1;
-                const uint4 e0 = pair_probe(tab, tab_shift, s, sk, &h0);
-                const uint4 e1 = pair_probe(tab, tab_shift, sp, s, &h1);
-                PairInfo right{kNone, kNone, kNone};
-                if (k != NIL) right = pair_finish(tab, tab_mask, s, sk, e0, h0);
-                R[i] = (uint16_t)right.rank; NS[i] = (uint16_t)right.product; MC[i] = (uint16_t)right.gate;
-                if (p != NIL) {
-                    const PairInfo left = pair_finish(tab, tab_mask, sp, s, e1, h1);
-                    R[p] = (uint16_t)left.rank; NS[p] = (uint16_t)left.product; MC[p] = (uint16_t)left.gate;
-                    if ((int)p < lo) D[(int)p / c] = 1;
+            for (int i0 = tid; i0 < n0; i0 += 4 * NT) {
+                uint4 e0[4], e1[4];
+                uint32_t h0[4], h1[4], s[4], sk[4], sp[4];
+                IT kk[4], pp[4];
+                bool on[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int i = i0 + j * NT;
+                    on[j] = i < n0 && F[i];
+                    kk[j] = NIL; pp[j] = NIL; s[j] = 0; sk[j] = 0; sp[j] = 0;
+                    if (on[j]) {
+                        F[i] = 0;
+                        kk[j] = NX[i];
+                        pp[j] = PV[i];
+                        s[j] = S[i];
+                        if (kk[j] != NIL) sk[j] = S[kk[j]];
+                        if (pp[j] != NIL) sp[j] = S[pp[j]];
+                    }
+                    e0[j] = pair_probe(tab, tab_shift, s[j], sk[j], &h0[j]);
+                    e1[j] = pair_probe(tab, tab_shift, sp[j], s[j], &h1[j]);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (!on[j]) continue;
+                    const int i = i0 + j * NT;
+                    PairInfo right{kNone, kNone, kNone};
+                    if (kk[j] != NIL) right = pair_finish(tab, tab_mask, s[j], sk[j], e0[j], h0[j]);
+                    R[i] = (uint16_t)right.rank; NS[i] = (uint16_t)right.product; MC[i] = (uint16_t)right.gate;
+                    if (pp[j] != NIL) {
+                        const PairInfo left = pair_finish(tab, tab_mask, sp[j], s[j], e1[j], h1[j]);
+                        const int p = (int)pp[j];
+                        R[p] = (uint16_t)left.rank; NS[p] = (uint16_t)left.product; MC[p] = (uint16_t)left.gate;
+                        D[p % NT] = 1;
+                    }
                 }
             }
         }
@@ -288,7 +304,7 @@ __device__ __forceinline__ void bpe_row(
         if (mine || D[tid]) {
             D[tid] = 0;
             cmin = kEmptyKey; cgate = kEmptyKey;
-            for (int i = lo; i < hi; ++i) {
+            for (int i = tid; i < n0; i += NT) {
                 const uint32_t r = R[i];
                 if (r != kNone) { cmin = umin(cmin, r); cgate = umin(cgate, MC[i]); }
             }
@@ -298,10 +314,13 @@ __device__ __forceinline__ void bpe_row(
     if (raw_out) {
         // chunk of a long row: hand back the symbol at every start position (kNone elsewhere);
         // the seam and gather kernels assemble the row
-        for (int i = lo; i < hi; ++i) raw_out[i] = stuck ? (uint16_t)kNone : S[i];
+        for (int i = tid; i < n0; i += NT) raw_out[i] = stuck ? (uint16_t)kNone : S[i];
         return;
     }
-    // compact the live symbols to the output
+    // compact the live symbols to the output: contiguous chunks per thread, once per row
+    const int c = (n0 + NT - 1) / NT;
+    const int lo = (tid * c < n0) ? tid * c : n0;
+    const int hi = (lo + c < n0) ? lo + c : n0;
     uint32_t live = 0;
     for (int i = lo; i < hi; ++i) live += (S[i] != kNone);
     uint32_t total;
@@ -315,7 +334,7 @@ __device__ __forceinline__ void bpe_row(
 
 // ---- long rows in chunks -------------------------------------------------------------------
 //
-// A row longer than the LDS capacity is cut into chunks of kChunkCore bytes, each extended by
+// A row longer than one extended chunk is cut into chunks of kChunkCore bytes, each extended by
 // kChunkOverlap bytes on both sides, and every extended chunk is merged on its own.  Two
 // neighbouring chunks A and B are then joined at a seam: a position p inside their overlap
 // where both runs end with a token boundary, the token ending at p is the same token in both,
@@ -326,9 +345,11 @@ __device__ __forceinline__ void bpe_row(
 // rule's product is only used by higher-ranked rules, so that merges happen in key order).
 // If an overlap holds no such p (e.g. a tandem repeat longer than the overlap), the row is
 // redone by the whole-row kernel.
-constexpr int kLdsCap = 4096;            // longest row / extended chunk the LDS kernel takes
-constexpr int kChunkOverlap = 512;
-constexpr int kChunkCore = kLdsCap - 2 * kChunkOverlap;
+constexpr int kLdsCap = 4096;            // longest piece any LDS kernel variant takes
+// 2048-byte extended chunks: 26 KB of LDS state, six workgroups per CU; measured faster than
+// 4096-byte chunks (fewer positions per thread, more chunks in flight)
+constexpr int kChunkOverlap = 256;
+constexpr int kChunkCore = 2048 - 2 * kChunkOverlap;
 constexpr int kLongThreads = 1024;
 constexpr int kLongGrid = 64;            // slabs of scratch for the whole-row fallback kernel
 
@@ -340,10 +361,11 @@ struct BpePlan {                          // device arrays inside the scratch bu
     int32_t *mc_row;      // [max_mc]
     int32_t *seam;        // [max_mc] seam to the right of a chunk (row position), -1 = none found
     int32_t *row_fail;    // [n_rows] 1 = redo the row with the whole-row kernel
-    uint16_t *chunk_sym;  // [max_mc][kLdsCap]
+    uint16_t *chunk_sym;  // [max_mc][ext]
     uint8_t *slabs;       // whole-row fallback state
     size_t slab_bytes, total_bytes;
     int64_t max_items, max_mc;
+    int core, overlap, ext;   // chunk core, overlap on each side, core + 2 * overlap
 };
 
 static size_t long_slab_bytes(int64_t max_len)
@@ -352,13 +374,29 @@ static size_t long_slab_bytes(int64_t max_len)
     return ((n * 17) + 255) & ~(size_t)255;
 }
 
+// chunk geometry: DNATOK_BPE_CHUNK="core,overlap" overrides the default (for experiments)
+static void chunk_geometry(int *core, int *overlap)
+{
+    static int c = 0, v = 0;
+    if (c == 0) {
+        c = kChunkCore; v = kChunkOverlap;
+        const char *env = getenv("DNATOK_BPE_CHUNK");
+        int ec = 0, ev = 0;
+        if (env && sscanf(env, "%d,%d", &ec, &ev) == 2 && ec >= 256 && ev >= 32 && ec > 2 * ev &&
+            ec + 2 * ev <= kLdsCap) { c = ec; v = ev; }
+    }
+    *core = c; *overlap = v;
+}
+
 static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t total)
 {
     BpePlan p{};
+    chunk_geometry(&p.core, &p.overlap);
+    p.ext = p.core + 2 * p.overlap;
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
-    const bool chunks = max_len > kLdsCap;
-    p.max_items = n_rows + (chunks ? total / kChunkCore + 1 : 0);
-    p.max_mc = chunks ? 2 * (total / kChunkCore) + 2 : 0;
+    const bool chunks = max_len > p.ext;
+    p.max_items = n_rows + (chunks ? total / p.core + 1 : 0);
+    p.max_mc = chunks ? 2 * (total / p.core) + 2 : 0;
     size_t o = 0;
     auto take = [&](size_t bytes) { size_t at = o; o = up(o + bytes); return at; };
     const size_t o_counts = take(64);
@@ -368,7 +406,7 @@ static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t
     const size_t o_mc_row = take(4 * (size_t)p.max_mc);
     const size_t o_seam = take(4 * (size_t)p.max_mc);
     const size_t o_fail = take(4 * (size_t)n_rows);
-    const size_t o_sym = take(2 * (size_t)kLdsCap * (size_t)p.max_mc);
+    const size_t o_sym = take(2 * (size_t)p.ext * (size_t)p.max_mc);
     p.slab_bytes = chunks ? long_slab_bytes(max_len) : 0;
     const int64_t slabs = n_rows < kLongGrid ? n_rows : kLongGrid;
     const size_t o_slabs = take(chunks ? p.slab_bytes * (size_t)slabs : 0);
@@ -402,8 +440,8 @@ __global__ __launch_bounds__(1024) void bpe_plan_kernel(
         if (row < n_rows) {
             const int64_t len = offsets[row + 1] - offsets[row];
             nc = 1;
-            if (len > kLdsCap && chunking) { nc = (uint32_t)((len + kChunkCore - 1) / kChunkCore); mc = nc; }
-            p.row_fail[row] = (len > kLdsCap && !chunking) ? 1 : 0;
+            if (len > p.ext && chunking) { nc = (uint32_t)((len + p.core - 1) / p.core); mc = nc; }
+            p.row_fail[row] = (len > p.ext && !chunking) ? 1 : 0;
         }
         const uint32_t inc0 = wave_inclusive_sum_u32(nc), inc1 = wave_inclusive_sum_u32(mc);
         if (lane == 63) { wt[0][wv] = inc0; wt[1][wv] = inc1; }
@@ -485,10 +523,10 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
             bpe_row<NT, uint16_t>(tab, mask, a.shift, b2s, a.out_remap, bytes + start, (int)len, S, R, NS, MC,
                                   NX, PV, F, D, red, tid, tok_tmp + start, lengths + row);
         } else {
-            const int64_t e0 = (int64_t)k * kChunkCore - kChunkOverlap < 0 ? 0 : (int64_t)k * kChunkCore - kChunkOverlap;
-            int64_t e1 = (int64_t)(k + 1) * kChunkCore + kChunkOverlap;
+            const int64_t e0 = (int64_t)k * p.core - p.overlap < 0 ? 0 : (int64_t)k * p.core - p.overlap;
+            int64_t e1 = (int64_t)(k + 1) * p.core + p.overlap;
             if (e1 > len) e1 = len;
-            uint16_t *raw = p.chunk_sym + (size_t)(p.mc_off[row] + k) * kLdsCap;
+            uint16_t *raw = p.chunk_sym + (size_t)(p.mc_off[row] + k) * p.ext;
             bpe_row<NT, uint16_t>(tab, mask, a.shift, b2s, a.out_remap, bytes + start + e0, (int)(e1 - e0),
                                   S, R, NS, MC, NX, PV, F, D, red, tid, nullptr, nullptr, raw);
         }
@@ -507,12 +545,12 @@ __global__ __launch_bounds__(256) void bpe_seam_kernel(const int64_t *__restrict
         const int32_t nc = p.mc_off[row + 1] - p.mc_off[row];
         if (k + 1 >= nc) continue;                                   // last chunk: no seam to the right
         const int64_t len = offsets[row + 1] - offsets[row];
-        const int64_t ea0 = (int64_t)k * kChunkCore - kChunkOverlap < 0 ? 0 : (int64_t)k * kChunkCore - kChunkOverlap;
-        int64_t ea1 = (int64_t)(k + 1) * kChunkCore + kChunkOverlap;
+        const int64_t ea0 = (int64_t)k * p.core - p.overlap < 0 ? 0 : (int64_t)k * p.core - p.overlap;
+        int64_t ea1 = (int64_t)(k + 1) * p.core + p.overlap;
         if (ea1 > len) ea1 = len;
-        const int64_t eb0 = (int64_t)(k + 1) * kChunkCore - kChunkOverlap;
-        const uint16_t *A = p.chunk_sym + (size_t)m * kLdsCap;       // A[i - ea0]
-        const uint16_t *B = p.chunk_sym + (size_t)(m + 1) * kLdsCap; // B[i - eb0]
+        const int64_t eb0 = (int64_t)(k + 1) * p.core - p.overlap;
+        const uint16_t *A = p.chunk_sym + (size_t)m * p.ext;         // A[i - ea0]
+        const uint16_t *B = p.chunk_sym + (size_t)(m + 1) * p.ext;   // B[i - eb0]
         uint32_t mine = 0xFFFFFFFFu;
         for (int64_t i = eb0 + threadIdx.x; i < ea1; i += 256) {
             const uint32_t sa = A[i - ea0];
@@ -552,12 +590,12 @@ __global__ __launch_bounds__(1024) void bpe_gather_kernel(
             const int64_t i = base + threadIdx.x;
             uint32_t sym = kNone;
             if (i < len) {
-                int32_t k = (int32_t)(i / kChunkCore);
+                int32_t k = (int32_t)(i / p.core);
                 if (k >= nc) k = nc - 1;
                 if (k > 0 && i < p.seam[m0 + k - 1]) --k;            // still left of the seam before chunk k
                 else if (k + 1 < nc && i >= p.seam[m0 + k]) ++k;     // already right of the seam after chunk k
-                const int64_t e0 = (int64_t)k * kChunkCore - kChunkOverlap < 0 ? 0 : (int64_t)k * kChunkCore - kChunkOverlap;
-                sym = p.chunk_sym[(size_t)(m0 + k) * kLdsCap + (i - e0)];
+                const int64_t e0 = (int64_t)k * p.core - p.overlap < 0 ? 0 : (int64_t)k * p.core - p.overlap;
+                sym = p.chunk_sym[(size_t)(m0 + k) * p.ext + (i - e0)];
             }
             const uint32_t live = sym != kNone;
             uint32_t total;
@@ -732,7 +770,7 @@ extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, co
     DNATOK_REQUIRE(t && offsets && lengths, DNATOK_E_INVALID, "dnatok_bpe_encode: null argument");
     DNATOK_REQUIRE(n_rows >= 0 && max_len >= 0 && total >= 0, DNATOK_E_INVALID,
                    "dnatok_bpe_encode: negative size");
-    DNATOK_REQUIRE(max_len < (int64_t)1 << 31 && total / kChunkCore + n_rows < (int64_t)1 << 30, DNATOK_E_TOO_LARGE,
+    DNATOK_REQUIRE(max_len < (int64_t)1 << 31 && total / 256 + n_rows < (int64_t)1 << 30, DNATOK_E_TOO_LARGE,
                    "dnatok_bpe_encode: batch too large for 32-bit work indices");
     if (n_rows == 0) return DNATOK_OK;
     DNATOK_REQUIRE(total == 0 || (bytes && tok_tmp), DNATOK_E_INVALID, "dnatok_bpe_encode: null buffer");
@@ -747,7 +785,7 @@ extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, co
     static const char *variant_env = getenv("DNATOK_BPE_VARIANT");
     static const char *chunk_env = getenv("DNATOK_BPE_NO_CHUNKS");
     const int variant = variant_env ? atoi(variant_env) : 0;
-    const bool long_rows = max_len > kLdsCap;
+    const bool long_rows = max_len > p.ext;
     const int chunking = (long_rows && t->monotone && !chunk_env) ? 1 : 0;
     bpe_plan_kernel<<<1, 1024, 0, s>>>(offsets, n_rows, chunking, p);
     DNATOK_HIP_TRY(hipGetLastError());
@@ -755,9 +793,13 @@ extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, co
     // the LDS capacity variant follows the longest row (or the chunk size for longer rows):
     // less LDS per workgroup means more workgroups per CU
     int rc;
-    if (variant == 3)            rc = launch_lds<64, 4, kLdsCap>(a, bytes, offsets, p, tok_tmp, lengths, s);
-    else if (max_len <= 1024)    rc = launch_lds<256, 1, 1024>(a, bytes, offsets, p, tok_tmp, lengths, s);
-    else if (max_len <= 2048)    rc = launch_lds<256, 1, 2048>(a, bytes, offsets, p, tok_tmp, lengths, s);
+    const int64_t work_len = max_len < p.ext ? max_len : p.ext;    // longest piece the LDS kernel sees
+    if (variant == 3 && max_len <= 1024)      rc = launch_lds<64, 4, 1024>(a, bytes, offsets, p, tok_tmp, lengths, s);
+    else if (variant == 4 && max_len <= 1024) rc = launch_lds<64, 8, 1024>(a, bytes, offsets, p, tok_tmp, lengths, s);
+    else if (variant == 5)                    rc = launch_lds<1024, 1, kLdsCap>(a, bytes, offsets, p, tok_tmp, lengths, s);
+    else if (work_len <= 1024)   rc = launch_lds<256, 1, 1024>(a, bytes, offsets, p, tok_tmp, lengths, s);
+    else if (work_len <= 2048)   rc = launch_lds<256, 1, 2048>(a, bytes, offsets, p, tok_tmp, lengths, s);
+    else if (variant == 6)       rc = launch_lds<512, 1, kLdsCap>(a, bytes, offsets, p, tok_tmp, lengths, s);
     else                         rc = launch_lds<256, 1, kLdsCap>(a, bytes, offsets, p, tok_tmp, lengths, s);
     if (rc) return rc;
     if (long_rows) {

@@ -284,6 +284,18 @@ def test_bpe_long_rows(bpe):
         np.testing.assert_array_equal(r, e)
 
 
+def test_bpe_rows_without_a_seam_fall_back_to_the_whole_row_kernel(bpe):
+    """Tandem repeats far longer than the chunk overlap: neighbouring chunk runs can stay out
+    of phase, no seam is accepted, and the row is redone by the whole-row kernel."""
+    which, enc, bo = bpe
+    say(f"bpe{which} seam fallback")
+    seqs = ["A" * 30000, "ACGTC" * 5000, "AC" * 4000 + "ACGTTGCA" * 2500,
+            wl.config4_bpe32000(1, 9000, seed=3).strings()[0]]
+    b = util.batch_from_strings(seqs)
+    for s, r, e in zip(seqs, bpe_rows(enc, b), bo.encode_batch(b.data, b.offsets)):
+        np.testing.assert_array_equal(r, e, err_msg=s[:20])
+
+
 def test_bpe_c4_golden():
     say("bpe32000 C4 32x100k")
     cfg = util.tokenizer_json("32000")
