@@ -394,6 +394,9 @@ def main() -> None:
     ap.add_argument("--per-call", action="store_true", help="time one exact batch instead of the sustained form")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy, the known-size kernel that the "
+                         "FETCH_SIZE / WRITE_SIZE counters are scaled by when profiling")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this backend and this benchmark are single-GPU (rows are independent; "
@@ -426,6 +429,22 @@ def main() -> None:
                      "device_ms_per_step": dev_ms},
         "bit_exact_vs_golden": True,
     }
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
+    traffic_file = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(traffic_file):
+        with open(traffic_file) as fh:
+            known = json.load(fh).get(f"{args.config}:{'per_call' if args.per_call else 'sustained'}")
+        if known and known.get("bases_per_step") == int(w.bases):
+            result["roofline"]["traffic"] = known["hbm_bytes_per_launch"]
+            result["roofline"]["traffic_source"] = known["source"]
 
     if not args.no_cpu:
         cores = os.cpu_count() or 1
