@@ -470,6 +470,14 @@ def main() -> None:
             del ww
             torch.cuda.empty_cache()
         result["per_call"] = per_call
+        if not args.no_cpu:
+            # the BPE configurations next to the HF CPU tokenizer of the same run (bounded samples)
+            hf_rows = {}
+            for cfg, cap in (("C3", 0), ("C4", 400_000), ("C5", 1_500_000)):
+                if cfg == args.config:
+                    continue
+                hf_rows[cfg] = {"threads_1": hf_cpu(cfg, 1, cap), f"threads_{cores}": hf_cpu(cfg, cores, cap)}
+            result["hf_tokenizers_cpu_other_configs"] = hf_rows
         sustained = {}
         for cfg in ["C1", "C3"]:
             if cfg == args.config and not args.per_call:

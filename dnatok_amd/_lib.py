@@ -37,6 +37,10 @@ def lib() -> ctypes.CDLL:
         raise DnatokError(
             f"{LIB_PATH} is missing: build it with `python -m dnatok_amd.build` "
             "(hipcc --offload-arch=gfx950). There is no fallback path.")
+    # torch ships its own HIP runtime (soname libamdhip64.so.7); loading it first lets the
+    # library's dependency resolve to that same copy instead of a second runtime from /opt/rocm,
+    # which would not see the device torch's copy already holds.
+    import torch  # noqa: F401
     L = ctypes.CDLL(LIB_PATH)
     L.dnatok_version.restype = c_int
     L.dnatok_last_error.restype = c_char_p
