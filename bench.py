@@ -118,9 +118,12 @@ class CharDense(Workload):
 
 
 class KmerPadded(Workload):
-    """C2: 256 x 6000 bp 6-mer tokenizer; padded int32 ids + uint8 mask + lengths."""
+    """C2: 256 x 6000 bp 6-mer tokenizer; padded int32 ids + uint8 mask + lengths.
 
-    def __init__(self, n_batches: int, t_cap: int = 6000):
+    The output buffers hold 6016 cells per row: room for the worst case (every base of a
+    6000 bp row spelled on its own), rounded up to whole 128-byte lines for ids and mask."""
+
+    def __init__(self, n_batches: int, t_cap: int = 6016):
         from dnatok_amd import encoders, hf_tokenizers as hf, kmer_tables, workloads as wl
         import torch
         vocab = hf.kmer_vocab(6)

@@ -1,20 +1,24 @@
 // Non-overlapping k-mer encoder with per-window fallback, tail handling, padding and mask.
 //
-// Persistent workgroups stage the tables in LDS once; after that every wave works alone:
-// it takes a row and walks it in steps of 256 units (a unit is a k-base window, or one of
-// the trailing len % k characters).  Each lane owns 4 consecutive units: it loads its 4k
-// bytes, turns them into base-5 digits through the LDS digit table, and looks the window up
-// in the LDS table of the 4^k N-free windows.
+// Persistent workgroups stage the tables in LDS once; after that every wave works alone on
+// rows dealt round-robin.  A wave walks its row in steps of 256 units (a unit is a k-base window, or one of the trailing
+// len % k characters).  Each lane owns 4 consecutive units: it loads its 4k bytes, turns them
+// into base-4 digits through the LDS digit table, and looks the window up in the LDS table of
+// the 4^k N-free windows.
 //
-//   * Step without exceptions (the common case): every lane holds 4 plain windows, so token
-//     positions are known without a scan and each lane issues one 16-byte id store and one
-//     4-byte mask store (a wave covers 1 KiB + 256 B contiguous).
-//   * Step with exceptions (a window holding N or a byte outside the alphabet, a window
-//     without an id, the ragged end of a row): unit token counts are prefix-summed across
-//     the wave with a DPP scan (no barrier) and every lane writes at its own offset.  When
-//     the table spells every non-plain window character by character (the usual grid-aligned
-//     tokenizer), the spelled tokens come from 5 LDS entries; otherwise from the global
-//     5^k entry table and its expansion lists.
+//   * Plain step (every lane holds 4 plain windows, and the row's write position is 16-byte
+//     aligned): token positions are known without a scan; each lane issues one 16-byte id
+//     store and one 4-byte mask store (a wave covers 1 KiB + 256 B contiguous).
+//   * Any other step (a window holding N or a byte outside the alphabet, a window without an
+//     id, the ragged end of a row, or a write position that an earlier expansion left off the
+//     16-byte grid): unit token counts are prefix-summed across the wave with a DPP scan, the
+//     lanes drop their tokens into a per-wave LDS staging area at their scanned positions,
+//     and the wave writes the staged run back out as aligned 16-byte groups.  The up-to-3
+//     tokens that do not fill a group stay in LDS for the next step of the row.  A step that
+//     yields more tokens than the staging area holds is staged in several passes.
+//     When the table spells every non-plain window character by character (the usual
+//     grid-aligned tokenizer), the spelled tokens come from an LDS table; otherwise from the
+//     global 5^k entry table and its expansion lists.
 //
 // Traffic: 1 byte read per base, 5 bytes written per token.
 #include "common.hpp"
@@ -49,67 +53,68 @@ struct KmerArgs {
 constexpr int kKmerThreads = 256;
 constexpr int kUnitsPerLane = 4;
 constexpr int kWaveUnits = 64 * kUnitsPerLane;          // units one wave handles per step
+// Staging area of one wave: kStageCap tokens in scanned order (+ room to read the last group whole).
+constexpr int kStageCap = 512;
+constexpr int kStageWords = kStageCap + 8;
 
 // LDS digit entries: 0..3 for A C G T; flags above every window code (4^8 = 1 << 16) for N and
 // for a byte outside the alphabet, so that "window code < 4^k" means "k plain bases".
 constexpr uint32_t kDigN = 1u << 16;
 constexpr uint32_t kDigBad = 1u << 17;
+// byte offset past the end of every row descriptor (its stores are dropped), and the cache
+// policy bits of the buffer stores (streaming: the output is not read again by the kernel)
+constexpr uint32_t kDropOffset = 0x80000000u;
+constexpr int kStoreAux = 2;
 
-typedef int32_t int4v __attribute__((ext_vector_type(4)));
-// the same vectors at element alignment: a row's token position is not a multiple of 4 once a
-// window has expanded, and global stores only need the element alignment
+// 4 ids at element alignment (the compiler may not assume more; the addresses the kernels
+// form are 16-byte aligned wherever the row layout allows)
 typedef int32_t int4v_a4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef int32_t int4v __attribute__((ext_vector_type(4)));
 typedef uint32_t u32_a1 __attribute__((aligned(1)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-__global__ void zero_i32_kernel(int32_t *p) { *p = 0; }
+__global__ void kmer_init_kernel(int32_t *max_len) { *max_len = 0; }
 
-__device__ __forceinline__ void store4(int32_t *out, uint8_t *mout, int p, const int32_t *t)
+// Stores the group of 4 cells [e, e + 4) of a row whose cells are addressed from the
+// 16-byte-aligned pointer pair (outA, moutA); only cells inside [lo, hi) are written.
+__device__ __forceinline__ void store_group(int32_t *outA, uint8_t *moutA, int e, int lo, int hi,
+                                            const int32_t *v, uint32_t mbyte)
 {
-    int4v_a4 v = {t[0], t[1], t[2], t[3]};
-    __builtin_nontemporal_store(v, reinterpret_cast<int4v_a4 *>(out + p));
-    if (mout) __builtin_nontemporal_store((u32_a1)0x01010101u, reinterpret_cast<u32_a1 *>(mout + p));
-}
-
-__device__ __forceinline__ void store1(int32_t *out, uint8_t *mout, int p, int t_cap, int32_t v)
-{
-    if (p < t_cap) {
-        out[p] = v;
-        if (mout) mout[p] = 1;
-    }
-}
-
-typedef int32_t int2v_a4 __attribute__((ext_vector_type(2), aligned(4)));
-typedef uint16_t u16_a1 __attribute__((aligned(1)));
-
-// N consecutive tokens (a spelled window) with as few stores as possible.
-template <int N>
-__device__ __forceinline__ void storeN(int32_t *out, uint8_t *mout, int p, int t_cap, const int32_t *t)
-{
-    if (p + N <= t_cap) {
-        int i = 0;
-#pragma unroll
-        for (; i + 4 <= N; i += 4) {
-            int4v_a4 v = {t[i], t[i + 1], t[i + 2], t[i + 3]};
-            *reinterpret_cast<int4v_a4 *>(out + p + i) = v;
-            if (mout) *reinterpret_cast<u32_a1 *>(mout + p + i) = 0x01010101u;
-        }
-        if (i + 2 <= N) {
-            int2v_a4 v = {t[i], t[i + 1]};
-            *reinterpret_cast<int2v_a4 *>(out + p + i) = v;
-            if (mout) *reinterpret_cast<u16_a1 *>(mout + p + i) = (uint16_t)0x0101u;
-            i += 2;
-        }
-        if (i < N) {
-            out[p + i] = t[i];
-            if (mout) mout[p + i] = 1;
-        }
+    if (e >= lo && e + 4 <= hi) {
+        int4v_a4 x = {v[0], v[1], v[2], v[3]};
+        __builtin_nontemporal_store(x, reinterpret_cast<int4v_a4 *>(outA + e));
+        if (moutA) __builtin_nontemporal_store((u32_a1)(mbyte * 0x01010101u), reinterpret_cast<u32_a1 *>(moutA + e));
     } else {
 #pragma unroll
-        for (int i = 0; i < N; ++i) store1(out, mout, p + i, t_cap, t[i]);
+        for (int i = 0; i < 4; ++i) {
+            if (e + i >= lo && e + i < hi) {
+                outA[e + i] = v[i];
+                if (moutA) moutA[e + i] = (uint8_t)mbyte;
+            }
+        }
     }
 }
 
-template <int K, bool LUT4_LDS, bool CHARS>
+// Cells [from, to) of a row get the pad id and mask 0; the whole wave takes part.
+__device__ __forceinline__ void pad_cells(int32_t *outA, uint8_t *moutA, int mis, int from, int to,
+                                          int32_t pad_id, int lane)
+{
+    const int lo = mis + from, hi = mis + to;
+    const int32_t v[4] = {pad_id, pad_id, pad_id, pad_id};
+    for (int e = (lo & ~3) + 4 * lane; e < hi; e += 4 * 64) store_group(outA, moutA, e, lo, hi, v, 0u);
+}
+
+// Orders the LDS traffic of the lanes of one wave (they run in lockstep; this only keeps the
+// compiler from moving LDS accesses across the point).
+__device__ __forceinline__ void wave_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <int K, bool LUT4_LDS, bool CHARS, bool HAS_MASK>
 __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
     KmerArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
     int64_t n_rows, int64_t t_cap, int64_t fill_to, int32_t *__restrict__ ids,
@@ -121,6 +126,7 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
     __shared__ int32_t s_single[256];
     __shared__ int32_t s_lut4[LUT4_LDS ? POW4 : 1];
     __shared__ int32_t s_spell[256];     // token a byte is spelled with inside a non-plain window
+    __shared__ __attribute__((aligned(16))) int32_t s_stage[kKmerThreads / 64][kStageWords];
 
     for (int i = threadIdx.x; i < 256; i += kKmerThreads) {
         const int d = a.digit[i];
@@ -134,9 +140,13 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
     __syncthreads();          // the only workgroup barrier: from here on every wave runs alone
 
     const int lane = threadIdx.x & 63;
-    const int64_t wave = (int64_t)blockIdx.x * (kKmerThreads / 64) + (threadIdx.x >> 6);
-    const int64_t n_waves = (int64_t)gridDim.x * (kKmerThreads / 64);
+    int32_t *const buf = s_stage[__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6))];
+    const int cap = t_cap > INT_MAX - 16 ? INT_MAX - 16 : (int)t_cap;
+    const int fill = fill_to > cap ? cap : (int)fill_to;
     int64_t wave_max = 0;
+    const int wave_in_wg = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int64_t wave = (int64_t)blockIdx.x * (kKmerThreads / 64) + wave_in_wg;
+    const int64_t n_waves = (int64_t)gridDim.x * (kKmerThreads / 64);
 
     for (int64_t row = wave; row < n_rows; row += n_waves) {
         const int64_t row_start = offsets[row];
@@ -146,29 +156,77 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
         const int n_units = full + (len - full * K);
         const uint8_t *src = bytes + row_start;
         int32_t *out = ids + row * t_cap;
-        uint8_t *mout = mask ? mask + row * t_cap : nullptr;
-        const int cap = t_cap > INT_MAX ? INT_MAX : (int)t_cap;
+        // cells are addressed from the 16-byte boundary at or below the row's first cell
+        const int mis = (int)((reinterpret_cast<uintptr_t>(out) >> 2) & 3);
+        int32_t *outA = out - mis;
+        uint8_t *moutA = HAS_MASK ? mask + row * t_cap - mis : nullptr;
+        const int lo = mis, hi_cap = mis + cap;
         int running = 0;
         int32_t my_status = 0;
 
-        // software pipeline: the bytes of the next step are requested before this step is decoded
-        uint32_t wn[K];
+        // The row's bytes are read through a buffer descriptor: a read past the row's end
+        // returns 0 (never a base) instead of faulting, so the bytes of the next step are
+        // requested without a branch, one step ahead of their use.
+        const __amdgpu_buffer_rsrc_t rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(src), (short)0, len, 0x00020000);
+        auto fetch = [&](uint32_t (&dst)[K], int unit0) {
+            const int off = (unit0 + lane * kUnitsPerLane) * K;       // 4 windows = 4K bytes, unaligned
+            int i = 0;
 #pragma unroll
-        for (int i = 0; i < K; ++i) wn[i] = 0;             // byte 0 is never a base
-        if (lane * kUnitsPerLane + kUnitsPerLane <= full) memcpy(wn, src + lane * kUnitsPerLane * K, 4 * K);
+            for (; i + 4 <= K; i += 4) {
+                const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off + 4 * i, 0, 0);
+                dst[i] = v.x; dst[i + 1] = v.y; dst[i + 2] = v.z; dst[i + 3] = v.w;
+            }
+            if (i + 2 <= K) {
+                const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, off + 4 * i, 0, 0);
+                dst[i] = v.x; dst[i + 1] = v.y;
+                i += 2;
+            }
+            if (i < K) dst[i] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, off + 4 * i, 0, 0);
+        };
+        // Stores of whole 4-cell groups go through buffer descriptors of the row as well: a lane
+        // that has nothing to store points past the descriptor's end and the hardware drops its
+        // store.  Every kind of step therefore issues the same stores (ids, mask) with no branch
+        // around them, and the wait for the bytes requested one step earlier (the counter is in
+        // issue order) can leave them in flight.
+        const int vec_cap = cap < 0x1FFFFFF0 ? cap : 0x1FFFFFF0;      // cells a descriptor reaches
+        const __amdgpu_buffer_rsrc_t rs_ids =
+            __builtin_amdgcn_make_buffer_rsrc(out, (short)0, vec_cap * 4, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rs_msk = __builtin_amdgcn_make_buffer_rsrc(
+            HAS_MASK ? mask + row * t_cap : reinterpret_cast<uint8_t *>(out), (short)0, HAS_MASK ? vec_cap : 0,
+            0x00020000);
+        // group of 4 cells starting at row cell r (whole = inside the row and the descriptor)
+        auto store_vec = [&](bool whole, int r, const int32_t *v) {
+            const int voff = whole ? r * 4 : (int)kDropOffset;
+            const u32x4 x = {(uint32_t)v[0], (uint32_t)v[1], (uint32_t)v[2], (uint32_t)v[3]};
+            __builtin_amdgcn_raw_buffer_store_b128(x, rs_ids, voff, 0, kStoreAux);
+            if (HAS_MASK)
+                __builtin_amdgcn_raw_buffer_store_b32(0x01010101u, rs_msk, whole ? r : (int)kDropOffset, 0, kStoreAux);
+        };
 
+        uint32_t w[K], wn[K];
+        uint32_t code[kUnitsPerLane];
+        int32_t t[kUnitsPerLane] = {0, 0, 0, 0};
+        // digit of byte bi of this lane (LDS lookup)
+        auto digit_of = [&](int bi) -> uint32_t { return s_dig[(w[bi >> 2] >> (8 * (bi & 3))) & 255u]; };
+
+        // Waits for the bytes requested last.  Every way through a step that issues more memory
+        // operations than the stores of store_vec starts with this: the compiler then knows the
+        // request has landed on those ways, and on the remaining ones it can count the stores
+        // between the request and its use exactly, and leave them in flight at the wait.
+        auto settle = [&]() {
+#pragma unroll
+            for (int i = 0; i < K; ++i) asm volatile("" ::"v"(wn[i]));
+        };
+        fetch(wn, 0);
+        settle();
         for (int u0 = 0; u0 < n_units; u0 += kWaveUnits) {
             const int ub = u0 + lane * kUnitsPerLane;
             const bool lane_full = ub + kUnitsPerLane <= full;     // 4 whole windows
             const bool empty = ub >= n_units;
-            uint32_t w[K];
 #pragma unroll
-            for (int i = 0; i < K; ++i) { w[i] = wn[i]; wn[i] = 0; }
-            if (ub + kWaveUnits + kUnitsPerLane <= full)            // 4 windows = 4K bytes, unaligned
-                memcpy(wn, src + (ub + kWaveUnits) * K, 4 * K);
-            // digit of byte bi of this lane (LDS lookup)
-            auto digit_of = [&](int bi) -> uint32_t { return s_dig[(w[bi >> 2] >> (8 * (bi & 3))) & 255u]; };
-            uint32_t code[kUnitsPerLane];
+            for (int i = 0; i < K; ++i) w[i] = wn[i];
+            fetch(wn, u0 + kWaveUnits);
 #pragma unroll
             for (int j = 0; j < kUnitsPerLane; ++j) {
                 uint32_t c = 0;
@@ -176,7 +234,6 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
                 for (int i = 0; i < K; ++i) c = (c << 2) + digit_of(j * K + i);
                 code[j] = c;
             }
-            int32_t t[kUnitsPerLane];
 #pragma unroll
             for (int j = 0; j < kUnitsPerLane; ++j) {
                 const uint32_t idx = code[j] & (POW4 - 1);
@@ -186,27 +243,34 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
             const bool fast = lane_full && any_flag < POW4 && (t[0] | t[1] | t[2] | t[3]) >= 0;
             const uint64_t fast_mask = __ballot(fast);
             const uint64_t rest_mask = __ballot(!fast && !empty);
+            const int A = mis + running;           // cell the step's first token goes to
 
-            if (rest_mask == 0) {
-                // every lane is plain or past the end: positions are known without a scan
-                const int p = running + lane * kUnitsPerLane;
-                if (fast) {
-                    if (p + 4 <= cap) {
-                        store4(out, mout, p, t);
-                    } else {
+            // what the step's common store (one 4-cell group per lane) will write
+            bool sv_whole = false;
+            int sv_r = 0;
+            int32_t sv_v[4] = {0, 0, 0, 0};
+
+            if (rest_mask == 0 && (A & 3) == 0) {
+                // every lane is plain or past the end, and the run starts on a 16-byte boundary:
+                // positions are known without a scan
+                const int r = running + lane * kUnitsPerLane;
+                sv_whole = fast && r + 4 <= vec_cap;
+                sv_r = r;
 #pragma unroll
-                        for (int j = 0; j < kUnitsPerLane; ++j) store1(out, mout, p + j, cap, t[j]);
-                    }
+                for (int j = 0; j < kUnitsPerLane; ++j) sv_v[j] = t[j];
+                if (__ballot(fast && !sv_whole)) {                 // row cut at t_cap
+                    settle();
+                    if (fast && !sv_whole) store_group(outA, moutA, mis + r, lo, hi_cap, t, 1u);
                 }
                 running += kUnitsPerLane * (int)__popcll(fast_mask);
-                continue;
-            }
-
-            // ---- step with exceptions ----
+            } else {
+            // ---- staged step ----
             // per unit: cnt = number of tokens; ex/ey = entry of a window that is not plain
             int32_t cnt[kUnitsPerLane], ex[kUnitsPerLane], ey[kUnitsPerLane];
             uint32_t lane_cnt = 0;
-            if (lane_full) {
+            if (fast) {
+                lane_cnt = kUnitsPerLane;
+            } else if (lane_full) {
 #pragma unroll
                 for (int j = 0; j < kUnitsPerLane; ++j) {
                     ex[j] = 0; ey[j] = 0;
@@ -269,79 +333,148 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
 
             const uint32_t inc = wave_inclusive_sum_u32(lane_cnt);
             const uint32_t step_total = __builtin_amdgcn_readlane(inc, 63);
-            int p = running + (int)(inc - lane_cnt);
+            // staged index 0 is cell A & ~3; the first `carry` entries are the tokens the previous
+            // step left over (at the start of a row: cells of the neighbouring row, never written)
+            const uint32_t carry = (uint32_t)(A & 3);
+            const uint32_t n_avail = carry + step_total;
+            const uint32_t s0 = carry + (inc - lane_cnt);
+            const bool last_step = u0 + kWaveUnits >= n_units;
+            const int A_end = A + (int)step_total;
+            const int hi = last_step && A_end < hi_cap ? A_end : hi_cap;
 
-            if (fast) {
-                if (p + 4 <= cap) {
-                    store4(out, mout, p, t);
-                } else {
-#pragma unroll
-                    for (int j = 0; j < kUnitsPerLane; ++j) store1(out, mout, p + j, cap, t[j]);
-                }
-            } else if (lane_full) {
-#pragma unroll
-                for (int j = 0; j < kUnitsPerLane; ++j) {
-                    if (code[j] < POW4 && t[j] >= 0) {
-                        store1(out, mout, p, cap, t[j]);
-                        ++p;
-                    } else if (CHARS) {
-                        int32_t sp[K];
-#pragma unroll
-                        for (int i = 0; i < K; ++i) {
-                            const int bi = j * K + i;
-                            sp[i] = s_spell[(w[bi >> 2] >> (8 * (bi & 3))) & 255u];
-                        }
-                        storeN<K>(out, mout, p, cap, sp);
-                        p += K;
-                    } else if (ex[j] >= 0) {
-                        store1(out, mout, p, cap, ex[j]);
-                        ++p;
-                    } else if (ex[j] == INT_MIN) {
-                        store1(out, mout, p, cap, a.missing_id);
-                        ++p;
-                    } else {
-                        for (int e = 0; e < -ex[j]; ++e) store1(out, mout, p + e, cap, a.flat[ey[j] + e]);
-                        p += -ex[j];
-                    }
-                }
-            } else if (!empty) {
-#pragma unroll 1
-                for (int j = 0; j < kUnitsPerLane; ++j) {
-                    const int u = ub + j;
-                    if (u < full) {
-                        uint32_t c = 0;
-                        int c5 = 0;
-#pragma unroll
-                        for (int i = 0; i < K; ++i) {
-                            const uint32_t v = s_dig[src[u * K + i]];
-                            c = (c << 2) + v;
-                            c5 = c5 * 5 + ((v & (kDigN | kDigBad)) ? 4 : (int)v);
-                        }
-                        int32_t id = -1;
-                        if (c < POW4) id = LUT4_LDS ? s_lut4[c] : a.lut4[c];
-                        if (id >= 0) {
-                            store1(out, mout, p, cap, id);
-                            ++p;
-                        } else {
-                            const int2 e = a.entry[c5];
-                            if (e.x >= 0 || e.x == INT_MIN) {
-                                store1(out, mout, p, cap, e.x >= 0 ? e.x : a.missing_id);
-                                ++p;
-                            } else {
-                                for (int q = 0; q < -e.x; ++q) store1(out, mout, p + q, cap, a.flat[e.y + q]);
-                                p += -e.x;
+            // the lanes' tokens in scanned order; put(s, tok) places token s of the staged run
+            auto produce = [&](auto put) {
+                uint32_t s = s0;
+                if (fast) {
+    #pragma unroll
+                    for (int j = 0; j < kUnitsPerLane; ++j) put(s + j, t[j]);
+                } else if (lane_full) {
+    #pragma unroll
+                    for (int j = 0; j < kUnitsPerLane; ++j) {
+                        if (code[j] < POW4 && t[j] >= 0) {
+                            put(s, t[j]);
+                            ++s;
+                        } else if (CHARS) {
+    #pragma unroll
+                            for (int i = 0; i < K; ++i) {
+                                const int bi = j * K + i;
+                                put(s + i, s_spell[(w[bi >> 2] >> (8 * (bi & 3))) & 255u]);
                             }
+                            s += K;
+                        } else if (ex[j] >= 0) {
+                            put(s, ex[j]);
+                            ++s;
+                        } else if (ex[j] == INT_MIN) {
+                            put(s, a.missing_id);
+                            ++s;
+                        } else {
+                            for (int e = 0; e < -ex[j]; ++e) put(s + e, a.flat[ey[j] + e]);
+                            s += -ex[j];
                         }
-                    } else if (u < n_units) {
-                        store1(out, mout, p, cap, s_single[src[full * K + (u - full)]]);
-                        ++p;
                     }
+                } else if (!empty) {
+    #pragma unroll 1
+                    for (int j = 0; j < kUnitsPerLane; ++j) {
+                        const int u = ub + j;
+                        if (u < full) {
+                            uint32_t c = 0;
+                            int c5 = 0;
+    #pragma unroll
+                            for (int i = 0; i < K; ++i) {
+                                const uint32_t v = s_dig[src[u * K + i]];
+                                c = (c << 2) + v;
+                                c5 = c5 * 5 + ((v & (kDigN | kDigBad)) ? 4 : (int)v);
+                            }
+                            int32_t id = -1;
+                            if (c < POW4) id = LUT4_LDS ? s_lut4[c] : a.lut4[c];
+                            if (id >= 0) {
+                                put(s, id);
+                                ++s;
+                            } else {
+                                const int2 e = a.entry[c5];
+                                if (e.x >= 0 || e.x == INT_MIN) {
+                                    put(s, e.x >= 0 ? e.x : a.missing_id);
+                                    ++s;
+                                } else {
+                                    for (int q = 0; q < -e.x; ++q) put(s + q, a.flat[e.y + q]);
+                                    s += -e.x;
+                                }
+                            }
+                        } else if (u < n_units) {
+                            put(s, s_single[src[full * K + (u - full)]]);
+                            ++s;
+                        }
+                    }
+                }
+            };
+            auto group_at = [&](uint32_t g, int32_t *v) {
+                const int4v x = *reinterpret_cast<const int4v *>(buf + 4 * g);
+                v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+            };
+
+            if (n_avail <= (uint32_t)kStageCap) {
+                produce([&](uint32_t s, int32_t tok) { buf[s] = tok; });
+                wave_sync();
+                // whole groups; the row's last step also writes the group it leaves unfilled
+                const uint32_t n_groups = last_step ? (n_avail + 3) >> 2 : n_avail >> 2;
+                const int e0 = A & ~3;
+                {
+                    // groups 0..63: one per lane, left to the step's common store
+                    const int e = e0 + 4 * lane;
+                    const bool mine = (uint32_t)lane < n_groups;
+                    group_at(lane, sv_v);
+                    sv_whole = mine && e >= lo && e + 4 <= hi && e - mis + 4 <= vec_cap;
+                    sv_r = e - mis;
+                    if (__ballot(mine && !sv_whole)) {             // row's first or last cells
+                        settle();
+                        if (mine && !sv_whole) store_group(outA, moutA, e, lo, hi, sv_v, 1u);
+                    }
+                }
+                if (n_groups > 64) {
+                    settle();
+                    for (uint32_t g = lane + 64; g < n_groups; g += 64) {
+                        int32_t v[4];
+                        group_at(g, v);
+                        store_group(outA, moutA, e0 + 4 * (int)g, lo, hi, v, 1u);
+                    }
+                }
+                const uint32_t left = last_step ? 0u : (n_avail & 3);
+                int32_t keep = 0;
+                if ((uint32_t)lane < left) keep = buf[(n_avail & ~3u) + lane];
+                wave_sync();
+                if ((uint32_t)lane < left) buf[lane] = keep;
+            } else {
+                // more than kStageCap tokens in one step: staged and written out in several passes
+                settle();
+                for (uint32_t pass = 0; pass < n_avail; pass += kStageCap) {
+                    produce([&](uint32_t s, int32_t tok) {
+                        const uint32_t rel = s - pass;
+                        if (rel < (uint32_t)kStageCap) buf[rel] = tok;
+                    });
+                    wave_sync();
+                    const bool final_pass = pass + kStageCap >= n_avail;
+                    const uint32_t count = final_pass ? n_avail - pass : (uint32_t)kStageCap;
+                    const uint32_t n_groups = final_pass && last_step ? (count + 3) >> 2 : count >> 2;
+                    const int e0 = (A & ~3) + (int)pass;
+                    for (uint32_t g = lane; g < n_groups; g += 64) {
+                        int32_t v[4];
+                        group_at(g, v);
+                        store_group(outA, moutA, e0 + 4 * (int)g, lo, hi, v, 1u);
+                    }
+                    const uint32_t left = final_pass && !last_step ? (count & 3) : 0u;
+                    int32_t keep = 0;
+                    if ((uint32_t)lane < left) keep = buf[(count & ~3u) + lane];
+                    wave_sync();
+                    if ((uint32_t)lane < left) buf[lane] = keep;
+                    wave_sync();
                 }
             }
             running += (int)step_total;
+            }
+            store_vec(sv_whole, sv_r, sv_v);
         }
 
-        const int64_t stored = running < cap ? running : cap;
+        const int stored = running < cap ? running : cap;
         int32_t st = 0;
         if (__ballot(my_status & DNATOK_ROW_INVALID_BYTE)) st |= DNATOK_ROW_INVALID_BYTE;
         if (__ballot(my_status & DNATOK_ROW_MISSING_KMER)) st |= DNATOK_ROW_MISSING_KMER;
@@ -351,12 +484,7 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
             if (status) status[row] = st;
         }
         if (stored > wave_max) wave_max = stored;
-        if (fill_to > 0) {
-            for (int64_t p = stored + lane; p < fill_to; p += 64) {
-                out[p] = a.pad_id;
-                if (mout) mout[p] = 0;
-            }
-        }
+        if (fill > stored) pad_cells(outA, moutA, mis, stored, fill, a.pad_id, lane);
     }
     // one atomic per wave at most, skipped when another wave already published a larger value
     if (max_len && lane == 0 && wave_max > 0 &&
@@ -370,18 +498,17 @@ __global__ __launch_bounds__(256) void pad_to_max_kernel(
     int32_t *__restrict__ ids, uint8_t *__restrict__ mask, const int32_t *__restrict__ lengths,
     int64_t n_rows, int64_t t_cap, const int32_t *__restrict__ max_len, int32_t pad_id)
 {
-    const int64_t fill = *max_len;
+    const int fill = *max_len;
     const int lane = threadIdx.x & 63;
     const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     const int64_t n_waves = (int64_t)gridDim.x * (blockDim.x >> 6);
     for (int64_t row = wave; row < n_rows; row += n_waves) {
-        int64_t len = lengths[row];
-        if (len > t_cap) len = t_cap;
+        int len = lengths[row];
         if (len < 0) len = 0;
-        for (int64_t p = len + lane; p < fill; p += 64) {
-            ids[row * t_cap + p] = pad_id;
-            if (mask) mask[row * t_cap + p] = 0;
-        }
+        if (len >= fill) continue;
+        int32_t *out = ids + row * t_cap;
+        const int mis = (int)((reinterpret_cast<uintptr_t>(out) >> 2) & 3);
+        pad_cells(out - mis, mask ? mask + row * t_cap - mis : nullptr, mis, len, fill, pad_id, lane);
     }
 }
 
@@ -392,13 +519,6 @@ int launch_pad_to_max(int32_t *ids, uint8_t *mask, const int32_t *lengths, int64
     if (blocks > 256 * 16) blocks = 256 * 16;
     if (blocks < 1) blocks = 1;
     pad_to_max_kernel<<<(int)blocks, 256, 0, s>>>(ids, mask, lengths, n_rows, t_cap, max_len, pad_id);
-    DNATOK_HIP_TRY(hipGetLastError());
-    return DNATOK_OK;
-}
-
-int launch_zero_i32(int32_t *p, hipStream_t s)
-{
-    zero_i32_kernel<<<1, 1, 0, s>>>(p);
     DNATOK_HIP_TRY(hipGetLastError());
     return DNATOK_OK;
 }
@@ -513,20 +633,23 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
                    "dnatok_kmer_encode_padded: fill_to = 0 needs max_len");
     if (n_rows == 0) return DNATOK_OK;
     hipStream_t s = (hipStream_t)stream;
-    if (max_len) {
-        int rc = launch_zero_i32(max_len, s);
-        if (rc) return rc;
-    }
     KmerArgs a{t->digit, t->single, t->lut4, t->entry, t->flat, t->pad_id, t->missing_id};
-    // persistent waves: the tables are staged into LDS once per workgroup, rows are dealt
-    // round-robin to waves
+    if (max_len) {
+        kmer_init_kernel<<<1, 1, 0, s>>>(max_len);
+        DNATOK_HIP_TRY(hipGetLastError());
+    }
+    // persistent waves: the tables are staged into LDS once per workgroup
     const int64_t want = (n_rows + kKmerThreads / 64 - 1) / (kKmerThreads / 64);
+#define LAUNCH3(KK, L, C, M)                                                                      \
+    do {                                                                                          \
+        static const int resident = resident_workgroups(kmer_rows_kernel<KK, L, C, M>, kKmerThreads, 0, 4); \
+        const int64_t grid = want < resident ? want : resident;                                   \
+        kmer_rows_kernel<KK, L, C, M><<<(int)grid, kKmerThreads, 0, s>>>(                         \
+            a, bytes, offsets, n_rows, t_cap, fill_to, ids, mask, lengths, status, max_len);      \
+    } while (0)
 #define LAUNCH2(KK, L, C)                                                                         \
     do {                                                                                          \
-        static const int resident = resident_workgroups(kmer_rows_kernel<KK, L, C>, kKmerThreads, 0, 4); \
-        const int64_t grid = want < resident ? want : resident;                                   \
-        kmer_rows_kernel<KK, L, C><<<(int)grid, kKmerThreads, 0, s>>>(                            \
-            a, bytes, offsets, n_rows, t_cap, fill_to, ids, mask, lengths, status, max_len);      \
+        if (mask) LAUNCH3(KK, L, C, true); else LAUNCH3(KK, L, C, false);                         \
     } while (0)
 #define LAUNCH(KK, L)                                                                             \
     do {                                                                                          \
@@ -543,6 +666,7 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
     }
 #undef LAUNCH
 #undef LAUNCH2
+#undef LAUNCH3
     DNATOK_HIP_TRY(hipGetLastError());
     if (fill_to == 0) return launch_pad_to_max(ids, mask, lengths, n_rows, t_cap, max_len, t->pad_id, s);
     return DNATOK_OK;

@@ -7,7 +7,15 @@ namespace dnatok {
 
 int launch_pad_to_max(int32_t *ids, uint8_t *mask, const int32_t *lengths, int64_t n_rows,
                       int64_t t_cap, const int32_t *max_len, int32_t pad_id, hipStream_t s);
-int launch_zero_i32(int32_t *p, hipStream_t s);
+
+__global__ void zero_i32_kernel(int32_t *p) { *p = 0; }
+
+static int launch_zero_i32(int32_t *p, hipStream_t s)
+{
+    zero_i32_kernel<<<1, 1, 0, s>>>(p);
+    DNATOK_HIP_TRY(hipGetLastError());
+    return DNATOK_OK;
+}
 
 constexpr int kScanThreads = 1024;
 

@@ -363,14 +363,16 @@ class DNATok:
     def _encode_kmer_device(self, seqs, data, offsets, lens) -> Tuple[torch.Tensor, torch.Tensor]:
         from ._lib import lib  # noqa: F401  (fail early if the library is missing)
         k = int(self.kmer_k)
+        # row stride of the output buffers: a multiple of 128 cells keeps every row of ids and of
+        # the mask on cache-line boundaries, which the store path of the kernel is built around
         t_cap = int(lens.max()) + 4
-        t_cap += (-t_cap) % 4
+        t_cap += (-t_cap) % 128
         ids, mask, lengths, status, longest = self._kmer_enc.encode_padded(data, offsets, t_cap, fill_to=0)
         width = int(longest.item())                      # one scalar: the output shape
         if self.token_len is not None and self.token_len > width:
             extra = int(self.token_len)
             ids, mask, lengths, status, longest = self._kmer_enc.encode_padded(
-                data, offsets, max(t_cap, extra + (-extra) % 4), fill_to=extra)
+                data, offsets, max(t_cap, extra + (-extra) % 128), fill_to=extra)
             width = extra
         ids, mask = ids[:, :width], mask[:, :width]
         bad = status.cpu().numpy()
@@ -466,7 +468,7 @@ class DNATok:
         data = u8_cpu.to(device, non_blocking=True).reshape(-1)
         offsets = torch.arange(b + 1, dtype=torch.int64, device=device) * t
         if self._kmer_enc is not None:
-            t_cap = t + 4 + (-(t + 4)) % 4
+            t_cap = t + 4 + (-(t + 4)) % 128
             ids, mask, lengths, status, longest = self._kmer_enc.encode_padded(data, offsets, t_cap, fill_to=0)
             if int(status.abs().max().item()) & 3:
                 raise RuntimeError("k-mer bytes path: a row needs the tokenizer's own answer")
