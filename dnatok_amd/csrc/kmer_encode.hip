@@ -1,21 +1,24 @@
 // Non-overlapping k-mer encoder with per-window fallback, tail handling, padding and mask.
 //
 // Persistent workgroups stage the tables in LDS once; after that every wave works alone on
-// rows dealt round-robin.  A wave walks its row in steps of 256 units (a unit is a k-base window, or one of the trailing
-// len % k characters).  Each lane owns 4 consecutive units: it loads its 4k bytes, turns them
-// into base-4 digits through the LDS digit table, and looks the window up in the LDS table of
-// the 4^k N-free windows.
+// rows dealt round-robin.  A wave walks its row in steps of 256 units (a unit is a k-base
+// window, or one of the trailing len % k characters).  Each lane owns 4 consecutive units: it
+// takes its 4k bytes (requested one step earlier through a buffer descriptor of the row),
+// turns them into base-4 digits through the LDS digit table, and looks the window up in the
+// LDS table of the 4^k N-free windows.
 //
-//   * Plain step (every lane holds 4 plain windows, and the row's write position is 16-byte
-//     aligned): token positions are known without a scan; each lane issues one 16-byte id
-//     store and one 4-byte mask store (a wave covers 1 KiB + 256 B contiguous).
+//   * Plain step (every lane holds 4 plain windows or lies past the row's end, and the row's
+//     write position is on a 128-byte line): token positions are known without a scan; each
+//     lane issues one 16-byte id store and one 4-byte mask store (a wave covers 1 KiB + 256 B
+//     contiguous).
 //   * Any other step (a window holding N or a byte outside the alphabet, a window without an
-//     id, the ragged end of a row, or a write position that an earlier expansion left off the
-//     16-byte grid): unit token counts are prefix-summed across the wave with a DPP scan, the
-//     lanes drop their tokens into a per-wave LDS staging area at their scanned positions,
-//     and the wave writes the staged run back out as aligned 16-byte groups.  The up-to-3
-//     tokens that do not fill a group stay in LDS for the next step of the row.  A step that
-//     yields more tokens than the staging area holds is staged in several passes.
+//     id, the ragged end of a row, or a write position that an earlier expansion moved off
+//     the line grid): unit token counts are prefix-summed across the wave with a DPP scan,
+//     the lanes drop their tokens into a per-wave LDS staging area at their scanned
+//     positions, and the wave writes the staged run back out as 16-byte groups, whole
+//     128-byte lines at a time.  The tokens past the last whole line stay in LDS for the
+//     next step of the row.  A step that yields more tokens than the staging area holds is
+//     staged in several passes.
 //     When the table spells every non-plain window character by character (the usual
 //     grid-aligned tokenizer), the spelled tokens come from an LDS table; otherwise from the
 //     global 5^k entry table and its expansion lists.
@@ -56,6 +59,11 @@ constexpr int kWaveUnits = 64 * kUnitsPerLane;          // units one wave handle
 // Staging area of one wave: kStageCap tokens in scanned order (+ room to read the last group whole).
 constexpr int kStageCap = 512;
 constexpr int kStageWords = kStageCap + 8;
+// A shifted run is written out in whole units of kFlushCells cells (one 128-byte line of ids;
+// a multiple of 4 that divides kStageCap); the cells past the last whole unit wait in LDS for
+// the next step of the row, so that no line of the output is written in two pieces.
+constexpr int kFlushCells = 32;
+constexpr uint32_t kFlushMask = kFlushCells - 1;
 
 // LDS digit entries: 0..3 for A C G T; flags above every window code (4^8 = 1 << 16) for N and
 // for a byte outside the alphabet, so that "window code < 4^k" means "k plain bases".
@@ -250,7 +258,7 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
             int sv_r = 0;
             int32_t sv_v[4] = {0, 0, 0, 0};
 
-            if (rest_mask == 0 && (A & 3) == 0) {
+            if (rest_mask == 0 && (A & (int)kFlushMask) == 0) {
                 // every lane is plain or past the end, and the run starts on a 16-byte boundary:
                 // positions are known without a scan
                 const int r = running + lane * kUnitsPerLane;
@@ -333,9 +341,10 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
 
             const uint32_t inc = wave_inclusive_sum_u32(lane_cnt);
             const uint32_t step_total = __builtin_amdgcn_readlane(inc, 63);
-            // staged index 0 is cell A & ~3; the first `carry` entries are the tokens the previous
-            // step left over (at the start of a row: cells of the neighbouring row, never written)
-            const uint32_t carry = (uint32_t)(A & 3);
+            // staged index 0 is the cell at the last multiple of kFlushCells at or below A; the first
+            // `carry` entries are the tokens the previous step left over (at the start of a row:
+            // cells of the neighbouring row, never written)
+            const uint32_t carry = (uint32_t)A & kFlushMask;
             const uint32_t n_avail = carry + step_total;
             const uint32_t s0 = carry + (inc - lane_cnt);
             const bool last_step = u0 + kWaveUnits >= n_units;
@@ -416,8 +425,8 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
                 produce([&](uint32_t s, int32_t tok) { buf[s] = tok; });
                 wave_sync();
                 // whole groups; the row's last step also writes the group it leaves unfilled
-                const uint32_t n_groups = last_step ? (n_avail + 3) >> 2 : n_avail >> 2;
-                const int e0 = A & ~3;
+                const uint32_t n_groups = last_step ? (n_avail + 3) >> 2 : (n_avail & ~kFlushMask) >> 2;
+                const int e0 = A & ~(int)kFlushMask;
                 {
                     // groups 0..63: one per lane, left to the step's common store
                     const int e = e0 + 4 * lane;
@@ -438,9 +447,9 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
                         store_group(outA, moutA, e0 + 4 * (int)g, lo, hi, v, 1u);
                     }
                 }
-                const uint32_t left = last_step ? 0u : (n_avail & 3);
+                const uint32_t left = last_step ? 0u : (n_avail & kFlushMask);
                 int32_t keep = 0;
-                if ((uint32_t)lane < left) keep = buf[(n_avail & ~3u) + lane];
+                if ((uint32_t)lane < left) keep = buf[(n_avail & ~kFlushMask) + lane];
                 wave_sync();
                 if ((uint32_t)lane < left) buf[lane] = keep;
             } else {
@@ -454,16 +463,16 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
                     wave_sync();
                     const bool final_pass = pass + kStageCap >= n_avail;
                     const uint32_t count = final_pass ? n_avail - pass : (uint32_t)kStageCap;
-                    const uint32_t n_groups = final_pass && last_step ? (count + 3) >> 2 : count >> 2;
-                    const int e0 = (A & ~3) + (int)pass;
+                    const uint32_t n_groups = final_pass && last_step ? (count + 3) >> 2 : (count & ~kFlushMask) >> 2;
+                    const int e0 = (A & ~(int)kFlushMask) + (int)pass;
                     for (uint32_t g = lane; g < n_groups; g += 64) {
                         int32_t v[4];
                         group_at(g, v);
                         store_group(outA, moutA, e0 + 4 * (int)g, lo, hi, v, 1u);
                     }
-                    const uint32_t left = final_pass && !last_step ? (count & 3) : 0u;
+                    const uint32_t left = final_pass && !last_step ? (count & kFlushMask) : 0u;
                     int32_t keep = 0;
-                    if ((uint32_t)lane < left) keep = buf[(count & ~3u) + lane];
+                    if ((uint32_t)lane < left) keep = buf[(count & ~kFlushMask) + lane];
                     wave_sync();
                     if ((uint32_t)lane < left) buf[lane] = keep;
                     wave_sync();
