@@ -150,18 +150,23 @@ class KmerPadded(Workload):
         self.bases = host.size
         self.kernel = "kmer_rows_kernel"
         self.name = (f"C2 non-overlapping 6-mer vocab-4106, 256x6000 bp batches, "
-                     f"{n_batches} distinct batch(es) per call, pad to longest row")
+                     f"{n_batches} distinct batch(es) per call, pad to longest row "
+                     f"(width of the previous call passed as the guess)")
+        self.width_guess = 0
         self.step()
         torch.cuda.synchronize()
         lengths = self.out[2].cpu().numpy()
         t_max = int(self.out[4].item())
+        self.width_guess = t_max
         assert t_max == int(lengths.max())
         # 1 B/base read; int32 id + uint8 mask for every cell of [rows, T_max]; int32 length per row
         self.algorithmic_bytes = host.size + 5 * self.n_rows * t_max + 4 * self.n_rows
         self.t_max = t_max
 
     def step(self):
-        self.enc.encode_padded(self.data, self.off, self.t_cap, fill_to=0, out=self.out)
+        # a stream of batches: the width of the previous call is the guess for this one
+        self.enc.encode_padded(self.data, self.off, self.t_cap, fill_to=0, width_guess=self.width_guess,
+                               out=self.out)
 
     def check(self):
         from tests.golden import check as util

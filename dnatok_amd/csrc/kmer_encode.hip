@@ -501,33 +501,48 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
         atomicMax(max_len, (int32_t)wave_max);
 }
 
-// Pads every row from its stored length up to the batch maximum found on the device.
-// One wave per row.
+// Pads every row from its stored length up to the batch maximum found on the device.  A wave
+// reads the lengths of kPadRows rows at once, then pads the rows that fall short one after
+// the other, so that the stores of all of them are in flight together.
+#ifndef DNATOK_PAD_ROWS
+#define DNATOK_PAD_ROWS 8
+#endif
+constexpr int kPadRows = DNATOK_PAD_ROWS;
+
 __global__ __launch_bounds__(256) void pad_to_max_kernel(
     int32_t *__restrict__ ids, uint8_t *__restrict__ mask, const int32_t *__restrict__ lengths,
-    int64_t n_rows, int64_t t_cap, const int32_t *__restrict__ max_len, int32_t pad_id)
+    int64_t n_rows, int64_t t_cap, const int32_t *__restrict__ max_len, int32_t pad_id, int32_t already)
 {
     const int fill = *max_len;
+    if (fill <= already) return;          // every row is padded this far already
     const int lane = threadIdx.x & 63;
     const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     const int64_t n_waves = (int64_t)gridDim.x * (blockDim.x >> 6);
-    for (int64_t row = wave; row < n_rows; row += n_waves) {
-        int len = lengths[row];
-        if (len < 0) len = 0;
-        if (len >= fill) continue;
-        int32_t *out = ids + row * t_cap;
-        const int mis = (int)((reinterpret_cast<uintptr_t>(out) >> 2) & 3);
-        pad_cells(out - mis, mask ? mask + row * t_cap - mis : nullptr, mis, len, fill, pad_id, lane);
+    for (int64_t base = wave * kPadRows; base < n_rows; base += n_waves * kPadRows) {
+        int len = fill;
+        if (lane < kPadRows && base + lane < n_rows) {
+            len = lengths[base + lane];
+            if (len < already) len = already;
+        }
+        uint64_t todo = __ballot(len < fill);
+        while (todo) {
+            const int l = __builtin_ctzll(todo);
+            todo &= todo - 1;
+            const int from = __builtin_amdgcn_readlane(len, l);
+            int32_t *out = ids + (base + l) * t_cap;
+            const int mis = (int)((reinterpret_cast<uintptr_t>(out) >> 2) & 3);
+            pad_cells(out - mis, mask ? mask + (base + l) * t_cap - mis : nullptr, mis, from, fill, pad_id, lane);
+        }
     }
 }
 
 int launch_pad_to_max(int32_t *ids, uint8_t *mask, const int32_t *lengths, int64_t n_rows,
-                      int64_t t_cap, const int32_t *max_len, int32_t pad_id, hipStream_t s)
+                      int64_t t_cap, const int32_t *max_len, int32_t pad_id, int32_t already, hipStream_t s)
 {
-    int64_t blocks = (n_rows + 3) / 4;
+    int64_t blocks = (n_rows + 4 * kPadRows - 1) / (4 * kPadRows);
     if (blocks > 256 * 16) blocks = 256 * 16;
     if (blocks < 1) blocks = 1;
-    pad_to_max_kernel<<<(int)blocks, 256, 0, s>>>(ids, mask, lengths, n_rows, t_cap, max_len, pad_id);
+    pad_to_max_kernel<<<(int)blocks, 256, 0, s>>>(ids, mask, lengths, n_rows, t_cap, max_len, pad_id, already);
     DNATOK_HIP_TRY(hipGetLastError());
     return DNATOK_OK;
 }
@@ -636,10 +651,18 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
 {
     DNATOK_REQUIRE(t && offsets && ids && lengths, DNATOK_E_INVALID,
                    "dnatok_kmer_encode_padded: null argument");
-    DNATOK_REQUIRE(n_rows >= 0 && t_cap >= 0 && fill_to >= 0 && fill_to <= t_cap, DNATOK_E_INVALID,
-                   "dnatok_kmer_encode_padded: need 0 <= fill_to <= t_cap");
+    DNATOK_REQUIRE(n_rows >= 0 && t_cap >= 0 && fill_to <= t_cap, DNATOK_E_INVALID,
+                   "dnatok_kmer_encode_padded: need fill_to <= t_cap");
     DNATOK_REQUIRE(fill_to > 0 || max_len, DNATOK_E_INVALID,
-                   "dnatok_kmer_encode_padded: fill_to = 0 needs max_len");
+                   "dnatok_kmer_encode_padded: fill_to <= 0 needs max_len");
+    // fill_to < 0: pad to the longest row; -fill_to is the caller's guess of that width.  Rows are
+    // padded to the guess while they are written (next to the cells just stored, which is far
+    // cheaper than coming back to every row), the pass after the kernel pads what is missing.
+    const bool to_longest = fill_to <= 0;
+    int64_t guess = to_longest ? -fill_to : 0;
+    if (guess > t_cap) guess = t_cap;
+    if (guess > INT_MAX - 16) guess = INT_MAX - 16;
+    if (to_longest) fill_to = guess;
     if (n_rows == 0) return DNATOK_OK;
     hipStream_t s = (hipStream_t)stream;
     KmerArgs a{t->digit, t->single, t->lut4, t->entry, t->flat, t->pad_id, t->missing_id};
@@ -677,6 +700,7 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
 #undef LAUNCH2
 #undef LAUNCH3
     DNATOK_HIP_TRY(hipGetLastError());
-    if (fill_to == 0) return launch_pad_to_max(ids, mask, lengths, n_rows, t_cap, max_len, t->pad_id, s);
+    if (to_longest)
+        return launch_pad_to_max(ids, mask, lengths, n_rows, t_cap, max_len, t->pad_id, (int32_t)guess, s);
     return DNATOK_OK;
 }

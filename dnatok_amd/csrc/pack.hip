@@ -6,7 +6,7 @@
 namespace dnatok {
 
 int launch_pad_to_max(int32_t *ids, uint8_t *mask, const int32_t *lengths, int64_t n_rows,
-                      int64_t t_cap, const int32_t *max_len, int32_t pad_id, hipStream_t s);
+                      int64_t t_cap, const int32_t *max_len, int32_t pad_id, int32_t already, hipStream_t s);
 
 __global__ void zero_i32_kernel(int32_t *p) { *p = 0; }
 
@@ -151,6 +151,6 @@ extern "C" int dnatok_pad_rows(const int32_t *tok_tmp, const int64_t *in_offsets
     pad_rows_kernel<<<wave_grid(n_rows), 256, 0, s>>>(tok_tmp, in_offsets, lengths, n_rows, remap,
                                                       pad_id, t_cap, fill_to, ids, mask, max_len);
     DNATOK_HIP_TRY(hipGetLastError());
-    if (fill_to == 0) return launch_pad_to_max(ids, mask, lengths, n_rows, t_cap, max_len, pad_id, s);
+    if (fill_to == 0) return launch_pad_to_max(ids, mask, lengths, n_rows, t_cap, max_len, pad_id, 0, s);
     return DNATOK_OK;
 }

@@ -367,8 +367,11 @@ class DNATok:
         # the mask on cache-line boundaries, which the store path of the kernel is built around
         t_cap = int(lens.max()) + 4
         t_cap += (-t_cap) % 128
-        ids, mask, lengths, status, longest = self._kmer_enc.encode_padded(data, offsets, t_cap, fill_to=0)
+        # the width of the previous batch is a good guess of this one's in a stream of batches
+        ids, mask, lengths, status, longest = self._kmer_enc.encode_padded(
+            data, offsets, t_cap, fill_to=0, width_guess=getattr(self, "_kmer_width_guess", 0))
         width = int(longest.item())                      # one scalar: the output shape
+        self._kmer_width_guess = width
         if self.token_len is not None and self.token_len > width:
             extra = int(self.token_len)
             ids, mask, lengths, status, longest = self._kmer_enc.encode_padded(

@@ -135,9 +135,11 @@ class KmerEncoder:
                 pass
 
     def encode_padded(self, data: torch.Tensor, offsets: torch.Tensor, t_cap: int, *,
-                      fill_to: int = 0, want_mask: bool = True, out=None):
+                      fill_to: int = 0, width_guess: int = 0, want_mask: bool = True, out=None):
         """Returns (ids[B, t_cap], mask, lengths[B], status[B], max_len[1]); with fill_to = 0 the
-        rows are padded to the device-side maximum, view ``ids[:, :max_len]``."""
+        rows are padded to the device-side maximum, view ``ids[:, :max_len]``.  ``width_guess``
+        (only with fill_to = 0) is the caller's guess of that maximum, e.g. the width of the
+        previous batch of a stream: rows are padded that far while they are written."""
         _require_cuda(data, torch.uint8, "data")
         _require_cuda(offsets, torch.int64, "offsets")
         n_rows = offsets.numel() - 1
@@ -151,7 +153,8 @@ class KmerEncoder:
         else:
             ids, mask, lengths, status, max_len = out
         _lib.check(_lib.lib().dnatok_kmer_encode_padded(
-            self._h, _ptr(data), _ptr(offsets), n_rows, int(t_cap), int(fill_to), _ptr(ids),
+            self._h, _ptr(data), _ptr(offsets), n_rows, int(t_cap),
+            int(fill_to) if fill_to > 0 else -min(int(width_guess), int(t_cap)), _ptr(ids),
             _ptr(mask), _ptr(lengths), _ptr(status), _ptr(max_len), _stream()),
             "dnatok_kmer_encode_padded")
         return ids, mask, lengths, status, max_len

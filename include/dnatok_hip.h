@@ -94,7 +94,11 @@ void dnatok_kmer_table_destroy(dnatok_kmer_t *t);
  * stored row length (NULL allowed).
  * fill_to > 0: every row is padded to column fill_to (<= t_cap).
  * fill_to = 0: rows are padded to the longest row of the batch, found on the device, so the
- *              caller may view ids[:, :max_len] without a second pass over the data. */
+ *              caller may view ids[:, :max_len] without a second pass over the data.
+ * fill_to < 0: as fill_to = 0, with -fill_to as the caller's guess of that longest row (say,
+ *              the width of the previous batch of a stream).  Rows are padded to the guess while
+ *              they are written and only what is missing afterwards; a guess that is too small
+ *              or too large costs time, never correctness (cells past max_len are unspecified). */
 int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *bytes, const int64_t *offsets,
                               int64_t n_rows, int64_t t_cap, int64_t fill_to,
                               int32_t *ids, uint8_t *mask, int32_t *lengths, int32_t *status,

@@ -162,6 +162,33 @@ def test_kmer_ragged_all_k(k):
         np.testing.assert_array_equal(mask[:, :width].cpu().numpy(), emask)
 
 
+def test_kmer_pad_to_longest_with_width_guess():
+    """fill_to = 0 with a guess of the longest row: a guess below, at or above the true width
+    gives the same ids / mask / lengths / max_len inside [:, :max_len]."""
+    say("kmer width guess")
+    k = 6
+    vocab = hf.kmer_vocab(k)
+    t = kmer_tables.tables_from_vocab(vocab, k, 0)
+    enc = encoders.KmerEncoder(k, t.digit, t.kmer_lut, t.single, pad_id=1, missing_id=0,
+                               exp_off=t.exp_off, exp_len=t.exp_len, exp_flat=t.exp_flat)
+    b = wl.config2_kmer(64, 3000, seed=77, n_fraction=0.02)
+    data, off = to_dev(b)
+    ref = enc.encode_padded(data, off, 3008, fill_to=0)
+    torch.cuda.synchronize()
+    width = int(ref[4].item())
+    erows, _ = O.kmer_encode(O.kmer_tables_from_vocab(vocab, k, 0), b.data, b.offsets)
+    eids, emask = O.pad_rows(erows, 1, width)
+    np.testing.assert_array_equal(ref[0][:, :width].cpu().numpy(), eids)
+    for guess in (1, width - 37, width, width + 5, 3008, 10 ** 9):
+        got = enc.encode_padded(data, off, 3008, fill_to=0, width_guess=guess)
+        torch.cuda.synchronize()
+        assert int(got[4].item()) == width
+        np.testing.assert_array_equal(got[0][:, :width].cpu().numpy(), eids)
+        np.testing.assert_array_equal(got[1][:, :width].cpu().numpy(), emask)
+        np.testing.assert_array_equal(got[2].cpu().numpy(), ref[2].cpu().numpy())
+        np.testing.assert_array_equal(got[3].cpu().numpy(), ref[3].cpu().numpy())
+
+
 def test_kmer_general_tables_not_spelled():
     """Tables whose N windows are not spelled character by character: N windows that have an
     id of their own, expansions of other lengths, and windows with nothing at all."""
