@@ -249,30 +249,15 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
             }
             const uint32_t any_flag = code[0] | code[1] | code[2] | code[3];
             const bool fast = lane_full && any_flag < POW4 && (t[0] | t[1] | t[2] | t[3]) >= 0;
-            const uint64_t fast_mask = __ballot(fast);
             const uint64_t rest_mask = __ballot(!fast && !empty);
             const int A = mis + running;           // cell the step's first token goes to
 
-            // what the step's common store (one 4-cell group per lane) will write
-            bool sv_whole = false;
-            int sv_r = 0;
-            int32_t sv_v[4] = {0, 0, 0, 0};
-
-            if (rest_mask == 0 && (A & (int)kFlushMask) == 0) {
-                // every lane is plain or past the end, and the run starts on a 16-byte boundary:
-                // positions are known without a scan
-                const int r = running + lane * kUnitsPerLane;
-                sv_whole = fast && r + 4 <= vec_cap;
-                sv_r = r;
-#pragma unroll
-                for (int j = 0; j < kUnitsPerLane; ++j) sv_v[j] = t[j];
-                if (__ballot(fast && !sv_whole)) {                 // row cut at t_cap
-                    settle();
-                    if (fast && !sv_whole) store_group(outA, moutA, mis + r, lo, hi_cap, t, 1u);
-                }
-                running += kUnitsPerLane * (int)__popcll(fast_mask);
-            } else {
-            // ---- staged step ----
+            // Tokens per unit and per lane, and their prefix sum over the wave.  Done for every
+            // step, also the plain ones that know their positions without it: the step's token
+            // count is then a scalar defined on one path only.  (A scalar that only one side of
+            // a branch defines is given a filler definition read from an arbitrary vector
+            // register; when that register is one the next step's bytes are being loaded into,
+            // the filler waits for the load.)
             // per unit: cnt = number of tokens; ex/ey = entry of a window that is not plain
             int32_t cnt[kUnitsPerLane], ex[kUnitsPerLane], ey[kUnitsPerLane];
             uint32_t lane_cnt = 0;
@@ -341,6 +326,26 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
 
             const uint32_t inc = wave_inclusive_sum_u32(lane_cnt);
             const uint32_t step_total = __builtin_amdgcn_readlane(inc, 63);
+
+            // what the step's common store (one 4-cell group per lane) will write
+            bool sv_whole = false;
+            int sv_r = 0;
+            int32_t sv_v[4] = {0, 0, 0, 0};
+
+            if (rest_mask == 0 && (A & (int)kFlushMask) == 0) {
+                // every lane is plain or past the end, and the run starts on a 16-byte boundary:
+                // positions are known without a scan
+                const int r = running + lane * kUnitsPerLane;
+                sv_whole = fast && r + 4 <= vec_cap;
+                sv_r = r;
+#pragma unroll
+                for (int j = 0; j < kUnitsPerLane; ++j) sv_v[j] = t[j];
+                if (__ballot(fast && !sv_whole)) {                 // row cut at t_cap
+                    settle();
+                    if (fast && !sv_whole) store_group(outA, moutA, mis + r, lo, hi_cap, t, 1u);
+                }
+            } else {
+            // ---- staged step ----
             // staged index 0 is the cell at the last multiple of kFlushCells at or below A; the first
             // `carry` entries are the tokens the previous step left over (at the start of a row:
             // cells of the neighbouring row, never written)
@@ -478,9 +483,9 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
                     wave_sync();
                 }
             }
-            running += (int)step_total;
             }
             store_vec(sv_whole, sv_r, sv_v);
+            running += (int)step_total;
         }
 
         const int stored = running < cap ? running : cap;
