@@ -28,6 +28,7 @@
 
 #include <limits.h>
 #include <string.h>
+#include <atomic>
 #include <vector>
 
 struct dnatok_kmer_table {
@@ -41,7 +42,18 @@ struct dnatok_kmer_table {
     int32_t *lut4;           // [4^k]  id of an ACGT-only window, or -1
     int2 *entry;             // [5^k]  {id, 0} | {-len, offset into flat} | {INT_MIN, 0} = nothing known
     int32_t *flat;           // expansion lists
+    // Running maxima of pad-to-longest calls.  A call takes the next of kMaxSlots slots (calls in
+    // flight on different streams use different slots).  A slot is two 64-bit words: the running
+    // maximum, tagged in its upper half with the slot's generation, and the generation itself,
+    // which the padding pass of a call bumps when it is done with the maximum.  A maximum of a
+    // later call is therefore larger than anything an earlier call left behind, and the slot
+    // never has to be cleared (a launch saved per call; replays of a captured call stay exact).
+    unsigned long long *max_slots;
+    mutable std::atomic<uint32_t> call_seq;
 };
+
+constexpr int kMaxSlots = 16;
+constexpr int kMaxSlotStride = 32;       // 64-bit words between two slots (one 256-byte line each)
 
 namespace dnatok {
 
@@ -83,6 +95,12 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 __global__ void kmer_init_kernel(int32_t *max_len) { *max_len = 0; }
+
+// Where a pad-to-longest call keeps its running maximum: slot[0] = generation << 32 | maximum,
+// slot[1] = generation.
+struct MaxRef {
+    unsigned long long *slot;
+};
 
 // Stores the group of 4 cells [e, e + 4) of a row whose cells are addressed from the
 // 16-byte-aligned pointer pair (outA, moutA); only cells inside [lo, hi) are written.
@@ -127,7 +145,7 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
     KmerArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
     int64_t n_rows, int64_t t_cap, int64_t fill_to, int32_t *__restrict__ ids,
     uint8_t *__restrict__ mask, int32_t *__restrict__ lengths, int32_t *__restrict__ status,
-    int32_t *__restrict__ max_len)
+    int32_t *__restrict__ max_len, MaxRef mref)
 {
     constexpr uint32_t POW4 = 1u << (2 * K);
     __shared__ uint32_t s_dig[256];
@@ -152,6 +170,7 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
     const int cap = t_cap > INT_MAX - 16 ? INT_MAX - 16 : (int)t_cap;
     const int fill = fill_to > cap ? cap : (int)fill_to;
     int64_t wave_max = 0;
+    const unsigned long long slot_gen = mref.slot ? mref.slot[1] : 0ull;
     const int wave_in_wg = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int64_t wave = (int64_t)blockIdx.x * (kKmerThreads / 64) + wave_in_wg;
     const int64_t n_waves = (int64_t)gridDim.x * (kKmerThreads / 64);
@@ -501,9 +520,15 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
         if (fill > stored) pad_cells(outA, moutA, mis, stored, fill, a.pad_id, lane);
     }
     // one atomic per wave at most, skipped when another wave already published a larger value
-    if (max_len && lane == 0 && wave_max > 0 &&
-        (int64_t)__builtin_nontemporal_load(max_len) < wave_max)
+    if (mref.slot) {
+        // (the first wave publishes even a maximum of 0: the slot then carries this call's tag)
+        const unsigned long long v = (slot_gen << 32) | (unsigned long long)wave_max;
+        if (lane == 0 && (wave_max > 0 || wave == 0) && __builtin_nontemporal_load(mref.slot) < v)
+            atomicMax(mref.slot, v);
+    } else if (max_len && lane == 0 && wave_max > 0 &&
+               (int64_t)__builtin_nontemporal_load(max_len) < wave_max) {
         atomicMax(max_len, (int32_t)wave_max);
+    }
 }
 
 // Pads every row from its stored length up to the batch maximum found on the device.  A wave
@@ -516,9 +541,19 @@ constexpr int kPadRows = DNATOK_PAD_ROWS;
 
 __global__ __launch_bounds__(256) void pad_to_max_kernel(
     int32_t *__restrict__ ids, uint8_t *__restrict__ mask, const int32_t *__restrict__ lengths,
-    int64_t n_rows, int64_t t_cap, const int32_t *__restrict__ max_len, int32_t pad_id, int32_t already)
+    int64_t n_rows, int64_t t_cap, int32_t *__restrict__ max_len, int32_t pad_id, int32_t already, MaxRef mref)
 {
-    const int fill = *max_len;
+    int fill;
+    if (mref.slot) {
+        // the maximum is in the call's slot; the slot's next user gets the next generation
+        fill = (int)(uint32_t)mref.slot[0];
+        if (blockIdx.x == 0 && threadIdx.x == 0) {
+            *max_len = fill;
+            mref.slot[1] = mref.slot[1] + 1;
+        }
+    } else {
+        fill = *max_len;
+    }
     if (fill <= already) return;          // every row is padded this far already
     const int lane = threadIdx.x & 63;
     const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -541,15 +576,21 @@ __global__ __launch_bounds__(256) void pad_to_max_kernel(
     }
 }
 
-int launch_pad_to_max(int32_t *ids, uint8_t *mask, const int32_t *lengths, int64_t n_rows,
-                      int64_t t_cap, const int32_t *max_len, int32_t pad_id, int32_t already, hipStream_t s)
+static int launch_pad(int32_t *ids, uint8_t *mask, const int32_t *lengths, int64_t n_rows, int64_t t_cap,
+                      int32_t *max_len, int32_t pad_id, int32_t already, MaxRef mref, hipStream_t s)
 {
     int64_t blocks = (n_rows + 4 * kPadRows - 1) / (4 * kPadRows);
     if (blocks > 256 * 16) blocks = 256 * 16;
     if (blocks < 1) blocks = 1;
-    pad_to_max_kernel<<<(int)blocks, 256, 0, s>>>(ids, mask, lengths, n_rows, t_cap, max_len, pad_id, already);
+    pad_to_max_kernel<<<(int)blocks, 256, 0, s>>>(ids, mask, lengths, n_rows, t_cap, max_len, pad_id, already, mref);
     DNATOK_HIP_TRY(hipGetLastError());
     return DNATOK_OK;
+}
+
+int launch_pad_to_max(int32_t *ids, uint8_t *mask, const int32_t *lengths, int64_t n_rows,
+                      int64_t t_cap, int32_t *max_len, int32_t pad_id, int32_t already, hipStream_t s)
+{
+    return launch_pad(ids, mask, lengths, n_rows, t_cap, max_len, pad_id, already, MaxRef{nullptr}, s);
 }
 
 }  // namespace dnatok
@@ -613,7 +654,8 @@ extern "C" int dnatok_kmer_table_create(int k, const int8_t *digit_h, const int3
     const size_t o_lut4 = up(o_single + 256 * 4);
     const size_t o_entry = up(o_lut4 + pow4 * 4);
     const size_t o_flat = up(o_entry + pow5 * sizeof(int2));
-    const size_t bytes = up(o_flat + (has_exp ? n_flat * 4 : 0)) + 256;
+    const size_t o_slots = up(o_flat + (has_exp ? n_flat * 4 : 0));
+    const size_t bytes = up(o_slots + (size_t)kMaxSlots * kMaxSlotStride * 8) + 256;
     std::vector<uint8_t> host(bytes, 0);
     memcpy(&host[o_digit], digit_h, 256);
     memcpy(&host[o_single], single_h, 256 * 4);
@@ -637,6 +679,8 @@ extern "C" int dnatok_kmer_table_create(int k, const int8_t *digit_h, const int3
     t->lut4 = (int32_t *)(b + o_lut4);
     t->entry = (int2 *)(b + o_entry);
     t->flat = (int32_t *)(b + o_flat);
+    t->max_slots = (unsigned long long *)(b + o_slots);
+    t->call_seq.store(0);
     *out = t;
     return DNATOK_OK;
 }
@@ -671,7 +715,11 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
     if (n_rows == 0) return DNATOK_OK;
     hipStream_t s = (hipStream_t)stream;
     KmerArgs a{t->digit, t->single, t->lut4, t->entry, t->flat, t->pad_id, t->missing_id};
-    if (max_len) {
+    MaxRef mref{nullptr};
+    if (to_longest) {
+        const uint32_t seq = t->call_seq.fetch_add(1, std::memory_order_relaxed);
+        mref.slot = t->max_slots + (size_t)(seq % kMaxSlots) * kMaxSlotStride;
+    } else if (max_len) {
         kmer_init_kernel<<<1, 1, 0, s>>>(max_len);
         DNATOK_HIP_TRY(hipGetLastError());
     }
@@ -682,7 +730,7 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
         static const int resident = resident_workgroups(kmer_rows_kernel<KK, L, C, M>, kKmerThreads, 0, 4); \
         const int64_t grid = want < resident ? want : resident;                                   \
         kmer_rows_kernel<KK, L, C, M><<<(int)grid, kKmerThreads, 0, s>>>(                         \
-            a, bytes, offsets, n_rows, t_cap, fill_to, ids, mask, lengths, status, max_len);      \
+            a, bytes, offsets, n_rows, t_cap, fill_to, ids, mask, lengths, status, max_len, mref); \
     } while (0)
 #define LAUNCH2(KK, L, C)                                                                         \
     do {                                                                                          \
@@ -706,6 +754,6 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
 #undef LAUNCH3
     DNATOK_HIP_TRY(hipGetLastError());
     if (to_longest)
-        return launch_pad_to_max(ids, mask, lengths, n_rows, t_cap, max_len, t->pad_id, (int32_t)guess, s);
+        return launch_pad(ids, mask, lengths, n_rows, t_cap, max_len, t->pad_id, (int32_t)guess, mref, s);
     return DNATOK_OK;
 }

@@ -6,7 +6,7 @@
 namespace dnatok {
 
 int launch_pad_to_max(int32_t *ids, uint8_t *mask, const int32_t *lengths, int64_t n_rows,
-                      int64_t t_cap, const int32_t *max_len, int32_t pad_id, int32_t already, hipStream_t s);
+                      int64_t t_cap, int32_t *max_len, int32_t pad_id, int32_t already, hipStream_t s);
 
 __global__ void zero_i32_kernel(int32_t *p) { *p = 0; }
 

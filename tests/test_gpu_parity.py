@@ -189,6 +189,48 @@ def test_kmer_pad_to_longest_with_width_guess():
         np.testing.assert_array_equal(got[3].cpu().numpy(), ref[3].cpu().numpy())
 
 
+def test_kmer_pad_to_longest_replayed_from_a_graph(kmer_enc):
+    """A captured pad-to-longest call, replayed over changing input: every replay reports the
+    longest row of its own input (first a batch with long rows, then shorter ones, then long
+    again), and matches the eager call."""
+    say("kmer graph replay")
+    n, length = 32, 2400
+    batches = [wl.config2_kmer(n, length, seed=5, n_fraction=0.05),
+               wl.config2_kmer(n, length, seed=6, n_fraction=0.0),
+               wl.config2_kmer(n, length, seed=7, n_fraction=0.01),
+               wl.config2_kmer(n, length, seed=8, n_fraction=0.08)]
+    data = torch.zeros(n * length, dtype=torch.uint8, device=DEV)
+    off = torch.arange(n + 1, dtype=torch.int64, device=DEV) * length
+    t_cap = 2432
+    out = (torch.empty((n, t_cap), dtype=torch.int32, device=DEV), torch.empty((n, t_cap), dtype=torch.uint8, device=DEV),
+           torch.empty(n, dtype=torch.int32, device=DEV), torch.empty(n, dtype=torch.int32, device=DEV),
+           torch.empty(1, dtype=torch.int32, device=DEV))
+    data.copy_(torch.from_numpy(batches[0].data))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        kmer_enc.encode_padded(data, off, t_cap, fill_to=0, out=out)        # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        kmer_enc.encode_padded(data, off, t_cap, fill_to=0, out=out)
+    widths = []
+    for b in batches + batches[:2]:
+        data.copy_(torch.from_numpy(b.data))
+        graph.replay()
+        torch.cuda.synchronize()
+        width = int(out[4].item())
+        widths.append(width)
+        got_ids, got_mask = out[0][:, :width].cpu().numpy(), out[1][:, :width].cpu().numpy()
+        eager = kmer_enc.encode_padded(data, off, t_cap, fill_to=0)
+        torch.cuda.synchronize()
+        assert int(eager[4].item()) == width == int(out[2].max().item())
+        np.testing.assert_array_equal(got_ids, eager[0][:, :width].cpu().numpy())
+        np.testing.assert_array_equal(got_mask, eager[1][:, :width].cpu().numpy())
+    assert widths[1] == length // 6 and widths[0] > widths[1] and widths[3] > widths[2] > widths[1]
+
+
 def test_kmer_general_tables_not_spelled():
     """Tables whose N windows are not spelled character by character: N windows that have an
     id of their own, expansions of other lengths, and windows with nothing at all."""
