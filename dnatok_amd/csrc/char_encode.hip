@@ -31,6 +31,7 @@ constexpr int kCharSteps = 4;                                   // dwords per la
 constexpr int kCharTile = kCharThreads * 4 * kCharSteps;        // 4096 bases per tile
 
 typedef int32_t int4v __attribute__((ext_vector_type(4)));
+typedef int32_t int4v_a4 __attribute__((ext_vector_type(4), aligned(4)));   // only the mask's 4-byte alignment is required
 
 __device__ __forceinline__ int4v lookup4(const int32_t *lut, uint32_t w)
 {
@@ -76,8 +77,12 @@ __global__ __launch_bounds__(kCharThreads) void char_packed_kernel(
                     if ((r + 3) % row_len == 0) v.w = start[w[s] >> 24];
                 }
                 __builtin_nontemporal_store(v, reinterpret_cast<int4v *>(ids + i));
-                if (HAS_MASK)
-                    __builtin_nontemporal_store(0x01010101u, reinterpret_cast<uint32_t *>(mask + i));
+            }
+            // the mask of a whole tile is 4096 ones: one 16-byte store per lane covers it
+            if (HAS_MASK) {
+                const int4v_a4 ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+                __builtin_nontemporal_store(
+                    ones, reinterpret_cast<int4v_a4 *>(mask + tile * kCharTile + (int64_t)threadIdx.x * 16));
             }
         } else {
             // last, partial tile: position by position
