@@ -138,17 +138,19 @@ __device__ __forceinline__ uint32_t team_exclusive_sum(uint32_t v, uint32_t *red
     return carry + inc - v;
 }
 
-// One row.  tid = index in the team; S/R/NS/MC/NX/PV/F hold n0 entries; D holds NT bytes;
-// red holds 4 * (NT / 64) words.  Tokens go to out[0 .. *out_len).
+// One row.  tid = index in the team; S/R/NS/MC/NX/PV hold n0 entries, Q (the merges of the
+// current round) n0 / 2; D holds NT bytes; red holds 4 * (NT / 64) + 4 words.  Tokens go to
+// out[0 .. *out_len).
 template <int NT, typename IT>
 __device__ __forceinline__ void bpe_row(
     const uint4 *tab, uint32_t tab_mask, uint32_t tab_shift, const uint16_t *byte_to_sym,
     const int32_t *out_remap, const uint8_t *__restrict__ src, const int n0, uint16_t *S, uint16_t *R,
-    uint16_t *NS, uint16_t *MC, IT *NX, IT *PV, uint8_t *F, uint8_t *D, uint32_t *red, const int tid,
+    uint16_t *NS, uint16_t *MC, IT *NX, IT *PV, IT *Q, uint8_t *D, uint32_t *red, const int tid,
     int32_t *__restrict__ out, int32_t *__restrict__ out_len, uint16_t *__restrict__ raw_out = nullptr)
 {
     constexpr IT NIL = (IT)~(IT)0;
     const int wv = (NT == 64) ? 0 : (tid >> 6);
+    uint32_t *qn = red + 4 * (NT / 64);        // number of merges queued in the current round
     // position i belongs to thread i % NT: in every pass the lanes of a wave touch consecutive
     // positions, so the LDS state arrays are read and written without bank conflicts
 
@@ -156,9 +158,9 @@ __device__ __forceinline__ void bpe_row(
         S[i] = byte_to_sym[src[i]];
         NX[i] = (i + 1 < n0) ? (IT)(i + 1) : NIL;
         PV[i] = (i > 0) ? (IT)(i - 1) : NIL;
-        F[i] = 0;
     }
     D[tid] = 0;
+    if (tid == 0) *qn = 0;
     team_sync<NT>();
 
     // initial pair of every position, four table probes in flight at a time
@@ -207,8 +209,7 @@ __device__ __forceinline__ void bpe_row(
         }
         const uint32_t limit = single ? rmin + 1 : gate;
 
-        // decide (reads only, except the owner's own flags)
-        bool mine = false;
+        // decide (reads only); a pair that merges is put on the round's queue
         if (cmin < limit) {
             for (int i = tid; i < n0; i += NT) {
                 const uint32_t r = R[i];
@@ -238,70 +239,66 @@ __device__ __forceinline__ void bpe_row(
                     }
                     m = ((chain | chain_r) & 1u) == 0;
                 }
-                if (m) { F[i] = 1; mine = true; }
+                if (m) Q[atomicAdd(qn, 1u)] = (IT)i;
             }
         }
         team_sync<NT>();
+        const int nm = (int)*qn;                   // merges of this round (they do not overlap)
 
-        // apply: position i absorbs its right neighbour j
-        if (mine) {
-            for (int i = tid; i < n0; i += NT) {
-                if (!F[i]) continue;
-                const IT j = NX[i];
-                const IT k = NX[j];
-                S[i] = NS[i];
-                S[j] = (uint16_t)kNone;
-                R[j] = (uint16_t)kNone;
-                NX[i] = k;
-                if (k != NIL) PV[k] = (IT)i;
-                D[(int)j % NT] = 1;           // j's owner must refresh its cached minimum
-            }
+        // apply: position i absorbs its right neighbour j; one merge per thread and pass
+        for (int m = tid; m < nm; m += NT) {
+            const IT i = Q[m];
+            const IT j = NX[i];
+            const IT k = NX[j];
+            S[i] = NS[i];
+            S[j] = (uint16_t)kNone;
+            R[j] = (uint16_t)kNone;
+            NX[i] = k;
+            if (k != NIL) PV[k] = i;
+            D[(int)(j % NT)] = 1;             // j's owner must refresh its cached minimum
         }
         team_sync<NT>();
 
-        // re-rank the two pairs around every new symbol; the probes of four positions (eight
-        // table reads) are in flight together
-        if (mine) {
-            for (int i0 = tid; i0 < n0; i0 += 4 * NT) {
-                uint4 e0[4], e1[4];
-                uint32_t h0[4], h1[4], s[4], sk[4], sp[4];
-                IT kk[4], pp[4];
-                bool on[4];
+        // re-rank the two pairs around every new symbol: probe 2m is the pair (new, right
+        // neighbour), probe 2m + 1 the pair (left neighbour, new).  The probes are dealt evenly to
+        // the threads, four table reads in flight per thread.
+        for (int p0 = tid; p0 < 2 * nm; p0 += 4 * NT) {
+            uint4 e[4];
+            uint32_t h[4], sa[4], sb[4];
+            IT target[4];
+            bool valid[4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int i = i0 + j * NT;
-                    on[j] = i < n0 && F[i];
-                    kk[j] = NIL; pp[j] = NIL; s[j] = 0; sk[j] = 0; sp[j] = 0;
-                    if (on[j]) {
-                        F[i] = 0;
-                        kk[j] = NX[i];
-                        pp[j] = PV[i];
-                        s[j] = S[i];
-                        if (kk[j] != NIL) sk[j] = S[kk[j]];
-                        if (pp[j] != NIL) sp[j] = S[pp[j]];
-                    }
-                    e0[j] = pair_probe(tab, tab_shift, s[j], sk[j], &h0[j]);
-                    e1[j] = pair_probe(tab, tab_shift, sp[j], s[j], &h1[j]);
-                }
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    if (!on[j]) continue;
-                    const int i = i0 + j * NT;
-                    PairInfo right{kNone, kNone, kNone};
-                    if (kk[j] != NIL) right = pair_finish(tab, tab_mask, s[j], sk[j], e0[j], h0[j]);
-                    R[i] = (uint16_t)right.rank; NS[i] = (uint16_t)right.product; MC[i] = (uint16_t)right.gate;
-                    if (pp[j] != NIL) {
-                        const PairInfo left = pair_finish(tab, tab_mask, sp[j], s[j], e1[j], h1[j]);
-                        const int p = (int)pp[j];
-                        R[p] = (uint16_t)left.rank; NS[p] = (uint16_t)left.product; MC[p] = (uint16_t)left.gate;
-                        D[p % NT] = 1;
+            for (int j = 0; j < 4; ++j) {
+                const int p = p0 + j * NT;
+                sa[j] = 0; sb[j] = 0; target[j] = NIL; valid[j] = false;
+                if (p < 2 * nm) {
+                    const IT i = Q[p >> 1];
+                    if (p & 1) {
+                        const IT pp = PV[i];
+                        target[j] = pp;
+                        if (pp != NIL) { sa[j] = S[pp]; sb[j] = S[i]; valid[j] = true; }
+                    } else {
+                        const IT kk = NX[i];
+                        target[j] = i;
+                        if (kk != NIL) { sa[j] = S[i]; sb[j] = S[kk]; valid[j] = true; }
                     }
                 }
+                e[j] = pair_probe(tab, tab_shift, sa[j], sb[j], &h[j]);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (target[j] == NIL) continue;       // no probe, or no left neighbour
+                PairInfo pi{kNone, kNone, kNone};
+                if (valid[j]) pi = pair_finish(tab, tab_mask, sa[j], sb[j], e[j], h[j]);
+                const int q = (int)target[j];
+                R[q] = (uint16_t)pi.rank; NS[q] = (uint16_t)pi.product; MC[q] = (uint16_t)pi.gate;
+                D[q % NT] = 1;
             }
         }
         team_sync<NT>();
+        if (tid == 0) *qn = 0;                     // seen by the next round's decide (a sync lies between)
 
-        if (mine || D[tid]) {
+        if (D[tid]) {
             D[tid] = 0;
             cmin = kEmptyKey; cgate = kEmptyKey;
             for (int i = tid; i < n0; i += NT) {
@@ -371,7 +368,7 @@ struct BpePlan {                          // device arrays inside the scratch bu
 static size_t long_slab_bytes(int64_t max_len)
 {
     const size_t n = ((size_t)max_len + 7) & ~(size_t)7;
-    return ((n * 17) + 255) & ~(size_t)255;
+    return ((n * 18) + 255) & ~(size_t)255;
 }
 
 // chunk geometry: DNATOK_BPE_CHUNK="core,overlap" overrides the default (for experiments)
@@ -489,14 +486,14 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     for (int i = threadIdx.x; i < 256; i += NT * TEAMS) b2s[i] = a.byte_to_sym[i];
     const int team = threadIdx.x / NT, tid = threadIdx.x % NT;
     int32_t *next_item = reinterpret_cast<int32_t *>(sp) + team; sp += 16 * sizeof(int32_t);
-    uint32_t *red = reinterpret_cast<uint32_t *>(sp) + team * (4 * (NT / 64)); sp += TEAMS * 4 * (NT / 64) * 4;
+    uint32_t *red = reinterpret_cast<uint32_t *>(sp) + team * (4 * (NT / 64) + 4); sp += TEAMS * (4 * (NT / 64) + 4) * 4;
     uint16_t *S = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
     uint16_t *R = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
     uint16_t *NS = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
     uint16_t *MC = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
     uint16_t *NX = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
     uint16_t *PV = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
-    uint8_t *F = sp + (size_t)team * CAP; sp += (size_t)TEAMS * CAP;
+    uint16_t *Q = reinterpret_cast<uint16_t *>(sp) + (size_t)team * (CAP / 2); sp += (size_t)TEAMS * CAP;
     uint8_t *D = sp + (size_t)team * NT;
     __syncthreads();
 
@@ -521,14 +518,14 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
             if (tid == 0) lengths[row] = len > CAP ? -1 : 0;
         } else if (nc == 1) {
             bpe_row<NT, uint16_t>(tab, mask, a.shift, b2s, a.out_remap, bytes + start, (int)len, S, R, NS, MC,
-                                  NX, PV, F, D, red, tid, tok_tmp + start, lengths + row);
+                                  NX, PV, Q, D, red, tid, tok_tmp + start, lengths + row);
         } else {
             const int64_t e0 = (int64_t)k * p.core - p.overlap < 0 ? 0 : (int64_t)k * p.core - p.overlap;
             int64_t e1 = (int64_t)(k + 1) * p.core + p.overlap;
             if (e1 > len) e1 = len;
             uint16_t *raw = p.chunk_sym + (size_t)(p.mc_off[row] + k) * p.ext;
             bpe_row<NT, uint16_t>(tab, mask, a.shift, b2s, a.out_remap, bytes + start + e0, (int)(e1 - e0),
-                                  S, R, NS, MC, NX, PV, F, D, red, tid, nullptr, nullptr, raw);
+                                  S, R, NS, MC, NX, PV, Q, D, red, tid, nullptr, nullptr, raw);
         }
         team_sync<NT>();
     }
@@ -615,7 +612,7 @@ __global__ __launch_bounds__(NT) void bpe_long_kernel(
     int64_t n_rows, int64_t max_len, BpePlan p, int32_t *__restrict__ tok_tmp,
     int32_t *__restrict__ lengths)
 {
-    __shared__ uint32_t red[4 * (NT / 64)];
+    __shared__ uint32_t red[4 * (NT / 64) + 4];
     __shared__ uint8_t D[NT];
     __shared__ uint16_t b2s[256];
     for (int i = threadIdx.x; i < 256; i += NT) b2s[i] = a.byte_to_sym[i];
@@ -638,9 +635,9 @@ __global__ __launch_bounds__(NT) void bpe_long_kernel(
         uint16_t *R = S + n;
         uint16_t *NS = R + n;
         uint16_t *MC = NS + n;
-        uint8_t *F = reinterpret_cast<uint8_t *>(MC + n);
+        uint32_t *Q = reinterpret_cast<uint32_t *>(MC + n);      // n / 2 entries
         bpe_row<NT, uint32_t>(a.tab, mask, a.shift, b2s, a.out_remap, bytes + start, (int)len, S, R, NS, MC,
-                              NX, PV, F, D, red, threadIdx.x, tok_tmp + start, lengths + row);
+                              NX, PV, Q, D, red, threadIdx.x, tok_tmp + start, lengths + row);
         __syncthreads();
     }
 }
@@ -665,7 +662,9 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
         DNATOK_REQUIRE(byte_to_id_h[i] >= 0 && byte_to_id_h[i] < n_symbols, DNATOK_E_INVALID,
                        "dnatok_bpe_table_create: byte_to_id[%d] out of range", i);
     uint32_t slots = 64, shift = 26;
-    while (slots < (uint32_t)n_merges * 2u + 2u) { slots <<= 1; --shift; }
+    // 8 slots per rule: a pair that has no rule (most probes in the later rounds) is then
+    // answered by its first probe nearly always, and a wave's probe is as slow as its slowest lane
+    while (slots < (uint32_t)n_merges * 8u + 2u) { slots <<= 1; --shift; }
     std::vector<uint4> tab(slots, uint4{kEmptyKey, kNone, 0, 0});
     std::vector<uint32_t> slot_of(n_merges > 0 ? n_merges : 1, 0xFFFFFFFFu);
     std::vector<uint32_t> first_use(n_symbols, 0xFFFFFFFFu);   // lowest rank using a symbol
@@ -744,7 +743,7 @@ template <int NT, int TEAMS, int CAP>
 int launch_lds(const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets, const BpePlan &p,
                int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
 {
-    const size_t lds = 512 + 64 + (size_t)TEAMS * 4 * (NT / 64) * 4 + (size_t)TEAMS * CAP * 13 + (size_t)TEAMS * NT + 64;
+    const size_t lds = 512 + 64 + (size_t)TEAMS * (4 * (NT / 64) + 4) * 4 + (size_t)TEAMS * CAP * 13 + (size_t)TEAMS * NT + 64;
     auto kern = bpe_lds_kernel<NT, TEAMS, CAP>;
     static bool attr_set = false;
     if (!attr_set) {
