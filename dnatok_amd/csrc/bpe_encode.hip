@@ -138,33 +138,35 @@ __device__ __forceinline__ uint32_t team_exclusive_sum(uint32_t v, uint32_t *red
     return carry + inc - v;
 }
 
-// One row.  tid = index in the team; S/R/NS/MC/NX/PV hold n0 entries, Q (the merges of the
-// current round) n0 / 2; D holds NT bytes; red holds 4 * (NT / 64) + 4 words.  Tokens go to
-// out[0 .. *out_len).
+// What the engine keeps per position, in one record so that a step along a chain of candidates
+// is one read: rank of the pair the position starts (kNone = no rule / dead), right and left
+// live neighbour, symbol.  8 bytes with 16-bit links (LDS kernels), 16 bytes with 32-bit links
+// (whole-row kernel, state in global memory).
+template <typename IT>
+struct alignas(4 * sizeof(IT)) PosRec {
+    IT r, nx, pv, s;
+};
+
+// One row.  tid = index in the team; P/NS/MC hold n0 entries, Q (the merges of the current round)
+// n0 / 2; D holds NT bytes; red holds 4 * (NT / 64) + 4 words.  Tokens go to out[0 .. *out_len).
 template <int NT, typename IT>
 __device__ __forceinline__ void bpe_row(
     const uint4 *tab, uint32_t tab_mask, uint32_t tab_shift, const uint16_t *byte_to_sym,
-    const int32_t *out_remap, const uint8_t *__restrict__ src, const int n0, uint16_t *S, uint16_t *R,
-    uint16_t *NS, uint16_t *MC, IT *NX, IT *PV, IT *Q, uint8_t *D, uint32_t *red, const int tid,
+    const int32_t *out_remap, const uint8_t *__restrict__ src, const int n0, PosRec<IT> *P,
+    uint16_t *NS, uint16_t *MC, IT *Q, uint8_t *D, uint32_t *red, const int tid,
     int32_t *__restrict__ out, int32_t *__restrict__ out_len, uint16_t *__restrict__ raw_out = nullptr)
 {
     constexpr IT NIL = (IT)~(IT)0;
+    constexpr IT DEAD = (IT)kNone;
     const int wv = (NT == 64) ? 0 : (tid >> 6);
     uint32_t *qn = red + 4 * (NT / 64);        // number of merges queued in the current round
     // position i belongs to thread i % NT: in every pass the lanes of a wave touch consecutive
     // positions, so the LDS state arrays are read and written without bank conflicts
 
-    for (int i = tid; i < n0; i += NT) {
-        S[i] = byte_to_sym[src[i]];
-        NX[i] = (i + 1 < n0) ? (IT)(i + 1) : NIL;
-        PV[i] = (i > 0) ? (IT)(i - 1) : NIL;
-    }
+    // symbols, links and the initial pair of every position, four table probes in flight at a time
+    uint32_t cmin = kEmptyKey, cgate = kEmptyKey;
     D[tid] = 0;
     if (tid == 0) *qn = 0;
-    team_sync<NT>();
-
-    // initial pair of every position, four table probes in flight at a time
-    uint32_t cmin = kEmptyKey, cgate = kEmptyKey;
     for (int i0 = tid; i0 < n0; i0 += 4 * NT) {
         uint4 e[4];
         uint32_t h[4], sa[4], sb[4];
@@ -172,9 +174,9 @@ __device__ __forceinline__ void bpe_row(
         for (int j = 0; j < 4; ++j) {
             const int i = i0 + j * NT;
             const bool ok = i + 1 < n0;
-            sa[j] = ok ? S[i] : 0u;
-            sb[j] = ok ? S[i + 1] : 0u;
-            e[j] = pair_probe(tab, tab_shift, sa[j], sb[j], &h[j]);
+            sa[j] = i < n0 ? byte_to_sym[src[i]] : 0u;
+            sb[j] = ok ? byte_to_sym[src[i + 1]] : 0u;
+            e[j] = pair_probe(tab, tab_shift, ok ? sa[j] : 0u, sb[j], &h[j]);
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -182,7 +184,13 @@ __device__ __forceinline__ void bpe_row(
             if (i >= n0) continue;
             PairInfo pi{kNone, kNone, kNone};
             if (i + 1 < n0) pi = pair_finish(tab, tab_mask, sa[j], sb[j], e[j], h[j]);
-            R[i] = (uint16_t)pi.rank; NS[i] = (uint16_t)pi.product; MC[i] = (uint16_t)pi.gate;
+            PosRec<IT> x;
+            x.r = (IT)pi.rank;
+            x.nx = (i + 1 < n0) ? (IT)(i + 1) : NIL;
+            x.pv = (i > 0) ? (IT)(i - 1) : NIL;
+            x.s = (IT)sa[j];
+            P[i] = x;
+            NS[i] = (uint16_t)pi.product; MC[i] = (uint16_t)pi.gate;
             if (pi.rank != kNone) { cmin = umin(cmin, pi.rank); cgate = umin(cgate, pi.gate); }
         }
     }
@@ -193,7 +201,7 @@ __device__ __forceinline__ void bpe_row(
     for (;;) {
         if (--budget < 0) { stuck = true; break; }   // cannot happen; keeps the loop bounded
         uint32_t rmin, gate;
-        team_min2<NT>(cmin, cgate, red + flip * (NT / 64) * 2, wv, rmin, gate);
+        team_min2<NT>(cmin, cgate, red + flip * (NT / 64) * 2, wv, rmin, gate);   // (syncs the team)
         flip ^= 1;
         if (rmin >= kNone) break;
         const bool single = gate <= rmin;          // non-monotone table: one merge this round
@@ -202,7 +210,7 @@ __device__ __forceinline__ void bpe_row(
             uint32_t mypos = kEmptyKey;
             if (cmin == rmin)
                 for (int i = tid; i < n0; i += NT)
-                    if (R[i] == rmin) { mypos = (uint32_t)i; break; }
+                    if (P[i].r == rmin) { mypos = (uint32_t)i; break; }
             uint32_t dummy;
             team_min2<NT>(mypos, mypos, red + flip * (NT / 64) * 2, wv, leftmost, dummy);
             flip ^= 1;
@@ -212,30 +220,27 @@ __device__ __forceinline__ void bpe_row(
         // decide (reads only); a pair that merges is put on the round's queue
         if (cmin < limit) {
             for (int i = tid; i < n0; i += NT) {
-                const uint32_t r = R[i];
+                const PosRec<IT> x = P[i];
+                const uint32_t r = x.r;
                 if (r >= limit) continue;
                 bool m;
                 if (single) {
                     m = ((uint32_t)i == leftmost);
                 } else {
-                    uint32_t chain = 0;
-                    IT p = (IT)i;
-                    uint32_t rp = r;
-                    for (;;) {                       // candidates to the left with key <= ours
-                        const IT q = PV[p];
-                        if (q == NIL) break;
-                        const uint32_t rq = R[q];
-                        if (rq > rp) break;
-                        ++chain; p = q; rp = rq;
+                    // both neighbours' records are requested together
+                    PosRec<IT> yl = P[x.pv != NIL ? x.pv : (IT)i];
+                    PosRec<IT> yr = P[x.nx != NIL ? x.nx : (IT)i];
+                    uint32_t chain = 0, rp = r;
+                    IT q = x.pv;
+                    while (q != NIL && yl.r <= rp) {      // candidates to the left with key <= ours
+                        ++chain; rp = yl.r; q = yl.pv;
+                        if (q != NIL) yl = P[q];
                     }
                     uint32_t chain_r = 0;
-                    p = (IT)i; rp = r;
-                    for (;;) {                       // candidates to the right with key < ours
-                        const IT q = NX[p];
-                        if (q == NIL) break;
-                        const uint32_t rq = R[q];
-                        if (rq >= rp) break;
-                        ++chain_r; p = q; rp = rq;
+                    rp = r; q = x.nx;
+                    while (q != NIL && yr.r < rp) {       // candidates to the right with key < ours
+                        ++chain_r; rp = yr.r; q = yr.nx;
+                        if (q != NIL) yr = P[q];
                     }
                     m = ((chain | chain_r) & 1u) == 0;
                 }
@@ -248,13 +253,13 @@ __device__ __forceinline__ void bpe_row(
         // apply: position i absorbs its right neighbour j; one merge per thread and pass
         for (int m = tid; m < nm; m += NT) {
             const IT i = Q[m];
-            const IT j = NX[i];
-            const IT k = NX[j];
-            S[i] = NS[i];
-            S[j] = (uint16_t)kNone;
-            R[j] = (uint16_t)kNone;
-            NX[i] = k;
-            if (k != NIL) PV[k] = i;
+            const IT j = P[i].nx;
+            const IT k = P[j].nx;
+            P[i].s = (IT)NS[i];
+            P[i].nx = k;
+            P[j].s = DEAD;
+            P[j].r = DEAD;
+            if (k != NIL) P[k].pv = i;
             D[(int)(j % NT)] = 1;             // j's owner must refresh its cached minimum
         }
         team_sync<NT>();
@@ -273,14 +278,13 @@ __device__ __forceinline__ void bpe_row(
                 sa[j] = 0; sb[j] = 0; target[j] = NIL; valid[j] = false;
                 if (p < 2 * nm) {
                     const IT i = Q[p >> 1];
+                    const PosRec<IT> x = P[i];
                     if (p & 1) {
-                        const IT pp = PV[i];
-                        target[j] = pp;
-                        if (pp != NIL) { sa[j] = S[pp]; sb[j] = S[i]; valid[j] = true; }
+                        target[j] = x.pv;
+                        if (x.pv != NIL) { sa[j] = P[x.pv].s; sb[j] = x.s; valid[j] = true; }
                     } else {
-                        const IT kk = NX[i];
                         target[j] = i;
-                        if (kk != NIL) { sa[j] = S[i]; sb[j] = S[kk]; valid[j] = true; }
+                        if (x.nx != NIL) { sa[j] = x.s; sb[j] = P[x.nx].s; valid[j] = true; }
                     }
                 }
                 e[j] = pair_probe(tab, tab_shift, sa[j], sb[j], &h[j]);
@@ -291,7 +295,7 @@ __device__ __forceinline__ void bpe_row(
                 PairInfo pi{kNone, kNone, kNone};
                 if (valid[j]) pi = pair_finish(tab, tab_mask, sa[j], sb[j], e[j], h[j]);
                 const int q = (int)target[j];
-                R[q] = (uint16_t)pi.rank; NS[q] = (uint16_t)pi.product; MC[q] = (uint16_t)pi.gate;
+                P[q].r = (IT)pi.rank; NS[q] = (uint16_t)pi.product; MC[q] = (uint16_t)pi.gate;
                 D[q % NT] = 1;
             }
         }
@@ -302,7 +306,7 @@ __device__ __forceinline__ void bpe_row(
             D[tid] = 0;
             cmin = kEmptyKey; cgate = kEmptyKey;
             for (int i = tid; i < n0; i += NT) {
-                const uint32_t r = R[i];
+                const uint32_t r = P[i].r;
                 if (r != kNone) { cmin = umin(cmin, r); cgate = umin(cgate, MC[i]); }
             }
         }
@@ -311,7 +315,7 @@ __device__ __forceinline__ void bpe_row(
     if (raw_out) {
         // chunk of a long row: hand back the symbol at every start position (kNone elsewhere);
         // the seam and gather kernels assemble the row
-        for (int i = tid; i < n0; i += NT) raw_out[i] = stuck ? (uint16_t)kNone : S[i];
+        for (int i = tid; i < n0; i += NT) raw_out[i] = stuck ? (uint16_t)kNone : (uint16_t)P[i].s;
         return;
     }
     // compact the live symbols to the output: contiguous chunks per thread, once per row
@@ -319,12 +323,12 @@ __device__ __forceinline__ void bpe_row(
     const int lo = (tid * c < n0) ? tid * c : n0;
     const int hi = (lo + c < n0) ? lo + c : n0;
     uint32_t live = 0;
-    for (int i = lo; i < hi; ++i) live += (S[i] != kNone);
+    for (int i = lo; i < hi; ++i) live += ((uint32_t)P[i].s != kNone);
     uint32_t total;
     uint32_t off = team_exclusive_sum<NT>(live, red, wv, total);
     for (int i = lo; i < hi; ++i) {
-        const uint32_t s = S[i];
-        if (s != kNone) out[off++] = out_remap ? out_remap[s] : (int32_t)s;
+        const uint32_t sy = P[i].s;
+        if (sy != kNone) out[off++] = out_remap ? out_remap[sy] : (int32_t)sy;
     }
     if (tid == 0) *out_len = stuck ? -2 : (int32_t)total;
 }
@@ -368,7 +372,7 @@ struct BpePlan {                          // device arrays inside the scratch bu
 static size_t long_slab_bytes(int64_t max_len)
 {
     const size_t n = ((size_t)max_len + 7) & ~(size_t)7;
-    return ((n * 18) + 255) & ~(size_t)255;
+    return ((n * 22) + 255) & ~(size_t)255;     // 16 (records) + 2 + 2 (product, gate) + 2 (queue)
 }
 
 // chunk geometry: DNATOK_BPE_CHUNK="core,overlap" overrides the default (for experiments)
@@ -487,12 +491,9 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     const int team = threadIdx.x / NT, tid = threadIdx.x % NT;
     int32_t *next_item = reinterpret_cast<int32_t *>(sp) + team; sp += 16 * sizeof(int32_t);
     uint32_t *red = reinterpret_cast<uint32_t *>(sp) + team * (4 * (NT / 64) + 4); sp += TEAMS * (4 * (NT / 64) + 4) * 4;
-    uint16_t *S = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
-    uint16_t *R = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
+    PosRec<uint16_t> *P = reinterpret_cast<PosRec<uint16_t> *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 8;
     uint16_t *NS = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
     uint16_t *MC = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
-    uint16_t *NX = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
-    uint16_t *PV = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
     uint16_t *Q = reinterpret_cast<uint16_t *>(sp) + (size_t)team * (CAP / 2); sp += (size_t)TEAMS * CAP;
     uint8_t *D = sp + (size_t)team * NT;
     __syncthreads();
@@ -517,15 +518,15 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
             // too long: left to the whole-row kernel (row_fail is set); empty: no tokens
             if (tid == 0) lengths[row] = len > CAP ? -1 : 0;
         } else if (nc == 1) {
-            bpe_row<NT, uint16_t>(tab, mask, a.shift, b2s, a.out_remap, bytes + start, (int)len, S, R, NS, MC,
-                                  NX, PV, Q, D, red, tid, tok_tmp + start, lengths + row);
+            bpe_row<NT, uint16_t>(tab, mask, a.shift, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC,
+                                  Q, D, red, tid, tok_tmp + start, lengths + row);
         } else {
             const int64_t e0 = (int64_t)k * p.core - p.overlap < 0 ? 0 : (int64_t)k * p.core - p.overlap;
             int64_t e1 = (int64_t)(k + 1) * p.core + p.overlap;
             if (e1 > len) e1 = len;
             uint16_t *raw = p.chunk_sym + (size_t)(p.mc_off[row] + k) * p.ext;
             bpe_row<NT, uint16_t>(tab, mask, a.shift, b2s, a.out_remap, bytes + start + e0, (int)(e1 - e0),
-                                  S, R, NS, MC, NX, PV, Q, D, red, tid, nullptr, nullptr, raw);
+                                  P, NS, MC, Q, D, red, tid, nullptr, nullptr, raw);
         }
         team_sync<NT>();
     }
@@ -605,7 +606,7 @@ __global__ __launch_bounds__(1024) void bpe_gather_kernel(
 }
 
 // Whole-row kernel for rows above the LDS capacity that could not be chunked: one workgroup per
-// row, state in global scratch (17 bytes / base).
+// row, state in global scratch (22 bytes / base).
 template <int NT>
 __global__ __launch_bounds__(NT) void bpe_long_kernel(
     BpeArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
@@ -629,15 +630,12 @@ __global__ __launch_bounds__(NT) void bpe_long_kernel(
             continue;
         }
         const size_t n = ((size_t)len + 7) & ~(size_t)7;
-        uint32_t *NX = reinterpret_cast<uint32_t *>(slab);
-        uint32_t *PV = NX + n;
-        uint16_t *S = reinterpret_cast<uint16_t *>(PV + n);
-        uint16_t *R = S + n;
-        uint16_t *NS = R + n;
+        PosRec<uint32_t> *P = reinterpret_cast<PosRec<uint32_t> *>(slab);
+        uint16_t *NS = reinterpret_cast<uint16_t *>(P + n);
         uint16_t *MC = NS + n;
         uint32_t *Q = reinterpret_cast<uint32_t *>(MC + n);      // n / 2 entries
-        bpe_row<NT, uint32_t>(a.tab, mask, a.shift, b2s, a.out_remap, bytes + start, (int)len, S, R, NS, MC,
-                              NX, PV, Q, D, red, threadIdx.x, tok_tmp + start, lengths + row);
+        bpe_row<NT, uint32_t>(a.tab, mask, a.shift, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC,
+                              Q, D, red, threadIdx.x, tok_tmp + start, lengths + row);
         __syncthreads();
     }
 }
