@@ -361,6 +361,7 @@ struct BpePlan {                          // device arrays inside the scratch bu
     int32_t *item_row;    // [max_items]
     int32_t *mc_row;      // [max_mc]
     int32_t *seam;        // [max_mc] seam to the right of a chunk (row position), -1 = none found
+    int32_t *cnt;         // [max_mc] tokens of a chunk between the seams on its two sides
     int32_t *row_fail;    // [n_rows] 1 = redo the row with the whole-row kernel
     uint16_t *chunk_sym;  // [max_mc][ext]
     uint8_t *slabs;       // whole-row fallback state
@@ -406,6 +407,7 @@ static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t
     const size_t o_item_row = take(4 * (size_t)p.max_items);
     const size_t o_mc_row = take(4 * (size_t)p.max_mc);
     const size_t o_seam = take(4 * (size_t)p.max_mc);
+    const size_t o_cnt = take(4 * (size_t)p.max_mc);
     const size_t o_fail = take(4 * (size_t)n_rows);
     const size_t o_sym = take(2 * (size_t)p.ext * (size_t)p.max_mc);
     p.slab_bytes = chunks ? long_slab_bytes(max_len) : 0;
@@ -419,6 +421,7 @@ static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t
         p.item_row = (int32_t *)(base + o_item_row);
         p.mc_row = (int32_t *)(base + o_mc_row);
         p.seam = (int32_t *)(base + o_seam);
+        p.cnt = (int32_t *)(base + o_cnt);
         p.row_fail = (int32_t *)(base + o_fail);
         p.chunk_sym = (uint16_t *)(base + o_sym);
         p.slabs = base + o_slabs;
@@ -569,39 +572,74 @@ __global__ __launch_bounds__(256) void bpe_seam_kernel(const int64_t *__restrict
     }
 }
 
-// One workgroup per multi-chunk row: tokens of chunk k between seam k-1 and seam k, compacted.
-__global__ __launch_bounds__(1024) void bpe_gather_kernel(
-    BpeArgs a, const int64_t *__restrict__ offsets, int64_t n_rows, BpePlan p,
-    int32_t *__restrict__ tok_tmp, int32_t *__restrict__ lengths)
+// The part of a row that chunk k contributes: from the seam on its left to the seam on its right.
+struct ChunkSpan {
+    int32_t row, k, nc;
+    int64_t lo, hi, e0;       // owned row positions [lo, hi); e0 = row position of the chunk's first symbol
+};
+
+__device__ __forceinline__ ChunkSpan chunk_span(const int64_t *offsets, const BpePlan &p, int32_t m)
 {
-    __shared__ uint32_t red[16];
+    ChunkSpan c;
+    c.row = p.mc_row[m];
+    c.k = m - p.mc_off[c.row];
+    c.nc = p.mc_off[c.row + 1] - p.mc_off[c.row];
+    const int64_t len = offsets[c.row + 1] - offsets[c.row];
+    c.e0 = (int64_t)c.k * p.core - p.overlap < 0 ? 0 : (int64_t)c.k * p.core - p.overlap;
+    c.lo = c.k > 0 ? p.seam[m - 1] : 0;
+    c.hi = c.k + 1 < c.nc ? p.seam[m] : len;
+    return c;
+}
+
+// One workgroup per chunk of a multi-chunk row: how many tokens it contributes.
+__global__ __launch_bounds__(256) void bpe_count_kernel(const int64_t *__restrict__ offsets, BpePlan p)
+{
+    __shared__ uint32_t red[8];
+    const int32_t n_mc = p.counts[1];
+    for (int32_t m = blockIdx.x; m < n_mc; m += gridDim.x) {
+        const ChunkSpan c = chunk_span(offsets, p, m);
+        if (p.row_fail[c.row]) continue;                 // (the same for the whole workgroup)
+        const uint16_t *sym = p.chunk_sym + (size_t)m * p.ext;
+        uint32_t live = 0;
+        for (int64_t i = c.lo + threadIdx.x; i < c.hi; i += 256) live += sym[i - c.e0] != kNone;
+        uint32_t total;
+        (void)team_exclusive_sum<256>(live, red, threadIdx.x >> 6, total);
+        if (threadIdx.x == 0) p.cnt[m] = (int32_t)total;
+    }
+}
+
+// One workgroup per chunk: its tokens, compacted, behind those of the row's earlier chunks.
+__global__ __launch_bounds__(256) void bpe_gather_kernel(
+    BpeArgs a, const int64_t *__restrict__ offsets, BpePlan p, int32_t *__restrict__ tok_tmp,
+    int32_t *__restrict__ lengths)
+{
+    __shared__ uint32_t red[8];
     const int wv = threadIdx.x >> 6;
-    for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
-        const int32_t nc = p.mc_off[row + 1] - p.mc_off[row];
-        if (nc <= 1 || p.row_fail[row]) continue;
-        const int32_t m0 = p.mc_off[row];
-        const int64_t start = offsets[row];
-        const int64_t len = offsets[row + 1] - start;
-        int32_t *out = tok_tmp + start;
-        int64_t written = 0;
-        for (int64_t base = 0; base < len; base += 1024) {
-            const int64_t i = base + threadIdx.x;
-            uint32_t sym = kNone;
-            if (i < len) {
-                int32_t k = (int32_t)(i / p.core);
-                if (k >= nc) k = nc - 1;
-                if (k > 0 && i < p.seam[m0 + k - 1]) --k;            // still left of the seam before chunk k
-                else if (k + 1 < nc && i >= p.seam[m0 + k]) ++k;     // already right of the seam after chunk k
-                const int64_t e0 = (int64_t)k * p.core - p.overlap < 0 ? 0 : (int64_t)k * p.core - p.overlap;
-                sym = p.chunk_sym[(size_t)(m0 + k) * p.ext + (i - e0)];
-            }
-            const uint32_t live = sym != kNone;
-            uint32_t total;
-            const uint32_t off = team_exclusive_sum<1024>(live, red, wv, total);
-            if (live) out[written + off] = a.out_remap ? a.out_remap[sym] : (int32_t)sym;
-            written += total;
+    const int32_t n_mc = p.counts[1];
+    for (int32_t m = blockIdx.x; m < n_mc; m += gridDim.x) {
+        const ChunkSpan c = chunk_span(offsets, p, m);
+        if (p.row_fail[c.row]) continue;
+        // tokens of the row's chunks before this one
+        uint32_t before = 0;
+        for (int32_t j = threadIdx.x; j < c.k; j += 256) before += (uint32_t)p.cnt[m - c.k + j];
+        uint32_t base;
+        (void)team_exclusive_sum<256>(before, red, wv, base);
+        // this chunk: a contiguous piece of the span per thread, in position order
+        const uint16_t *sym = p.chunk_sym + (size_t)m * p.ext;
+        const int64_t n = c.hi - c.lo;
+        const int64_t per = (n + 255) / 256;
+        const int64_t t0 = c.lo + (int64_t)threadIdx.x * per < c.hi ? c.lo + (int64_t)threadIdx.x * per : c.hi;
+        const int64_t t1 = t0 + per < c.hi ? t0 + per : c.hi;
+        uint32_t live = 0;
+        for (int64_t i = t0; i < t1; ++i) live += sym[i - c.e0] != kNone;
+        uint32_t total;
+        uint32_t off = base + team_exclusive_sum<256>(live, red, wv, total);
+        int32_t *out = tok_tmp + offsets[c.row];
+        for (int64_t i = t0; i < t1; ++i) {
+            const uint32_t sy = sym[i - c.e0];
+            if (sy != kNone) out[off++] = a.out_remap ? a.out_remap[sy] : (int32_t)sy;
         }
-        if (threadIdx.x == 0) lengths[row] = (int32_t)written;
+        if (threadIdx.x == 0 && c.k + 1 == c.nc) lengths[c.row] = (int32_t)(base + total);
     }
 }
 
@@ -804,8 +842,9 @@ extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, co
             int64_t g = p.max_mc < 4096 ? p.max_mc : 4096;
             bpe_seam_kernel<<<(int)(g < 1 ? 1 : g), 256, 0, s>>>(offsets, p);
             DNATOK_HIP_TRY(hipGetLastError());
-            int64_t gr = n_rows < 1024 ? n_rows : 1024;
-            bpe_gather_kernel<<<(int)gr, 1024, 0, s>>>(a, offsets, n_rows, p, tok_tmp, lengths);
+            bpe_count_kernel<<<(int)(g < 1 ? 1 : g), 256, 0, s>>>(offsets, p);
+            DNATOK_HIP_TRY(hipGetLastError());
+            bpe_gather_kernel<<<(int)(g < 1 ? 1 : g), 256, 0, s>>>(a, offsets, p, tok_tmp, lengths);
             DNATOK_HIP_TRY(hipGetLastError());
         }
         const int64_t slabs = n_rows < kLongGrid ? n_rows : kLongGrid;

@@ -51,63 +51,81 @@ __global__ __launch_bounds__(kScanThreads) void scan_lengths_kernel(
     if (threadIdx.x == 0) out_offsets[n_rows] = carry;
 }
 
+constexpr int kPackTile = 4096;          // output cells one workgroup copies
+
+// Packed layout.  A workgroup takes kPackTile consecutive cells of the packed output, finds the
+// first row that reaches into them (binary search in out_offsets) and copies row piece after
+// row piece, so that the work per workgroup is the same whether the batch is 4096 short rows
+// or a few very long ones.
 __global__ __launch_bounds__(256) void pack_copy_kernel(
-    const int32_t *__restrict__ tok_tmp, const int64_t *__restrict__ in_offsets,
-    const int32_t *__restrict__ lengths, int64_t n_rows, const int32_t *__restrict__ remap,
-    const int64_t *__restrict__ out_offsets, int32_t *__restrict__ ids_out,
-    uint8_t *__restrict__ mask_out)
+    const int32_t *__restrict__ tok_tmp, const int64_t *__restrict__ in_offsets, int64_t n_rows,
+    const int32_t *__restrict__ remap, const int64_t *__restrict__ out_offsets,
+    int32_t *__restrict__ ids_out, uint8_t *__restrict__ mask_out)
 {
-    const int lane = threadIdx.x & 63;
-    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int64_t n_waves = (int64_t)gridDim.x * 4;
-    for (int64_t row = wave; row < n_rows; row += n_waves) {
-        const int64_t len = lengths[row];
-        const int32_t *src = tok_tmp + in_offsets[row];
-        const int64_t o = out_offsets[row];
-        for (int64_t j = lane; j < len; j += 64) {
-            int32_t v = src[j];
-            if (remap) v = remap[v];
-            ids_out[o + j] = v;
-            if (mask_out) mask_out[o + j] = 1;
+    const int64_t total = out_offsets[n_rows];
+    for (int64_t o0 = (int64_t)blockIdx.x * kPackTile; o0 < total; o0 += (int64_t)gridDim.x * kPackTile) {
+        const int64_t o1 = o0 + kPackTile < total ? o0 + kPackTile : total;
+        // last row with out_offsets[row] <= o0 (every thread does the same 20-odd steps)
+        int64_t lo = 0, hi = n_rows;
+        while (hi - lo > 1) {
+            const int64_t mid = (lo + hi) >> 1;
+            if (out_offsets[mid] <= o0) lo = mid; else hi = mid;
+        }
+        for (int64_t row = lo; row < n_rows; ++row) {
+            const int64_t r0 = out_offsets[row], r1 = out_offsets[row + 1];
+            if (r0 >= o1) break;
+            const int64_t c0 = r0 > o0 ? r0 : o0, c1 = r1 < o1 ? r1 : o1;
+            const int32_t *src = tok_tmp + in_offsets[row] - r0;       // src[o] for r0 <= o < r1
+            for (int64_t o = c0 + threadIdx.x; o < c1; o += 256) {
+                int32_t v = src[o];
+                if (remap) v = remap[v];
+                ids_out[o] = v;
+                if (mask_out) mask_out[o] = 1;
+            }
         }
     }
 }
 
+constexpr int kPadTile = 2048;           // cells of one row that one workgroup handles
+
+// Padded layout: workgroup (row, tile) copies the row's tokens that fall into its tile of
+// columns and pads the rest of the tile up to fill_to.
 __global__ __launch_bounds__(256) void pad_rows_kernel(
     const int32_t *__restrict__ tok_tmp, const int64_t *__restrict__ in_offsets,
-    const int32_t *__restrict__ lengths, int64_t n_rows, const int32_t *__restrict__ remap,
-    int32_t pad_id, int64_t t_cap, int64_t fill_to, int32_t *__restrict__ ids,
-    uint8_t *__restrict__ mask, int32_t *__restrict__ max_len)
+    const int32_t *__restrict__ lengths, int64_t n_rows, int64_t tiles_per_row,
+    const int32_t *__restrict__ remap, int32_t pad_id, int64_t t_cap, int64_t fill_to,
+    int32_t *__restrict__ ids, uint8_t *__restrict__ mask, int32_t *__restrict__ max_len)
 {
-    const int lane = threadIdx.x & 63;
-    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int64_t n_waves = (int64_t)gridDim.x * 4;
-    for (int64_t row = wave; row < n_rows; row += n_waves) {
+    const int64_t n_tiles = n_rows * tiles_per_row;
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int64_t row = tile / tiles_per_row;
+        const int64_t c0 = (tile - row * tiles_per_row) * kPadTile;
         int64_t len = lengths[row];
         if (len < 0) len = 0;
         if (len > t_cap) len = t_cap;
+        if (c0 == 0 && max_len && threadIdx.x == 0) atomicMax(max_len, (int32_t)len);
+        const int64_t end = len > fill_to ? len : fill_to;            // cells of the row that get written
+        if (c0 >= end) continue;
+        const int64_t c1 = c0 + kPadTile < end ? c0 + kPadTile : end;
         const int32_t *src = tok_tmp + in_offsets[row];
         int32_t *o = ids + row * t_cap;
         uint8_t *m = mask ? mask + row * t_cap : nullptr;
-        for (int64_t j = lane; j < len; j += 64) {
-            int32_t v = src[j];
-            if (remap) v = remap[v];
+        for (int64_t j = c0 + threadIdx.x; j < c1; j += 256) {
+            int32_t v = pad_id;
+            if (j < len) {
+                v = src[j];
+                if (remap) v = remap[v];
+            }
             o[j] = v;
-            if (m) m[j] = 1;
+            if (m) m[j] = j < len ? 1 : 0;
         }
-        for (int64_t j = len + lane; j < fill_to; j += 64) {
-            o[j] = pad_id;
-            if (m) m[j] = 0;
-        }
-        if (max_len && lane == 0) atomicMax(max_len, (int32_t)len);
     }
 }
 
-static int wave_grid(int64_t n_rows)
+static int capped_grid(int64_t want)
 {
-    int64_t g = (n_rows + 3) / 4;
-    if (g > 256 * 16) g = 256 * 16;
-    return (int)(g < 1 ? 1 : g);
+    if (want > 256 * 32) want = 256 * 32;
+    return (int)(want < 1 ? 1 : want);
 }
 
 }  // namespace dnatok
@@ -127,8 +145,10 @@ extern "C" int dnatok_pack_ragged(const int32_t *tok_tmp, const int64_t *in_offs
     DNATOK_HIP_TRY(hipGetLastError());
     if (n_rows == 0) return DNATOK_OK;
     DNATOK_REQUIRE(tok_tmp && ids_out, DNATOK_E_INVALID, "dnatok_pack_ragged: null buffer");
-    pack_copy_kernel<<<wave_grid(n_rows), 256, 0, s>>>(tok_tmp, in_offsets, lengths, n_rows, remap,
-                                                       out_offsets, ids_out, mask_out);
+    // the packed size is only known on the device: a fixed grid strides over its tiles, and
+    // workgroups past the end find nothing to do
+    pack_copy_kernel<<<256 * 16, 256, 0, s>>>(
+        tok_tmp, in_offsets, n_rows, remap, out_offsets, ids_out, mask_out);
     DNATOK_HIP_TRY(hipGetLastError());
     return DNATOK_OK;
 }
@@ -148,8 +168,9 @@ extern "C" int dnatok_pad_rows(const int32_t *tok_tmp, const int64_t *in_offsets
         int rc = launch_zero_i32(max_len, s);
         if (rc) return rc;
     }
-    pad_rows_kernel<<<wave_grid(n_rows), 256, 0, s>>>(tok_tmp, in_offsets, lengths, n_rows, remap,
-                                                      pad_id, t_cap, fill_to, ids, mask, max_len);
+    const int64_t tiles_per_row = t_cap > 0 ? (t_cap + kPadTile - 1) / kPadTile : 1;
+    pad_rows_kernel<<<capped_grid(n_rows * tiles_per_row), 256, 0, s>>>(
+        tok_tmp, in_offsets, lengths, n_rows, tiles_per_row, remap, pad_id, t_cap, fill_to, ids, mask, max_len);
     DNATOK_HIP_TRY(hipGetLastError());
     if (fill_to == 0) return launch_pad_to_max(ids, mask, lengths, n_rows, t_cap, max_len, pad_id, 0, s);
     return DNATOK_OK;
