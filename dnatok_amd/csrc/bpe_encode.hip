@@ -13,17 +13,21 @@
 //     key merges.  Overlaps form chains of strictly decreasing key, along which the decision
 //     alternates, so each candidate walks its left and right chain and merges iff both have
 //     even length (for a run x x x x this is "every other one from the left", HF's tie rule);
-//   * merges are applied in a doubly linked list over the original positions (a merge keeps
-//     the left position), the two neighbour pairs of each new symbol are re-ranked through
-//     the hashed merge table, and only the threads whose positions changed refresh their
-//     cached minima.
+//   * the pairs that merge go onto a per-round queue; the queue deals the apply work (one merge
+//     per thread) and the re-rank work (two table probes per merge) evenly to the team, whatever
+//     positions the merges sit at.  Merges are applied in a doubly linked list over the original
+//     positions (a merge keeps the left position); rank, links and symbol of a position sit in one
+//     record, so a step along a chain is one read; the two neighbour pairs of each new symbol are
+//     re-ranked through the hashed merge table, and only the threads whose positions changed
+//     refresh their cached minima.
 //
 // A table in which some rule's product is used by a LOWER-ranked rule (possible when two
 // rules produce the same string) makes G <= rmin; such a round merges only the single
 // smallest-key pair, which is exactly HF's next step.
 //
-// State lives in LDS for rows up to the LDS capacity (symbols, ranks and links as uint16),
-// and in a global scratch area (L2-resident) for longer rows.
+// State lives in LDS for rows up to the LDS capacity (13 bytes per position: an 8-byte record,
+// product and gate of the position's pair, and the queue), and in a global scratch area
+// (L2-resident, 32-bit links) for longer rows that cannot be cut into chunks.
 #include "common.hpp"
 
 #include <stdlib.h>
@@ -817,11 +821,8 @@ extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, co
     hipStream_t s = (hipStream_t)stream;
     BpeArgs a{t->tab, t->byte_to_sym, t->out_remap, t->slots, t->shift, t->n_merges};
 
-    static const char *variant_env = getenv("DNATOK_BPE_VARIANT");
-    static const char *chunk_env = getenv("DNATOK_BPE_NO_CHUNKS");
-    const int variant = variant_env ? atoi(variant_env) : 0;
     const bool long_rows = max_len > p.ext;
-    const int chunking = (long_rows && t->monotone && !chunk_env) ? 1 : 0;
+    const int chunking = (long_rows && t->monotone) ? 1 : 0;
     bpe_plan_kernel<<<1, 1024, 0, s>>>(offsets, n_rows, chunking, p);
     DNATOK_HIP_TRY(hipGetLastError());
 
@@ -829,12 +830,8 @@ extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, co
     // less LDS per workgroup means more workgroups per CU
     int rc;
     const int64_t work_len = max_len < p.ext ? max_len : p.ext;    // longest piece the LDS kernel sees
-    if (variant == 3 && max_len <= 1024)      rc = launch_lds<64, 4, 1024>(a, bytes, offsets, p, tok_tmp, lengths, s);
-    else if (variant == 4 && max_len <= 1024) rc = launch_lds<64, 8, 1024>(a, bytes, offsets, p, tok_tmp, lengths, s);
-    else if (variant == 5)                    rc = launch_lds<1024, 1, kLdsCap>(a, bytes, offsets, p, tok_tmp, lengths, s);
-    else if (work_len <= 1024)   rc = launch_lds<256, 1, 1024>(a, bytes, offsets, p, tok_tmp, lengths, s);
+    if (work_len <= 1024)        rc = launch_lds<256, 1, 1024>(a, bytes, offsets, p, tok_tmp, lengths, s);
     else if (work_len <= 2048)   rc = launch_lds<256, 1, 2048>(a, bytes, offsets, p, tok_tmp, lengths, s);
-    else if (variant == 6)       rc = launch_lds<512, 1, kLdsCap>(a, bytes, offsets, p, tok_tmp, lengths, s);
     else                         rc = launch_lds<256, 1, kLdsCap>(a, bytes, offsets, p, tok_tmp, lengths, s);
     if (rc) return rc;
     if (long_rows) {
