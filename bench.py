@@ -393,6 +393,33 @@ def hf_cpu(config: str, threads: int, max_bases: int) -> dict | None:
         return {"error": f"{type(e).__name__}: {e}"}
 
 
+def fused_embed_extra():
+    """Fused byte -> id -> embedding row kernel on one C1 batch (64 x 8192 bases), bf16 rows of 512:
+    1 byte read and 1 KiB written per base; checked against the two-step torch form."""
+    import torch
+    from dnatok_amd import encoders, hf_tokenizers as hf, workloads as wl
+    vocab = hf.char_vocab()
+    lut = np.zeros(256, dtype=np.int32)
+    for ch in "ACGTN":
+        lut[ord(ch)] = vocab[ch]
+    enc = encoders.CharEncoder(lut, 1)
+    data = _dev(wl.config1_char().data)
+    weight = torch.randn((len(vocab), 512), device="cuda").to(torch.bfloat16)
+    out = torch.empty((data.numel(), 512), dtype=torch.bfloat16, device="cuda")
+    enc.embed_packed(data, weight, out=out)
+    ids, _ = enc.encode_packed(data)
+    assert torch.equal(out.view(torch.int16), weight[ids.long()].view(torch.int16)), "fused embedding gather differs"
+
+    class W:
+        def step(self):
+            enc.embed_packed(data, weight, out=out)
+    wm, dm = time_steps(W(), 20, 3)
+    by = data.numel() * (1 + 1024)
+    return {"workload": "C1 batch 64x8192 bases -> bf16 [B, T, 512]", "ms_per_call": wm, "device_ms_per_call": dm,
+            "mbp_per_s": data.numel() / (wm * 1e-3) / 1e6, "algorithmic_bytes": by,
+            "hbm_frac": by / (dm * 1e-3) / 1e9 / HBM_PEAK_GBS, "kernel": "char_embed_kernel"}
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -497,6 +524,7 @@ def main() -> None:
             del ww
             torch.cuda.empty_cache()
         result["sustained"] = sustained
+        result["fused_embedding_gather"] = fused_embed_extra()
 
     print(json.dumps(result), flush=True)
 

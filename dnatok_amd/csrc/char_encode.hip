@@ -238,6 +238,96 @@ extern "C" int dnatok_char_encode_packed(const dnatok_char_t *t, const uint8_t *
     return DNATOK_OK;
 }
 
+namespace dnatok {
+
+// Fused byte -> id -> embedding row: out[i, :] = emb[table[bytes[i]], :] without the id tensor in
+// between.  A wave reads 64 bytes with one load, then copies the 64 rows one after the other,
+// 16 bytes per lane and instruction (the row pointer is wave-uniform, so a copy instruction covers
+// 1 KiB of the source row and 1 KiB of the output).  Write-bound: row_bytes per base.
+constexpr int64_t kEmbedLdsBytes = 48 * 1024;      // embedding tables up to this size are staged in LDS
+
+template <bool HAS_START, bool IN_LDS>
+__global__ __launch_bounds__(kCharThreads) void char_embed_kernel(
+    const uint8_t *__restrict__ bytes, int64_t total, int64_t row_len,
+    const CharTableDev *__restrict__ tab, const uint8_t *__restrict__ emb, int32_t n_vocab,
+    int64_t row_bytes, uint8_t *__restrict__ out)
+{
+    __shared__ int32_t lut[256];
+    __shared__ int32_t start[256];
+    extern __shared__ __align__(16) uint8_t s_emb[];          // the whole table when IN_LDS
+    lut[threadIdx.x] = tab->lut[threadIdx.x];
+    if (HAS_START) start[threadIdx.x] = tab->start[threadIdx.x];
+    if (IN_LDS)
+        for (int64_t o = (int64_t)threadIdx.x * 16; o < n_vocab * row_bytes; o += kCharThreads * 16)
+            *reinterpret_cast<int4v *>(s_emb + o) = *reinterpret_cast<const int4v *>(emb + o);
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * (kCharThreads / 64) + (threadIdx.x >> 6);
+    const int64_t n_waves = (int64_t)gridDim.x * (kCharThreads / 64);
+    for (int64_t base = wave * 64; base < total; base += n_waves * 64) {
+        const int64_t i = base + lane;
+        int32_t id = -1;
+        if (i < total) {
+            const uint8_t c = bytes[i];
+            id = (HAS_START && i % row_len == 0) ? start[c] : lut[c];
+            if (id < 0 || id >= n_vocab) id = -1;                     // no such row: zeros
+        }
+        const int n_here = total - base < 64 ? (int)(total - base) : 64;
+        // four rows per pass, so that four loads are in flight before the first store
+        for (int b0 = 0; b0 < n_here; b0 += 4) {
+            for (int64_t o = (int64_t)lane * 16; o < row_bytes; o += 64 * 16) {
+                int4v v[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int32_t rid = __builtin_amdgcn_readlane(id, (b0 + j) & 63);
+                    v[j] = int4v{0, 0, 0, 0};
+                    if (rid >= 0) {
+                        const int64_t at = (int64_t)rid * row_bytes + o;
+                        v[j] = IN_LDS ? *reinterpret_cast<const int4v *>(s_emb + at)
+                                      : *reinterpret_cast<const int4v *>(emb + at);
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (b0 + j < n_here)
+                        __builtin_nontemporal_store(v[j], reinterpret_cast<int4v *>(out + (base + b0 + j) * row_bytes + o));
+            }
+        }
+    }
+}
+
+}  // namespace dnatok
+
+extern "C" int dnatok_char_embed_packed(const dnatok_char_t *t, const uint8_t *bytes, int64_t total,
+                                        int64_t row_len, const void *emb, int32_t n_vocab,
+                                        int64_t row_bytes, void *out, void *stream)
+{
+    DNATOK_REQUIRE(t, DNATOK_E_INVALID, "dnatok_char_embed_packed: null argument");
+    DNATOK_REQUIRE(total >= 0 && row_len >= 0 && n_vocab > 0 && row_bytes > 0, DNATOK_E_INVALID,
+                   "dnatok_char_embed_packed: bad size");
+    if (total == 0) return DNATOK_OK;
+    DNATOK_REQUIRE(bytes && emb && out, DNATOK_E_INVALID, "dnatok_char_embed_packed: null buffer");
+    DNATOK_REQUIRE(((uintptr_t)emb & 15) == 0 && ((uintptr_t)out & 15) == 0 && (row_bytes & 15) == 0,
+                   DNATOK_E_INVALID,
+                   "dnatok_char_embed_packed: embedding rows and output must be 16-byte aligned "
+                   "(row_bytes a multiple of 16)");
+    hipStream_t s = (hipStream_t)stream;
+    const int grid = grid_for((total + 255) / 256);
+    const bool use_start = t->has_start && row_len > 0;
+    const int64_t table_bytes = (int64_t)n_vocab * row_bytes;
+    const bool in_lds = table_bytes <= kEmbedLdsBytes;
+    const size_t lds = in_lds ? (size_t)table_bytes : 0;
+#define LAUNCH(S, L)                                                                              \
+    char_embed_kernel<S, L><<<grid, kCharThreads, lds, s>>>(bytes, total, use_start ? row_len : 1, t->dev, \
+                                                            (const uint8_t *)emb, n_vocab, row_bytes, (uint8_t *)out)
+    if (use_start) { if (in_lds) LAUNCH(true, true); else LAUNCH(true, false); }
+    else           { if (in_lds) LAUNCH(false, true); else LAUNCH(false, false); }
+#undef LAUNCH
+    DNATOK_HIP_TRY(hipGetLastError());
+    return DNATOK_OK;
+}
+
 extern "C" int dnatok_char_encode_padded(const dnatok_char_t *t, const uint8_t *bytes,
                                          const int64_t *offsets, int64_t n_rows, int64_t t_out,
                                          int pad_left, int32_t *ids, uint8_t *mask, void *stream)

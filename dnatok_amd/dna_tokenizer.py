@@ -479,6 +479,21 @@ class DNATok:
         ids, _ = self._char_enc.encode_packed(data, row_len=t)
         return ids.view(b, t).to(torch.int64)
 
+    def fused_tokenize_gather(self, ascii_bytes: torch.Tensor, embed_weight: torch.Tensor,
+                              device="cuda") -> torch.Tensor:
+        """``embed_weight[ascii_lut[ascii_bytes]]`` in one kernel: uint8 [B, T] (host or device)
+        and a [V, D] device weight -> [B, T, D] of the weight's dtype; the id tensor is never
+        written (reference: _fused_tokenize_gather, 3465-3532, a Triton kernel there).
+        Single-nucleotide tokenizers only."""
+        self._require_ready()
+        if self._char_enc is None or self._kmer_enc is not None or self.bpe_backend is not None:
+            raise RuntimeError("the fused kernel serves single-nucleotide table tokenizers")
+        b, t = ascii_bytes.shape
+        data = ascii_bytes.to(device, non_blocking=True).reshape(-1)
+        weight = embed_weight if embed_weight.is_contiguous() else embed_weight.contiguous()
+        out = self._char_enc.embed_packed(data, weight, row_len=t)
+        return out.view(b, t, weight.shape[1])
+
     # ------------------------------------------------------------------ embedding
 
     def iter_embed_tokens_in_slices(self, ids: torch.Tensor, emb_batch: int, device) -> Iterator[torch.Tensor]:

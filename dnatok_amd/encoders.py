@@ -103,6 +103,24 @@ class CharEncoder:
         return ids, (mask if want_mask else None)
 
 
+    def embed_packed(self, data: torch.Tensor, weight: torch.Tensor, *, row_len: int = 0,
+                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """out[i, :] = weight[lut[data[i]], :] in one kernel (no id tensor).  ``weight`` is a
+        contiguous [V, D] device tensor of any dtype whose rows are a multiple of 16 bytes."""
+        _require_cuda(data, torch.uint8, "data")
+        if not (weight.is_cuda and weight.dim() == 2 and weight.is_contiguous()):
+            raise ValueError("weight must be a contiguous [V, D] device tensor")
+        total = data.numel()
+        row_bytes = weight.shape[1] * weight.element_size()
+        if out is None:
+            out = torch.empty((total, weight.shape[1]), dtype=weight.dtype, device=data.device)
+        _lib.check(_lib.lib().dnatok_char_embed_packed(self._h, _ptr(data), total, int(row_len), _ptr(weight),
+                                                       int(weight.shape[0]), int(row_bytes), _ptr(out),
+                                                       _stream()),
+                   "dnatok_char_embed_packed")
+        return out
+
+
 class KmerEncoder:
     """Grid-aligned k-mer windows with per-window fallback (C ABI: dnatok_kmer_*)."""
 

@@ -66,6 +66,15 @@ int dnatok_char_encode_padded(const dnatok_char_t *t, const uint8_t *bytes, cons
 int dnatok_char_encode_packed(const dnatok_char_t *t, const uint8_t *bytes, int64_t total,
                               int64_t row_len, int32_t *ids, uint8_t *mask, void *stream);
 
+/* Fused tokenize + embedding gather: out[i, :] = emb[lut[bytes[i]], :] for i < total, without the
+ * id tensor in between.  Replaces DNATok._fused_tokenize_gather (src/dna_tokenizer.py:3465-3532,
+ * a Triton kernel there).  emb is [n_vocab] rows of row_bytes bytes each (any element type; rows
+ * and output 16-byte aligned, row_bytes a multiple of 16), out is [total] rows of row_bytes.
+ * An id outside [0, n_vocab) gives a row of zeros.  row_len as in dnatok_char_encode_packed. */
+int dnatok_char_embed_packed(const dnatok_char_t *t, const uint8_t *bytes, int64_t total,
+                             int64_t row_len, const void *emb, int32_t n_vocab, int64_t row_bytes,
+                             void *out, void *stream);
+
 /* ---------------------------------------------------------------------------------------
  * Non-overlapping k-mer encoder (grid-aligned windows, per-window fallback, tail as single
  * characters).  Replaces DNATok._encode_batch_kmer_numpy_partial (src/dna_tokenizer.py:

@@ -89,6 +89,28 @@ def test_char_packed_start_table():
         np.testing.assert_array_equal(ids.cpu().numpy().reshape(9, row_len), eids)
 
 
+@pytest.mark.parametrize("dtype,dim", [(torch.bfloat16, 512), (torch.float32, 36), (torch.float16, 8)])
+def test_char_fused_embedding_gather(dtype, dim):
+    """out[i, :] = weight[lut[byte[i]], :], compared with the two-step torch form; also with a
+    first-column table, an id without a row (zeros) and a byte count that is no multiple of 64."""
+    say(f"char fused embed {dtype} D={dim}")
+    lut = util.char_lut()
+    rng = np.random.default_rng(dim)
+    weight = torch.from_numpy(rng.standard_normal((int(lut.max()) + 1, dim)).astype(np.float32)).to(DEV).to(dtype)
+    for start, n_vocab_cut in ((None, 0), (lut + 0, 0), (None, 2)):
+        enc = encoders.CharEncoder(lut, pad_id=1, start_lut=start)
+        b = wl.config1_char(5, 1000 + 37, seed=dim)
+        data, _ = to_dev(b)
+        w = weight[:weight.shape[0] - n_vocab_cut].contiguous()
+        out = enc.embed_packed(data, w, row_len=1037)
+        torch.cuda.synchronize()
+        ids = torch.from_numpy(O.char_encode_packed(lut, b.data)).to(DEV).long()
+        ok = ids < w.shape[0]
+        ref = torch.zeros((ids.numel(), dim), dtype=dtype, device=DEV)
+        ref[ok] = w[ids[ok]]
+        assert torch.equal(out.view(torch.uint8), ref.view(torch.uint8))
+
+
 def test_char_c5_packed(char_enc):
     say("char C5 packed")
     b = wl.config5_ragged()
