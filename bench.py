@@ -420,6 +420,40 @@ def fused_embed_extra():
             "hbm_frac": by / (dm * 1e-3) / 1e9 / HBM_PEAK_GBS, "kernel": "char_embed_kernel"}
 
 
+def unpack_2bit_extra():
+    """2-bit packed bases -> int32 ids, sustained form: 340 distinct C1 batches (178 Mbp) packed on
+    the host by the library, one launch; 0.25 byte read and 4 bytes written per base; checked
+    against the byte path's ids wherever the text is ACGT (N travels as A)."""
+    import torch
+    from dnatok_amd import encoders, hf_tokenizers as hf
+    vocab = hf.char_vocab()
+    lut = np.zeros(256, dtype=np.int32)
+    for ch in "ACGTN":
+        lut[ord(ch)] = vocab[ch]
+    enc = encoders.CharEncoder(lut, 1)
+    n_rows = 64 * 340
+    host = many_batches_uniform(n_rows, 8192, 7001, n_rate=0.001).reshape(n_rows, 8192)
+    t0 = time.perf_counter()
+    packed_h = encoders.pack_2bit_host(torch.from_numpy(host))
+    pack_s = time.perf_counter() - t0
+    packed = packed_h.to("cuda")
+    ids = torch.empty((n_rows, 8192), dtype=torch.int32, device="cuda")
+    enc.unpack_2bit(packed, 8192, out=ids)
+    want = lut[host[-64:]].copy()
+    want[host[-64:] == ord("N")] = lut[ord("A")]
+    assert np.array_equal(ids[-64:].cpu().numpy(), want), "2-bit unpack differs"
+
+    class W:
+        def step(self):
+            enc.unpack_2bit(packed, 8192, out=ids)
+    wm, dm = time_steps(W(), 10, 2)
+    by = host.size * 4 + host.size // 4
+    return {"workload": "340 C1 batches (64x8192 bases each), 2-bit packed -> int32 ids", "ms_per_call": wm,
+            "device_ms_per_call": dm, "mbp_per_s": host.size / (wm * 1e-3) / 1e6, "algorithmic_bytes": by,
+            "hbm_frac": by / (dm * 1e-3) / 1e9 / HBM_PEAK_GBS, "kernel": "char_unpack2bit_kernel",
+            "host_pack_mbp_per_s_1_core": host.size / pack_s / 1e6}
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -525,6 +559,7 @@ def main() -> None:
             torch.cuda.empty_cache()
         result["sustained"] = sustained
         result["fused_embedding_gather"] = fused_embed_extra()
+        result["unpack_2bit"] = unpack_2bit_extra()
 
     print(json.dumps(result), flush=True)
 

@@ -328,6 +328,125 @@ extern "C" int dnatok_char_embed_packed(const dnatok_char_t *t, const uint8_t *b
     return DNATOK_OK;
 }
 
+namespace dnatok {
+
+// 2-bit packed bases (4 per byte, first base in the low bits, codes A C G T = 0 1 2 3) -> ids.
+// HBM-bound and write-dominated: 0.25 byte read and sizeof(OUT) bytes written per base.  The
+// workgroup first builds, in LDS, the four ids of every one of the 256 possible packed bytes;
+// a lane then reads one packed byte (a wave covers 64 contiguous bytes), looks its four ids up
+// with one LDS read and stores them contiguously (a wave covers 1 KiB of int32 ids).  Giving a
+// lane four packed bytes and 64 contiguous output bytes instead measures 7 x slower: the four
+// stores of a wave then each touch 64 lines.
+constexpr int kUnpackSteps = 8;                                  // packed bytes per lane per tile
+constexpr int kUnpackTile = kCharThreads * kUnpackSteps;         // 2048 packed bytes = 8192 bases
+
+template <typename OUT> struct Quad;
+template <> struct Quad<uint8_t> { typedef uint32_t type; };
+template <> struct Quad<int32_t> { typedef int4v type; };
+template <> struct Quad<int64_t> { typedef int64_t type __attribute__((ext_vector_type(4))); };
+
+template <typename OUT>
+__device__ __forceinline__ typename Quad<OUT>::type make_quad(int4v v);
+template <> __device__ __forceinline__ uint32_t make_quad<uint8_t>(int4v v)
+{
+    return (uint32_t)(v.x & 255) | ((uint32_t)(v.y & 255) << 8) | ((uint32_t)(v.z & 255) << 16) |
+           ((uint32_t)v.w << 24);
+}
+template <> __device__ __forceinline__ int4v make_quad<int32_t>(int4v v) { return v; }
+template <> __device__ __forceinline__ Quad<int64_t>::type make_quad<int64_t>(int4v v)
+{
+    return Quad<int64_t>::type{(int64_t)v.x, (int64_t)v.y, (int64_t)v.z, (int64_t)v.w};
+}
+
+// QUADS: row_len % 4 == 0 and ids aligned to 4 elements, so the packed stream and the output are
+// both flat and every packed byte owns one aligned group of four cells.  Otherwise rows are
+// ceil(row_len / 4) packed bytes each and cells are stored one by one.
+template <typename OUT, bool HAS_START, bool QUADS>
+__global__ __launch_bounds__(kCharThreads) void char_unpack2bit_kernel(
+    const uint8_t *__restrict__ packed, int64_t n_rows, int64_t row_len, int64_t row_packed,
+    const CharTableDev *__restrict__ tab, OUT *__restrict__ ids)
+{
+    __shared__ int4v quad[256];
+    __shared__ int32_t first[4];
+    {
+        const int32_t a = tab->lut['A'], c = tab->lut['C'], g = tab->lut['G'], t = tab->lut['T'];
+        auto pick = [&](uint32_t code) { return code == 0 ? a : code == 1 ? c : code == 2 ? g : t; };
+        const uint32_t b = threadIdx.x;
+        quad[b] = int4v{pick(b & 3u), pick((b >> 2) & 3u), pick((b >> 4) & 3u), pick(b >> 6)};
+        if (HAS_START && b < 4) first[b] = tab->start[(int)"ACGT"[b]];
+    }
+    __syncthreads();
+
+    const int64_t n_packed = n_rows * row_packed;
+    const int64_t n_tiles = (n_packed + kUnpackTile - 1) / kUnpackTile;
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int64_t p0 = tile * kUnpackTile + threadIdx.x;
+        uint8_t w[kUnpackSteps];
+#pragma unroll
+        for (int s = 0; s < kUnpackSteps; ++s) {
+            const int64_t p = p0 + s * kCharThreads;
+            w[s] = p < n_packed ? __builtin_nontemporal_load(packed + p) : (uint8_t)0;
+        }
+#pragma unroll
+        for (int s = 0; s < kUnpackSteps; ++s) {
+            const int64_t p = p0 + s * kCharThreads;
+            if (p >= n_packed) continue;
+            int4v v = quad[w[s]];
+            if (QUADS) {
+                if (HAS_START && (p * 4) % row_len == 0) v.x = first[w[s] & 3u];
+                __builtin_nontemporal_store(make_quad<OUT>(v),
+                                            reinterpret_cast<typename Quad<OUT>::type *>(ids + p * 4));
+            } else {
+                const int64_t b = p / row_packed;
+                const int64_t col = (p - b * row_packed) * 4;
+                if (HAS_START && col == 0) v.x = first[w[s] & 3u];
+                OUT *o = ids + b * row_len + col;
+                const int32_t vs[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    if (col + k < row_len) o[k] = (OUT)vs[k];
+            }
+        }
+    }
+}
+
+template <typename OUT>
+static int launch_unpack2bit(const dnatok_char_table *t, const uint8_t *packed, int64_t n_rows,
+                             int64_t row_len, void *ids, hipStream_t s)
+{
+    const int64_t row_packed = (row_len + 3) / 4;
+    const int64_t n_tiles = (n_rows * row_packed + kUnpackTile - 1) / kUnpackTile;
+    const int grid = grid_for(n_tiles);
+    const bool quads = row_len % 4 == 0 && ((uintptr_t)ids % (4 * sizeof(OUT))) == 0;
+#define LAUNCH(S, Q)                                                                             \
+    char_unpack2bit_kernel<OUT, S, Q><<<grid, kCharThreads, 0, s>>>(packed, n_rows, row_len,      \
+                                                                     row_packed, t->dev, (OUT *)ids)
+    if (t->has_start) { if (quads) LAUNCH(true, true); else LAUNCH(true, false); }
+    else              { if (quads) LAUNCH(false, true); else LAUNCH(false, false); }
+#undef LAUNCH
+    DNATOK_HIP_TRY(hipGetLastError());
+    return DNATOK_OK;
+}
+
+}  // namespace dnatok
+
+extern "C" int dnatok_char_unpack_2bit(const dnatok_char_t *t, const uint8_t *packed, int64_t n_rows,
+                                       int64_t row_len, void *ids, int32_t id_bytes, void *stream)
+{
+    DNATOK_REQUIRE(t, DNATOK_E_INVALID, "dnatok_char_unpack_2bit: null argument");
+    DNATOK_REQUIRE(n_rows >= 0 && row_len >= 0, DNATOK_E_INVALID, "dnatok_char_unpack_2bit: negative size");
+    DNATOK_REQUIRE(id_bytes == 1 || id_bytes == 4 || id_bytes == 8, DNATOK_E_INVALID,
+                   "dnatok_char_unpack_2bit: id_bytes must be 1, 4 or 8 (got %d)", (int)id_bytes);
+    if (n_rows == 0 || row_len == 0) return DNATOK_OK;
+    DNATOK_REQUIRE(packed && ids, DNATOK_E_INVALID, "dnatok_char_unpack_2bit: null buffer");
+    DNATOK_REQUIRE(((uintptr_t)ids % (size_t)id_bytes) == 0, DNATOK_E_INVALID,
+                   "dnatok_char_unpack_2bit: ids not aligned to its element size");
+    hipStream_t s = (hipStream_t)stream;
+    if (id_bytes == 1) return launch_unpack2bit<uint8_t>(t, packed, n_rows, row_len, ids, s);
+    if (id_bytes == 4) return launch_unpack2bit<int32_t>(t, packed, n_rows, row_len, ids, s);
+    return launch_unpack2bit<int64_t>(t, packed, n_rows, row_len, ids, s);
+}
+
 extern "C" int dnatok_char_encode_padded(const dnatok_char_t *t, const uint8_t *bytes,
                                          const int64_t *offsets, int64_t n_rows, int64_t t_out,
                                          int pad_left, int32_t *ids, uint8_t *mask, void *stream)

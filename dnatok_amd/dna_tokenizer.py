@@ -17,6 +17,7 @@ re-tokenized by the tokenizer object itself, as the reference does
 """
 from __future__ import annotations
 
+import inspect
 import logging
 import os
 from typing import Any, Iterator, List, Optional, Sequence, Tuple
@@ -98,9 +99,15 @@ class DNATok:
         self._kmer_enc: Optional[encoders.KmerEncoder] = None
         self._kmer_tables: Optional[kmer_tables.KmerTables] = None
         self._staging_bytes_cpu: Optional[torch.Tensor] = None
+        self._packed_2bit_cpu: Optional[torch.Tensor] = None
+        self._dev_ping: Optional[torch.Tensor] = None
+        self._dev_pong: Optional[torch.Tensor] = None
 
     def free_buffers(self) -> None:
         self._staging_bytes_cpu = None
+        self._packed_2bit_cpu = None
+        self._dev_ping = None
+        self._dev_pong = None
 
     # ------------------------------------------------------------- tokenizer access
 
@@ -447,7 +454,9 @@ class DNATok:
     # ------------------------------------------------------------------ bytes path
 
     def encode_batch_to_ascii_bytes(self, seqs: List[str]) -> torch.Tensor:
-        """Equal-length strings -> persistent pinned uint8 [B, T] (reference: 2594-2651)."""
+        """Equal-length strings -> persistent pinned uint8 [B, T]; with ``normalize_case`` the
+        bytes are upper-cased, with ``handle_invalid_chars`` (and no separate invalid id) bytes
+        outside ACGTN become N (reference: 2594-2651).  One join, one native pass."""
         if not seqs:
             raise ValueError("No sequences provided for encoding.")
         t = len(seqs[0])
@@ -460,7 +469,50 @@ class DNATok:
                                                   pin_memory=torch.cuda.is_available())
         out = self._staging_bytes_cpu[:need].view(len(seqs), t)
         out.copy_(torch.frombuffer(bytearray(buf), dtype=torch.uint8).view(len(seqs), t))
+        to_n = self.handle_invalid_chars and (self.invalid_char_id is None or self.invalid_char_id == self.id_N)
+        if self.normalize_case or to_n:
+            encoders.clean_ascii_host(out, upper_case=self.normalize_case, invalid_to_n=to_n)
         return out
+
+    def encode_batch_to_packed_2bit(self, seqs: List[str]) -> Tuple[torch.Tensor, int]:
+        """Equal-length strings -> (pinned uint8 [B, ceil(T/4)], T): four bases per byte, first
+        base in the low bits, A C G T = 0 1 2 3; N and every other byte travel as code 0
+        (reference: 3143-3210).  A quarter of the bytes path's PCIe payload."""
+        if not seqs:
+            raise ValueError("No sequences provided.")
+        ascii_rows = self.encode_batch_to_ascii_bytes(seqs)
+        b, t = ascii_rows.shape
+        tp = (t + 3) // 4
+        if self._packed_2bit_cpu is None or tuple(self._packed_2bit_cpu.shape) != (b, tp):
+            self._packed_2bit_cpu = torch.empty((b, tp), dtype=torch.uint8, pin_memory=torch.cuda.is_available())
+        encoders.pack_2bit_host(ascii_rows, out=self._packed_2bit_cpu)
+        return self._packed_2bit_cpu, t
+
+    def _unpack_2bit(self, packed_cpu: torch.Tensor, t_true: int, device, dtype: torch.dtype) -> torch.Tensor:
+        self._require_ready()
+        if self._char_enc is None or self._kmer_enc is not None or self.bpe_backend is not None:
+            raise RuntimeError("the 2-bit path serves single-nucleotide table tokenizers")
+        if packed_cpu.dim() != 2 or packed_cpu.dtype != torch.uint8:
+            raise TypeError("packed must be a uint8 [B, ceil(T/4)] tensor")
+        packed = packed_cpu.to(device, non_blocking=True).contiguous()
+        return self._char_enc.unpack_2bit(packed, int(t_true), dtype=dtype)
+
+    def _unpack_2bit_to_ids_cuda(self, packed_cpu: torch.Tensor, T_true: int, device="cuda") -> torch.Tensor:
+        """H2D of the packed bytes, then unpack + table lookup in one kernel -> int64 [B, T]
+        (reference: 3212-3275)."""
+        return self._unpack_2bit(packed_cpu, T_true, device, torch.int64)
+
+    def _unpack_2bit_to_ids_cuda_u8(self, packed_cpu: torch.Tensor, T_true: int, device="cuda") -> torch.Tensor:
+        """Same for vocabularies of at most 256 ids; the result is int64 like the reference's
+        (3278-3330), written by the kernel directly."""
+        if not self._ascii_lut_fits_uint8():
+            raise RuntimeError("uint8 IDs path requires vocab <= 256.")
+        return self._unpack_2bit(packed_cpu, T_true, device, torch.int64)
+
+    def _ascii_lut_fits_uint8(self) -> bool:
+        if self.ascii_lut is None:
+            return False
+        return int(np.max(self.ascii_lut, initial=0)) <= 255 and int(self.id_pad) <= 255
 
     def ids_from_ascii_bytes_cuda(self, u8_cpu: torch.Tensor, device="cuda") -> torch.Tensor:
         """uint8 [B, T] on the host -> int64 ids on the GPU (reference: 2653-2723, 2826-2940)."""
@@ -496,14 +548,99 @@ class DNATok:
 
     # ------------------------------------------------------------------ embedding
 
-    def iter_embed_tokens_in_slices(self, ids: torch.Tensor, emb_batch: int, device) -> Iterator[torch.Tensor]:
-        dev = torch.device(device)
-        for s in range(0, ids.shape[0], max(1, int(emb_batch))):
-            chunk = ids[s:s + emb_batch].to(dev, dtype=torch.long, non_blocking=True)
-            out = self.embedder.embed_tokens(chunk)
-            yield out.float() if self.force_fp32_outputs and out.is_floating_point() else out
+    def _embed_call(self, ids_dev: torch.Tensor) -> torch.Tensor:
+        kwargs = {}
+        try:
+            if "rc_invariant" in inspect.signature(self.embedder.embed_tokens).parameters:
+                kwargs["rc_invariant"] = False
+        except (TypeError, ValueError):
+            pass
+        with torch.amp.autocast(device_type="cuda", dtype=torch.float16, enabled=ids_dev.is_cuda):
+            out = self.embedder.embed_tokens(ids_dev, **kwargs)
+        return out.float() if self.force_fp32_outputs and out.is_floating_point() else out
 
-    iter_embed_tokens_pipelined = iter_embed_tokens_in_slices
+    def _ids_micro_bs_for_T(self, t: int, emb_batch: int) -> int:
+        """Rows per embed call: emb_batch, capped so that a call holds at most
+        ids_max_tokens_per_call tokens (reference: 2322-2339)."""
+        cap = max(1, int(self.ids_max_tokens_per_call) // max(1, int(t)))
+        return max(1, min(int(emb_batch), cap))
+
+    def iter_embed_tokens_in_slices(self, ids: torch.Tensor, emb_batch: int, device) -> Iterator[torch.Tensor]:
+        """One slice after the other on the current stream (reference: 2377-2452)."""
+        dev = torch.device(device)
+        if ids.dim() != 2 or ids.shape[0] == 0:
+            return
+        step = self._ids_micro_bs_for_T(int(ids.shape[1]), emb_batch)
+        for s in range(0, ids.shape[0], step):
+            chunk = ids[s:s + step].to(dev, dtype=torch.long, non_blocking=True)
+            yield self._embed_call(chunk)
+
+    def iter_embed_tokens_pipelined(self, ids_cpu: torch.Tensor, emb_batch: int, device="cuda", *,
+                                    use_int32_h2d: Optional[bool] = None) -> Iterator[torch.Tensor]:
+        """Two device buffers and a copy stream: the H2D copy of slice i+1 (int32 over the bus
+        when ``use_int32_h2d``, widened on the device) runs while ``embed_tokens`` works on
+        slice i (reference: 2454-2591).  A slice's buffer is handed out again only after the
+        compute stream has passed the embed call that read it."""
+        dev = torch.device(device)
+        if dev.type != "cuda" or not torch.cuda.is_available() or ids_cpu.is_cuda:
+            yield from self.iter_embed_tokens_in_slices(ids_cpu, emb_batch, device)
+            return
+        if ids_cpu.dim() != 2:
+            raise ValueError("ids must be [B, T]")
+        b, t = int(ids_cpu.shape[0]), int(ids_cpu.shape[1])
+        if b == 0:
+            return
+        if use_int32_h2d is None:
+            use_int32_h2d = self.prefer_int32_h2d
+        wire = torch.int32 if use_int32_h2d else torch.int64
+        src = ids_cpu if ids_cpu.dtype == wire else ids_cpu.to(wire)
+        if not src.is_pinned():
+            src = src.pin_memory()
+        step = self._ids_micro_bs_for_T(t, emb_batch)
+        if (self._dev_ping is None or self._dev_ping.device != dev or self._dev_ping.dtype != wire
+                or self._dev_ping.shape[0] < step or self._dev_ping.shape[1] != t):
+            self._dev_ping = torch.empty((step, t), dtype=wire, device=dev)
+            self._dev_pong = torch.empty((step, t), dtype=wire, device=dev)
+        bufs = (self._dev_ping, self._dev_pong)
+        compute = torch.cuda.current_stream(dev)
+        copy_stream = torch.cuda.Stream(device=dev)                 # default priority
+        copied = (torch.cuda.Event(), torch.cuda.Event())
+        consumed = (torch.cuda.Event(), torch.cuda.Event())
+        starts = list(range(0, b, step))
+
+        def schedule(i: int) -> None:
+            lo = starts[i]
+            hi = min(b, lo + step)
+            which = i & 1
+            with torch.cuda.stream(copy_stream):
+                if i >= 2:
+                    copy_stream.wait_event(consumed[which])         # the embed call that read it
+                else:
+                    copy_stream.wait_stream(compute)                # whatever used the buffers before
+                bufs[which][:hi - lo].copy_(src[lo:hi], non_blocking=True)
+                copied[which].record(copy_stream)
+
+        schedule(0)
+        if len(starts) > 1:
+            schedule(1)
+        for i, lo in enumerate(starts):
+            hi = min(b, lo + step)
+            which = i & 1
+            compute.wait_event(copied[which])
+            buf = bufs[which][:hi - lo]
+            ids_dev = buf.to(torch.long)
+            if ids_dev.data_ptr() != buf.data_ptr():                # widened copy: the buffer is free after it
+                consumed[which].record(compute)
+                if i + 2 < len(starts):
+                    schedule(i + 2)
+                out = self._embed_call(ids_dev)
+            else:                                                   # embed_tokens reads the buffer itself
+                out = self._embed_call(ids_dev)
+                consumed[which].record(compute)
+                if i + 2 < len(starts):
+                    schedule(i + 2)
+            yield out
+        compute.wait_stream(copy_stream)
 
     def embed_from_strings(self, seqs: List[str], emb_batch: int, device, *, path: str = "ids"
                            ) -> Iterator[torch.Tensor]:

@@ -49,6 +49,37 @@ def bytes_from_strings(seqs: Sequence[str], device="cuda") -> Tuple[torch.Tensor
     return data, torch.from_numpy(offsets).to(device), lens
 
 
+def clean_ascii_host(buf: torch.Tensor, *, upper_case: bool, invalid_to_n: bool) -> int:
+    """In place on a contiguous host uint8 tensor: a-z -> A-Z, then bytes outside ACGTN -> 'N'
+    (one pass; reference: DNATok._encode_ascii_bytes_impl, src/dna_tokenizer.py:2637-2649).
+    Returns how many bytes were replaced."""
+    if buf.is_cuda or buf.dtype != torch.uint8 or not buf.is_contiguous():
+        raise ValueError("buf must be a contiguous uint8 tensor on the host")
+    n = ctypes.c_int64(0)
+    _lib.check(_lib.lib().dnatok_host_clean_ascii(ctypes.c_void_p(buf.data_ptr()), buf.numel(), int(upper_case),
+                                                  int(invalid_to_n), ctypes.byref(n)),
+               "dnatok_host_clean_ascii")
+    return int(n.value)
+
+
+def pack_2bit_host(ascii_rows: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Host uint8 [B, T] ASCII -> host uint8 [B, ceil(T/4)], four bases per byte, first base in
+    the low bits, A C G T = 0 1 2 3, anything else 0 (reference:
+    DNATok.encode_batch_to_packed_2bit, src/dna_tokenizer.py:3143-3210)."""
+    if ascii_rows.is_cuda or ascii_rows.dtype != torch.uint8 or ascii_rows.dim() != 2 or not ascii_rows.is_contiguous():
+        raise ValueError("ascii_rows must be a contiguous uint8 [B, T] tensor on the host")
+    b, t = ascii_rows.shape
+    tp = (t + 3) // 4
+    if out is None:
+        out = torch.empty((b, tp), dtype=torch.uint8, pin_memory=torch.cuda.is_available())
+    if tuple(out.shape) != (b, tp) or out.is_cuda or out.dtype != torch.uint8 or not out.is_contiguous():
+        raise ValueError("out must be a contiguous uint8 [B, ceil(T/4)] tensor on the host")
+    _lib.check(_lib.lib().dnatok_host_pack_2bit(ctypes.c_void_p(ascii_rows.data_ptr()), b, t,
+                                                ctypes.c_void_p(out.data_ptr())),
+               "dnatok_host_pack_2bit")
+    return out
+
+
 class CharEncoder:
     """ids = table[byte] with padding and mask (C ABI: dnatok_char_*)."""
 
@@ -118,6 +149,28 @@ class CharEncoder:
                                                        int(weight.shape[0]), int(row_bytes), _ptr(out),
                                                        _stream()),
                    "dnatok_char_embed_packed")
+        return out
+
+
+    def unpack_2bit(self, packed: torch.Tensor, row_len: int, *, dtype: torch.dtype = torch.int32,
+                    out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Device uint8 [B, ceil(row_len/4)] of 2-bit codes -> ids [B, row_len] of ``dtype``
+        (uint8, int32 or int64): ids = lut["ACGT"[code]], column 0 from the start table."""
+        _require_cuda(packed, torch.uint8, "packed")
+        if packed.dim() != 2 or packed.shape[1] != (int(row_len) + 3) // 4:
+            raise ValueError("packed must be [B, ceil(row_len / 4)]")
+        if dtype not in (torch.uint8, torch.int32, torch.int64):
+            raise ValueError("dtype must be uint8, int32 or int64")
+        b = packed.shape[0]
+        if out is None:
+            out = torch.empty((b, int(row_len)), dtype=dtype, device=packed.device)
+        elif tuple(out.shape) != (b, int(row_len)):
+            raise ValueError("out must be [B, row_len]")
+        else:
+            _require_cuda(out, dtype, "out")
+        _lib.check(_lib.lib().dnatok_char_unpack_2bit(self._h, _ptr(packed), b, int(row_len), _ptr(out),
+                                                      out.element_size(), _stream()),
+                   "dnatok_char_unpack_2bit")
         return out
 
 

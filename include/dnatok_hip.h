@@ -75,6 +75,30 @@ int dnatok_char_embed_packed(const dnatok_char_t *t, const uint8_t *bytes, int64
                              int64_t row_len, const void *emb, int32_t n_vocab, int64_t row_bytes,
                              void *out, void *stream);
 
+/* 2-bit packed bases -> ids.  packed is uint8[n_rows, ceil(row_len / 4)] on the device: four bases
+ * per byte, the first in the low two bits, codes A C G T = 0 1 2 3 (what dnatok_host_pack_2bit
+ * writes).  ids is [n_rows, row_len] of id_bytes-wide integers (1: uint8, 4: int32, 8: int64);
+ * ids[b, t] = lut["ACGT"[code]], column 0 from the start table when the table has one.  Replaces
+ * DNATok._unpack_2bit_to_ids_cuda / _unpack_2bit_to_ids_cuda_u8 (src/dna_tokenizer.py:3212-3330). */
+int dnatok_char_unpack_2bit(const dnatok_char_t *t, const uint8_t *packed, int64_t n_rows,
+                            int64_t row_len, void *ids, int32_t id_bytes, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Host-side ingest (CPU code, host pointers, no device work).
+ * ------------------------------------------------------------------------------------- */
+
+/* In place: a-z -> A-Z when upper_case; then, when invalid_to_n, every byte outside ACGTN (outside
+ * ACGTNacgtn when upper_case = 0) becomes 'N'.  *n_replaced (may be NULL) counts those.  Replaces the
+ * numpy passes of DNATok._encode_ascii_bytes_impl (src/dna_tokenizer.py:2637-2649). */
+int dnatok_host_clean_ascii(uint8_t *bytes_h, int64_t n, int upper_case, int invalid_to_n,
+                            int64_t *n_replaced);
+
+/* ASCII rows uint8[n_rows, row_len] -> packed uint8[n_rows, ceil(row_len / 4)]:
+ * byte = c0 | c1 << 2 | c2 << 4 | c3 << 6 with A C G T (either case) = 0 1 2 3 and every other byte,
+ * N included, 0; the last byte of a row is filled with 0 codes.  Replaces
+ * DNATok.encode_batch_to_packed_2bit (src/dna_tokenizer.py:3143-3210). */
+int dnatok_host_pack_2bit(const uint8_t *ascii_h, int64_t n_rows, int64_t row_len, uint8_t *packed_h);
+
 /* ---------------------------------------------------------------------------------------
  * Non-overlapping k-mer encoder (grid-aligned windows, per-window fallback, tail as single
  * characters).  Replaces DNATok._encode_batch_kmer_numpy_partial (src/dna_tokenizer.py:

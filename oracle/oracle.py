@@ -79,6 +79,51 @@ def char_encode_packed(lut, data: np.ndarray) -> np.ndarray:
     return ids
 
 
+def clean_ascii(data: np.ndarray, upper_case: bool, invalid_to_n: bool) -> np.ndarray:
+    """Upper-case a-z, then bytes outside ACGTN (ACGTNacgtn without upper-casing) -> 'N'
+    (reference: src/dna_tokenizer.py:2637-2649).  Pinned by hand-written cases in
+    tests/test_oracle.py."""
+    arr = np.array(data, dtype=np.uint8, copy=True)
+    if upper_case:
+        lower = (arr >= ord("a")) & (arr <= ord("z"))
+        arr[lower] -= 32
+    if invalid_to_n:
+        valid = np.frombuffer(b"ACGTN" if upper_case else b"ACGTNacgtn", dtype=np.uint8)
+        arr[~np.isin(arr, valid)] = ord("N")
+    return arr
+
+
+def pack_2bit(ascii_rows: np.ndarray) -> np.ndarray:
+    """uint8 [B, T] ASCII -> uint8 [B, ceil(T/4)], byte = c0 | c1<<2 | c2<<4 | c3<<6 with
+    A C G T (either case) = 0 1 2 3, everything else 0, rows filled up with code 0
+    (reference: src/dna_tokenizer.py:3129-3141, 3195-3209).  Pinned by known bytes
+    ("ACGT" -> 0xE4, "TTTT" -> 0xFF, "CA" -> 0x01) and by the round trip through
+    ``unpack_2bit_ids`` in tests/test_oracle.py."""
+    code = np.zeros(256, dtype=np.uint8)
+    for j, ch in enumerate("ACGT"):
+        code[ord(ch)] = j
+        code[ord(ch.lower())] = j
+    b, t = ascii_rows.shape
+    tp = (t + 3) // 4
+    codes = np.zeros((b, tp * 4), dtype=np.uint8)
+    codes[:, :t] = code[ascii_rows]
+    c = codes.reshape(b, tp, 4)
+    return (c[..., 0] | (c[..., 1] << 2) | (c[..., 2] << 4) | (c[..., 3] << 6)).astype(np.uint8)
+
+
+def unpack_2bit_ids(lut, packed: np.ndarray, t_true: int, start_lut=None) -> np.ndarray:
+    """Packed uint8 [B, ceil(T/4)] -> int64 ids [B, T]: lut["ACGT"[code]], column 0 from the
+    start table (reference: src/dna_tokenizer.py:3232-3275)."""
+    lut = np.asarray(lut)
+    acgt = np.frombuffer(b"ACGT", dtype=np.uint8)
+    b, tp = packed.shape
+    codes = np.stack([(packed >> s) & 3 for s in (0, 2, 4, 6)], axis=2).reshape(b, tp * 4)[:, :t_true]
+    ids = lut[acgt[codes]].astype(np.int64)
+    if start_lut is not None and t_true > 0:
+        ids[:, 0] = np.asarray(start_lut)[acgt[codes[:, 0]]]
+    return ids
+
+
 # --------------------------------------------------------------- k-mer
 
 def base5_digits(fold_case: bool = False) -> np.ndarray:

@@ -143,6 +143,48 @@ def test_ids_and_bytes_paths_feed_the_same_ids():
     assert all(torch.equal(x, y) for x, y in zip(out_ids, out_bytes))
 
 
+def test_two_bit_path_feeds_the_same_ids_as_the_bytes_path():
+    tok = SimpleCharTokenizer()
+    h = DNATok(RecordingEmbedder(tok), normalize_case=True, handle_invalid_chars=True)
+    h.discover()
+    for t in (64, 67):
+        seqs = random_seqs(9, t, alphabet="ACGTacgt", seed=t)
+        packed, t_true = h.encode_batch_to_packed_2bit(seqs)
+        assert t_true == t and tuple(packed.shape) == (9, (t + 3) // 4) and packed.dtype == torch.uint8
+        ids = h._unpack_2bit_to_ids_cuda(packed, t_true, "cuda")
+        assert ids.dtype == torch.int64 and ids.is_cuda
+        assert torch.equal(ids, h.ids_from_ascii_bytes_cuda(h.encode_batch_to_ascii_bytes(seqs)))
+        assert torch.equal(ids.cpu(), tok(seqs, padding=True, return_tensors="pt")["input_ids"])
+        assert torch.equal(ids, h._unpack_2bit_to_ids_cuda_u8(packed, t_true, "cuda"))
+    # N and every other byte travel as code 0 and come back as A
+    packed, t_true = h.encode_batch_to_packed_2bit(["ANxT"])
+    assert h._unpack_2bit_to_ids_cuda(packed, t_true, "cuda").tolist() == [[1, 1, 1, 4]]
+    # the staging bytes are cleaned the way the reference cleans them
+    assert bytes(h.encode_batch_to_ascii_bytes(["acgtnx-R"]).numpy().tobytes()) == b"ACGTNNNN"
+
+
+@pytest.mark.parametrize("use_i32", [True, False])
+def test_pipelined_streamer_equals_slices(use_i32):
+    tok = SimpleCharTokenizer()
+    emb = RecordingEmbedder(tok).to("cuda")
+    h = DNATok(emb, ids_max_tokens_per_call=3 * 128, force_fp32_outputs=True)
+    h.discover()
+    g = torch.Generator().manual_seed(5)
+    ids = torch.randint(0, 6, (23, 128), generator=g, dtype=torch.int64)        # 8 slices of <= 3 rows
+    seen = []
+    orig = emb.embed_tokens
+    emb.embed_tokens = lambda input_ids, rc_invariant=False: (seen.append(input_ids.clone()), orig(input_ids))[1]
+    for _ in range(2):                                                       # the second pass reuses the buffers
+        seen.clear()
+        outs = list(h.iter_embed_tokens_pipelined(ids, emb_batch=8, device="cuda", use_int32_h2d=use_i32))
+        torch.cuda.synchronize()
+        assert [o.shape[0] for o in outs] == [3] * 7 + [2]
+        assert torch.equal(torch.cat(seen).cpu(), ids)
+        ref = list(h.iter_embed_tokens_in_slices(ids, emb_batch=8, device="cuda"))
+        assert all(torch.equal(a, b) for a, b in zip(outs, ref)) and len(outs) == len(ref)
+    assert list(h.iter_embed_tokens_pipelined(ids[:0], 8, "cuda")) == []
+
+
 def test_kmer_discover_and_encode():
     tok = MockKmerTokenizer(4)
     h = DNATok(RecordingEmbedder(tok))

@@ -111,6 +111,29 @@ def test_char_fused_embedding_gather(dtype, dim):
         assert torch.equal(out.view(torch.uint8), ref.view(torch.uint8))
 
 
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.int32, torch.int64])
+def test_char_unpack_2bit(dtype):
+    """2-bit packed rows -> ids of three widths, rows of every length mod 4 (the flat and the
+    row-by-row kernel), with and without a first-column table; packed by the host function of
+    the library, checked against the oracle's unpack of the oracle's packing."""
+    lut = util.char_lut()
+    rng = np.random.default_rng(11)
+    alphabet = np.frombuffer(b"ACGTNacgt", dtype=np.uint8)
+    for start in (None, lut + 3):
+        enc = encoders.CharEncoder(lut, pad_id=1, start_lut=start)
+        for b, t in ((3, 1), (5, 7), (4, 64), (7, 1001), (2, 8190), (64, 8192), (300, 516)):
+            say(f"char unpack 2bit {dtype} B={b} T={t} start={start is not None}")
+            rows = rng.choice(alphabet, size=(b, t))
+            packed = encoders.pack_2bit_host(torch.from_numpy(rows))
+            np.testing.assert_array_equal(packed.numpy(), O.pack_2bit(rows))
+            out = torch.full((b * t + 8,), 77, dtype=dtype, device=DEV)       # guard cells behind the rows
+            ids = enc.unpack_2bit(packed.to(DEV), t, dtype=dtype, out=out[:b * t].view(b, t))
+            torch.cuda.synchronize()
+            want = O.unpack_2bit_ids(lut, packed.numpy(), t, start_lut=start)
+            np.testing.assert_array_equal(ids.cpu().numpy().astype(np.int64), want)
+            assert bool((out[b * t:] == 77).all())
+
+
 def test_char_c5_packed(char_enc):
     say("char C5 packed")
     b = wl.config5_ragged()

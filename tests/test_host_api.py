@@ -2,6 +2,7 @@
 (the reference's own CPU unit tests, tests/test_gputok_bpe_backend.py:319-425), tokenizer.json
 handling, and the compat tokenizer classes."""
 import numpy as np
+import pytest
 
 from dnatok_amd import dnatok_compat, hf_tokenizers as hf
 from dnatok_amd.gputok_bpe_backend import (_compile_normalizer, _compile_normalizer_step, _extract_merges,
@@ -80,3 +81,40 @@ def test_compat_tokenizers():
     tk = hf.build_char_tokenizer()
     s = "ACGTNNACGTTTGACN"
     assert tk.encode(s, add_special_tokens=False).ids == nt.encode(s)
+
+
+# ------------------------------------------------------------------ host ingest (C ABI, CPU code)
+
+def test_host_clean_ascii_matches_oracle():
+    import torch
+    from dnatok_amd import encoders
+    from oracle import oracle as O
+    rng = np.random.default_rng(3)
+    raw = rng.integers(0, 256, size=10_000, dtype=np.uint8)
+    raw[::3] = rng.choice(np.frombuffer(b"ACGTNacgtn", dtype=np.uint8), size=raw[::3].size)
+    for upper in (False, True):
+        for to_n in (False, True):
+            buf = torch.from_numpy(raw.copy())
+            n = encoders.clean_ascii_host(buf, upper_case=upper, invalid_to_n=to_n)
+            want = O.clean_ascii(raw, upper, to_n)
+            assert np.array_equal(buf.numpy(), want)
+            if to_n:
+                up = O.clean_ascii(raw, upper, False)
+                assert n == int((up != want).sum())
+    assert encoders.clean_ascii_host(torch.empty(0, dtype=torch.uint8), upper_case=True, invalid_to_n=True) == 0
+
+
+def test_host_pack_2bit_matches_oracle():
+    import torch
+    from dnatok_amd import encoders
+    from oracle import oracle as O
+    rng = np.random.default_rng(4)
+    for b, t in ((1, 1), (3, 4), (5, 7), (2, 64), (9, 1001), (64, 8192)):
+        rows = rng.choice(np.frombuffer(b"ACGTNacgtnX", dtype=np.uint8), size=(b, t))
+        got = encoders.pack_2bit_host(torch.from_numpy(rows)).numpy()
+        assert got.shape == (b, (t + 3) // 4)
+        assert np.array_equal(got, O.pack_2bit(rows))
+    assert encoders.pack_2bit_host(torch.from_numpy(np.frombuffer(b"ACGT", dtype=np.uint8).reshape(1, 4).copy())
+                                   ).numpy().tolist() == [[0xE4]]
+    with pytest.raises(ValueError):
+        encoders.pack_2bit_host(torch.zeros(4, dtype=torch.uint8))

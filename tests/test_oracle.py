@@ -181,3 +181,37 @@ def test_kernel_vocab_first_seen_order():
     assert vocab[256:] == ["AC", "ACG", "GT", "CG"]       # 'CG' is interned before 'A'+'CG' reuses 'ACG'
     assert a.tolist() == [65, 256, 71, 65] and b2.tolist() == [67, 71, 84, 259]
     assert n.tolist() == [256, 257, 258, 257]
+
+
+# ------------------------------------------------------------------ 2-bit ingest
+
+def test_pack_2bit_known_bytes_and_round_trip():
+    as_rows = lambda s: np.frombuffer(s.encode(), dtype=np.uint8).reshape(1, -1)
+    assert O.pack_2bit(as_rows("ACGT")).tolist() == [[0xE4]]            # 0 | 1<<2 | 2<<4 | 3<<6
+    assert O.pack_2bit(as_rows("TTTT")).tolist() == [[0xFF]]
+    assert O.pack_2bit(as_rows("CA")).tolist() == [[0x01]]              # filled up with code 0
+    assert O.pack_2bit(as_rows("acgtN")).tolist() == [[0xE4, 0x00]]     # case folded, N travels as A
+    assert O.pack_2bit(as_rows("AAAAG")).tolist() == [[0x00, 0x02]]
+    # every packed byte spells its four bases back, first base in the low bits
+    lut = np.arange(256, dtype=np.int64)                                # id = ASCII code
+    every = np.arange(256, dtype=np.uint8).reshape(1, 256)
+    ids = O.unpack_2bit_ids(lut, every, 1024)[0].reshape(256, 4)
+    for b in (0, 1, 0x1B, 0xE4, 0xFF):
+        want = ["ACGT"[(b >> (2 * j)) & 3] for j in range(4)]
+        assert [chr(x) for x in ids[b]] == want
+    # round trip on ACGT text of every length mod 4; N reads back as A
+    rng = np.random.default_rng(5)
+    for t in (1, 2, 3, 4, 5, 63, 64, 257):
+        rows = rng.choice(np.frombuffer(b"ACGT", dtype=np.uint8), size=(7, t))
+        assert np.array_equal(O.unpack_2bit_ids(lut, O.pack_2bit(rows), t), rows)
+    start = lut + 1000
+    got = O.unpack_2bit_ids(lut, O.pack_2bit(as_rows("GATN")), 4, start_lut=start)
+    assert got.tolist() == [[ord("G") + 1000, ord("A"), ord("T"), ord("A")]]
+
+
+def test_clean_ascii_cases():
+    raw = np.frombuffer(b"acgtnACGTNxX-?rR", dtype=np.uint8)
+    assert O.clean_ascii(raw, False, False).tobytes() == b"acgtnACGTNxX-?rR"
+    assert O.clean_ascii(raw, True, False).tobytes() == b"ACGTNACGTNXX-?RR"
+    assert O.clean_ascii(raw, False, True).tobytes() == b"acgtnACGTNNNNNNN"
+    assert O.clean_ascii(raw, True, True).tobytes() == b"ACGTNACGTNNNNNNN"
