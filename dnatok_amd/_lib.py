@@ -21,7 +21,29 @@ EXPORTS = [
     "dnatok_kmer_table_create", "dnatok_kmer_table_destroy", "dnatok_kmer_encode_padded",
     "dnatok_bpe_table_create", "dnatok_bpe_table_destroy", "dnatok_bpe_scratch_bytes",
     "dnatok_bpe_encode", "dnatok_pack_ragged", "dnatok_pad_rows",
+    "dnatok_normalize_bounds", "dnatok_normalize_rows",
 ]
+
+
+class NormStep(ctypes.Structure):
+    """dnatok_norm_step of include/dnatok_hip.h."""
+    _fields_ = [("kind", c_int32), ("flags", c_int32), ("pattern_len", c_int32), ("content_len", c_int32),
+                ("pattern", ctypes.c_uint8 * 16), ("content", ctypes.c_uint8 * 16)]
+
+    @classmethod
+    def make(cls, kind: int, flags: int = 0, pattern: bytes = b"", content: bytes = b"") -> "NormStep":
+        if len(pattern) > 16 or len(content) > 16:
+            raise ValueError("normalizer pattern / content longer than 16 bytes")
+        st = cls(kind, flags, len(pattern), len(content))
+        for i, c in enumerate(pattern):
+            st.pattern[i] = c
+        for i, c in enumerate(content):
+            st.content[i] = c
+        return st
+
+
+NORM_STRIP, NORM_REPLACE, NORM_REPLACE_RUN, NORM_PREPEND, NORM_LOWERCASE = 1, 2, 3, 4, 5
+
 
 _lib = None
 
@@ -75,6 +97,10 @@ def lib() -> ctypes.CDLL:
                                      c_void_p, c_void_p, c_void_p]
     L.dnatok_pad_rows.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int32, c_int64,
                                   c_int64, c_void_p, c_void_p, c_void_p, c_void_p]
+    L.dnatok_normalize_bounds.argtypes = [c_void_p, c_int32, c_int64, c_int64, c_int64, POINTER(c_int64),
+                                          POINTER(c_int64), POINTER(c_size_t)]
+    L.dnatok_normalize_rows.argtypes = [c_void_p, c_int32, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                                        c_void_p, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]
     for name in EXPORTS:
         getattr(L, name)          # AttributeError here means the library is stale
     _lib = L

@@ -79,7 +79,7 @@ class DnatokBpeKernel:
         if b == 0:
             return (torch.empty((0, 0), dtype=torch.int32, device="cuda"),
                     torch.empty((0,), dtype=torch.int32, device="cuda"))
-        data, offsets, lens = encoders.bytes_from_strings(texts, "cuda")
+        data, offsets, lens = encoders.bytes_from_strings(texts, "cuda", encoding="utf-8")
         t_max = max(int(lens.max()), 1)
         total = int(data.numel())
         if impl.tok is None or impl.tok.numel() < max(total, 1):

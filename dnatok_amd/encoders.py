@@ -34,16 +34,26 @@ def _require_cuda(t: torch.Tensor, dtype: torch.dtype, name: str) -> None:
         raise ValueError(f"{name} must be a contiguous {dtype} tensor on the GPU")
 
 
-def bytes_from_strings(seqs: Sequence[str], device="cuda") -> Tuple[torch.Tensor, torch.Tensor, np.ndarray]:
-    """Concatenate ASCII strings into one device uint8 buffer + device int64 offsets.
+def bytes_from_strings(seqs: Sequence[str], device="cuda", encoding: str = "ascii"
+                       ) -> Tuple[torch.Tensor, torch.Tensor, np.ndarray]:
+    """Concatenate strings into one device uint8 buffer + device int64 offsets.
 
     Returns (data, offsets, host_lengths).  One join and one H2D copy per call
     (reference: DNATokBPE::tokenize_batch, src/dnatok_bpe_kernel/dnatok_bpe.cu:872-887).
+    ``encoding`` = "ascii": one byte per character, non-ASCII characters become ``?`` (what the
+    table paths of the reference do, src/dna_tokenizer.py:1793); "utf-8": the bytes the
+    reference's BPE kernel sees, since its binding receives ``std::string``.
     """
-    lens = np.fromiter((len(s) for s in seqs), dtype=np.int64, count=len(seqs))
+    joined = "".join(seqs)
+    if encoding == "utf-8" and not joined.isascii():
+        parts = [s.encode("utf-8") for s in seqs]
+        lens = np.fromiter((len(p) for p in parts), dtype=np.int64, count=len(parts))
+        buf = b"".join(parts)
+    else:
+        lens = np.fromiter((len(s) for s in seqs), dtype=np.int64, count=len(seqs))
+        buf = joined.encode("ascii", errors="replace")
     offsets = np.zeros(len(seqs) + 1, dtype=np.int64)
     np.cumsum(lens, out=offsets[1:])
-    buf = "".join(seqs).encode("ascii", errors="replace")
     host = torch.frombuffer(bytearray(buf), dtype=torch.uint8) if buf else torch.empty(0, dtype=torch.uint8)
     data = host.to(device)
     return data, torch.from_numpy(offsets).to(device), lens
@@ -78,6 +88,45 @@ def pack_2bit_host(ascii_rows: torch.Tensor, out: Optional[torch.Tensor] = None)
                                                 ctypes.c_void_p(out.data_ptr())),
                "dnatok_host_pack_2bit")
     return out
+
+
+class RowNormalizer:
+    """A tokenizer normalizer as a device program over ragged rows of bytes
+    (C ABI: dnatok_normalize_rows).  ``steps`` are ``_lib.NormStep`` records."""
+
+    def __init__(self, steps):
+        self.steps = list(steps)
+        self._arr = (_lib.NormStep * max(len(self.steps), 1))(*self.steps)
+        self._scratch: Optional[torch.Tensor] = None
+        rc = _lib.lib().dnatok_normalize_bounds(self._arr, len(self.steps), 0, 0, 0, None, None, None)
+        _lib.check(rc, "dnatok_normalize_bounds")
+
+    def bounds(self, n_rows: int, total: int, max_len: int) -> Tuple[int, int, int]:
+        """(total bytes, longest row, scratch bytes): upper bounds after the steps."""
+        t, m, sc = ctypes.c_int64(0), ctypes.c_int64(0), ctypes.c_size_t(0)
+        _lib.check(_lib.lib().dnatok_normalize_bounds(self._arr, len(self.steps), int(n_rows), int(total),
+                                                      int(max_len), ctypes.byref(t), ctypes.byref(m),
+                                                      ctypes.byref(sc)), "dnatok_normalize_bounds")
+        return int(t.value), int(m.value), int(sc.value)
+
+    def apply(self, data: torch.Tensor, offsets: torch.Tensor, total: int, max_len: int
+              ) -> Tuple[torch.Tensor, torch.Tensor, int, int]:
+        """(bytes, offsets, total bound, longest-row bound) of the normalized rows; the real
+        sizes stay on the device (``offsets[-1]``)."""
+        _require_cuda(data, torch.uint8, "data")
+        _require_cuda(offsets, torch.int64, "offsets")
+        n_rows = offsets.numel() - 1
+        out_total, out_max, need = self.bounds(n_rows, total, max_len)
+        if self._scratch is None or self._scratch.numel() < need or self._scratch.device != data.device:
+            self._scratch = torch.empty(max(need, 1), dtype=torch.uint8, device=data.device)   # grow-only
+        out = torch.empty(max(out_total, 1), dtype=torch.uint8, device=data.device)
+        out_offsets = torch.empty(n_rows + 1, dtype=torch.int64, device=data.device)
+        _lib.check(_lib.lib().dnatok_normalize_rows(self._arr, len(self.steps), _ptr(data), _ptr(offsets), n_rows,
+                                                    int(total), int(max_len), _ptr(out), out.numel(),
+                                                    _ptr(out_offsets), _ptr(self._scratch),
+                                                    self._scratch.numel(), _stream()),
+                   "dnatok_normalize_rows")
+        return out, out_offsets, out_total, out_max
 
 
 class CharEncoder:

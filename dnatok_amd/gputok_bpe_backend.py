@@ -24,7 +24,7 @@ from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple
 
 import torch
 
-from . import bpe_vocab, encoders
+from . import _lib, bpe_vocab, encoders
 
 
 # ------------------------------------------------------------------ tokenizer.json
@@ -107,6 +107,86 @@ def _compile_normalizer(cfg: Dict[str, Any]) -> Optional[Callable[[str], str]]:
     return fn
 
 
+_PLAIN = _re.compile(r"[A-Za-z0-9_ \-]")
+_RUN_RX = _re.compile(r"^(\\?.)(?:\{(\d+),\}|\+)$", _re.S)
+
+
+def _has_border(p: bytes) -> bool:
+    return any(p[:k] == p[len(p) - k:] for k in range(1, len(p)))
+
+
+def _device_steps_of(step: Dict[str, Any]) -> Optional[List[_lib.NormStep]]:
+    """One HF normalizer step as device steps (C ABI: dnatok_norm_step), or None when the
+    device pass cannot express it: a regex other than ``^``, ``c{n,}``, ``c+`` or a plain
+    literal, a literal that overlaps itself or is empty, anything longer than 16 bytes.  The
+    device steps act on the UTF-8 bytes of ASCII rows exactly as the callables of
+    ``_compile_normalizer_step`` act on the strings."""
+    if not isinstance(step, dict):
+        return None
+    kind = step.get("type")
+    try:
+        if kind == "Strip":
+            flags = (1 if step.get("strip_left", True) else 0) | (2 if step.get("strip_right", True) else 0)
+            return [_lib.NormStep.make(_lib.NORM_STRIP, flags)] if flags else []
+        if kind == "Replace":
+            pattern = step.get("pattern")
+            content = str(step.get("content", "")).encode("utf-8")
+            if isinstance(pattern, dict) and "String" in pattern:
+                lit = str(pattern["String"]).encode("utf-8")
+                if not lit or _has_border(lit) or not lit.isascii():
+                    return None
+                return [_lib.NormStep.make(_lib.NORM_REPLACE, 0, lit, content)]
+            if isinstance(pattern, dict) and "Regex" in pattern:
+                rx = str(pattern["Regex"])
+                if b"\\" in content:                      # group references / escapes in the replacement
+                    return None
+                if rx == "^":
+                    return [_lib.NormStep.make(_lib.NORM_PREPEND, 0, b"", content)]
+                m = _RUN_RX.match(rx)
+                if m:
+                    ch = m.group(1)
+                    if len(ch) == 2:                        # escaped: only punctuation escapes are literal
+                        ch = ch[1] if not ch[1].isalnum() else ""
+                    elif not _PLAIN.fullmatch(ch):
+                        ch = ""
+                    n = int(m.group(2)) if m.group(2) is not None else 1
+                    if len(ch) == 1 and ch.isascii() and 1 <= n <= 64:
+                        return [_lib.NormStep.make(_lib.NORM_REPLACE_RUN, n, ch.encode(), content)]
+                    return None
+                if rx and all(_PLAIN.fullmatch(c) for c in rx) and not _has_border(rx.encode()):
+                    return [_lib.NormStep.make(_lib.NORM_REPLACE, 0, rx.encode(), content)]
+            return None
+        if kind == "Prepend":
+            return [_lib.NormStep.make(_lib.NORM_PREPEND, 0, b"", str(step.get("prepend", "")).encode("utf-8"))]
+        if kind == "Lowercase":
+            return [_lib.NormStep.make(_lib.NORM_LOWERCASE)]
+        if kind in (None, "NFC", "NFKC", "NFD", "NFKD", "StripAccents"):
+            return []
+        if kind == "Sequence":
+            out: List[_lib.NormStep] = []
+            for sub in step.get("normalizers", []):
+                part = _device_steps_of(sub)
+                if part is None:
+                    return None
+                out.extend(part)
+            return out
+    except ValueError:                                      # longer than the step record holds
+        return None
+    return None
+
+
+def _compile_device_normalizer(cfg: Dict[str, Any]) -> Optional["encoders.RowNormalizer"]:
+    """The tokenizer's normalizer as a device program, or None (no normalizer, or one the
+    device pass cannot express: the host callables are used then)."""
+    norm = cfg.get("normalizer")
+    if norm is None:
+        return None
+    steps = _device_steps_of(norm)
+    if steps is None:
+        return None
+    return encoders.RowNormalizer(steps)
+
+
 def _extract_merges(cfg: Dict[str, Any]) -> List[str]:
     """Merges as ``"a b"`` strings in rank order (reference: 251-262)."""
     out: List[str] = []
@@ -171,11 +251,14 @@ class GPUTokBPEBackend:
                                "this backend ships the 'dnatok' engine only")
         self.tokenizer = hf_tokenizer
         self.engine = engine
+        self.normalize_on_device = True
         cfg = _read_tokenizer_json(hf_tokenizer)
         ok, reason = _supported_tokenizer(cfg)
         if not ok:
             raise RuntimeError(f"GPUTokBPEBackend cannot accelerate this tokenizer: {reason}")
         self._normalize = _compile_normalizer(cfg)
+        # the same steps as a device program, used for all-ASCII batches; None: host callables
+        self._normalize_device = _compile_device_normalizer(cfg) if self._normalize is not None else None
         self._merges: List[str] = _extract_merges(cfg)
         if not self._merges:
             raise RuntimeError("Tokenizer has no merges; nothing to accelerate.")
@@ -255,13 +338,23 @@ class GPUTokBPEBackend:
                      ) -> Tuple[torch.Tensor, torch.Tensor]:
         if not seqs:
             raise ValueError("No sequences provided.")
-        norm = [self._normalize(s) for s in seqs] if self._normalize is not None else list(seqs)
         dev = torch.device(device) if not isinstance(device, torch.device) else device
         if dev.type != "cuda":
             raise RuntimeError("GPUTokBPEBackend.encode_batch runs on the GPU only (device='cuda')")
-        data, offsets, lens = encoders.bytes_from_strings(norm, dev)
+        if self._normalize is None:
+            data, offsets, lens = encoders.bytes_from_strings(seqs, dev, encoding="utf-8")
+            t_cap = int(lens.max())
+        elif self._normalize_device is not None and self.normalize_on_device and "".join(seqs).isascii():
+            # raw bytes up, normalizer steps as compaction passes on the device; the sizes after
+            # them stay on the device, the engine is sized by their upper bounds
+            data, offsets, lens = encoders.bytes_from_strings(seqs, dev, encoding="utf-8")
+            data, offsets, _, t_cap = self._normalize_device.apply(data, offsets, int(lens.sum()), int(lens.max()))
+        else:
+            norm = [self._normalize(s) for s in seqs]
+            data, offsets, lens = encoders.bytes_from_strings(norm, dev, encoding="utf-8")
+            t_cap = int(lens.max())
         b = len(seqs)
-        t_cap = max(int(lens.max()), 1)
+        t_cap = max(t_cap, 1)
         ids32, mask, lengths, longest = self.encode_device(data, offsets, t_cap)
         width = int(longest.item())                       # the one host sync: the output shape
         if int(lengths.min().item()) < 0:

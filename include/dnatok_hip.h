@@ -188,6 +188,49 @@ int dnatok_pad_rows(const int32_t *tok_tmp, const int64_t *in_offsets, const int
                     int64_t n_rows, const int32_t *remap, int32_t pad_id, int64_t t_cap,
                     int64_t fill_to, int32_t *ids, uint8_t *mask, int32_t *max_len, void *stream);
 
+/* ---------------------------------------------------------------------------------------
+ * Tokenizer normalizer on the device: the steps GPUTokBPEBackend compiles from a
+ * tokenizer.json "normalizer" and applies string by string on the host before the kernel
+ * (_compile_normalizer_step / _compile_normalizer, src/gputok_bpe_backend.py:179-248; applied at
+ * 531-535), here applied to the ragged rows of bytes already on the device.
+ * ------------------------------------------------------------------------------------- */
+
+#define DNATOK_NORM_MAX_BYTES   16   /* longest pattern / replacement / prefix of a step */
+
+#define DNATOK_NORM_STRIP        1   /* flags bit 0: left, bit 1: right; ASCII whitespace as str.strip() */
+#define DNATOK_NORM_REPLACE      2   /* every occurrence of pattern -> content (str.replace); the pattern
+                                        must not overlap itself (no proper prefix equal to a suffix) */
+#define DNATOK_NORM_REPLACE_RUN  3   /* every maximal run of the byte pattern[0] that is at least `flags`
+                                        long -> one content (the regex  c{n,}  with n = flags, 1..64) */
+#define DNATOK_NORM_PREPEND      4   /* content in front of every row, empty rows included */
+#define DNATOK_NORM_LOWERCASE    5   /* A-Z -> a-z */
+
+typedef struct dnatok_norm_step {
+    int32_t kind;
+    int32_t flags;
+    int32_t pattern_len;
+    int32_t content_len;
+    uint8_t pattern[DNATOK_NORM_MAX_BYTES];
+    uint8_t content[DNATOK_NORM_MAX_BYTES];
+} dnatok_norm_step;
+
+/* Host-side arithmetic (steps_h is a host array): upper bounds of the total bytes and of the
+ * longest row after the steps, for a batch of n_rows rows of `total` bytes whose longest row has
+ * max_len bytes, and the bytes of device scratch dnatok_normalize_rows needs.  Also validates the
+ * steps.  Any of the three outputs may be NULL. */
+int dnatok_normalize_bounds(const dnatok_norm_step *steps_h, int32_t n_steps, int64_t n_rows,
+                            int64_t total, int64_t max_len, int64_t *out_total, int64_t *out_max_len,
+                            size_t *scratch_bytes);
+
+/* Applies the steps in order to rows bytes[offsets[b] .. offsets[b+1]) (offsets[0] = 0,
+ * offsets[n_rows] = total) and writes the rows back to back into out_bytes (capacity at least the
+ * out_total bound) with their boundaries in out_offsets int64[n_rows + 1].  The input is left
+ * untouched; sizes after the first step exist only on the device, so nothing is read back. */
+int dnatok_normalize_rows(const dnatok_norm_step *steps_h, int32_t n_steps, const uint8_t *bytes,
+                          const int64_t *offsets, int64_t n_rows, int64_t total, int64_t max_len,
+                          uint8_t *out_bytes, int64_t out_capacity, int64_t *out_offsets,
+                          void *scratch, size_t scratch_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -257,6 +257,117 @@ def test_bpe_backend_with_normalizer():
         assert ids[i, :len(e.ids)].tolist() == e.ids and int(mask[i].sum()) == len(e.ids)
 
 
+def _rows_to_device(rows):
+    from dnatok_amd import encoders
+    return encoders.bytes_from_strings(rows, "cuda", encoding="utf-8")
+
+
+def _rows_from_device(data, offsets):
+    off = offsets.cpu().numpy()
+    raw = data.cpu().numpy().tobytes()
+    return [raw[off[i]:off[i + 1]].decode("utf-8") for i in range(len(off) - 1)]
+
+
+NORMALIZER_CASES = [
+    {"type": "Strip", "strip_left": True, "strip_right": True},
+    {"type": "Strip", "strip_left": True, "strip_right": False},
+    {"type": "Strip", "strip_left": False, "strip_right": True},
+    {"type": "Replace", "pattern": {"Regex": "N{10,}"}, "content": "-"},
+    {"type": "Replace", "pattern": {"Regex": "N{10,}"}, "content": ""},
+    {"type": "Replace", "pattern": {"Regex": "N+"}, "content": "<run-of-N>"},
+    {"type": "Replace", "pattern": {"Regex": "N{3,}"}, "content": "0123456789abcdef"},
+    {"type": "Replace", "pattern": {"String": "N"}, "content": "nn"},
+    {"type": "Replace", "pattern": {"String": "ACG"}, "content": "x"},
+    {"type": "Replace", "pattern": {"String": "GT"}, "content": "[gt-pair]"},
+    {"type": "Replace", "pattern": {"Regex": "^"}, "content": "_"},
+    {"type": "Prepend", "prepend": "\u2581"},
+    {"type": "Lowercase"},
+    {"type": "Sequence", "normalizers": [
+        {"type": "Strip", "strip_left": True, "strip_right": True},
+        {"type": "Replace", "pattern": {"Regex": "N{10,}"}, "content": "-"},
+        {"type": "Prepend", "prepend": "_"},
+        {"type": "NFC"},
+        {"type": "Lowercase"}]},
+    {"type": "Sequence", "normalizers": [
+        {"type": "Lowercase"},
+        {"type": "Replace", "pattern": {"String": "acgt"}, "content": "ACGTACGT"},
+        {"type": "Replace", "pattern": {"Regex": "n{2,}"}, "content": "N"},
+        {"type": "Replace", "pattern": {"String": "TA"}, "content": ""}]},
+]
+
+
+@pytest.mark.parametrize("case", range(len(NORMALIZER_CASES)))
+def test_device_normalizer_equals_the_host_callables(case):
+    """Every normalizer step the device pass expresses, on rows built to hit its edges: empty
+    rows (also first and last), rows of nothing but whitespace or N, runs of 9 / 10 / 11 N at row
+    starts and ends, runs and matches that straddle the 16-position lane spans and the
+    4096-position tiles; expected values from the str -> str callables (the reference's form)."""
+    from dnatok_amd.gputok_bpe_backend import _compile_normalizer_step, _device_steps_of
+    from dnatok_amd import encoders
+    step = NORMALIZER_CASES[case]
+    host = _compile_normalizer_step(step)
+    steps = _device_steps_of(step)
+    assert host is not None and steps is not None
+    rng = random.Random(case)
+    rows = ["", "N" * 9, "N" * 10, "N" * 11, "  \t ", " ", "ACGT", "  ACGTN" + "N" * 12 + "ACG \n", "",
+            "N" * 10 + "A" + "N" * 9 + "C" + "N" * 30, "GTGTGT", "ACGACGAC", "TTACGTTTA", "NNN", "N", "G", "T" + "N" * 4095,
+            "N" * 5000, "\x1c\x1fAC\x0b\x0c", ""]
+    for n in (15, 16, 17, 31, 33, 4090, 4096, 4100, 9000):
+        body = "".join(rng.choice("ACGTN") for _ in range(n))
+        rows.append(body)
+        rows.append("A" * (n - 5) + "N" * 12 + body[:7])          # a run across the n-th position
+        rows.append("C" * (n - 2) + "ACGT" + "GT" * 3)            # matches across it
+    rng.shuffle(rows)
+    rows = [""] + rows + [""]
+    data, offsets, lens = _rows_to_device(rows)
+    norm = encoders.RowNormalizer(steps)
+    out, out_off, total_bound, longest_bound = norm.apply(data, offsets, int(lens.sum()), int(lens.max()))
+    torch.cuda.synchronize()
+    want = [host(r) for r in rows]
+    got = _rows_from_device(out, out_off)
+    assert got == want
+    want_bytes = [len(w.encode("utf-8")) for w in want]
+    assert sum(want_bytes) <= total_bound and max(want_bytes) <= longest_bound
+    # the input is left as it was
+    assert _rows_from_device(data, offsets) == rows
+    # no rows at all, and one empty row
+    for few in ([], [""]):
+        d2, o2, l2 = _rows_to_device(few)
+        out2, off2, _, _ = norm.apply(d2, o2, 0, 0)
+        assert _rows_from_device(out2, off2) == [host(r) for r in few]
+
+
+def test_bpe_backend_normalizes_on_the_device_like_on_the_host():
+    import json
+    from tokenizers import Tokenizer
+    cfg = dict(util.tokenizer_json("4096"))
+    cfg["normalizer"] = {"type": "Sequence", "normalizers": [
+        {"type": "Strip", "strip_left": True, "strip_right": True},
+        {"type": "Replace", "pattern": {"Regex": "N{10,}"}, "content": "N"}]}
+    tk = Tokenizer.from_str(json.dumps(cfg))
+    be = GPUTokBPEBackend(tk)
+    assert be._normalize_device is not None and be.normalize_on_device
+    random.seed(3)
+    seqs = []
+    for _ in range(200):
+        n = random.choice([0, 1, 5, 64, 500, 3000, 9000])
+        body = "".join(random.choice("ACGT") for _ in range(n))
+        if n > 40 and random.random() < 0.7:
+            at = random.randrange(n - 30)
+            body = body[:at] + "N" * random.choice([3, 9, 10, 11, 25]) + body[at + 25:]
+        seqs.append(random.choice(["", " ", "  "]) + body + random.choice(["", "\n", " "]))
+    ids, mask = be.encode_batch(seqs)
+    be.normalize_on_device = False
+    ids_h, mask_h = be.encode_batch(seqs)
+    assert torch.equal(ids, ids_h) and torch.equal(mask, mask_h)
+    for i, e in enumerate(tk.encode_batch(seqs, add_special_tokens=False)):
+        assert ids[i, :len(e.ids)].tolist() == e.ids and int(mask[i].sum()) == len(e.ids)
+    # a regex the device pass does not express keeps the host callables
+    cfg["normalizer"] = {"type": "Replace", "pattern": {"Regex": "[NX]{2,}"}, "content": "N"}
+    be2 = GPUTokBPEBackend(Tokenizer.from_str(json.dumps(cfg)))
+    assert be2._normalize_device is None and be2._normalize is not None
+
+
 def test_dnatok_routes_bpe_tokenizers_to_the_backend():
     tk = hf.load_bpe_tokenizer("4096")
 

@@ -118,3 +118,49 @@ def test_host_pack_2bit_matches_oracle():
                                    ).numpy().tolist() == [[0xE4]]
     with pytest.raises(ValueError):
         encoders.pack_2bit_host(torch.zeros(4, dtype=torch.uint8))
+
+
+# ------------------------------------------------------------------ device normalizer: host-side compile
+
+def test_device_normalizer_compile_and_validation():
+    import ctypes
+    from dnatok_amd import _lib
+    from dnatok_amd.gputok_bpe_backend import _device_steps_of
+    kinds = lambda step: [(s.kind, s.flags, bytes(s.pattern[:s.pattern_len]), bytes(s.content[:s.content_len]))
+                          for s in _device_steps_of(step)]
+    assert kinds({"type": "Strip", "strip_left": True, "strip_right": False}) == [(_lib.NORM_STRIP, 1, b"", b"")]
+    assert kinds({"type": "Strip", "strip_left": False, "strip_right": False}) == []
+    assert kinds({"type": "Replace", "pattern": {"Regex": "N{10,}"}, "content": "-"}) == \
+        [(_lib.NORM_REPLACE_RUN, 10, b"N", b"-")]
+    assert kinds({"type": "Replace", "pattern": {"Regex": "N+"}, "content": ""}) == [(_lib.NORM_REPLACE_RUN, 1, b"N", b"")]
+    assert kinds({"type": "Replace", "pattern": {"Regex": "\\-{2,}"}, "content": "-"}) == \
+        [(_lib.NORM_REPLACE_RUN, 2, b"-", b"-")]
+    assert kinds({"type": "Replace", "pattern": {"Regex": "^"}, "content": "_"}) == [(_lib.NORM_PREPEND, 0, b"", b"_")]
+    assert kinds({"type": "Replace", "pattern": {"String": "AC"}, "content": "x"}) == [(_lib.NORM_REPLACE, 0, b"AC", b"x")]
+    assert kinds({"type": "Prepend", "prepend": "\u2581"}) == [(_lib.NORM_PREPEND, 0, b"", "\u2581".encode())]
+    assert kinds({"type": "Sequence", "normalizers": [{"type": "NFKC"}, {"type": "Lowercase"}]}) == \
+        [(_lib.NORM_LOWERCASE, 0, b"", b"")]
+    for not_on_device in (
+            {"type": "Replace", "pattern": {"Regex": "[NX]{2,}"}, "content": "N"},      # a character class
+            {"type": "Replace", "pattern": {"Regex": ".{3,}"}, "content": "N"},         # any character
+            {"type": "Replace", "pattern": {"Regex": "\\d+"}, "content": "N"},          # a class escape
+            {"type": "Replace", "pattern": {"Regex": "(N)\\1"}, "content": "N"},
+            {"type": "Replace", "pattern": {"Regex": "N{10,}"}, "content": "\\g<0>"},   # group reference
+            {"type": "Replace", "pattern": {"Regex": "N{100,}"}, "content": "N"},       # longer than the window
+            {"type": "Replace", "pattern": {"String": "AA"}, "content": "x"},           # overlaps itself
+            {"type": "Replace", "pattern": {"String": "ATA"}, "content": "x"},
+            {"type": "Replace", "pattern": {"String": ""}, "content": "x"},
+            {"type": "Replace", "pattern": {"String": "ACGTACGTACGTACGTA"[:17] + "C"}, "content": "x"},
+            {"type": "Prepend", "prepend": "x" * 17},
+            {"type": "BertNormalizer"}):
+        assert _device_steps_of(not_on_device) is None, not_on_device
+    # the library validates the records itself as well
+    L = _lib.lib()
+    bad = (_lib.NormStep * 1)(_lib.NormStep.make(_lib.NORM_REPLACE, 0, b"AA", b"x"))
+    assert L.dnatok_normalize_bounds(bad, 1, 1, 10, 10, None, None, None) == -1
+    assert b"overlaps itself" in L.dnatok_last_error()
+    run = (_lib.NormStep * 2)(_lib.NormStep.make(_lib.NORM_REPLACE_RUN, 3, b"N", b"0123456789"),
+                              _lib.NormStep.make(_lib.NORM_PREPEND, 0, b"", b"__"))
+    t, m, sc = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_size_t()
+    assert L.dnatok_normalize_bounds(run, 2, 4, 100, 30, ctypes.byref(t), ctypes.byref(m), ctypes.byref(sc)) == 0
+    assert (t.value, m.value) == (33 * 10 + 1 + 8, 100 + 2) and sc.value >= 2 * t.value
