@@ -16,7 +16,8 @@ LIB_PATH = os.path.join(_HERE, "libdnatok_hip.so")
 EXPORTS = [
     "dnatok_version", "dnatok_last_error",
     "dnatok_char_table_create", "dnatok_char_table_destroy",
-    "dnatok_char_encode_padded", "dnatok_char_encode_packed", "dnatok_char_embed_packed",
+    "dnatok_char_encode_padded", "dnatok_char_encode_padded_as", "dnatok_char_encode_packed",
+    "dnatok_char_embed_packed",
     "dnatok_char_unpack_2bit", "dnatok_host_clean_ascii", "dnatok_host_pack_2bit",
     "dnatok_kmer_table_create", "dnatok_kmer_table_destroy", "dnatok_kmer_encode_padded",
     "dnatok_bpe_table_create", "dnatok_bpe_table_destroy", "dnatok_bpe_scratch_bytes",
@@ -72,6 +73,8 @@ def lib() -> ctypes.CDLL:
     L.dnatok_char_table_destroy.restype = None
     L.dnatok_char_encode_padded.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int,
                                             c_void_p, c_void_p, c_void_p]
+    L.dnatok_char_encode_padded_as.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int,
+                                               c_void_p, c_int32, c_void_p, c_void_p]
     L.dnatok_char_encode_packed.argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_void_p,
                                             c_void_p, c_void_p]
     L.dnatok_char_embed_packed.argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int32,

@@ -43,6 +43,30 @@ __device__ __forceinline__ int4v lookup4(const int32_t *lut, uint32_t w)
     return v;
 }
 
+// Four ids of one of the output widths (uint8, int16, int32, int64) as one store.
+template <typename OUT> struct Quad;
+template <> struct Quad<uint8_t> { typedef uint32_t type; };
+template <> struct Quad<int16_t> { typedef int16_t type __attribute__((ext_vector_type(4))); };
+template <> struct Quad<int32_t> { typedef int4v type; };
+template <> struct Quad<int64_t> { typedef int64_t type __attribute__((ext_vector_type(4))); };
+
+template <typename OUT>
+__device__ __forceinline__ typename Quad<OUT>::type make_quad(int4v v);
+template <> __device__ __forceinline__ uint32_t make_quad<uint8_t>(int4v v)
+{
+    return (uint32_t)(v.x & 255) | ((uint32_t)(v.y & 255) << 8) | ((uint32_t)(v.z & 255) << 16) |
+           ((uint32_t)v.w << 24);
+}
+template <> __device__ __forceinline__ Quad<int16_t>::type make_quad<int16_t>(int4v v)
+{
+    return Quad<int16_t>::type{(int16_t)v.x, (int16_t)v.y, (int16_t)v.z, (int16_t)v.w};
+}
+template <> __device__ __forceinline__ int4v make_quad<int32_t>(int4v v) { return v; }
+template <> __device__ __forceinline__ Quad<int64_t>::type make_quad<int64_t>(int4v v)
+{
+    return Quad<int64_t>::type{(int64_t)v.x, (int64_t)v.y, (int64_t)v.z, (int64_t)v.w};
+}
+
 // Flat stream; requires bytes 4-byte aligned, ids 16-byte aligned, mask 4-byte aligned.
 template <bool HAS_MASK, bool HAS_START>
 __global__ __launch_bounds__(kCharThreads) void char_packed_kernel(
@@ -102,13 +126,14 @@ __global__ __launch_bounds__(kCharThreads) void char_packed_kernel(
 }
 
 // Ragged rows to a padded [n_rows, t_out] matrix.  One tile = 1024 output columns of one row.
-// ALIGNED: t_out % 4 == 0 and ids / mask bases are 16- / 4-byte aligned, so each lane stores
-// its 4 columns with one 16-byte and one 4-byte store.
-template <bool HAS_MASK, bool HAS_START, bool ALIGNED>
+// ALIGNED: t_out % 4 == 0, the ids base is aligned to four ids and the mask base to 4 bytes, so
+// each lane stores its 4 columns with one store of four ids and one 4-byte store.  OUT is the
+// width the ids are written in.
+template <typename OUT, bool HAS_MASK, bool HAS_START, bool ALIGNED>
 __global__ __launch_bounds__(kCharThreads) void char_padded_kernel(
     const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets, int64_t n_rows,
     int64_t t_out, int64_t tiles_per_row, int pad_left, int32_t pad_id,
-    const CharTableDev *__restrict__ tab, int32_t *__restrict__ ids, uint8_t *__restrict__ mask)
+    const CharTableDev *__restrict__ tab, OUT *__restrict__ ids, uint8_t *__restrict__ mask)
 {
     __shared__ int32_t lut[256];
     __shared__ int32_t start[256];
@@ -148,17 +173,17 @@ __global__ __launch_bounds__(kCharThreads) void char_padded_kernel(
                 }
             }
         }
-        int32_t *o = ids + b * t_out + col0;
+        OUT *o = ids + b * t_out + col0;
         if (ALIGNED) {
-            int4v vv = {v[0], v[1], v[2], v[3]};
-            __builtin_nontemporal_store(vv, reinterpret_cast<int4v *>(o));
+            const int4v vv = {v[0], v[1], v[2], v[3]};
+            __builtin_nontemporal_store(make_quad<OUT>(vv), reinterpret_cast<typename Quad<OUT>::type *>(o));
             if (HAS_MASK)
                 __builtin_nontemporal_store(m, reinterpret_cast<uint32_t *>(mask + b * t_out + col0));
         } else {
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 if (col0 + k < t_out) {
-                    o[k] = v[k];
+                    o[k] = (OUT)v[k];
                     if (HAS_MASK) mask[b * t_out + col0 + k] = (uint8_t)((m >> (8 * k)) & 1u);
                 }
             }
@@ -340,24 +365,6 @@ namespace dnatok {
 constexpr int kUnpackSteps = 8;                                  // packed bytes per lane per tile
 constexpr int kUnpackTile = kCharThreads * kUnpackSteps;         // 2048 packed bytes = 8192 bases
 
-template <typename OUT> struct Quad;
-template <> struct Quad<uint8_t> { typedef uint32_t type; };
-template <> struct Quad<int32_t> { typedef int4v type; };
-template <> struct Quad<int64_t> { typedef int64_t type __attribute__((ext_vector_type(4))); };
-
-template <typename OUT>
-__device__ __forceinline__ typename Quad<OUT>::type make_quad(int4v v);
-template <> __device__ __forceinline__ uint32_t make_quad<uint8_t>(int4v v)
-{
-    return (uint32_t)(v.x & 255) | ((uint32_t)(v.y & 255) << 8) | ((uint32_t)(v.z & 255) << 16) |
-           ((uint32_t)v.w << 24);
-}
-template <> __device__ __forceinline__ int4v make_quad<int32_t>(int4v v) { return v; }
-template <> __device__ __forceinline__ Quad<int64_t>::type make_quad<int64_t>(int4v v)
-{
-    return Quad<int64_t>::type{(int64_t)v.x, (int64_t)v.y, (int64_t)v.z, (int64_t)v.w};
-}
-
 // QUADS: row_len % 4 == 0 and ids aligned to 4 elements, so the packed stream and the output are
 // both flat and every packed byte owns one aligned group of four cells.  Otherwise rows are
 // ceil(row_len / 4) packed bytes each and cells are stored one by one.
@@ -447,24 +454,22 @@ extern "C" int dnatok_char_unpack_2bit(const dnatok_char_t *t, const uint8_t *pa
     return launch_unpack2bit<int64_t>(t, packed, n_rows, row_len, ids, s);
 }
 
-extern "C" int dnatok_char_encode_padded(const dnatok_char_t *t, const uint8_t *bytes,
-                                         const int64_t *offsets, int64_t n_rows, int64_t t_out,
-                                         int pad_left, int32_t *ids, uint8_t *mask, void *stream)
+namespace dnatok {
+
+template <typename OUT>
+static int launch_char_padded(const dnatok_char_table *t, const uint8_t *bytes, const int64_t *offsets,
+                              int64_t n_rows, int64_t t_out, int pad_left, void *ids_v, uint8_t *mask,
+                              hipStream_t s)
 {
-    DNATOK_REQUIRE(t && offsets, DNATOK_E_INVALID, "dnatok_char_encode_padded: null argument");
-    DNATOK_REQUIRE(n_rows >= 0 && t_out >= 0, DNATOK_E_INVALID,
-                   "dnatok_char_encode_padded: negative size");
-    if (n_rows == 0 || t_out == 0) return DNATOK_OK;
-    DNATOK_REQUIRE(ids, DNATOK_E_INVALID, "dnatok_char_encode_padded: null output");
-    hipStream_t s = (hipStream_t)stream;
+    OUT *ids = (OUT *)ids_v;
     const int64_t tiles_per_row = (t_out + kCharThreads * 4 - 1) / (kCharThreads * 4);
     const int grid = grid_for(n_rows * tiles_per_row);
-    const bool aligned = (t_out % 4 == 0) && ((uintptr_t)ids & 15) == 0 && ((uintptr_t)mask & 3) == 0;
+    const bool aligned = (t_out % 4 == 0) && ((uintptr_t)ids % (4 * sizeof(OUT))) == 0 && ((uintptr_t)mask & 3) == 0;
     const bool hs = t->has_start;
-#define LAUNCH(M, S, A)                                                                          \
-    char_padded_kernel<M, S, A><<<grid, kCharThreads, 0, s>>>(bytes, offsets, n_rows, t_out,      \
-                                                              tiles_per_row, pad_left, t->pad_id, \
-                                                              t->dev, ids, mask)
+#define LAUNCH(M, S, A)                                                                               \
+    char_padded_kernel<OUT, M, S, A><<<grid, kCharThreads, 0, s>>>(bytes, offsets, n_rows, t_out,      \
+                                                                   tiles_per_row, pad_left, t->pad_id, \
+                                                                   t->dev, ids, mask)
     if (mask) {
         if (hs) { if (aligned) LAUNCH(true, true, true); else LAUNCH(true, true, false); }
         else    { if (aligned) LAUNCH(true, false, true); else LAUNCH(true, false, false); }
@@ -475,4 +480,36 @@ extern "C" int dnatok_char_encode_padded(const dnatok_char_t *t, const uint8_t *
 #undef LAUNCH
     DNATOK_HIP_TRY(hipGetLastError());
     return DNATOK_OK;
+}
+
+}  // namespace dnatok
+
+extern "C" int dnatok_char_encode_padded_as(const dnatok_char_t *t, const uint8_t *bytes,
+                                            const int64_t *offsets, int64_t n_rows, int64_t t_out,
+                                            int pad_left, void *ids, int32_t id_bytes, uint8_t *mask,
+                                            void *stream)
+{
+    DNATOK_REQUIRE(t && offsets, DNATOK_E_INVALID, "dnatok_char_encode_padded: null argument");
+    DNATOK_REQUIRE(n_rows >= 0 && t_out >= 0, DNATOK_E_INVALID,
+                   "dnatok_char_encode_padded: negative size");
+    DNATOK_REQUIRE(id_bytes == 1 || id_bytes == 2 || id_bytes == 4 || id_bytes == 8, DNATOK_E_INVALID,
+                   "dnatok_char_encode_padded: id_bytes must be 1, 2, 4 or 8 (got %d)", (int)id_bytes);
+    if (n_rows == 0 || t_out == 0) return DNATOK_OK;
+    DNATOK_REQUIRE(ids, DNATOK_E_INVALID, "dnatok_char_encode_padded: null output");
+    DNATOK_REQUIRE(((uintptr_t)ids % (size_t)id_bytes) == 0, DNATOK_E_INVALID,
+                   "dnatok_char_encode_padded: ids not aligned to its element size");
+    hipStream_t s = (hipStream_t)stream;
+    switch (id_bytes) {
+    case 1: return launch_char_padded<uint8_t>(t, bytes, offsets, n_rows, t_out, pad_left, ids, mask, s);
+    case 2: return launch_char_padded<int16_t>(t, bytes, offsets, n_rows, t_out, pad_left, ids, mask, s);
+    case 4: return launch_char_padded<int32_t>(t, bytes, offsets, n_rows, t_out, pad_left, ids, mask, s);
+    default: return launch_char_padded<int64_t>(t, bytes, offsets, n_rows, t_out, pad_left, ids, mask, s);
+    }
+}
+
+extern "C" int dnatok_char_encode_padded(const dnatok_char_t *t, const uint8_t *bytes,
+                                         const int64_t *offsets, int64_t n_rows, int64_t t_out,
+                                         int pad_left, int32_t *ids, uint8_t *mask, void *stream)
+{
+    return dnatok_char_encode_padded_as(t, bytes, offsets, n_rows, t_out, pad_left, ids, 4, mask, stream);
 }

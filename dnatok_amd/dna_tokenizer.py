@@ -430,6 +430,18 @@ class DNATok:
         k = int(self.kmer_k) if self.kmer_k else 1
         max_chars = int(max_tokens) * k
         seqs = [s[:max_chars] for s in seqs]
+        max_id = max(int(self.vocab_size) - 1, int(self.id_pad))
+        narrow = _smallest_dtype(max_id)
+        if self._char_enc is not None and self._kmer_enc is None and self.bpe_backend is None:
+            # single-nucleotide tables: one kernel writes the final width, padding side and dtype
+            data, offsets, lens = encoders.bytes_from_strings(seqs, "cuda")
+            target = int(lens.max())
+            if pad_to_max:
+                target = max(target, int(max_tokens))
+            if pad_multiple > 1 and target % pad_multiple:
+                target += pad_multiple - target % pad_multiple
+            return self._char_enc.encode_padded(data, offsets, target, pad_left=(self.padding_side == "left"),
+                                                dtype=narrow)
         old = self.token_len
         self.token_len = None
         try:
@@ -445,11 +457,9 @@ class DNATok:
             extra = target - ids.shape[1]
             pad_i = torch.full((ids.shape[0], extra), int(self.id_pad), dtype=ids.dtype, device=ids.device)
             pad_m = torch.zeros((ids.shape[0], extra), dtype=torch.uint8, device=ids.device)
-            left = self.padding_side == "left" and self._char_enc is not None
-            ids = torch.cat([pad_i, ids] if left else [ids, pad_i], dim=1)
-            mask = torch.cat([pad_m, mask] if left else [mask, pad_m], dim=1)
-        max_id = max(int(self.vocab_size) - 1, int(self.id_pad))
-        return ids.to(_smallest_dtype(max_id)), mask
+            ids = torch.cat([ids, pad_i], dim=1)
+            mask = torch.cat([mask, pad_m], dim=1)
+        return ids.to(narrow), mask
 
     # ------------------------------------------------------------------ bytes path
 

@@ -153,18 +153,25 @@ class CharEncoder:
                 pass
 
     def encode_padded(self, data: torch.Tensor, offsets: torch.Tensor, t_out: int, *,
-                      pad_left: bool = False, want_mask: bool = True,
+                      pad_left: bool = False, want_mask: bool = True, dtype: torch.dtype = torch.int32,
                       ids: Optional[torch.Tensor] = None, mask: Optional[torch.Tensor] = None):
+        """Ragged rows -> ids [B, t_out] of ``dtype`` (uint8, int16, int32 or int64) and mask
+        uint8 [B, t_out], padded with the pad id on the right, or on the left with ``pad_left``."""
         _require_cuda(data, torch.uint8, "data")
         _require_cuda(offsets, torch.int64, "offsets")
+        if dtype not in (torch.uint8, torch.int16, torch.int32, torch.int64):
+            raise ValueError("dtype must be uint8, int16, int32 or int64")
         n_rows = offsets.numel() - 1
         if ids is None:
-            ids = torch.empty((n_rows, t_out), dtype=torch.int32, device=data.device)
+            ids = torch.empty((n_rows, t_out), dtype=dtype, device=data.device)
+        else:
+            _require_cuda(ids, dtype, "ids")
         if want_mask and mask is None:
             mask = torch.empty((n_rows, t_out), dtype=torch.uint8, device=data.device)
-        _lib.check(_lib.lib().dnatok_char_encode_padded(self._h, _ptr(data), _ptr(offsets), n_rows,
-                                                        int(t_out), int(pad_left), _ptr(ids),
-                                                        _ptr(mask if want_mask else None), _stream()),
+        _lib.check(_lib.lib().dnatok_char_encode_padded_as(self._h, _ptr(data), _ptr(offsets), n_rows,
+                                                           int(t_out), int(pad_left), _ptr(ids),
+                                                           ids.element_size(),
+                                                           _ptr(mask if want_mask else None), _stream()),
                    "dnatok_char_encode_padded")
         return ids, (mask if want_mask else None)
 

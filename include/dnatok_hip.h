@@ -60,6 +60,15 @@ int dnatok_char_encode_padded(const dnatok_char_t *t, const uint8_t *bytes, cons
                               int64_t n_rows, int64_t t_out, int pad_left,
                               int32_t *ids, uint8_t *mask, void *stream);
 
+/* The same with ids of id_bytes-wide integers (1: uint8, 2: int16, 4: int32, 8: int64; an id that
+ * does not fit is cut to the width): what DNATok.encode_batch_with_padding returns once it has
+ * narrowed its ids to the smallest type that holds the vocabulary (src/dna_tokenizer.py:2150-2236),
+ * written directly in that type, padded on either side, at any width t_out (a fixed token_len, a
+ * multiple of pad_multiple). */
+int dnatok_char_encode_padded_as(const dnatok_char_t *t, const uint8_t *bytes, const int64_t *offsets,
+                                 int64_t n_rows, int64_t t_out, int pad_left,
+                                 void *ids, int32_t id_bytes, uint8_t *mask, void *stream);
+
 /* Flat stream: ids[i] = lut[bytes[i]], i < total; mask (may be NULL) is set to 1.
  * row_len > 0 declares equal-length rows, so that positions i % row_len == 0 use the start
  * table; row_len = 0 means no row structure.  This is also the dense [B, T] -> [B, T] case. */

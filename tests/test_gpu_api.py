@@ -143,6 +143,42 @@ def test_ids_and_bytes_paths_feed_the_same_ids():
     assert all(torch.equal(x, y) for x, y in zip(out_ids, out_bytes))
 
 
+@pytest.mark.parametrize("side", ["left", "right"])
+def test_char_encode_batch_with_padding_follows_the_reference_form(side):
+    """Single-nucleotide tokenizers: truncate to max_tokens, pad with N to the longest (or to
+    max_tokens), round up to pad_multiple, overwrite the padding with the pad id, narrow the ids
+    (the steps of the reference, src/dna_tokenizer.py:2150-2236, done here with numpy)."""
+    tok = SimpleCharTokenizer()
+    tok.padding_side = side
+    h = DNATok(RecordingEmbedder(tok))
+    h.discover()
+    assert h.padding_side == side
+    seqs = random_seqs(1, 50, seed=1) + random_seqs(1, 3, seed=2) + random_seqs(1, 37, seed=3) + ["A"]
+    for max_tokens, pad_to_max, mult in ((40, False, 16), (100, True, 16), (100, False, 1), (37, False, 8), (64, True, 1)):
+        ids, mask = h.encode_batch_with_padding(seqs, max_tokens, pad_to_max=pad_to_max, pad_multiple=mult)
+        cut = [s[:max_tokens] for s in seqs]
+        target = max(len(s) for s in cut)
+        if pad_to_max:
+            target = max(target, max_tokens)
+        if mult > 1 and target % mult:
+            target += mult - target % mult
+        want = np.full((len(cut), target), tok.pad_token_id, dtype=np.int64)
+        want_mask = np.zeros((len(cut), target), dtype=np.uint8)
+        for i, sq in enumerate(cut):
+            row = [tok.vocab[c] for c in sq]
+            if side == "left":
+                want[i, target - len(row):] = row
+                want_mask[i, target - len(row):] = 1
+            else:
+                want[i, :len(row)] = row
+                want_mask[i, :len(row)] = 1
+        assert ids.dtype == torch.uint8 and mask.dtype == torch.uint8 and ids.is_cuda
+        np.testing.assert_array_equal(ids.cpu().numpy().astype(np.int64), want)
+        np.testing.assert_array_equal(mask.cpu().numpy(), want_mask)
+    with pytest.raises(ValueError, match="Empty batch"):
+        h.encode_batch_with_padding([], 10)
+
+
 def test_two_bit_path_feeds_the_same_ids_as_the_bytes_path():
     tok = SimpleCharTokenizer()
     h = DNATok(RecordingEmbedder(tok), normalize_case=True, handle_invalid_chars=True)

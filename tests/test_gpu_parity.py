@@ -111,6 +111,34 @@ def test_char_fused_embedding_gather(dtype, dim):
         assert torch.equal(out.view(torch.uint8), ref.view(torch.uint8))
 
 
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.int16, torch.int32, torch.int64])
+def test_char_padded_in_every_id_width(dtype):
+    """Ragged rows padded on either side, ids written as uint8 / int16 / int32 / int64: widths
+    that are and are not a multiple of 4 (one store of four ids, or id by id), a first-column table,
+    an id that needs more than 8 bits (cut to the width, like a cast)."""
+    lut = util.char_lut().copy()
+    lut[ord("G")] = 300                                               # does not fit uint8
+    rng = np.random.default_rng(2)
+    for start in (None, lut + 5):
+        enc = encoders.CharEncoder(lut, pad_id=1, start_lut=start)
+        for t_out in (1, 7, 64, 1001, 4100):
+            lens = rng.integers(0, t_out + 40, size=33)
+            lens[0], lens[1] = 0, t_out
+            rows = [rng.choice(np.frombuffer(b"ACGTN", dtype=np.uint8), size=int(n)) for n in lens]
+            offsets = np.zeros(len(rows) + 1, dtype=np.int64)
+            offsets[1:] = np.cumsum(lens)
+            data = np.concatenate(rows) if offsets[-1] else np.zeros(0, dtype=np.uint8)
+            d_data, d_off = torch.from_numpy(data).to(DEV), torch.from_numpy(offsets).to(DEV)
+            for pad_left in (False, True):
+                say(f"char padded {dtype} t_out={t_out} left={pad_left} start={start is not None}")
+                ids, mask = enc.encode_padded(d_data, d_off, t_out, pad_left=pad_left, dtype=dtype)
+                torch.cuda.synchronize()
+                eids, emask = O.char_encode_padded(lut, data, offsets, t_out, 1, start_lut=start, pad_left=pad_left)
+                want = torch.from_numpy(eids).to(dtype)                # the cast an int32 result would get
+                assert ids.dtype == dtype and torch.equal(ids.cpu(), want)
+                np.testing.assert_array_equal(mask.cpu().numpy(), emask)
+
+
 @pytest.mark.parametrize("dtype", [torch.uint8, torch.int32, torch.int64])
 def test_char_unpack_2bit(dtype):
     """2-bit packed rows -> ids of three widths, rows of every length mod 4 (the flat and the
