@@ -1,0 +1,289 @@
+"""``python -m dnatok_amd.dnatok_cli``: info / encode / validate / bench from a shell.
+
+The four commands of the reference's command line (src/dnatok_cli.py:162-307) with the same
+options and the same output fields.  ``--model`` names a tokenizer that can be had without a
+network: a directory or ``tokenizer.json`` on disk (loaded with ``tokenizers.Tokenizer.from_file``
+and, for directories, ``transformers.AutoTokenizer`` when that works offline), or one of the
+built-in synthetic tokenizers of the benchmark configurations:
+
+    char      single nucleotides, NTv3 vocabulary order     (kernel: char)
+    ntv3      the NTv3 compat tokenizer class                (kernel: char)
+    evo2      byte-level ids, id = ord(c)                    (kernel: char)
+    kmer6     non-overlapping 6-mers, grid-aligned fallback  (kernel: k-mer)
+    bpe4096   BPE trained on the synthetic corpus            (kernel: BPE engine)
+    bpe32000  BPE with the 32000 vocabulary                  (kernel: BPE engine)
+
+All encoding runs on the GPU through libdnatok_hip.so; the reference tokenizer it is compared
+with runs on the host.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import random
+import sys
+import time
+from typing import Any, List, Optional, Tuple
+
+BUILTIN = ("char", "ntv3", "evo2", "kmer6", "bpe4096", "bpe32000")
+
+
+class _TokenizerCall:
+    """``tokenizers.Tokenizer`` behind the call style DNATok probes (``tok(texts, ...)``)."""
+
+    def __init__(self, tk, pad_id: int = 0, padding_side: str = "right"):
+        self.backend_tokenizer = tk
+        self._tk = tk
+        self.pad_token_id = pad_id
+        self.padding_side = padding_side
+        self.vocab_size = tk.get_vocab_size()
+
+    def get_vocab(self):
+        return self._tk.get_vocab()
+
+    def to_str(self):
+        return self._tk.to_str()
+
+    def __call__(self, texts, add_special_tokens=False, **_):
+        single = isinstance(texts, str)
+        rows = [e.ids for e in self._tk.encode_batch([texts] if single else list(texts),
+                                                     add_special_tokens=add_special_tokens)]
+        return {"input_ids": rows[0] if single else rows}
+
+
+def _load_tokenizer(model: str):
+    from . import dnatok_compat, hf_tokenizers as hf
+    if model == "char":
+        return _TokenizerCall(hf.build_char_tokenizer(), pad_id=hf.char_vocab()["<pad>"])
+    if model == "ntv3":
+        return dnatok_compat.NTv3Tokenizer()
+    if model == "evo2":
+        return dnatok_compat.Evo2ByteTokenizer()
+    if model == "kmer6":
+        return _TokenizerCall(hf.build_kmer_tokenizer(6), pad_id=hf.kmer_vocab(6)["<pad>"])
+    if model in ("bpe4096", "bpe32000"):
+        tk = hf.load_bpe_tokenizer(model[3:])
+        return _TokenizerCall(tk, pad_id=tk.token_to_id("[PAD]"))
+    path = model
+    if os.path.isdir(path):
+        try:
+            os.environ.setdefault("HF_HUB_OFFLINE", "1")
+            from transformers import AutoTokenizer
+            return AutoTokenizer.from_pretrained(path, local_files_only=True)
+        except Exception:
+            path = os.path.join(path, "tokenizer.json")
+    if os.path.isfile(path):
+        from tokenizers import Tokenizer
+        tk = Tokenizer.from_file(path)
+        pad = tk.padding["pad_id"] if tk.padding else (tk.token_to_id("[PAD]") or tk.token_to_id("<pad>") or 0)
+        return _TokenizerCall(tk, pad_id=int(pad))
+    raise SystemExit(f"--model {model!r}: not a built-in name ({', '.join(BUILTIN)}) and not a path on disk")
+
+
+def _build_dnatok(model: str, device: str):
+    import torch
+    from .dna_tokenizer import DNATok
+    tok = _load_tokenizer(model)
+
+    class _Embedder:
+        def __init__(self, t):
+            self.tokenizer = t
+            size = getattr(t, "vocab_size", 0)
+            size = int(size) if isinstance(size, int) and size else len(t.get_vocab())
+            self.embed_table = torch.nn.Embedding(size + 4, 16).to(device)
+
+        def embed_tokens(self, ids):
+            return self.embed_table(ids)
+
+    dn = DNATok(_Embedder(tok), normalize_case=False, handle_invalid_chars=False)
+    dn.discover()
+    return tok, dn
+
+
+def _detect_path(dn) -> str:
+    if getattr(dn, "kmer_k", None) is not None:
+        return f"kmer-{dn.kmer_k}"
+    if getattr(dn, "bpe_backend", None) is not None:
+        return "gpu-bpe-kernel"
+    if getattr(dn, "ascii_lut", None) is not None and dn.use_ids_path:
+        return "ascii-lut"
+    return "hf-fallback"
+
+
+def _default_device() -> str:
+    import torch
+    return "cuda" if torch.cuda.is_available() else "cpu"
+
+
+def _emit(payload: Any, as_json: bool) -> None:
+    if as_json:
+        json.dump(payload, sys.stdout, indent=2)
+        print()
+    elif isinstance(payload, dict):
+        width = max(map(len, payload)) if payload else 0
+        for k, v in payload.items():
+            print(f"  {k:<{width}}  {v}")
+    else:
+        print(payload)
+
+
+def _strip_pad(row: List[int], pad: int, side: str) -> List[int]:
+    if side == "left":
+        j = 0
+        while j < len(row) and row[j] == pad:
+            j += 1
+        return row[j:]
+    j = len(row)
+    while j > 0 and row[j - 1] == pad:
+        j -= 1
+    return row[:j]
+
+
+def _hf_ids(tok, seqs: List[str]) -> List[List[int]]:
+    out = tok(seqs, add_special_tokens=False, padding=False, truncation=False, return_tensors=None)
+    rows = out["input_ids"]
+    return [r.tolist() if hasattr(r, "tolist") else list(r) for r in rows]
+
+
+def cmd_info(args) -> int:
+    device = args.device or _default_device()
+    tok, dn = _build_dnatok(args.model, device)
+    size = getattr(tok, "vocab_size", 0)
+    _emit({
+        "model": args.model,
+        "tokenizer_class": type(tok).__name__,
+        "vocab_size": int(size) if isinstance(size, int) and size else len(tok.get_vocab()),
+        "selected_path": _detect_path(dn),
+        "device": device,
+        "kmer_k": dn.kmer_k,
+        "has_ascii_lut": dn.ascii_lut is not None,
+        "has_gpu_bpe_backend": dn.bpe_backend is not None,
+        "has_cached_lmm": dn.lmm_bpe is not None,
+        "padding_side": dn.padding_side,
+        "id_pad": int(dn.id_pad),
+    }, args.json)
+    return 0
+
+
+def cmd_encode(args) -> int:
+    device = args.device or _default_device()
+    _, dn = _build_dnatok(args.model, device)
+    ids = _strip_pad(dn.encode_batch_to_ids([args.seq])[0].tolist(), int(dn.id_pad), dn.padding_side)
+    _emit({
+        "model": args.model,
+        "sequence": args.seq[:80] + ("..." if len(args.seq) > 80 else ""),
+        "sequence_length_bp": len(args.seq),
+        "n_tokens": len(ids),
+        "token_ids": ids if args.json else ids[:32] + (["..."] if len(ids) > 32 else []),
+        "selected_path": _detect_path(dn),
+    }, args.json)
+    return 0
+
+
+def cmd_validate(args) -> int:
+    """Bit identity with the tokenizer itself on n random ACGT sequences of one length."""
+    device = args.device or _default_device()
+    tok, dn = _build_dnatok(args.model, device)
+    rng = random.Random(args.seed)
+    seqs = ["".join(rng.choices("ACGT", k=args.window)) for _ in range(args.n)]
+    ours = dn.encode_batch_to_ids(seqs).cpu().tolist()
+    theirs = _hf_ids(tok, seqs)
+    pad = int(dn.id_pad)
+    n_match, first = 0, None
+    for i, s in enumerate(seqs):
+        row = _strip_pad(ours[i], pad, dn.padding_side)
+        if row == list(theirs[i]):
+            n_match += 1
+        elif first is None:
+            first = {"i": i, "seq_head": s[:40], "dnatok_head": row[:8], "hf_head": list(theirs[i])[:8]}
+    _emit({
+        "model": args.model,
+        "n_sequences": args.n,
+        "n_match": n_match,
+        "n_mismatch": args.n - n_match,
+        "match_rate": n_match / max(args.n, 1),
+        "selected_path": _detect_path(dn),
+        "first_mismatch": first,
+    }, args.json)
+    return 0 if n_match == args.n else 1
+
+
+def cmd_bench(args) -> int:
+    """Strings in, ids out, chunk by chunk: this backend beside the tokenizer on the host."""
+    device = args.device or _default_device()
+    os.environ["RAYON_NUM_THREADS"] = str(args.hf_threads)
+    os.environ["TOKENIZERS_PARALLELISM"] = "true" if args.hf_threads > 1 else "false"
+    tok, dn = _build_dnatok(args.model, device)
+    rng = random.Random(args.seed)
+    seqs = ["".join(rng.choices("ACGT", k=args.window)) for _ in range(args.n)]
+    bp_total = sum(map(len, seqs))
+    tok(seqs[:min(args.chunk, args.n)], add_special_tokens=False)
+    dn.encode_batch_to_ids(seqs[:min(args.chunk, args.n)])
+    t0 = time.perf_counter()
+    for i in range(0, args.n, args.chunk):
+        tok(seqs[i:i + args.chunk], add_special_tokens=False)
+    t_hf = time.perf_counter() - t0
+    import torch
+    if device == "cuda":
+        torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(0, args.n, args.chunk):
+        dn.encode_batch_to_ids(seqs[i:i + args.chunk])
+    if device == "cuda":
+        torch.cuda.synchronize()
+    t_dn = time.perf_counter() - t0
+    _emit({
+        "model": args.model,
+        "n_sequences": args.n,
+        "window_bp": args.window,
+        "chunk": args.chunk,
+        "total_bp": bp_total,
+        "hf_threads": args.hf_threads,
+        "hf_time_s": round(t_hf, 4),
+        "hf_mbp_per_s": round(bp_total / t_hf / 1e6, 2),
+        "dnatok_time_s": round(t_dn, 4),
+        "dnatok_mbp_per_s": round(bp_total / t_dn / 1e6, 2),
+        "speedup_dnatok_vs_hf": round(t_hf / t_dn, 2),
+        "selected_path": _detect_path(dn),
+        "device": device,
+    }, args.json)
+    return 0
+
+
+def main(argv: Optional[list] = None) -> int:
+    ap = argparse.ArgumentParser(prog="dnatok", description="DNA tokenization on the MI355X backend")
+    sub = ap.add_subparsers(dest="cmd", required=True)
+
+    def common(p):
+        p.add_argument("--model", required=True, help="built-in name (%s) or a tokenizer path" % ", ".join(BUILTIN))
+        p.add_argument("--device", default=None, help="cuda (default when a GPU is present)")
+        p.add_argument("--json", action="store_true", help="emit machine-readable JSON")
+
+    p = sub.add_parser("info", help="tokenizer family and the kernel it is routed to")
+    common(p)
+    p.set_defaults(fn=cmd_info)
+    p = sub.add_parser("encode", help="encode one sequence")
+    common(p)
+    p.add_argument("--seq", required=True, help="DNA sequence (ACGT[N])")
+    p.set_defaults(fn=cmd_encode)
+    p = sub.add_parser("validate", help="bit identity with the tokenizer on random sequences")
+    common(p)
+    p.add_argument("--n", type=int, default=500)
+    p.add_argument("--window", type=int, default=1024)
+    p.add_argument("--seed", type=int, default=42)
+    p.set_defaults(fn=cmd_validate)
+    p = sub.add_parser("bench", help="strings -> ids throughput beside the host tokenizer")
+    common(p)
+    p.add_argument("--n", type=int, default=1000)
+    p.add_argument("--window", type=int, default=4096)
+    p.add_argument("--chunk", type=int, default=32)
+    p.add_argument("--hf-threads", type=int, default=8)
+    p.add_argument("--seed", type=int, default=11)
+    p.set_defaults(fn=cmd_bench)
+    args = ap.parse_args(argv)
+    return int(args.fn(args))
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())

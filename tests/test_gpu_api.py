@@ -452,3 +452,23 @@ def test_bpe_kernel_wrapper_contract(tmp_path):
     assert torch.equal(kept.cpu(), torch.from_numpy(ids_h)) and not torch.equal(view.cpu(), kept.cpu())
     e_ids, e_len = k.tokenize_batch([])
     assert e_ids.shape == (0, 0) and e_len.shape == (0,)
+
+
+@pytest.mark.parametrize("model,path", [("char", "ascii-lut"), ("ntv3", "ascii-lut"), ("evo2", "ascii-lut"),
+                                        ("kmer6", "kmer-6"), ("bpe4096", "gpu-bpe-kernel")])
+def test_cli_info_encode_validate(model, path, capsys):
+    import json
+    from dnatok_amd import dnatok_cli
+    assert dnatok_cli.main(["info", "--model", model, "--json"]) == 0
+    info = json.loads(capsys.readouterr().out)
+    assert info["selected_path"] == path and info["device"] == "cuda"
+    assert dnatok_cli.main(["encode", "--model", model, "--seq", "ACGTACGTTTGACCA", "--json"]) == 0
+    enc = json.loads(capsys.readouterr().out)
+    assert enc["sequence_length_bp"] == 15 and enc["n_tokens"] == len(enc["token_ids"]) > 0
+    assert dnatok_cli.main(["validate", "--model", model, "--n", "40", "--window", "600", "--json"]) == 0
+    val = json.loads(capsys.readouterr().out)
+    assert val["n_match"] == 40 and val["n_mismatch"] == 0 and val["first_mismatch"] is None
+    assert dnatok_cli.main(["bench", "--model", model, "--n", "64", "--window", "512", "--chunk", "32",
+                            "--hf-threads", "2", "--json"]) == 0
+    b = json.loads(capsys.readouterr().out)
+    assert b["total_bp"] == 64 * 512 and b["dnatok_mbp_per_s"] > 0
