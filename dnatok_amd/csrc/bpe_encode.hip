@@ -359,7 +359,7 @@ constexpr int kLongThreads = 1024;
 constexpr int kLongGrid = 64;            // slabs of scratch for the whole-row fallback kernel
 
 struct BpePlan {                          // device arrays inside the scratch buffer
-    int32_t *counts;      // [0] items, [1] chunk items of multi-chunk rows, [2] work counter
+    int32_t *counts;      // [0] items, [1] chunk items of multi-chunk rows, [2] work counter, [3] failed rows
     int32_t *item_off;    // [n_rows + 1] first item of a row
     int32_t *mc_off;      // [n_rows + 1] first chunk slot of a row (multi-chunk rows only)
     int32_t *item_row;    // [max_items]
@@ -433,25 +433,42 @@ static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t
     return p;
 }
 
-// Work list: one item per short row, ceil(len / core) items per long row.  Single workgroup.
+// Work list: one item per short row, ceil(len / core) items per long row.  Single workgroup; a
+// thread takes four consecutive rows per step, so that 4096 rows are one round of loads and one
+// scan (the kernel is a chain of load latencies and barriers, not work).
+constexpr int kPlanRows = 4;
+constexpr uint32_t kPlanInline = 4;      // rows of more chunks than this are written out by their whole wave
+
 __global__ __launch_bounds__(1024) void bpe_plan_kernel(
     const int64_t *__restrict__ offsets, int64_t n_rows, int chunking, BpePlan p)
 {
     __shared__ uint32_t wt[2][16];
     __shared__ int32_t carry[2];
-    if (threadIdx.x == 0) { carry[0] = 0; carry[1] = 0; }
+    __shared__ int32_t fail_s;
+    if (threadIdx.x == 0) { carry[0] = 0; carry[1] = 0; fail_s = 0; }
     __syncthreads();
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    for (int64_t base = 0; base < n_rows; base += 1024) {
-        const int64_t row = base + threadIdx.x;
-        uint32_t nc = 0, mc = 0;
-        if (row < n_rows) {
-            const int64_t len = offsets[row + 1] - offsets[row];
-            nc = 1;
-            if (len > p.ext && chunking) { nc = (uint32_t)((len + p.core - 1) / p.core); mc = nc; }
-            p.row_fail[row] = (len > p.ext && !chunking) ? 1 : 0;
+    int32_t n_fail = 0;
+    for (int64_t base = 0; base < n_rows; base += 1024 * kPlanRows) {
+        const int64_t row0 = base + (int64_t)threadIdx.x * kPlanRows;
+        int64_t off[kPlanRows + 1];
+#pragma unroll
+        for (int r = 0; r <= kPlanRows; ++r) off[r] = row0 + r <= n_rows ? offsets[row0 + r] : 0;
+        uint32_t nc[kPlanRows], mc[kPlanRows], nc_sum = 0, mc_sum = 0;
+#pragma unroll
+        for (int r = 0; r < kPlanRows; ++r) {
+            nc[r] = 0; mc[r] = 0;
+            if (row0 + r < n_rows) {
+                const int64_t len = off[r + 1] - off[r];
+                nc[r] = 1;
+                if (len > p.ext && chunking) { nc[r] = (uint32_t)((len + p.core - 1) / p.core); mc[r] = nc[r]; }
+                const int fail = (len > p.ext && !chunking) ? 1 : 0;
+                p.row_fail[row0 + r] = fail;
+                n_fail += fail;
+            }
+            nc_sum += nc[r]; mc_sum += mc[r];
         }
-        const uint32_t inc0 = wave_inclusive_sum_u32(nc), inc1 = wave_inclusive_sum_u32(mc);
+        const uint32_t inc0 = wave_inclusive_sum_u32(nc_sum), inc1 = wave_inclusive_sum_u32(mc_sum);
         if (lane == 63) { wt[0][wv] = inc0; wt[1][wv] = inc1; }
         __syncthreads();
         uint32_t b0 = 0, b1 = 0, t0 = 0, t1 = 0;
@@ -461,23 +478,49 @@ __global__ __launch_bounds__(1024) void bpe_plan_kernel(
             t0 += wt[0][w]; t1 += wt[1][w];
         }
         const int32_t c0 = carry[0], c1 = carry[1];
-        if (row < n_rows) {
-            const int32_t io = c0 + (int32_t)(b0 + inc0 - nc), mo = c1 + (int32_t)(b1 + inc1 - mc);
-            p.item_off[row] = io;
-            p.mc_off[row] = mo;
-            for (uint32_t k = 0; k < nc; ++k) p.item_row[io + k] = (int32_t)row;
-            for (uint32_t k = 0; k < mc; ++k) { p.mc_row[mo + k] = (int32_t)row; p.seam[mo + k] = -1; }
+        int32_t io = c0 + (int32_t)(b0 + inc0 - nc_sum), mo = c1 + (int32_t)(b1 + inc1 - mc_sum);
+#pragma unroll
+        for (int r = 0; r < kPlanRows; ++r) {
+            const bool valid = row0 + r < n_rows;
+            const int32_t row = (int32_t)(row0 + r);
+            if (valid) {
+                p.item_off[row] = io;
+                p.mc_off[row] = mo;
+            }
+            // a row of many chunks has its entries written by the whole wave, the others by their lane
+            const bool big = valid && nc[r] > kPlanInline;
+            if (valid && !big) {
+                for (uint32_t k = 0; k < nc[r]; ++k) p.item_row[io + k] = row;
+                for (uint32_t k = 0; k < mc[r]; ++k) { p.mc_row[mo + k] = row; p.seam[mo + k] = -1; }
+            }
+            uint64_t todo = __ballot(big);
+            while (todo) {
+                const int src = __builtin_amdgcn_readfirstlane(__builtin_ctzll(todo));
+                todo &= todo - 1;
+                const int32_t b_row = __builtin_amdgcn_readlane(row, src);
+                const int32_t b_io = __builtin_amdgcn_readlane(io, src), b_mo = __builtin_amdgcn_readlane(mo, src);
+                const uint32_t b_nc = __builtin_amdgcn_readlane(nc[r], src), b_mc = __builtin_amdgcn_readlane(mc[r], src);
+                for (uint32_t k = lane; k < b_nc; k += 64) p.item_row[b_io + k] = b_row;
+                for (uint32_t k = lane; k < b_mc; k += 64) { p.mc_row[b_mo + k] = b_row; p.seam[b_mo + k] = -1; }
+            }
+            if (valid) {
+                io += (int32_t)nc[r];
+                mo += (int32_t)mc[r];
+            }
         }
         __syncthreads();
         if (threadIdx.x == 0) { carry[0] = c0 + (int32_t)t0; carry[1] = c1 + (int32_t)t1; }
         __syncthreads();
     }
+    if (n_fail) atomicAdd(&fail_s, n_fail);
+    __syncthreads();
     if (threadIdx.x == 0) {
         p.item_off[n_rows] = carry[0];
         p.mc_off[n_rows] = carry[1];
         p.counts[0] = carry[0];
         p.counts[1] = carry[1];
         p.counts[2] = 0;
+        p.counts[3] = fail_s;                         // rows left to the whole-row kernel (the seam kernel may add some)
     }
 }
 
@@ -569,7 +612,10 @@ __global__ __launch_bounds__(256) void bpe_seam_kernel(const int64_t *__restrict
         __syncthreads();
         if (threadIdx.x == 0) {
             const uint32_t b = umin(umin(best[0], best[1]), umin(best[2], best[3]));
-            if (b == 0xFFFFFFFFu) { p.seam[m] = -1; p.row_fail[row] = 1; }
+            if (b == 0xFFFFFFFFu) {
+                p.seam[m] = -1;
+                if (atomicExch(&p.row_fail[row], 1) == 0) atomicAdd(&p.counts[3], 1);
+            }
             else p.seam[m] = (int32_t)b;
         }
         __syncthreads();
@@ -658,6 +704,7 @@ __global__ __launch_bounds__(NT) void bpe_long_kernel(
     __shared__ uint32_t red[4 * (NT / 64) + 4];
     __shared__ uint8_t D[NT];
     __shared__ uint16_t b2s[256];
+    if (p.counts[3] == 0) return;                    // no row needs this kernel (the usual case)
     for (int i = threadIdx.x; i < 256; i += NT) b2s[i] = a.byte_to_sym[i];
     __syncthreads();
     // each workgroup owns one slab of scratch, sized for the longest row

@@ -5,18 +5,6 @@
 
 namespace dnatok {
 
-int launch_pad_to_max(int32_t *ids, uint8_t *mask, const int32_t *lengths, int64_t n_rows,
-                      int64_t t_cap, int32_t *max_len, int32_t pad_id, int32_t already, hipStream_t s);
-
-__global__ void zero_i32_kernel(int32_t *p) { *p = 0; }
-
-static int launch_zero_i32(int32_t *p, hipStream_t s)
-{
-    zero_i32_kernel<<<1, 1, 0, s>>>(p);
-    DNATOK_HIP_TRY(hipGetLastError());
-    return DNATOK_OK;
-}
-
 constexpr int kScanThreads = 1024;
 
 // out_offsets[b] = sum of max(lengths[0..b), 0); single workgroup, 1024 rows per step.
@@ -87,15 +75,58 @@ __global__ __launch_bounds__(256) void pack_copy_kernel(
 }
 
 constexpr int kPadTile = 2048;           // cells of one row that one workgroup handles
+constexpr int kPadFuseRows = 2048;       // up to this many rows every workgroup finds the longest row itself
+
+// Longest row (lengths cut to [0, t_cap]) of the batch, by one workgroup.
+__device__ __forceinline__ int32_t block_max_length(const int32_t *lengths, int64_t n_rows, int64_t t_cap,
+                                                    uint32_t *red)
+{
+    uint32_t m = 0;
+    for (int64_t i = threadIdx.x; i < n_rows; i += blockDim.x) {
+        int64_t v = lengths[i];
+        if (v < 0) v = 0;
+        if (v > t_cap) v = t_cap;
+        m = m > (uint32_t)v ? m : (uint32_t)v;
+    }
+    m = wave_max_u32(m);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    uint32_t all = 0;
+    for (unsigned w = 0; w < blockDim.x / 64; ++w) all = all > red[w] ? all : red[w];
+    return (int32_t)all;
+}
+
+__global__ __launch_bounds__(1024) void rows_max_kernel(const int32_t *__restrict__ lengths, int64_t n_rows,
+                                                        int64_t t_cap, int32_t *__restrict__ max_len)
+{
+    __shared__ uint32_t red[16];
+    const int32_t m = block_max_length(lengths, n_rows, t_cap, red);
+    if (threadIdx.x == 0) *max_len = m;
+}
 
 // Padded layout: workgroup (row, tile) copies the row's tokens that fall into its tile of
-// columns and pads the rest of the tile up to fill_to.
+// columns and pads the rest of the tile up to the width: fill_to, or with fill_to = 0 the longest
+// row of the batch.  That one is found by every workgroup for itself while the batch is small
+// (FUSED_MAX: the lengths are a few KB in L2, and no launch, atomic or second pass over the rows
+// is needed), and read from max_len, where rows_max_kernel has put it, otherwise.
+template <bool FUSED_MAX>
 __global__ __launch_bounds__(256) void pad_rows_kernel(
     const int32_t *__restrict__ tok_tmp, const int64_t *__restrict__ in_offsets,
     const int32_t *__restrict__ lengths, int64_t n_rows, int64_t tiles_per_row,
     const int32_t *__restrict__ remap, int32_t pad_id, int64_t t_cap, int64_t fill_to,
     int32_t *__restrict__ ids, uint8_t *__restrict__ mask, int32_t *__restrict__ max_len)
 {
+    __shared__ uint32_t red[4];
+    int64_t width = fill_to;
+    if (FUSED_MAX) {
+        if (fill_to == 0 || max_len) {
+            const int32_t longest = block_max_length(lengths, n_rows, t_cap, red);
+            if (fill_to == 0) width = longest;
+            if (max_len && blockIdx.x == 0 && threadIdx.x == 0) *max_len = longest;
+        }
+    } else if (fill_to == 0) {
+        width = *max_len;
+    }
     const int64_t n_tiles = n_rows * tiles_per_row;
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const int64_t row = tile / tiles_per_row;
@@ -103,8 +134,7 @@ __global__ __launch_bounds__(256) void pad_rows_kernel(
         int64_t len = lengths[row];
         if (len < 0) len = 0;
         if (len > t_cap) len = t_cap;
-        if (c0 == 0 && max_len && threadIdx.x == 0) atomicMax(max_len, (int32_t)len);
-        const int64_t end = len > fill_to ? len : fill_to;            // cells of the row that get written
+        const int64_t end = len > width ? len : width;                // cells of the row that get written
         if (c0 >= end) continue;
         const int64_t c1 = c0 + kPadTile < end ? c0 + kPadTile : end;
         const int32_t *src = tok_tmp + in_offsets[row];
@@ -164,14 +194,16 @@ extern "C" int dnatok_pad_rows(const int32_t *tok_tmp, const int64_t *in_offsets
     DNATOK_REQUIRE(fill_to > 0 || max_len, DNATOK_E_INVALID, "dnatok_pad_rows: fill_to = 0 needs max_len");
     if (n_rows == 0) return DNATOK_OK;
     hipStream_t s = (hipStream_t)stream;
-    if (max_len) {
-        int rc = launch_zero_i32(max_len, s);
-        if (rc) return rc;
-    }
     const int64_t tiles_per_row = t_cap > 0 ? (t_cap + kPadTile - 1) / kPadTile : 1;
-    pad_rows_kernel<<<capped_grid(n_rows * tiles_per_row), 256, 0, s>>>(
-        tok_tmp, in_offsets, lengths, n_rows, tiles_per_row, remap, pad_id, t_cap, fill_to, ids, mask, max_len);
+    const int grid = capped_grid(n_rows * tiles_per_row);
+    if (n_rows <= kPadFuseRows) {
+        pad_rows_kernel<true><<<grid, 256, 0, s>>>(tok_tmp, in_offsets, lengths, n_rows, tiles_per_row, remap, pad_id,
+                                                   t_cap, fill_to, ids, mask, max_len);
+    } else {
+        if (max_len) rows_max_kernel<<<1, 1024, 0, s>>>(lengths, n_rows, t_cap, max_len);
+        pad_rows_kernel<false><<<grid, 256, 0, s>>>(tok_tmp, in_offsets, lengths, n_rows, tiles_per_row, remap, pad_id,
+                                                    t_cap, fill_to, ids, mask, max_len);
+    }
     DNATOK_HIP_TRY(hipGetLastError());
-    if (fill_to == 0) return launch_pad_to_max(ids, mask, lengths, n_rows, t_cap, max_len, pad_id, 0, s);
     return DNATOK_OK;
 }
