@@ -582,10 +582,17 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     }
 }
 
-// One workgroup per chunk of a multi-chunk row: the seam with the chunk to its right.
+// One workgroup per chunk of a multi-chunk row: the seam with the chunk to its right.  The two
+// runs over the shared stretch (at most 2 x overlap positions) are staged in LDS first: the search
+// walks from token start to token start, a chain of dependent reads that is several times
+// shorter there than in L2.  (One wave per chunk instead of one workgroup was measured for this
+// kernel and the two after it: twice as slow, the per-lane loops over the chunk get too long.)
+constexpr int kSeamStage = 1024;          // positions of the shared stretch held in LDS
+
 __global__ __launch_bounds__(256) void bpe_seam_kernel(const int64_t *__restrict__ offsets, BpePlan p)
 {
     __shared__ uint32_t best[4];
+    __shared__ uint16_t sa_s[kSeamStage], sb_s[kSeamStage];
     const int32_t n_mc = p.counts[1];
     for (int32_t m = blockIdx.x; m < n_mc; m += gridDim.x) {
         const int32_t row = p.mc_row[m];
@@ -599,13 +606,21 @@ __global__ __launch_bounds__(256) void bpe_seam_kernel(const int64_t *__restrict
         const int64_t eb0 = (int64_t)(k + 1) * p.core - p.overlap;
         const uint16_t *A = p.chunk_sym + (size_t)m * p.ext;         // A[i - ea0]
         const uint16_t *B = p.chunk_sym + (size_t)(m + 1) * p.ext;   // B[i - eb0]
+        const int n = (int)(ea1 - eb0);                              // shared positions eb0 .. ea1
+        const bool staged = n <= kSeamStage;                         // (the same for the whole workgroup)
+        if (staged) {
+            for (int j = threadIdx.x; j < n; j += 256) { sa_s[j] = A[eb0 - ea0 + j]; sb_s[j] = B[j]; }
+            __syncthreads();
+        }
+        auto a_at = [&](int j) -> uint32_t { return staged ? sa_s[j] : A[eb0 - ea0 + j]; };
+        auto b_at = [&](int j) -> uint32_t { return staged ? sb_s[j] : B[j]; };
         uint32_t mine = 0xFFFFFFFFu;
-        for (int64_t i = eb0 + threadIdx.x; i < ea1; i += 256) {
-            const uint32_t sa = A[i - ea0];
-            if (sa == kNone || sa != B[i - eb0]) continue;
-            int64_t j = i + 1;                                       // next token start in A
-            while (j < ea1 && A[j - ea0] == kNone) ++j;
-            if (j < ea1 && A[j - ea0] == B[j - eb0]) { mine = (uint32_t)j; break; }
+        for (int i = threadIdx.x; i < n; i += 256) {
+            const uint32_t sa = a_at(i);
+            if (sa == kNone || sa != b_at(i)) continue;
+            int j = i + 1;                                           // next token start in A
+            while (j < n && a_at(j) == kNone) ++j;
+            if (j < n && a_at(j) == b_at(j)) { mine = (uint32_t)(eb0 + j); break; }
         }
         mine = wave_min_u32(mine);
         if ((threadIdx.x & 63) == 0) best[threadIdx.x >> 6] = mine;
@@ -615,8 +630,9 @@ __global__ __launch_bounds__(256) void bpe_seam_kernel(const int64_t *__restrict
             if (b == 0xFFFFFFFFu) {
                 p.seam[m] = -1;
                 if (atomicExch(&p.row_fail[row], 1) == 0) atomicAdd(&p.counts[3], 1);
+            } else {
+                p.seam[m] = (int32_t)b;
             }
-            else p.seam[m] = (int32_t)b;
         }
         __syncthreads();
     }
