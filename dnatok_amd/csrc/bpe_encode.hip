@@ -587,11 +587,19 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
 
     const uint32_t mask = a.slots - 1;
     const int32_t n_items = p.counts[0];
-    for (;;) {
-        if (tid == 0) *next_item = atomicAdd(&p.counts[2], 1);
-        team_sync<NT>();
-        const int32_t item = *next_item;
-        team_sync<NT>();
+    // A team's first item is its own number; only the items beyond one per team are handed out
+    // through the counter.  (Every team asking the counter at the start of the kernel is a
+    // thousand atomics on one address, about 12 ns each, before the last team has its row.)
+    const int32_t n_teams = (int32_t)gridDim.x * TEAMS;
+    int32_t item = (int32_t)blockIdx.x * TEAMS + team;
+    for (bool first = true;; first = false) {
+        if (!first) {
+            if (n_teams >= n_items) break;           // nothing was left for the counter
+            if (tid == 0) *next_item = n_teams + atomicAdd(&p.counts[2], 1);
+            team_sync<NT>();
+            item = *next_item;
+            team_sync<NT>();
+        }
         if (item >= n_items) break;
         const int32_t row = p.item_row[item];
         const int32_t k = item - p.item_off[row];
