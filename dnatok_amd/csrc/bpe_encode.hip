@@ -389,8 +389,11 @@ __device__ __forceinline__ void bpe_row(
 // redone by the whole-row kernel.
 constexpr int kLdsCap = 4096;            // longest piece any LDS kernel variant takes
 // 2048-byte extended chunks: 26 KB of LDS state, six workgroups per CU; measured faster than
-// 4096-byte chunks (fewer positions per thread, more chunks in flight)
-constexpr int kChunkOverlap = 256;
+// 4096-byte chunks (fewer positions per thread, more chunks in flight) and than 1408- or 1536-byte
+// ones (the overlap is work done twice: its share of a chunk decides).  Overlap: with 64 bytes 0.3 %
+// of the seams of the 32000-vocabulary benchmark rows (10 % tandem repeats of up to 180 bp) find no
+// position, with 96 none of 5,088, with 128 none of 35,200 (CPU count with the oracle).
+constexpr int kChunkOverlap = 128;
 constexpr int kChunkCore = 2048 - 2 * kChunkOverlap;
 constexpr int kLongThreads = 1024;
 constexpr int kLongGrid = 64;            // slabs of scratch for the whole-row fallback kernel
@@ -939,6 +942,8 @@ extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, co
     int rc;
     const int64_t work_len = max_len < p.ext ? max_len : p.ext;    // longest piece the LDS kernel sees
     if (work_len <= 1024)        rc = launch_lds<256, 1, 1024>(a, bytes, offsets, p, tok_tmp, lengths, s);
+    else if (work_len <= 1408)   rc = launch_lds<256, 1, 1408>(a, bytes, offsets, p, tok_tmp, lengths, s);
+    else if (work_len <= 1536)   rc = launch_lds<256, 1, 1536>(a, bytes, offsets, p, tok_tmp, lengths, s);
     else if (work_len <= 2048)   rc = launch_lds<256, 1, 2048>(a, bytes, offsets, p, tok_tmp, lengths, s);
     else                         rc = launch_lds<256, 1, kLdsCap>(a, bytes, offsets, p, tok_tmp, lengths, s);
     if (rc) return rc;
