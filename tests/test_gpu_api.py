@@ -373,6 +373,36 @@ def test_device_normalizer_equals_the_host_callables(case):
         assert _rows_from_device(out2, off2) == [host(r) for r in few]
 
 
+def test_device_normalizer_on_a_batch_above_8192_tiles():
+    """36 Mbases in 4000 rows: more than 8192 tiles of 4096 positions, where the tile sizes are
+    scanned by a launch of their own and two passes alternate between the scratch buffers."""
+    from dnatok_amd import encoders
+    from dnatok_amd.gputok_bpe_backend import _compile_normalizer_step, _device_steps_of
+    rng = np.random.default_rng(3)
+    n_rows = 4000
+    lens = rng.integers(100, 18_000, size=n_rows)
+    data = np.frombuffer(b"ACGTN", dtype=np.uint8)[rng.integers(0, 5, size=int(lens.sum()))].copy()
+    for at in rng.integers(0, data.size - 100, size=15_000):
+        data[at:at + rng.integers(1, 40)] = ord("N")
+    off = np.zeros(n_rows + 1, dtype=np.int64)
+    off[1:] = np.cumsum(lens)
+    assert data.size // 4096 > 8192
+    spec = {"type": "Sequence", "normalizers": [
+        {"type": "Replace", "pattern": {"Regex": "N{10,}"}, "content": "-"},
+        {"type": "Prepend", "prepend": "_"}, {"type": "Lowercase"},
+        {"type": "Replace", "pattern": {"String": "acg"}, "content": "ACGT"}]}
+    host = _compile_normalizer_step(spec)
+    norm = encoders.RowNormalizer(_device_steps_of(spec))
+    out, out_off, bound, _ = norm.apply(torch.from_numpy(data).cuda(), torch.from_numpy(off).cuda(),
+                                        int(off[-1]), int(lens.max()))
+    torch.cuda.synchronize()
+    oo, raw = out_off.cpu().numpy(), out.cpu().numpy()
+    assert oo[-1] <= bound
+    for i in range(n_rows):
+        want = host(data[off[i]:off[i + 1]].tobytes().decode()).encode()
+        assert raw[oo[i]:oo[i + 1]].tobytes() == want, i
+
+
 def test_bpe_backend_normalizes_on_the_device_like_on_the_host():
     import json
     from tokenizers import Tokenizer
