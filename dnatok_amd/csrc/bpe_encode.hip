@@ -723,12 +723,19 @@ __global__ __launch_bounds__(256) void bpe_count_kernel(const int64_t *__restric
 }
 
 // One workgroup per chunk: its tokens, compacted, behind those of the row's earlier chunks.
+// Positions are taken 256 at a time: a ballot per wave places every live symbol among its wave's,
+// the waves' counts go through LDS, all symbols (and their remapped ids) of a block of passes are
+// loaded before the first store, and a wave's stores go to consecutive cells.  (A contiguous piece
+// per thread with load, remap and store in one loop ran as a chain of dependent loads: the
+// stores may alias what the next iteration reads.)
 __global__ __launch_bounds__(256) void bpe_gather_kernel(
     BpeArgs a, const int64_t *__restrict__ offsets, BpePlan p, int32_t *__restrict__ tok_tmp,
     int32_t *__restrict__ lengths)
 {
+    constexpr int kPasses = 8;
     __shared__ uint32_t red[8];
-    const int wv = threadIdx.x >> 6;
+    __shared__ uint32_t wave_cnt[kPasses][4];
+    const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int32_t n_mc = p.counts[1];
     for (int32_t m = blockIdx.x; m < n_mc; m += gridDim.x) {
         const ChunkSpan c = chunk_span(offsets, p, m);
@@ -738,22 +745,41 @@ __global__ __launch_bounds__(256) void bpe_gather_kernel(
         for (int32_t j = threadIdx.x; j < c.k; j += 256) before += (uint32_t)p.cnt[m - c.k + j];
         uint32_t base;
         (void)team_exclusive_sum<256>(before, red, wv, base);
-        // this chunk: a contiguous piece of the span per thread, in position order
         const uint16_t *sym = p.chunk_sym + (size_t)m * p.ext;
-        const int64_t n = c.hi - c.lo;
-        const int64_t per = (n + 255) / 256;
-        const int64_t t0 = c.lo + (int64_t)threadIdx.x * per < c.hi ? c.lo + (int64_t)threadIdx.x * per : c.hi;
-        const int64_t t1 = t0 + per < c.hi ? t0 + per : c.hi;
-        uint32_t live = 0;
-        for (int64_t i = t0; i < t1; ++i) live += sym[i - c.e0] != kNone;
-        uint32_t total;
-        uint32_t off = base + team_exclusive_sum<256>(live, red, wv, total);
         int32_t *out = tok_tmp + offsets[c.row];
-        for (int64_t i = t0; i < t1; ++i) {
-            const uint32_t sy = sym[i - c.e0];
-            if (sy != kNone) out[off++] = a.out_remap ? a.out_remap[sy] : (int32_t)sy;
+        uint32_t done = base;
+        for (int64_t i0 = c.lo; i0 < c.hi; i0 += kPasses * 256) {
+            uint32_t sy[kPasses], ahead[kPasses];
+            int32_t val[kPasses];
+#pragma unroll
+            for (int k = 0; k < kPasses; ++k) {
+                const int64_t i = i0 + k * 256 + threadIdx.x;
+                sy[k] = i < c.hi ? (uint32_t)sym[i - c.e0] : kNone;
+            }
+#pragma unroll
+            for (int k = 0; k < kPasses; ++k) {
+                val[k] = (sy[k] != kNone && a.out_remap) ? a.out_remap[sy[k]] : (int32_t)sy[k];
+                const uint64_t live = __ballot(sy[k] != kNone);
+                ahead[k] = (uint32_t)__builtin_popcountll(live & ((1ull << lane) - 1ull));
+                if (lane == 0) wave_cnt[k][wv] = (uint32_t)__builtin_popcountll(live);
+            }
+            __syncthreads();
+            uint32_t at = done;
+#pragma unroll
+            for (int k = 0; k < kPasses; ++k) {
+                uint32_t mine = at;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const uint32_t n = wave_cnt[k][w];
+                    if (w < wv) mine += n;
+                    at += n;
+                }
+                if (sy[k] != kNone) out[mine + ahead[k]] = val[k];
+            }
+            done = at;
+            __syncthreads();                                 // wave_cnt is rewritten by the next block
         }
-        if (threadIdx.x == 0 && c.k + 1 == c.nc) lengths[c.row] = (int32_t)(base + total);
+        if (threadIdx.x == 0 && c.k + 1 == c.nc) lengths[c.row] = (int32_t)done;
     }
 }
 

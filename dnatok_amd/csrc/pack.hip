@@ -53,11 +53,19 @@ __global__ __launch_bounds__(256) void pack_copy_kernel(
     const int64_t total = out_offsets[n_rows];
     for (int64_t o0 = (int64_t)blockIdx.x * kPackTile; o0 < total; o0 += (int64_t)gridDim.x * kPackTile) {
         const int64_t o1 = o0 + kPackTile < total ? o0 + kPackTile : total;
-        // last row with out_offsets[row] <= o0 (every thread does the same 20-odd steps)
-        int64_t lo = 0, hi = n_rows;
+        // last row with out_offsets[row] <= o0.  Every wave searches for itself, 64 evenly spaced
+        // offsets per step: 4096 rows are two dependent loads instead of the twelve of a binary
+        // search (the search is a chain of load latencies at the start of every tile).
+        int64_t lo = 0, hi = n_rows;                  // out_offsets[lo] <= o0 < out_offsets[hi] (hi = n_rows: the total)
         while (hi - lo > 1) {
-            const int64_t mid = (lo + hi) >> 1;
-            if (out_offsets[mid] <= o0) lo = mid; else hi = mid;
+            const int64_t step = (hi - lo + 63) >> 6;
+            const int64_t idx = lo + (int64_t)(threadIdx.x & 63) * step;
+            const bool at_or_below = idx < hi && out_offsets[idx] <= o0;      // true for a prefix of the lanes (lane 0 always)
+            const int n_below = __builtin_popcountll(__ballot(at_or_below));
+            const int64_t last = lo + (int64_t)(n_below - 1) * step;
+            if (last + step < hi) hi = last + step;
+            lo = last;
+            if (step == 1) break;
         }
         for (int64_t row = lo; row < n_rows; ++row) {
             const int64_t r0 = out_offsets[row], r1 = out_offsets[row + 1];
