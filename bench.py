@@ -509,8 +509,8 @@ def main() -> None:
                          "FETCH_SIZE / WRITE_SIZE counters are scaled by when profiling")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this backend and this benchmark are single-GPU (rows are independent; "
-              "see DESIGN.md for how the path would shard). Run with --gpus 1.", file=sys.stderr)
+        print("bench.py: this backend and this benchmark are single-GPU (rows are independent: several "
+              "GPUs would each take a share of the rows, with no exchange). Run with --gpus 1.", file=sys.stderr)
         raise SystemExit(2)
 
     import torch
