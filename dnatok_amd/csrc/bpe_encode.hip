@@ -477,7 +477,6 @@ static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t
 // thread takes four consecutive rows per step, so that 4096 rows are one round of loads and one
 // scan (the kernel is a chain of load latencies and barriers, not work).
 constexpr int kPlanRows = 4;
-constexpr uint32_t kPlanInline = 4;      // rows of more chunks than this are written out by their whole wave
 
 __global__ __launch_bounds__(1024) void bpe_plan_kernel(
     const int64_t *__restrict__ offsets, int64_t n_rows, int chunking, BpePlan p)
@@ -527,22 +526,10 @@ __global__ __launch_bounds__(1024) void bpe_plan_kernel(
                 p.item_off[row] = io;
                 p.mc_off[row] = mo;
             }
-            // a row of many chunks has its entries written by the whole wave, the others by their lane
-            const bool big = valid && nc[r] > kPlanInline;
-            if (valid && !big) {
-                for (uint32_t k = 0; k < nc[r]; ++k) p.item_row[io + k] = row;
-                for (uint32_t k = 0; k < mc[r]; ++k) { p.mc_row[mo + k] = row; p.seam[mo + k] = -1; }
-            }
-            uint64_t todo = __ballot(big);
-            while (todo) {
-                const int src = __builtin_amdgcn_readfirstlane(__builtin_ctzll(todo));
-                todo &= todo - 1;
-                const int32_t b_row = __builtin_amdgcn_readlane(row, src);
-                const int32_t b_io = __builtin_amdgcn_readlane(io, src), b_mo = __builtin_amdgcn_readlane(mo, src);
-                const uint32_t b_nc = __builtin_amdgcn_readlane(nc[r], src), b_mc = __builtin_amdgcn_readlane(mc[r], src);
-                for (uint32_t k = lane; k < b_nc; k += 64) p.item_row[b_io + k] = b_row;
-                for (uint32_t k = lane; k < b_mc; k += 64) { p.mc_row[b_mo + k] = b_row; p.seam[b_mo + k] = -1; }
-            }
+            // the entries of the work list: a row that is one item here, the chunks of a chunked
+            // row in bpe_expand_kernel (a single workgroup writing tens of thousands of scattered
+            // words is bound by its one CU's store path)
+            if (valid && nc[r] == 1) p.item_row[io] = row;
             if (valid) {
                 io += (int32_t)nc[r];
                 mo += (int32_t)mc[r];
@@ -564,14 +551,41 @@ __global__ __launch_bounds__(1024) void bpe_plan_kernel(
     }
 }
 
+// item_row / mc_row of the chunked rows: one thread per row, a row of many chunks by its wave.
+__global__ __launch_bounds__(256) void bpe_expand_kernel(int64_t n_rows, BpePlan p)
+{
+    const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    int32_t io = 0, mo = 0, nc = 0;
+    if (row < n_rows) {
+        io = p.item_off[row];
+        mo = p.mc_off[row];
+        nc = p.mc_off[row + 1] - mo;                 // 0 for a row that is a single item
+    }
+    const bool big = nc > 8;
+    if (!big)
+        for (int32_t k = 0; k < nc; ++k) { p.item_row[io + k] = (int32_t)row; p.mc_row[mo + k] = (int32_t)row; }
+    uint64_t todo = __ballot(big);
+    while (todo) {
+        const int src = __builtin_amdgcn_readfirstlane(__builtin_ctzll(todo));
+        todo &= todo - 1;
+        const int32_t b_row = __builtin_amdgcn_readlane((int32_t)row, src);
+        const int32_t b_io = __builtin_amdgcn_readlane(io, src), b_mo = __builtin_amdgcn_readlane(mo, src);
+        const int32_t b_nc = __builtin_amdgcn_readlane(nc, src);
+        for (int32_t k = lane; k < b_nc; k += 64) { p.item_row[b_io + k] = b_row; p.mc_row[b_mo + k] = b_row; }
+    }
+}
+
 // Rows and chunks of at most CAP bytes, state in LDS (13 bytes per position); the merge table
 // stays in global memory (L2-resident) and is probed in batches.  NT = 64: every wave of the
 // workgroup takes its own item (no workgroup barrier after the set-up); NT = blockDim.x: the
-// workgroup shares an item.  Items are handed out through an atomic counter.
-template <int NT, int TEAMS, int CAP>
+// workgroup shares an item.  PLANNED: the items are those of the work list (rows and chunks of
+// long rows), handed out through an atomic counter.  Otherwise (no row of the batch is longer
+// than CAP) an item is a row, teams take rows round robin, and no work list is built at all.
+template <int NT, int TEAMS, int CAP, bool PLANNED>
 __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     BpeArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
-    BpePlan p, int32_t *__restrict__ tok_tmp, int32_t *__restrict__ lengths)
+    BpePlan p, int32_t n_rows, int32_t *__restrict__ tok_tmp, int32_t *__restrict__ lengths)
 {
     extern __shared__ __align__(16) uint8_t smem[];
     uint8_t *sp = smem;
@@ -589,7 +603,7 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     __syncthreads();
 
     const uint32_t mask = a.slots - 1;
-    const int32_t n_items = p.counts[0];
+    const int32_t n_items = PLANNED ? p.counts[0] : n_rows;
     // A team's first item is its own number; only the items beyond one per team are handed out
     // through the counter.  (Every team asking the counter at the start of the kernel is a
     // thousand atomics on one address, about 12 ns each, before the last team has its row.)
@@ -597,16 +611,23 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     int32_t item = (int32_t)blockIdx.x * TEAMS + team;
     for (bool first = true;; first = false) {
         if (!first) {
-            if (n_teams >= n_items) break;           // nothing was left for the counter
-            if (tid == 0) *next_item = n_teams + atomicAdd(&p.counts[2], 1);
-            team_sync<NT>();
-            item = *next_item;
-            team_sync<NT>();
+            if (PLANNED) {
+                if (n_teams >= n_items) break;       // nothing was left for the counter
+                if (tid == 0) *next_item = n_teams + atomicAdd(&p.counts[2], 1);
+                team_sync<NT>();
+                item = *next_item;
+                team_sync<NT>();
+            } else {
+                item += n_teams;
+            }
         }
         if (item >= n_items) break;
-        const int32_t row = p.item_row[item];
-        const int32_t k = item - p.item_off[row];
-        const int32_t nc = p.item_off[row + 1] - p.item_off[row];
+        int32_t row = item, k = 0, nc = 1;
+        if (PLANNED) {
+            row = p.item_row[item];
+            k = item - p.item_off[row];
+            nc = p.item_off[row + 1] - p.item_off[row];
+        }
         const int64_t start = offsets[row];
         const int64_t len = offsets[row + 1] - start;
         // one straight path per iteration (no `continue`): every lane of the team must come
@@ -917,24 +938,62 @@ extern "C" size_t dnatok_bpe_scratch_bytes(const dnatok_bpe_t *t, int64_t n_rows
 namespace {
 
 template <int NT, int TEAMS, int CAP>
-int launch_lds(const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets, const BpePlan &p,
-               int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
+constexpr size_t lds_bytes()
 {
-    const size_t lds = 512 + 64 + (size_t)TEAMS * (4 * (NT / 64) + 4) * 4 + (size_t)TEAMS * CAP * 13 + (size_t)TEAMS * NT + 64;
-    auto kern = bpe_lds_kernel<NT, TEAMS, CAP>;
+    return 512 + 64 + (size_t)TEAMS * (4 * (NT / 64) + 4) * 4 + (size_t)TEAMS * CAP * 13 + (size_t)TEAMS * NT + 64;
+}
+
+// Teams of the LDS kernel that are resident at once (the same for both of its forms).
+template <int NT, int TEAMS, int CAP>
+int64_t lds_resident_teams()
+{
+    static const int resident =
+        resident_workgroups(bpe_lds_kernel<NT, TEAMS, CAP, true>, NT * TEAMS, lds_bytes<NT, TEAMS, CAP>(), 2);
+    return (int64_t)resident * TEAMS;
+}
+
+template <int NT, int TEAMS, int CAP, bool PLANNED>
+int launch_lds_as(const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets, const BpePlan &p,
+                  int64_t n_rows, int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
+{
+    const size_t lds = lds_bytes<NT, TEAMS, CAP>();
+    auto kern = bpe_lds_kernel<NT, TEAMS, CAP, PLANNED>;
     static bool attr_set = false;
     if (!attr_set) {
         DNATOK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         attr_set = true;
     }
-    static const int resident = resident_workgroups(kern, NT * TEAMS, lds, 2);
-    int64_t grid = (p.max_items + TEAMS - 1) / TEAMS;
+    const int64_t items = PLANNED ? p.max_items : n_rows;
+    int64_t grid = (items + TEAMS - 1) / TEAMS;
+    const int64_t resident = lds_resident_teams<NT, TEAMS, CAP>() / TEAMS;
     if (grid > resident) grid = resident;
     if (grid < 1) grid = 1;
-    kern<<<(int)grid, NT * TEAMS, lds, s>>>(a, bytes, offsets, p, tok_tmp, lengths);
+    kern<<<(int)grid, NT * TEAMS, lds, s>>>(a, bytes, offsets, p, (int32_t)n_rows, tok_tmp, lengths);
     DNATOK_HIP_TRY(hipGetLastError());
     return DNATOK_OK;
+}
+
+// The work list (plan) is needed when rows are cut into chunks or left to the whole-row kernel,
+// and when there are more rows than resident teams: rows then are dealt through the list's
+// counter, since rows take different times and a fixed share per team ends in a long tail
+// (16 x 1024 rows of 1 KB: 0.60 ms with fixed shares, 0.46 ms dealt).  A batch of at most one row
+// per team needs neither list nor counter.
+template <int NT, int TEAMS, int CAP>
+int run_lds(bool long_rows, int chunking, const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets,
+            const BpePlan &p, int64_t n_rows, int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
+{
+    const bool planned = long_rows || n_rows > lds_resident_teams<NT, TEAMS, CAP>();
+    if (planned) {
+        bpe_plan_kernel<<<1, 1024, 0, s>>>(offsets, n_rows, chunking, p);
+        DNATOK_HIP_TRY(hipGetLastError());
+        if (chunking) {
+            bpe_expand_kernel<<<(int)((n_rows + 255) / 256), 256, 0, s>>>(n_rows, p);
+            DNATOK_HIP_TRY(hipGetLastError());
+        }
+        return launch_lds_as<NT, TEAMS, CAP, true>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    }
+    return launch_lds_as<NT, TEAMS, CAP, false>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
 }
 
 }  // namespace
@@ -960,18 +1019,15 @@ extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, co
 
     const bool long_rows = max_len > p.ext;
     const int chunking = (long_rows && t->monotone) ? 1 : 0;
-    bpe_plan_kernel<<<1, 1024, 0, s>>>(offsets, n_rows, chunking, p);
-    DNATOK_HIP_TRY(hipGetLastError());
-
     // the LDS capacity variant follows the longest row (or the chunk size for longer rows):
     // less LDS per workgroup means more workgroups per CU
     int rc;
     const int64_t work_len = max_len < p.ext ? max_len : p.ext;    // longest piece the LDS kernel sees
-    if (work_len <= 1024)        rc = launch_lds<256, 1, 1024>(a, bytes, offsets, p, tok_tmp, lengths, s);
-    else if (work_len <= 1408)   rc = launch_lds<256, 1, 1408>(a, bytes, offsets, p, tok_tmp, lengths, s);
-    else if (work_len <= 1536)   rc = launch_lds<256, 1, 1536>(a, bytes, offsets, p, tok_tmp, lengths, s);
-    else if (work_len <= 2048)   rc = launch_lds<256, 1, 2048>(a, bytes, offsets, p, tok_tmp, lengths, s);
-    else                         rc = launch_lds<256, 1, kLdsCap>(a, bytes, offsets, p, tok_tmp, lengths, s);
+    if (work_len <= 1024)        rc = run_lds<256, 1, 1024>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    else if (work_len <= 1408)   rc = run_lds<256, 1, 1408>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    else if (work_len <= 1536)   rc = run_lds<256, 1, 1536>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    else if (work_len <= 2048)   rc = run_lds<256, 1, 2048>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    else                         rc = run_lds<256, 1, kLdsCap>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
     if (rc) return rc;
     if (long_rows) {
         if (chunking) {
