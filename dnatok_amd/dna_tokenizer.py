@@ -102,12 +102,19 @@ class DNATok:
         self._packed_2bit_cpu: Optional[torch.Tensor] = None
         self._dev_ping: Optional[torch.Tensor] = None
         self._dev_pong: Optional[torch.Tensor] = None
+        self._graph = None
+        self._graph_shape: Optional[Tuple[int, int]] = None
+        self._graph_static_in: Optional[torch.Tensor] = None
+        self._graph_static_out: Optional[torch.Tensor] = None
 
     def free_buffers(self) -> None:
         self._staging_bytes_cpu = None
         self._packed_2bit_cpu = None
         self._dev_ping = None
         self._dev_pong = None
+        self._graph = None
+        self._graph_static_in = None
+        self._graph_static_out = None
 
     # ------------------------------------------------------------- tokenizer access
 
@@ -555,6 +562,48 @@ class DNATok:
         weight = embed_weight if embed_weight.is_contiguous() else embed_weight.contiguous()
         out = self._char_enc.embed_packed(data, weight, row_len=t)
         return out.view(b, t, weight.shape[1])
+
+    # ------------------------------------------------------------------ HIP graph
+
+    def _record_cuda_graph(self, seqs_template: List[str], device="cuda", emb_batch: int = 0) -> None:
+        """Capture the bytes -> ids kernel for one fixed [B, T] shape in a HIP graph: static
+        uint8 input and int64 output buffers, one kernel node (the ids are written as int64 by
+        the kernel, there is no cast node).  Replays take new bytes through
+        ``_replay_cuda_graph`` (reference: 3382-3427).  Single-nucleotide tokenizers."""
+        self._require_ready()
+        if not torch.cuda.is_available():
+            raise RuntimeError("HIP graphs need a GPU.")
+        if self._char_enc is None or self._kmer_enc is not None or self.bpe_backend is not None:
+            raise RuntimeError("the graph path serves single-nucleotide table tokenizers")
+        dev = torch.device(device)
+        ascii_cpu = self.encode_batch_to_ascii_bytes(seqs_template)
+        b, t = int(ascii_cpu.shape[0]), int(ascii_cpu.shape[1])
+        self._graph_shape = (b, t)
+        self._graph_static_in = torch.empty((b, t), dtype=torch.uint8, device=dev)
+        self._graph_static_out = torch.empty((b, t), dtype=torch.long, device=dev)
+        self._graph_offsets = torch.arange(b + 1, dtype=torch.int64, device=dev) * t
+        self._graph_static_in.copy_(ascii_cpu, non_blocking=True)
+        side = torch.cuda.Stream(device=dev)                       # default priority
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):                              # warm-up outside the capture
+            self._char_enc.encode_padded(self._graph_static_in.view(-1), self._graph_offsets, t, want_mask=False,
+                                         dtype=torch.int64, ids=self._graph_static_out)
+        torch.cuda.current_stream(dev).wait_stream(side)
+        self._graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self._graph):
+            self._char_enc.encode_padded(self._graph_static_in.view(-1), self._graph_offsets, t, want_mask=False,
+                                         dtype=torch.int64, ids=self._graph_static_out)
+
+    def _replay_cuda_graph(self, ascii_cpu: torch.Tensor) -> torch.Tensor:
+        """Copy new bytes into the graph's input buffer and replay it; returns the graph's
+        output buffer, which the next replay overwrites (reference: 3429-3451)."""
+        if getattr(self, "_graph", None) is None:
+            raise RuntimeError("CUDA graph not recorded.")
+        if tuple(ascii_cpu.shape) != self._graph_shape:
+            raise ValueError(f"Graph shape mismatch: recorded {self._graph_shape}, got {tuple(ascii_cpu.shape)}")
+        self._graph_static_in.copy_(ascii_cpu, non_blocking=True)
+        self._graph.replay()
+        return self._graph_static_out
 
     # ------------------------------------------------------------------ embedding
 

@@ -199,6 +199,28 @@ def test_two_bit_path_feeds_the_same_ids_as_the_bytes_path():
     assert bytes(h.encode_batch_to_ascii_bytes(["acgtnx-R"]).numpy().tobytes()) == b"ACGTNNNN"
 
 
+def test_recorded_graph_replays_with_new_bytes():
+    """The bytes -> ids kernel captured in a HIP graph: several replays with different inputs,
+    eager encodes and synchronisations in between, every replay checked against the eager ids."""
+    tok = SimpleCharTokenizer()
+    h = DNATok(RecordingEmbedder(tok))
+    h.discover()
+    with pytest.raises(RuntimeError, match="not recorded"):
+        h._replay_cuda_graph(torch.zeros((2, 2), dtype=torch.uint8))
+    h._record_cuda_graph(random_seqs(12, 200, seed=1), device="cuda", emb_batch=4)
+    for seed in (2, 3, 4, 5):
+        seqs = random_seqs(12, 200, seed=seed)
+        want = tok(seqs, padding=True, return_tensors="pt")["input_ids"]
+        staged = h.encode_batch_to_ascii_bytes(seqs)
+        got = h._replay_cuda_graph(staged)
+        assert got.dtype == torch.int64 and got.is_cuda
+        assert torch.equal(got.cpu(), want)
+        h.encode_batch_to_ids(random_seqs(3, 50, seed=seed + 10))     # eager work between the replays
+        torch.cuda.synchronize()
+    with pytest.raises(ValueError, match="shape mismatch"):
+        h._replay_cuda_graph(torch.zeros((12, 100), dtype=torch.uint8))
+
+
 @pytest.mark.parametrize("use_i32", [True, False])
 def test_pipelined_streamer_equals_slices(use_i32):
     tok = SimpleCharTokenizer()
