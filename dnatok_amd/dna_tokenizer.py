@@ -560,8 +560,12 @@ class DNATok:
         b, t = ascii_bytes.shape
         data = ascii_bytes.to(device, non_blocking=True).reshape(-1)
         weight = embed_weight if embed_weight.is_contiguous() else embed_weight.contiguous()
-        out = self._char_enc.embed_packed(data, weight, row_len=t)
+        # like the reference's kernel, this is weight[ascii_lut[bytes]]: the separate table for a
+        # row's first character is not applied here
+        out = self._char_enc.embed_packed(data, weight, row_len=0)
         return out.view(b, t, weight.shape[1])
+
+    _fused_tokenize_gather = fused_tokenize_gather
 
     # ------------------------------------------------------------------ HIP graph
 

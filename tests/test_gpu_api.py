@@ -199,6 +199,20 @@ def test_two_bit_path_feeds_the_same_ids_as_the_bytes_path():
     assert bytes(h.encode_batch_to_ascii_bytes(["acgtnx-R"]).numpy().tobytes()) == b"ACGTNNNN"
 
 
+def test_fused_tokenize_gather_equals_lookup_then_embedding():
+    tok = SimpleCharTokenizer()
+    emb = RecordingEmbedder(tok).to("cuda")
+    h = DNATok(emb)
+    h.discover()
+    seqs = random_seqs(6, 333, seed=8)
+    weight = torch.randn((8, 64), device="cuda").to(torch.bfloat16)
+    staged = h.encode_batch_to_ascii_bytes(seqs)
+    out = h._fused_tokenize_gather(staged, weight, "cuda")
+    ids = h.ids_from_ascii_bytes_cuda(staged)
+    assert out.shape == (6, 333, 64) and out.dtype == torch.bfloat16
+    assert torch.equal(out.view(torch.int16), weight[ids].view(torch.int16))
+
+
 def test_recorded_graph_replays_with_new_bytes():
     """The bytes -> ids kernel captured in a HIP graph: several replays with different inputs,
     eager encodes and synchronisations in between, every replay checked against the eager ids."""
