@@ -37,6 +37,7 @@
 struct dnatok_bpe_table {
     int32_t n_merges, n_symbols;
     uint32_t slots, shift;       // hash table size (power of two) and 32 - log2(slots)
+    uint32_t mul1, mul2;         // multipliers of the two hash functions
     int monotone;                // no rule's product is used by a lower-ranked rule
     void *blob;
     uint4 *tab;                  // [slots]  {key = a << 16 | b, rank, product | gate << 16, 0}
@@ -53,7 +54,7 @@ struct BpeArgs {
     const uint4 *tab;
     const uint16_t *byte_to_sym;
     const int32_t *out_remap;
-    uint32_t slots, shift;
+    uint32_t shift, mul1, mul2;
     int32_t n_merges;
 };
 
@@ -63,31 +64,46 @@ struct PairInfo {
     uint32_t rank, product, gate;
 };
 
-__host__ __device__ __forceinline__ uint32_t pair_hash(uint32_t key, uint32_t shift)
+// The merge table is a cuckoo hash: every rule sits in one of the two slots its key hashes to, so
+// a lookup is two independent reads issued together and never a chain of dependent ones.  (With
+// linear probing a wave's lookup was as slow as its unluckiest lane: two to three trips to L2 per
+// lookup even at one rule per eight slots.)
+struct PairTable {
+    const uint4 *tab;
+    uint32_t shift, mul1, mul2;
+};
+
+struct PairEntry {               // the three words of a slot that carry something
+    uint32_t x, y, z;
+};
+
+struct PairProbe {
+    PairEntry e1, e2;
+};
+
+__host__ __device__ __forceinline__ uint32_t pair_slot(uint32_t key, uint32_t mul, uint32_t shift)
 {
-    return (key * 0x9E3779B1u) >> shift;
+    return (key * mul) >> shift;
 }
 
-// First probe of the rule for (a, b): issued for several pairs back to back, so that their
-// memory latencies overlap; pair_finish resolves the (rare) collisions afterwards.
-__device__ __forceinline__ uint4 pair_probe(const uint4 *tab, uint32_t shift, uint32_t a, uint32_t b,
-                                            uint32_t *slot)
-{
-    const uint32_t h = pair_hash((a << 16) | b, shift);
-    *slot = h;
-    return tab[h];
-}
-
-__device__ __forceinline__ PairInfo pair_finish(const uint4 *tab, uint32_t mask, uint32_t a, uint32_t b,
-                                                uint4 e, uint32_t h)
+// Both reads of the rule for (a, b); issued for several pairs back to back, so that their memory
+// latencies overlap.  pair_finish picks the answer.
+__device__ __forceinline__ PairProbe pair_probe(const PairTable &t, uint32_t a, uint32_t b)
 {
     const uint32_t key = (a << 16) | b;
-    for (;;) {
-        if (e.x == key) return PairInfo{e.y, e.z & 0xFFFFu, e.z >> 16};
-        if (e.x == kEmptyKey) return PairInfo{kNone, kNone, kNone};
-        h = (h + 1) & mask;
-        e = tab[h];
-    }
+    PairProbe pr;
+    pr.e1 = *reinterpret_cast<const PairEntry *>(t.tab + pair_slot(key, t.mul1, t.shift));
+    pr.e2 = *reinterpret_cast<const PairEntry *>(t.tab + pair_slot(key, t.mul2, t.shift));
+    return pr;
+}
+
+__device__ __forceinline__ PairInfo pair_finish(uint32_t a, uint32_t b, const PairProbe &pr)
+{
+    const uint32_t key = (a << 16) | b;
+    const bool first = pr.e1.x == key;
+    const uint32_t y = first ? pr.e1.y : pr.e2.y, z = first ? pr.e1.z : pr.e2.z;
+    if (!first && pr.e2.x != key) return PairInfo{kNone, kNone, kNone};
+    return PairInfo{y, z & 0xFFFFu, z >> 16};
 }
 
 template <int NT>
@@ -155,39 +171,40 @@ struct alignas(4 * sizeof(IT)) PosRec {
 // n0 / 2; D holds NT bytes; red holds 4 * (NT / 64) + 4 words.  Tokens go to out[0 .. *out_len).
 template <int NT, typename IT>
 __device__ __forceinline__ void bpe_row(
-    const uint4 *tab, uint32_t tab_mask, uint32_t tab_shift, const uint16_t *byte_to_sym,
+    const PairTable pt, const uint16_t *byte_to_sym,
     const int32_t *out_remap, const uint8_t *__restrict__ src, const int n0, PosRec<IT> *P,
     uint16_t *NS, uint16_t *MC, IT *Q, uint8_t *D, uint32_t *red, const int tid,
     int32_t *__restrict__ out, int32_t *__restrict__ out_len, uint16_t *__restrict__ raw_out = nullptr)
 {
     constexpr IT NIL = (IT)~(IT)0;
     constexpr IT DEAD = (IT)kNone;
+    constexpr int kProbes = 2;
     const int wv = (NT == 64) ? 0 : (tid >> 6);
     uint32_t *qn = red + 4 * (NT / 64);        // number of merges queued in the current round
     // position i belongs to thread i % NT: in every pass the lanes of a wave touch consecutive
     // positions, so the LDS state arrays are read and written without bank conflicts
 
-    // symbols, links and the initial pair of every position, four table probes in flight at a time
+    // symbols, links and the initial pair of every position, kProbes pairs of table reads in flight at a time
     uint32_t cmin = kEmptyKey, cgate = kEmptyKey;
     D[tid] = 0;
     if (tid == 0) *qn = 0;
-    for (int i0 = tid; i0 < n0; i0 += 4 * NT) {
-        uint4 e[4];
-        uint32_t h[4], sa[4], sb[4];
+    for (int i0 = tid; i0 < n0; i0 += kProbes * NT) {
+        PairProbe e[kProbes];
+        uint32_t sa[kProbes], sb[kProbes];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < kProbes; ++j) {
             const int i = i0 + j * NT;
             const bool ok = i + 1 < n0;
             sa[j] = i < n0 ? byte_to_sym[src[i]] : 0u;
             sb[j] = ok ? byte_to_sym[src[i + 1]] : 0u;
-            e[j] = pair_probe(tab, tab_shift, ok ? sa[j] : 0u, sb[j], &h[j]);
+            e[j] = pair_probe(pt, ok ? sa[j] : 0u, sb[j]);
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < kProbes; ++j) {
             const int i = i0 + j * NT;
             if (i >= n0) continue;
             PairInfo pi{kNone, kNone, kNone};
-            if (i + 1 < n0) pi = pair_finish(tab, tab_mask, sa[j], sb[j], e[j], h[j]);
+            if (i + 1 < n0) pi = pair_finish(sa[j], sb[j], e[j]);
             PosRec<IT> x;
             x.r = (IT)pi.rank;
             x.nx = (i + 1 < n0) ? (IT)(i + 1) : NIL;
@@ -226,7 +243,9 @@ __device__ __forceinline__ void bpe_row(
             // the thread's positions four at a time: their records are read together, not one
             // after the other behind each candidate's chain walk.  (Reading the candidates'
             // neighbours ahead as well, and one queue atomic per wave instead of one per merge,
-            // were measured: the phase got 15-20 % slower.)
+            // were measured: the phase got 15-20 % slower.  So were the four candidates walking
+            // their chains in step: a long chain, e.g. inside a tandem repeat, then drags the
+            // loop body of all four along, and the 32000-vocabulary rows took 1.6 x as long.)
             for (int i0 = tid; i0 < n0; i0 += 4 * NT) {
               PosRec<IT> xs[4];
 #pragma unroll
@@ -282,14 +301,14 @@ __device__ __forceinline__ void bpe_row(
 
         // re-rank the two pairs around every new symbol: probe 2m is the pair (new, right
         // neighbour), probe 2m + 1 the pair (left neighbour, new).  The probes are dealt evenly to
-        // the threads, four table reads in flight per thread.
-        for (int p0 = tid; p0 < 2 * nm; p0 += 4 * NT) {
-            uint4 e[4];
-            uint32_t h[4], sa[4], sb[4];
-            IT target[4];
-            bool valid[4];
+        // the threads, kProbes pairs of table reads in flight per thread.
+        for (int p0 = tid; p0 < 2 * nm; p0 += kProbes * NT) {
+            PairProbe e[kProbes];
+            uint32_t sa[kProbes], sb[kProbes];
+            IT target[kProbes];
+            bool valid[kProbes];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < kProbes; ++j) {
                 const int p = p0 + j * NT;
                 sa[j] = 0; sb[j] = 0; target[j] = NIL; valid[j] = false;
                 if (p < 2 * nm) {
@@ -303,13 +322,13 @@ __device__ __forceinline__ void bpe_row(
                         if (x.nx != NIL) { sa[j] = x.s; sb[j] = P[x.nx].s; valid[j] = true; }
                     }
                 }
-                e[j] = pair_probe(tab, tab_shift, sa[j], sb[j], &h[j]);
+                e[j] = pair_probe(pt, sa[j], sb[j]);
             }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < kProbes; ++j) {
                 if (target[j] == NIL) continue;       // no probe, or no left neighbour
                 PairInfo pi{kNone, kNone, kNone};
-                if (valid[j]) pi = pair_finish(tab, tab_mask, sa[j], sb[j], e[j], h[j]);
+                if (valid[j]) pi = pair_finish(sa[j], sb[j], e[j]);
                 const int q = (int)target[j];
                 P[q].r = (IT)pi.rank; NS[q] = (uint16_t)pi.product; MC[q] = (uint16_t)pi.gate;
                 D[q % NT] = 1;
@@ -589,7 +608,7 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
 {
     extern __shared__ __align__(16) uint8_t smem[];
     uint8_t *sp = smem;
-    const uint4 *tab = a.tab;
+    const PairTable pt{a.tab, a.shift, a.mul1, a.mul2};
     uint16_t *b2s = reinterpret_cast<uint16_t *>(sp); sp += 512;
     for (int i = threadIdx.x; i < 256; i += NT * TEAMS) b2s[i] = a.byte_to_sym[i];
     const int team = threadIdx.x / NT, tid = threadIdx.x % NT;
@@ -602,7 +621,6 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     uint8_t *D = sp + (size_t)team * NT;
     __syncthreads();
 
-    const uint32_t mask = a.slots - 1;
     const int32_t n_items = PLANNED ? p.counts[0] : n_rows;
     // A team's first item is its own number; only the items beyond one per team are handed out
     // through the counter.  (Every team asking the counter at the start of the kernel is a
@@ -637,14 +655,14 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
             // too long: left to the whole-row kernel (row_fail is set); empty: no tokens
             if (tid == 0) lengths[row] = len > CAP ? -1 : 0;
         } else if (nc == 1) {
-            bpe_row<NT, uint16_t>(tab, mask, a.shift, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC,
+            bpe_row<NT, uint16_t>(pt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC,
                                   Q, D, red, tid, tok_tmp + start, lengths + row);
         } else {
             const int64_t e0 = (int64_t)k * p.core - p.overlap < 0 ? 0 : (int64_t)k * p.core - p.overlap;
             int64_t e1 = (int64_t)(k + 1) * p.core + p.overlap;
             if (e1 > len) e1 = len;
             uint16_t *raw = p.chunk_sym + (size_t)(p.mc_off[row] + k) * p.ext;
-            bpe_row<NT, uint16_t>(tab, mask, a.shift, b2s, a.out_remap, bytes + start + e0, (int)(e1 - e0),
+            bpe_row<NT, uint16_t>(pt, b2s, a.out_remap, bytes + start + e0, (int)(e1 - e0),
                                   P, NS, MC, Q, D, red, tid, nullptr, nullptr, raw);
         }
         team_sync<NT>();
@@ -820,7 +838,7 @@ __global__ __launch_bounds__(NT) void bpe_long_kernel(
     __syncthreads();
     // each workgroup owns one slab of scratch, sized for the longest row
     uint8_t *slab = p.slabs + (size_t)blockIdx.x * p.slab_bytes;
-    const uint32_t mask = a.slots - 1;
+    const PairTable pt{a.tab, a.shift, a.mul1, a.mul2};
     for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
         if (!p.row_fail[row]) continue;
         const int64_t start = offsets[row];
@@ -834,7 +852,7 @@ __global__ __launch_bounds__(NT) void bpe_long_kernel(
         uint16_t *NS = reinterpret_cast<uint16_t *>(P + n);
         uint16_t *MC = NS + n;
         uint32_t *Q = reinterpret_cast<uint32_t *>(MC + n);      // n / 2 entries
-        bpe_row<NT, uint32_t>(a.tab, mask, a.shift, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC,
+        bpe_row<NT, uint32_t>(pt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC,
                               Q, D, red, threadIdx.x, tok_tmp + start, lengths + row);
         __syncthreads();
     }
@@ -859,36 +877,55 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
     for (int i = 0; i < 256; ++i)
         DNATOK_REQUIRE(byte_to_id_h[i] >= 0 && byte_to_id_h[i] < n_symbols, DNATOK_E_INVALID,
                        "dnatok_bpe_table_create: byte_to_id[%d] out of range", i);
-    uint32_t slots = 64, shift = 26;
-    // 8 slots per rule: a pair that has no rule (most probes in the later rounds) is then
-    // answered by its first probe nearly always, and a wave's probe is as slow as its slowest lane
-    while (slots < (uint32_t)n_merges * 8u + 2u) { slots <<= 1; --shift; }
-    std::vector<uint4> tab(slots, uint4{kEmptyKey, kNone, 0, 0});
-    std::vector<uint32_t> slot_of(n_merges > 0 ? n_merges : 1, 0xFFFFFFFFu);
-    std::vector<uint32_t> first_use(n_symbols, 0xFFFFFFFFu);   // lowest rank using a symbol
     for (int32_t i = 0; i < n_merges; ++i) {
         const int32_t pa = pair_a_h[i], pb = pair_b_h[i], nid = new_id_h[i];
         DNATOK_REQUIRE(pa >= 0 && pa < n_symbols && pb >= 0 && pb < n_symbols && nid >= 0 && nid < n_symbols,
                        DNATOK_E_INVALID, "dnatok_bpe_table_create: merge %d has an id out of range", i);
-        const uint32_t key = ((uint32_t)pa << 16) | (uint32_t)pb;
-        uint32_t h = pair_hash(key, shift);
-        bool dup = false;
-        while (tab[h].x != kEmptyKey) {
-            if (tab[h].x == key) { dup = true; break; }
-            h = (h + 1) & (slots - 1);
+    }
+    // Four to eight slots per rule, far below the load at which two-choice cuckoo placement starts
+    // to fail; a placement that still fails is redone with other multipliers, then a larger table.
+    static const uint32_t kMul[8] = {0x9E3779B1u, 0x85EBCA6Bu, 0xC2B2AE35u, 0x27D4EB2Fu,
+                                     0x165667B1u, 0xD3A2646Du, 0xFD7046C5u, 0xB55A4F09u};
+    uint32_t slots = 64, shift = 26, mul1 = 0, mul2 = 0;
+    while (slots < (uint32_t)n_merges * 4u + 2u) { slots <<= 1; --shift; }
+    std::vector<uint4> tab;
+    std::vector<uint32_t> first_use;                           // lowest rank using a symbol
+    for (int attempt = 0;; ++attempt) {
+        DNATOK_REQUIRE(shift > 4, DNATOK_E_INVALID, "dnatok_bpe_table_create: the merge table could not be hashed");
+        mul1 = kMul[(2 * attempt) & 7]; mul2 = kMul[(2 * attempt + 1) & 7];
+        tab.assign(slots, uint4{kEmptyKey, kNone, 0, 0});
+        first_use.assign(n_symbols, 0xFFFFFFFFu);
+        bool placed = true;
+        for (int32_t i = 0; i < n_merges && placed; ++i) {
+            const uint32_t pa = (uint32_t)pair_a_h[i], pb = (uint32_t)pair_b_h[i];
+            const uint32_t key = (pa << 16) | pb;
+            if (tab[pair_slot(key, mul1, shift)].x == key || tab[pair_slot(key, mul2, shift)].x == key)
+                continue;                       // a repeated pair keeps its first rank
+            if (first_use[pa] == 0xFFFFFFFFu) first_use[pa] = (uint32_t)i;
+            if (first_use[pb] == 0xFFFFFFFFu) first_use[pb] = (uint32_t)i;
+            uint4 e{key, (uint32_t)i, (uint32_t)new_id_h[i], 0};
+            uint32_t came_from = 0xFFFFFFFFu;
+            placed = false;
+            for (int kick = 0; kick < 512; ++kick) {
+                const uint32_t h1 = pair_slot(e.x, mul1, shift), h2 = pair_slot(e.x, mul2, shift);
+                if (tab[h1].x == kEmptyKey) { tab[h1] = e; placed = true; break; }
+                if (tab[h2].x == kEmptyKey) { tab[h2] = e; placed = true; break; }
+                const uint32_t v = (h1 == came_from) ? h2 : h1;     // push out the entry of the other slot
+                const uint4 out_e = tab[v];
+                tab[v] = e; e = out_e; came_from = v;
+            }
         }
-        if (dup) continue;                      // a repeated pair keeps its first rank
-        tab[h] = uint4{key, (uint32_t)i, (uint32_t)nid, 0};
-        slot_of[i] = h;
-        if (first_use[pa] == 0xFFFFFFFFu) first_use[pa] = (uint32_t)i;
-        if (first_use[pb] == 0xFFFFFFFFu) first_use[pb] = (uint32_t)i;
+        if (placed) break;
+        if ((attempt & 3) == 3) { slots <<= 1; --shift; }
     }
     int monotone = 1;
-    for (int32_t i = 0; i < n_merges; ++i) {
-        const uint32_t fu = first_use[new_id_h[i]];
-        if (slot_of[i] != 0xFFFFFFFFu) tab[slot_of[i]].z |= (fu == 0xFFFFFFFFu ? kNone : fu) << 16;
-        if (fu <= (uint32_t)i) monotone = 0;
-    }
+    for (int32_t i = 0; i < n_merges; ++i)
+        if (first_use[new_id_h[i]] <= (uint32_t)i) monotone = 0;
+    for (uint4 &e : tab)
+        if (e.x != kEmptyKey) {
+            const uint32_t fu = first_use[e.z];
+            e.z |= (fu == 0xFFFFFFFFu ? kNone : fu) << 16;
+        }
     std::vector<uint16_t> b2s(256);
     for (int i = 0; i < 256; ++i) b2s[i] = (uint16_t)byte_to_id_h[i];
 
@@ -911,7 +948,7 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
     }
     dnatok_bpe_table *t = new dnatok_bpe_table();
     uint8_t *b = (uint8_t *)blob;
-    t->n_merges = n_merges; t->n_symbols = n_symbols; t->slots = slots; t->shift = shift;
+    t->n_merges = n_merges; t->n_symbols = n_symbols; t->slots = slots; t->shift = shift; t->mul1 = mul1; t->mul2 = mul2;
     t->monotone = monotone; t->blob = blob;
     t->tab = (uint4 *)(b + o_tab);
     t->byte_to_sym = (uint16_t *)(b + o_b2s);
@@ -1015,7 +1052,7 @@ extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, co
     DNATOK_REQUIRE(((uintptr_t)scratch & 255) == 0, DNATOK_E_INVALID, "dnatok_bpe_encode: scratch must be 256-byte aligned");
     const BpePlan p = make_plan((uint8_t *)scratch, n_rows, max_len, total);
     hipStream_t s = (hipStream_t)stream;
-    BpeArgs a{t->tab, t->byte_to_sym, t->out_remap, t->slots, t->shift, t->n_merges};
+    BpeArgs a{t->tab, t->byte_to_sym, t->out_remap, t->shift, t->mul1, t->mul2, t->n_merges};
 
     const bool long_rows = max_len > p.ext;
     const int chunking = (long_rows && t->monotone) ? 1 : 0;
