@@ -473,6 +473,24 @@ def test_bpe_nonmonotone_random_tables():
             np.testing.assert_array_equal(r, e, err_msg=f"trial {trial} {s} {merges}")
 
 
+def test_bpe_repeated_pair_keeps_its_first_rank():
+    """A pair listed twice: the later entry (another rank, another product) must never be used."""
+    say("bpe table with a repeated pair")
+    merges = [("A", "C"), ("AC", "G"), ("T", "T"), ("ACG", "TT"), ("G", "A")]
+    kv = bpe_vocab.KernelVocab(merges)
+    a, b2, n = list(kv.pair_a), list(kv.pair_b), list(kv.new_id)
+    a.insert(3, a[0]); b2.insert(3, b2[0]); n.insert(3, n[2])          # (A, C) again, giving TT's id
+    plain = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv))
+    twice = encoders.BpeEncoder(np.array(a, dtype=np.int32), np.array(b2, dtype=np.int32),
+                                np.array(n, dtype=np.int32), len(kv))
+    rng = random.Random(5)
+    seqs = ["".join(rng.choice("ACGT") for _ in range(rng.randint(1, 400))) for _ in range(50)]
+    b = util.batch_from_strings(seqs)
+    # ranks above the inserted entry shift by one, the ids produced do not
+    for r1, r2 in zip(bpe_rows(plain, b), bpe_rows(twice, b)):
+        np.testing.assert_array_equal(r1, r2)
+
+
 # ---------------------------------------------------------------- packer
 
 def test_c5_ragged_bpe_and_char_packed(char_enc):
