@@ -25,8 +25,8 @@
 // rules produce the same string) makes G <= rmin; such a round merges only the single
 // smallest-key pair, which is exactly HF's next step.
 //
-// State lives in LDS for rows up to the LDS capacity (13 bytes per position: an 8-byte record,
-// product and gate of the position's pair, and the queue), and in a global scratch area
+// State lives in LDS for rows up to the LDS capacity (15 bytes per position: an 8-byte record,
+// product and gate of the position's pair, and the two queues), and in a global scratch area
 // (L2-resident, 32-bit links) for longer rows that cannot be cut into chunks.
 #include "common.hpp"
 
@@ -168,12 +168,13 @@ struct alignas(4 * sizeof(IT)) PosRec {
 };
 
 // One row.  tid = index in the team; P/NS/MC hold n0 entries, Q (the merges of the current round)
-// n0 / 2; D holds NT bytes; red holds 4 * (NT / 64) + 4 words.  Tokens go to out[0 .. *out_len).
-template <int NT, typename IT>
+// n0 / 2, C (its candidates) n0; D holds NT bytes; PER > 0 says that n0 <= PER * NT, and every thread
+// then keeps the ranks of its own positions in registers as well; red holds 4 * (NT / 64) + 4 words.  Tokens go to out[0 .. *out_len).
+template <int NT, typename IT, int PER>
 __device__ __forceinline__ void bpe_row(
     const PairTable pt, const uint16_t *byte_to_sym,
     const int32_t *out_remap, const uint8_t *__restrict__ src, const int n0, PosRec<IT> *P,
-    uint16_t *NS, uint16_t *MC, IT *Q, uint8_t *D, uint32_t *red, const int tid,
+    uint16_t *NS, uint16_t *MC, IT *Q, IT *C, uint8_t *D, uint32_t *red, const int tid,
     int32_t *__restrict__ out, int32_t *__restrict__ out_len, uint16_t *__restrict__ raw_out = nullptr)
 {
     constexpr IT NIL = (IT)~(IT)0;
@@ -181,13 +182,14 @@ __device__ __forceinline__ void bpe_row(
     constexpr int kProbes = 2;
     const int wv = (NT == 64) ? 0 : (tid >> 6);
     uint32_t *qn = red + 4 * (NT / 64);        // number of merges queued in the current round
+    uint32_t *cn = qn + 1;                     // number of candidates queued in the current round
     // position i belongs to thread i % NT: in every pass the lanes of a wave touch consecutive
     // positions, so the LDS state arrays are read and written without bank conflicts
 
     // symbols, links and the initial pair of every position, kProbes pairs of table reads in flight at a time
     uint32_t cmin = kEmptyKey, cgate = kEmptyKey;
     D[tid] = 0;
-    if (tid == 0) *qn = 0;
+    if (tid == 0) { *qn = 0; *cn = 0; }
     for (int i0 = tid; i0 < n0; i0 += kProbes * NT) {
         PairProbe e[kProbes];
         uint32_t sa[kProbes], sb[kProbes];
@@ -216,6 +218,18 @@ __device__ __forceinline__ void bpe_row(
         }
     }
 
+    // ranks of the thread's own positions (position tid + k * NT is its k-th), kept up to date by
+    // the refresh at the end of every round: the candidates of a round are then found without
+    // reading LDS
+    uint32_t myr[PER > 0 ? PER : 1];
+    if (PER > 0) {
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+            const int i = tid + k * NT;
+            myr[k] = i < n0 ? (uint32_t)P[i].r : kNone;      // written by this thread just above
+        }
+    }
+
     int flip = 0;
     int budget = n0 + 8;                       // every round merges at least one pair
     bool stuck = false;
@@ -238,50 +252,68 @@ __device__ __forceinline__ void bpe_row(
         }
         const uint32_t limit = single ? rmin + 1 : gate;
 
-        // decide (reads only); a pair that merges is put on the round's queue
-        if (cmin < limit) {
-            // the thread's positions four at a time: their records are read together, not one
-            // after the other behind each candidate's chain walk.  (Reading the candidates'
-            // neighbours ahead as well, and one queue atomic per wave instead of one per merge,
-            // were measured: the phase got 15-20 % slower.  So were the four candidates walking
-            // their chains in step: a long chain, e.g. inside a tandem repeat, then drags the
-            // loop body of all four along, and the 32000-vocabulary rows took 1.6 x as long; the
-            // left and right chain of one candidate walked in one loop: 1.1-1.2 x; one queue atomic
-            // per thread for its four positions: 1.03 x.)
-            for (int i0 = tid; i0 < n0; i0 += 4 * NT) {
-              PosRec<IT> xs[4];
+        // decide (reads only); a pair that merges is put on the round's queue.  The candidates
+        // (pairs with a rank below the limit, typically a quarter of the live positions, spread
+        // unevenly over the threads) are first collected on a queue of their own and then dealt out
+        // one per thread: every thread walks one candidate's chains at a time, with all lanes of a
+        // wave busy, instead of its own positions one after the other with most lanes idle.
+        if (single) {
+            if (tid == 0) { Q[0] = (IT)leftmost; *qn = 1; }
+        } else {
+            const int lane = tid & 63;
+            constexpr int kBlocks = PER > 0 ? (PER + 3) / 4 : 1 << 20;
 #pragma unroll
-              for (int k = 0; k < 4; ++k) { const int i = i0 + k * NT; xs[k] = P[i < n0 ? i : tid]; }
+            for (int blk = 0; blk < kBlocks; ++blk) {     // the same trip count for every lane
+                const int b0 = blk * 4 * NT;
+                if (b0 >= n0) break;
+                uint64_t bal[4];
+                uint32_t total = 0;
 #pragma unroll
-              for (int k = 0; k < 4; ++k) {
-                const int i = i0 + k * NT;
-                if (i >= n0) continue;
-                const PosRec<IT> x = xs[k];
-                const uint32_t r = x.r;
-                if (r >= limit) continue;
-                bool m;
-                if (single) {
-                    m = ((uint32_t)i == leftmost);
-                } else {
-                    // both neighbours' records are requested together
-                    PosRec<IT> yl = P[x.pv != NIL ? x.pv : (IT)i];
-                    PosRec<IT> yr = P[x.nx != NIL ? x.nx : (IT)i];
-                    uint32_t chain = 0, rp = r;
-                    IT q = x.pv;
-                    while (q != NIL && yl.r <= rp) {      // candidates to the left with key <= ours
-                        ++chain; rp = yl.r; q = yl.pv;
-                        if (q != NIL) yl = P[q];
+                for (int k = 0; k < 4; ++k) {
+                    bool c;
+                    if (PER > 0) {
+                        c = blk * 4 + k < PER && myr[blk * 4 + k < PER ? blk * 4 + k : 0] < limit;
+                    } else {
+                        const int i = b0 + k * NT + tid;
+                        c = cmin < limit && i < n0 && (uint32_t)P[i].r < limit;
                     }
-                    uint32_t chain_r = 0;
-                    rp = r; q = x.nx;
-                    while (q != NIL && yr.r < rp) {       // candidates to the right with key < ours
-                        ++chain_r; rp = yr.r; q = yr.nx;
-                        if (q != NIL) yr = P[q];
-                    }
-                    m = ((chain | chain_r) & 1u) == 0;
+                    bal[k] = __ballot(c);
+                    total += (uint32_t)__builtin_popcountll(bal[k]);
                 }
-                if (m) Q[atomicAdd(qn, 1u)] = (IT)i;
-              }
+                if (total == 0) continue;                 // (uniform over the wave)
+                uint32_t at = 0;
+                if (lane == 0) at = atomicAdd(cn, total);
+                at = (uint32_t)__builtin_amdgcn_readfirstlane((int)at);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    if (bal[k] >> lane & 1ull)
+                        C[at + (uint32_t)__builtin_popcountll(bal[k] & ((1ull << lane) - 1ull))] =
+                            (IT)(b0 + k * NT + tid);
+                    at += (uint32_t)__builtin_popcountll(bal[k]);
+                }
+            }
+            team_sync<NT>();
+            const int ncand = (int)*cn;
+            for (int c = tid; c < ncand; c += NT) {
+                const int i = (int)C[c];
+                const PosRec<IT> x = P[i];
+                const uint32_t r = x.r;
+                // both neighbours' records are requested together
+                PosRec<IT> yl = P[x.pv != NIL ? x.pv : (IT)i];
+                PosRec<IT> yr = P[x.nx != NIL ? x.nx : (IT)i];
+                uint32_t chain = 0, rp = r;
+                IT q = x.pv;
+                while (q != NIL && yl.r <= rp) {          // candidates to the left with key <= ours
+                    ++chain; rp = yl.r; q = yl.pv;
+                    if (q != NIL) yl = P[q];
+                }
+                uint32_t chain_r = 0;
+                rp = r; q = x.nx;
+                while (q != NIL && yr.r < rp) {           // candidates to the right with key < ours
+                    ++chain_r; rp = yr.r; q = yr.nx;
+                    if (q != NIL) yr = P[q];
+                }
+                if (((chain | chain_r) & 1u) == 0) Q[atomicAdd(qn, 1u)] = (IT)i;
             }
         }
         team_sync<NT>();
@@ -337,14 +369,24 @@ __device__ __forceinline__ void bpe_row(
             }
         }
         team_sync<NT>();
-        if (tid == 0) *qn = 0;                     // seen by the next round's decide (a sync lies between)
+        if (tid == 0) { *qn = 0; *cn = 0; }        // seen by the next round's decide (a sync lies between)
 
         if (D[tid]) {
             D[tid] = 0;
             cmin = kEmptyKey; cgate = kEmptyKey;
-            for (int i = tid; i < n0; i += NT) {
-                const uint32_t r = P[i].r;
-                if (r != kNone) { cmin = umin(cmin, r); cgate = umin(cgate, MC[i]); }
+            if (PER > 0) {
+#pragma unroll
+                for (int k = 0; k < PER; ++k) {
+                    const int i = tid + k * NT;
+                    const uint32_t r = i < n0 ? (uint32_t)P[i].r : kNone;
+                    myr[k] = r;
+                    if (r != kNone) { cmin = umin(cmin, r); cgate = umin(cgate, MC[i]); }
+                }
+            } else {
+                for (int i = tid; i < n0; i += NT) {
+                    const uint32_t r = P[i].r;
+                    if (r != kNone) { cmin = umin(cmin, r); cgate = umin(cgate, MC[i]); }
+                }
             }
         }
     }
@@ -438,7 +480,7 @@ struct BpePlan {                          // device arrays inside the scratch bu
 static size_t long_slab_bytes(int64_t max_len)
 {
     const size_t n = ((size_t)max_len + 7) & ~(size_t)7;
-    return ((n * 22) + 255) & ~(size_t)255;     // 16 (records) + 2 + 2 (product, gate) + 2 (queue)
+    return ((n * 26) + 255) & ~(size_t)255;     // 16 (records) + 2 + 2 (product, gate) + 2 + 4 (queues)
 }
 
 // chunk geometry: DNATOK_BPE_CHUNK="core,overlap" overrides the default (for experiments)
@@ -597,7 +639,7 @@ __global__ __launch_bounds__(256) void bpe_expand_kernel(int64_t n_rows, BpePlan
     }
 }
 
-// Rows and chunks of at most CAP bytes, state in LDS (13 bytes per position); the merge table
+// Rows and chunks of at most CAP bytes, state in LDS (15 bytes per position); the merge table
 // stays in global memory (L2-resident) and is probed in batches.  NT = 64: every wave of the
 // workgroup takes its own item (no workgroup barrier after the set-up); NT = blockDim.x: the
 // workgroup shares an item.  PLANNED: the items are those of the work list (rows and chunks of
@@ -620,6 +662,7 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     uint16_t *NS = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
     uint16_t *MC = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
     uint16_t *Q = reinterpret_cast<uint16_t *>(sp) + (size_t)team * (CAP / 2); sp += (size_t)TEAMS * CAP;
+    uint16_t *C = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
     uint8_t *D = sp + (size_t)team * NT;
     __syncthreads();
 
@@ -657,15 +700,15 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
             // too long: left to the whole-row kernel (row_fail is set); empty: no tokens
             if (tid == 0) lengths[row] = len > CAP ? -1 : 0;
         } else if (nc == 1) {
-            bpe_row<NT, uint16_t>(pt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC,
-                                  Q, D, red, tid, tok_tmp + start, lengths + row);
+            bpe_row<NT, uint16_t, (CAP + NT - 1) / NT>(pt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC,
+                                  Q, C, D, red, tid, tok_tmp + start, lengths + row);
         } else {
             const int64_t e0 = (int64_t)k * p.core - p.overlap < 0 ? 0 : (int64_t)k * p.core - p.overlap;
             int64_t e1 = (int64_t)(k + 1) * p.core + p.overlap;
             if (e1 > len) e1 = len;
             uint16_t *raw = p.chunk_sym + (size_t)(p.mc_off[row] + k) * p.ext;
-            bpe_row<NT, uint16_t>(pt, b2s, a.out_remap, bytes + start + e0, (int)(e1 - e0),
-                                  P, NS, MC, Q, D, red, tid, nullptr, nullptr, raw);
+            bpe_row<NT, uint16_t, (CAP + NT - 1) / NT>(pt, b2s, a.out_remap, bytes + start + e0, (int)(e1 - e0),
+                                  P, NS, MC, Q, C, D, red, tid, nullptr, nullptr, raw);
         }
         team_sync<NT>();
     }
@@ -825,7 +868,7 @@ __global__ __launch_bounds__(256) void bpe_gather_kernel(
 }
 
 // Whole-row kernel for rows above the LDS capacity that could not be chunked: one workgroup per
-// row, state in global scratch (22 bytes / base).
+// row, state in global scratch (26 bytes / base).
 template <int NT>
 __global__ __launch_bounds__(NT) void bpe_long_kernel(
     BpeArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
@@ -854,8 +897,9 @@ __global__ __launch_bounds__(NT) void bpe_long_kernel(
         uint16_t *NS = reinterpret_cast<uint16_t *>(P + n);
         uint16_t *MC = NS + n;
         uint32_t *Q = reinterpret_cast<uint32_t *>(MC + n);      // n / 2 entries
-        bpe_row<NT, uint32_t>(pt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC,
-                              Q, D, red, threadIdx.x, tok_tmp + start, lengths + row);
+        uint32_t *C = Q + n / 2;                                 // n entries
+        bpe_row<NT, uint32_t, 0>(pt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC,
+                              Q, C, D, red, threadIdx.x, tok_tmp + start, lengths + row);
         __syncthreads();
     }
 }
@@ -979,7 +1023,7 @@ namespace {
 template <int NT, int TEAMS, int CAP>
 constexpr size_t lds_bytes()
 {
-    return 512 + 64 + (size_t)TEAMS * (4 * (NT / 64) + 4) * 4 + (size_t)TEAMS * CAP * 13 + (size_t)TEAMS * NT + 64;
+    return 512 + 64 + (size_t)TEAMS * (4 * (NT / 64) + 4) * 4 + (size_t)TEAMS * CAP * 15 + (size_t)TEAMS * NT + 64;
 }
 
 // Teams of the LDS kernel that are resident at once (the same for both of its forms).
