@@ -179,6 +179,9 @@ __device__ __forceinline__ void bpe_row(
 {
     constexpr IT NIL = (IT)~(IT)0;
     constexpr IT DEAD = (IT)kNone;
+    // pairs of table reads in flight per thread.  (Four cost 20 registers and a wave per SIMD; four
+    // for the first pairs only, or all bytes of a thread's positions requested before the first
+    // table read, gained nothing.)
     constexpr int kProbes = 2;
     const int wv = (NT == 64) ? 0 : (tid >> 6);
     uint32_t *qn = red + 4 * (NT / 64);        // number of merges queued in the current round
@@ -379,8 +382,9 @@ __device__ __forceinline__ void bpe_row(
                 for (int k = 0; k < PER; ++k) {
                     const int i = tid + k * NT;
                     const uint32_t r = i < n0 ? (uint32_t)P[i].r : kNone;
+                    const uint32_t g = MC[i < n0 ? i : tid];      // read beside the rank, not after it
                     myr[k] = r;
-                    if (r != kNone) { cmin = umin(cmin, r); cgate = umin(cgate, MC[i]); }
+                    if (r != kNone) { cmin = umin(cmin, r); cgate = umin(cgate, g); }
                 }
             } else {
                 for (int i = tid; i < n0; i += NT) {
@@ -451,7 +455,7 @@ __device__ __forceinline__ void bpe_row(
 // If an overlap holds no such p (e.g. a tandem repeat longer than the overlap), the row is
 // redone by the whole-row kernel.
 constexpr int kLdsCap = 4096;            // longest piece any LDS kernel variant takes
-// 2048-byte extended chunks: 26 KB of LDS state, six workgroups per CU; measured faster than
+// 2048-byte extended chunks: 31 KB of LDS state, five workgroups per CU; measured faster than
 // 4096-byte chunks (fewer positions per thread, more chunks in flight) and than 1408- or 1536-byte
 // ones (the overlap is work done twice: its share of a chunk decides).  Overlap: with 64 bytes 0.3 %
 // of the seams of the 32000-vocabulary benchmark rows (10 % tandem repeats of up to 180 bp) find no
