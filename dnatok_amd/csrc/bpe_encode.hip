@@ -264,35 +264,49 @@ __device__ __forceinline__ void bpe_row(
             if (tid == 0) { Q[0] = (IT)leftmost; *qn = 1; }
         } else {
             const int lane = tid & 63;
-            constexpr int kBlocks = PER > 0 ? (PER + 3) / 4 : 1 << 20;
-#pragma unroll
-            for (int blk = 0; blk < kBlocks; ++blk) {     // the same trip count for every lane
-                const int b0 = blk * 4 * NT;
-                if (b0 >= n0) break;
-                uint64_t bal[4];
+            if (PER > 0) {
+                // ranks from registers, one ballot per position of the thread, one queue atomic
+                // per wave and round
+                uint64_t bal[PER > 0 ? PER : 1];
                 uint32_t total = 0;
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    bool c;
-                    if (PER > 0) {
-                        c = blk * 4 + k < PER && myr[blk * 4 + k < PER ? blk * 4 + k : 0] < limit;
-                    } else {
-                        const int i = b0 + k * NT + tid;
-                        c = cmin < limit && i < n0 && (uint32_t)P[i].r < limit;
-                    }
-                    bal[k] = __ballot(c);
+                for (int k = 0; k < PER; ++k) {
+                    bal[k] = __ballot(myr[k] < limit);    // (kNone beyond the row's end: never below)
                     total += (uint32_t)__builtin_popcountll(bal[k]);
                 }
-                if (total == 0) continue;                 // (uniform over the wave)
-                uint32_t at = 0;
-                if (lane == 0) at = atomicAdd(cn, total);
-                at = (uint32_t)__builtin_amdgcn_readfirstlane((int)at);
+                if (total != 0) {                         // (uniform over the wave)
+                    uint32_t at = 0;
+                    if (lane == 0) at = atomicAdd(cn, total);
+                    at = (uint32_t)__builtin_amdgcn_readfirstlane((int)at);
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    if (bal[k] >> lane & 1ull)
-                        C[at + (uint32_t)__builtin_popcountll(bal[k] & ((1ull << lane) - 1ull))] =
-                            (IT)(b0 + k * NT + tid);
-                    at += (uint32_t)__builtin_popcountll(bal[k]);
+                    for (int k = 0; k < PER; ++k) {
+                        if (bal[k] >> lane & 1ull)
+                            C[at + (uint32_t)__builtin_popcountll(bal[k] & ((1ull << lane) - 1ull))] =
+                                (IT)(tid + k * NT);
+                        at += (uint32_t)__builtin_popcountll(bal[k]);
+                    }
+                }
+            } else {
+                for (int b0 = 0; b0 < n0; b0 += 4 * NT) {     // the same trip count for every lane
+                    uint64_t bal[4];
+                    uint32_t total = 0;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const int i = b0 + k * NT + tid;
+                        bal[k] = __ballot(cmin < limit && i < n0 && (uint32_t)P[i].r < limit);
+                        total += (uint32_t)__builtin_popcountll(bal[k]);
+                    }
+                    if (total == 0) continue;                 // (uniform over the wave)
+                    uint32_t at = 0;
+                    if (lane == 0) at = atomicAdd(cn, total);
+                    at = (uint32_t)__builtin_amdgcn_readfirstlane((int)at);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        if (bal[k] >> lane & 1ull)
+                            C[at + (uint32_t)__builtin_popcountll(bal[k] & ((1ull << lane) - 1ull))] =
+                                (IT)(b0 + k * NT + tid);
+                        at += (uint32_t)__builtin_popcountll(bal[k]);
+                    }
                 }
             }
             team_sync<NT>();
