@@ -175,7 +175,8 @@ __device__ __forceinline__ void bpe_row(
     const PairTable pt, const uint16_t *byte_to_sym,
     const int32_t *out_remap, const uint8_t *__restrict__ src, const int n0, PosRec<IT> *P,
     uint16_t *NS, uint16_t *MC, IT *Q, IT *C, uint8_t *D, uint32_t *red, const int tid,
-    int32_t *__restrict__ out, int32_t *__restrict__ out_len, uint16_t *__restrict__ raw_out = nullptr)
+    int32_t *__restrict__ out, int32_t *__restrict__ out_len, uint16_t *__restrict__ raw_out = nullptr,
+    const int mid_lo = 0, const int mid_hi = 0, int32_t *__restrict__ mid_out = nullptr)
 {
     constexpr IT NIL = (IT)~(IT)0;
     constexpr IT DEAD = (IT)kNone;
@@ -410,9 +411,19 @@ __device__ __forceinline__ void bpe_row(
     }
 
     if (raw_out) {
-        // chunk of a long row: hand back the symbol at every start position (kNone elsewhere);
-        // the seam and gather kernels assemble the row
-        for (int i = tid; i < n0; i += NT) raw_out[i] = stuck ? (uint16_t)kNone : (uint16_t)P[i].s;
+        // chunk of a long row: hand back the symbol at every start position (kNone elsewhere) and
+        // the number of tokens that start in [mid_lo, mid_hi), the stretch no neighbouring chunk
+        // shares; the seam and gather kernels assemble the row
+        uint32_t live = 0;
+        for (int i = tid; i < n0; i += NT) {
+            const uint16_t sy = stuck ? (uint16_t)kNone : (uint16_t)P[i].s;
+            raw_out[i] = sy;
+            live += (i >= mid_lo && i < mid_hi && sy != (uint16_t)kNone) ? 1u : 0u;
+        }
+        uint32_t total;
+        team_sync<NT>();                         // red may still be read by the last round's minimum
+        (void)team_exclusive_sum<NT>(live, red, wv, total);
+        if (tid == 0) *mid_out = (int32_t)total;
         return;
     }
     // Compact the live symbols to the output, in position order.  Position i = pass * NT + tid, so a
@@ -486,7 +497,8 @@ struct BpePlan {                          // device arrays inside the scratch bu
     int32_t *item_row;    // [max_items]
     int32_t *mc_row;      // [max_mc]
     int32_t *seam;        // [max_mc] seam to the right of a chunk (row position), -1 = none found
-    int32_t *cnt;         // [max_mc] tokens of a chunk between the seams on its two sides
+    int32_t *cnt;         // [max_mc][4] tokens of a chunk: in the stretch it shares with no other chunk, from the
+                          // seam on its left to that stretch, from that stretch to the seam on its right
     int32_t *row_fail;    // [n_rows] 1 = redo the row with the whole-row kernel
     uint16_t *chunk_sym;  // [max_mc][ext]
     uint8_t *slabs;       // whole-row fallback state
@@ -532,7 +544,7 @@ static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t
     const size_t o_item_row = take(4 * (size_t)p.max_items);
     const size_t o_mc_row = take(4 * (size_t)p.max_mc);
     const size_t o_seam = take(4 * (size_t)p.max_mc);
-    const size_t o_cnt = take(4 * (size_t)p.max_mc);
+    const size_t o_cnt = take(16 * (size_t)p.max_mc);
     const size_t o_fail = take(4 * (size_t)n_rows);
     const size_t o_sym = take(2 * (size_t)p.ext * (size_t)p.max_mc);
     p.slab_bytes = chunks ? long_slab_bytes(max_len) : 0;
@@ -724,9 +736,15 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
             const int64_t e0 = (int64_t)k * p.core - p.overlap < 0 ? 0 : (int64_t)k * p.core - p.overlap;
             int64_t e1 = (int64_t)(k + 1) * p.core + p.overlap;
             if (e1 > len) e1 = len;
-            uint16_t *raw = p.chunk_sym + (size_t)(p.mc_off[row] + k) * p.ext;
+            const int32_t m = p.mc_off[row] + k;
+            uint16_t *raw = p.chunk_sym + (size_t)m * p.ext;
+            // what the chunk shares with no other: from the end of the left overlap to the start of the right one
+            int64_t mid_lo = k > 0 ? (int64_t)k * p.core + p.overlap : 0;
+            if (mid_lo > len) mid_lo = len;
+            const int64_t mid_hi = k + 1 < nc ? (int64_t)(k + 1) * p.core - p.overlap : len;
             bpe_row<NT, uint16_t, (CAP + NT - 1) / NT>(pt, b2s, a.out_remap, bytes + start + e0, (int)(e1 - e0),
-                                  P, NS, MC, Q, C, D, red, tid, nullptr, nullptr, raw);
+                                  P, NS, MC, Q, C, D, red, tid, nullptr, nullptr, raw,
+                                  (int)(mid_lo - e0), (int)(mid_hi - e0), p.cnt + 4 * (size_t)m);
         }
         team_sync<NT>();
     }
@@ -741,7 +759,7 @@ constexpr int kSeamStage = 1024;          // positions of the shared stretch hel
 
 __global__ __launch_bounds__(256) void bpe_seam_kernel(const int64_t *__restrict__ offsets, BpePlan p)
 {
-    __shared__ uint32_t best[4];
+    __shared__ uint32_t best[4], red[8];
     __shared__ uint16_t sa_s[kSeamStage], sb_s[kSeamStage];
     const int32_t n_mc = p.counts[1];
     for (int32_t m = blockIdx.x; m < n_mc; m += gridDim.x) {
@@ -775,8 +793,8 @@ __global__ __launch_bounds__(256) void bpe_seam_kernel(const int64_t *__restrict
         mine = wave_min_u32(mine);
         if ((threadIdx.x & 63) == 0) best[threadIdx.x >> 6] = mine;
         __syncthreads();
+        const uint32_t b = umin(umin(best[0], best[1]), umin(best[2], best[3]));
         if (threadIdx.x == 0) {
-            const uint32_t b = umin(umin(best[0], best[1]), umin(best[2], best[3]));
             if (b == 0xFFFFFFFFu) {
                 p.seam[m] = -1;
                 if (atomicExch(&p.row_fail[row], 1) == 0) atomicAdd(&p.counts[3], 1);
@@ -784,6 +802,20 @@ __global__ __launch_bounds__(256) void bpe_seam_kernel(const int64_t *__restrict
                 p.seam[m] = (int32_t)b;
             }
         }
+        // tokens of A in the shared stretch left of the seam, tokens of B right of it: with each
+        // chunk's own count of its unshared stretch these are the chunks' shares of the row
+        uint32_t tail = 0, head = 0;
+        if (b != 0xFFFFFFFFu) {
+            const int cut = (int)((int64_t)b - eb0);
+            for (int i = threadIdx.x; i < n; i += 256) {
+                if (i < cut) tail += a_at(i) != kNone;
+                else head += b_at(i) != kNone;
+            }
+        }
+        uint32_t tail_all, head_all;
+        (void)team_exclusive_sum<256>(tail, red, threadIdx.x >> 6, tail_all);
+        (void)team_exclusive_sum<256>(head, red + 4, threadIdx.x >> 6, head_all);
+        if (threadIdx.x == 0) { p.cnt[4 * (size_t)m + 2] = (int32_t)tail_all; p.cnt[4 * (size_t)(m + 1) + 1] = (int32_t)head_all; }
         __syncthreads();
     }
 }
@@ -807,23 +839,6 @@ __device__ __forceinline__ ChunkSpan chunk_span(const int64_t *offsets, const Bp
     return c;
 }
 
-// One workgroup per chunk of a multi-chunk row: how many tokens it contributes.
-__global__ __launch_bounds__(256) void bpe_count_kernel(const int64_t *__restrict__ offsets, BpePlan p)
-{
-    __shared__ uint32_t red[8];
-    const int32_t n_mc = p.counts[1];
-    for (int32_t m = blockIdx.x; m < n_mc; m += gridDim.x) {
-        const ChunkSpan c = chunk_span(offsets, p, m);
-        if (p.row_fail[c.row]) continue;                 // (the same for the whole workgroup)
-        const uint16_t *sym = p.chunk_sym + (size_t)m * p.ext;
-        uint32_t live = 0;
-        for (int64_t i = c.lo + threadIdx.x; i < c.hi; i += 256) live += sym[i - c.e0] != kNone;
-        uint32_t total;
-        (void)team_exclusive_sum<256>(live, red, threadIdx.x >> 6, total);
-        if (threadIdx.x == 0) p.cnt[m] = (int32_t)total;
-    }
-}
-
 // One workgroup per chunk: its tokens, compacted, behind those of the row's earlier chunks.
 // Positions are taken 256 at a time: a ballot per wave places every live symbol among its wave's,
 // the waves' counts go through LDS, all symbols (and their remapped ids) of a block of passes are
@@ -844,7 +859,10 @@ __global__ __launch_bounds__(256) void bpe_gather_kernel(
         if (p.row_fail[c.row]) continue;
         // tokens of the row's chunks before this one
         uint32_t before = 0;
-        for (int32_t j = threadIdx.x; j < c.k; j += 256) before += (uint32_t)p.cnt[m - c.k + j];
+        for (int32_t j = threadIdx.x; j < c.k; j += 256) {
+            const int32_t *part = p.cnt + 4 * (size_t)(m - c.k + j);       // {unshared, after left seam, before right seam}
+            before += (uint32_t)(part[0] + (j > 0 ? part[1] : 0) + part[2]);
+        }
         uint32_t base;
         (void)team_exclusive_sum<256>(before, red, wv, base);
         const uint16_t *sym = p.chunk_sym + (size_t)m * p.ext;
@@ -1134,8 +1152,6 @@ extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, co
         if (chunking) {
             int64_t g = p.max_mc < 4096 ? p.max_mc : 4096;
             bpe_seam_kernel<<<(int)(g < 1 ? 1 : g), 256, 0, s>>>(offsets, p);
-            DNATOK_HIP_TRY(hipGetLastError());
-            bpe_count_kernel<<<(int)(g < 1 ? 1 : g), 256, 0, s>>>(offsets, p);
             DNATOK_HIP_TRY(hipGetLastError());
             bpe_gather_kernel<<<(int)(g < 1 ? 1 : g), 256, 0, s>>>(a, offsets, p, tok_tmp, lengths);
             DNATOK_HIP_TRY(hipGetLastError());
