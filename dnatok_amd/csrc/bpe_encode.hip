@@ -194,6 +194,35 @@ __device__ __forceinline__ void bpe_row(
     uint32_t cmin = kEmptyKey, cgate = kEmptyKey;
     D[tid] = 0;
     if (tid == 0) { *qn = 0; *cn = 0; }
+    // With PER > 0 the row's bytes come into LDS first (the candidate queue is free until the first
+    // round), 8 aligned bytes per thread: one trip to memory for the whole row instead of one per
+    // batch of table reads.  Only a word that reaches over the row's first or last byte is put
+    // together from single bytes, so that nothing outside the row is read.
+    uint8_t *stage = reinterpret_cast<uint8_t *>(C);
+    int head = 0;
+    if (PER > 0) {
+        const uintptr_t a0 = reinterpret_cast<uintptr_t>(src) & ~(uintptr_t)7;
+        head = (int)(reinterpret_cast<uintptr_t>(src) - a0);
+        const int n_words = (head + n0 + 7) >> 3;
+        for (int wd = tid; wd < n_words; wd += NT) {
+            const int first = 8 * wd - head;                  // row position of the word's first byte
+            uint2 v;
+            if (first >= 0 && first + 8 <= n0) {
+                v = *reinterpret_cast<const uint2 *>(a0 + 8 * (uintptr_t)wd);
+            } else {
+                uint32_t lo = 0, hi = 0;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    if (first + q >= 0 && first + q < n0) lo |= (uint32_t)src[first + q] << (8 * q);
+                    if (first + 4 + q >= 0 && first + 4 + q < n0) hi |= (uint32_t)src[first + 4 + q] << (8 * q);
+                }
+                v = uint2{lo, hi};
+            }
+            *reinterpret_cast<uint2 *>(stage + 8 * wd) = v;
+        }
+        team_sync<NT>();
+    }
+    auto byte_at = [&](int i) -> uint32_t { return PER > 0 ? stage[head + i] : src[i]; };
     for (int i0 = tid; i0 < n0; i0 += kProbes * NT) {
         PairProbe e[kProbes];
         uint32_t sa[kProbes], sb[kProbes];
@@ -201,8 +230,8 @@ __device__ __forceinline__ void bpe_row(
         for (int j = 0; j < kProbes; ++j) {
             const int i = i0 + j * NT;
             const bool ok = i + 1 < n0;
-            sa[j] = i < n0 ? byte_to_sym[src[i]] : 0u;
-            sb[j] = ok ? byte_to_sym[src[i + 1]] : 0u;
+            sa[j] = i < n0 ? byte_to_sym[byte_at(i)] : 0u;
+            sb[j] = ok ? byte_to_sym[byte_at(i + 1)] : 0u;
             e[j] = pair_probe(pt, ok ? sa[j] : 0u, sb[j]);
         }
 #pragma unroll
