@@ -519,12 +519,17 @@ constexpr int kChunkCore = 2048 - 2 * kChunkOverlap;
 constexpr int kLongThreads = 1024;
 constexpr int kLongGrid = 64;            // slabs of scratch for the whole-row fallback kernel
 
+// The work list: the chunks of all chunked rows first (the largest items), then the rows that are
+// one item each, in classes of falling length.  Items are handed out in that order, so the last
+// ones to start are short: with rows in their given order a 2 KB item that starts last leaves most
+// teams idle for its whole duration (ragged benchmark batch: 0.299 -> 0.289 ms).
+constexpr int kSingleClasses = 3;
+
 struct BpePlan {                          // device arrays inside the scratch buffer
-    int32_t *counts;      // [0] items, [1] chunk items of multi-chunk rows, [2] work counter, [3] failed rows
-    int32_t *item_off;    // [n_rows + 1] first item of a row
+    int32_t *counts;      // [0] items, [1] chunk items, [2] work counter, [3] failed rows, [4 + c] single rows of class c
     int32_t *mc_off;      // [n_rows + 1] first chunk slot of a row (multi-chunk rows only)
-    int32_t *item_row;    // [max_items]
-    int32_t *mc_row;      // [max_mc]
+    int4 *rec;           // [max_mc] a chunk item: {row, chunk of the row, chunks of the row, row length}
+    int32_t *single[kSingleClasses];   // [n_rows] each: the rows that are one item, longest class first
     int32_t *seam;        // [max_mc] seam to the right of a chunk (row position), -1 = none found
     int32_t *cnt;         // [max_mc][4] tokens of a chunk: in the stretch it shares with no other chunk, from the
                           // seam on its left to that stretch, from that stretch to the seam on its right
@@ -568,10 +573,10 @@ static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t
     size_t o = 0;
     auto take = [&](size_t bytes) { size_t at = o; o = up(o + bytes); return at; };
     const size_t o_counts = take(64);
-    const size_t o_item_off = take(4 * (size_t)(n_rows + 1));
     const size_t o_mc_off = take(4 * (size_t)(n_rows + 1));
-    const size_t o_item_row = take(4 * (size_t)p.max_items);
-    const size_t o_mc_row = take(4 * (size_t)p.max_mc);
+    const size_t o_rec = take(16 * (size_t)p.max_mc);
+    size_t o_single[kSingleClasses];
+    for (int c = 0; c < kSingleClasses; ++c) o_single[c] = take(4 * (size_t)n_rows);
     const size_t o_seam = take(4 * (size_t)p.max_mc);
     const size_t o_cnt = take(16 * (size_t)p.max_mc);
     const size_t o_fail = take(4 * (size_t)n_rows);
@@ -582,10 +587,9 @@ static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t
     p.total_bytes = o + 256;
     if (base) {
         p.counts = (int32_t *)(base + o_counts);
-        p.item_off = (int32_t *)(base + o_item_off);
         p.mc_off = (int32_t *)(base + o_mc_off);
-        p.item_row = (int32_t *)(base + o_item_row);
-        p.mc_row = (int32_t *)(base + o_mc_row);
+        p.rec = (int4 *)(base + o_rec);
+        for (int c = 0; c < kSingleClasses; ++c) p.single[c] = (int32_t *)(base + o_single[c]);
         p.seam = (int32_t *)(base + o_seam);
         p.cnt = (int32_t *)(base + o_cnt);
         p.row_fail = (int32_t *)(base + o_fail);
@@ -595,18 +599,20 @@ static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t
     return p;
 }
 
-// Work list: one item per short row, ceil(len / core) items per long row.  Single workgroup; a
-// thread takes four consecutive rows per step, so that 4096 rows are one round of loads and one
-// scan (the kernel is a chain of load latencies and barriers, not work).
+// Work list: ceil(len / core) chunk slots per long row, one entry in its length class per other
+// row.  Single workgroup; a thread takes four consecutive rows per step, so that 4096 rows are one
+// round of loads and one scan (the kernel is a chain of load latencies and barriers, not work).
 constexpr int kPlanRows = 4;
+constexpr int kPlanScans = 1 + kSingleClasses;
 
 __global__ __launch_bounds__(1024) void bpe_plan_kernel(
     const int64_t *__restrict__ offsets, int64_t n_rows, int chunking, BpePlan p)
 {
-    __shared__ uint32_t wt[2][16];
-    __shared__ int32_t carry[2];
+    __shared__ uint32_t wt[kPlanScans][16];
+    __shared__ int32_t carry[kPlanScans];
     __shared__ int32_t fail_s;
-    if (threadIdx.x == 0) { carry[0] = 0; carry[1] = 0; fail_s = 0; }
+    if (threadIdx.x < kPlanScans) carry[threadIdx.x] = 0;
+    if (threadIdx.x == 0) fail_s = 0;
     __syncthreads();
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     int32_t n_fail = 0;
@@ -615,86 +621,105 @@ __global__ __launch_bounds__(1024) void bpe_plan_kernel(
         int64_t off[kPlanRows + 1];
 #pragma unroll
         for (int r = 0; r <= kPlanRows; ++r) off[r] = row0 + r <= n_rows ? offsets[row0 + r] : 0;
-        uint32_t nc[kPlanRows], mc[kPlanRows], nc_sum = 0, mc_sum = 0;
+        // what a row adds to each scan: [0] chunk slots, [1 + c] one if it is a single row of class c
+        uint32_t add[kPlanRows][kPlanScans], sum[kPlanScans];
+#pragma unroll
+        for (int q = 0; q < kPlanScans; ++q) sum[q] = 0;
 #pragma unroll
         for (int r = 0; r < kPlanRows; ++r) {
-            nc[r] = 0; mc[r] = 0;
+#pragma unroll
+            for (int q = 0; q < kPlanScans; ++q) add[r][q] = 0;
             if (row0 + r < n_rows) {
                 const int64_t len = off[r + 1] - off[r];
-                nc[r] = 1;
-                if (len > p.ext && chunking) { nc[r] = (uint32_t)((len + p.core - 1) / p.core); mc[r] = nc[r]; }
+                if (len > p.ext && chunking) {
+                    add[r][0] = (uint32_t)((len + p.core - 1) / p.core);
+                } else {
+                    const int c = len > p.ext / 2 ? 0 : (len > p.ext / 4 ? 1 : 2);
+#pragma unroll
+                    for (int q = 0; q < kSingleClasses; ++q) add[r][1 + q] = q == c ? 1u : 0u;
+                }
                 const int fail = (len > p.ext && !chunking) ? 1 : 0;
                 p.row_fail[row0 + r] = fail;
                 n_fail += fail;
             }
-            nc_sum += nc[r]; mc_sum += mc[r];
-        }
-        const uint32_t inc0 = wave_inclusive_sum_u32(nc_sum), inc1 = wave_inclusive_sum_u32(mc_sum);
-        if (lane == 63) { wt[0][wv] = inc0; wt[1][wv] = inc1; }
-        __syncthreads();
-        uint32_t b0 = 0, b1 = 0, t0 = 0, t1 = 0;
 #pragma unroll
-        for (int w = 0; w < 16; ++w) {
-            if (w < wv) { b0 += wt[0][w]; b1 += wt[1][w]; }
-            t0 += wt[0][w]; t1 += wt[1][w];
+            for (int q = 0; q < kPlanScans; ++q) sum[q] += add[r][q];
         }
-        const int32_t c0 = carry[0], c1 = carry[1];
-        int32_t io = c0 + (int32_t)(b0 + inc0 - nc_sum), mo = c1 + (int32_t)(b1 + inc1 - mc_sum);
+        uint32_t inc[kPlanScans];
+#pragma unroll
+        for (int q = 0; q < kPlanScans; ++q) {
+            inc[q] = wave_inclusive_sum_u32(sum[q]);
+            if (lane == 63) wt[q][wv] = inc[q];
+        }
+        __syncthreads();
+        int32_t at[kPlanScans], tot[kPlanScans];
+#pragma unroll
+        for (int q = 0; q < kPlanScans; ++q) {
+            uint32_t b = 0, t = 0;
+#pragma unroll
+            for (int w = 0; w < 16; ++w) {
+                if (w < wv) b += wt[q][w];
+                t += wt[q][w];
+            }
+            at[q] = carry[q] + (int32_t)(b + inc[q] - sum[q]);
+            tot[q] = carry[q] + (int32_t)t;
+        }
 #pragma unroll
         for (int r = 0; r < kPlanRows; ++r) {
-            const bool valid = row0 + r < n_rows;
+            if (row0 + r >= n_rows) continue;
             const int32_t row = (int32_t)(row0 + r);
-            if (valid) {
-                p.item_off[row] = io;
-                p.mc_off[row] = mo;
-            }
-            // the entries of the work list: a row that is one item here, the chunks of a chunked
-            // row in bpe_expand_kernel (a single workgroup writing tens of thousands of scattered
-            // words is bound by its one CU's store path)
-            if (valid && nc[r] == 1) p.item_row[io] = row;
-            if (valid) {
-                io += (int32_t)nc[r];
-                mo += (int32_t)mc[r];
-            }
+            p.mc_off[row] = at[0];
+            // the entries of the chunks are written by bpe_expand_kernel (a single workgroup
+            // writing tens of thousands of scattered words is bound by its one CU's store path)
+#pragma unroll
+            for (int q = 0; q < kSingleClasses; ++q)
+                if (add[r][1 + q]) p.single[q][at[1 + q]] = row;
+#pragma unroll
+            for (int q = 0; q < kPlanScans; ++q) at[q] += (int32_t)add[r][q];
         }
         __syncthreads();
-        if (threadIdx.x == 0) { carry[0] = c0 + (int32_t)t0; carry[1] = c1 + (int32_t)t1; }
+        if (threadIdx.x < kPlanScans) {
+#pragma unroll
+            for (int q = 0; q < kPlanScans; ++q) if ((int)threadIdx.x == q) carry[q] = tot[q];
+        }
         __syncthreads();
     }
     if (n_fail) atomicAdd(&fail_s, n_fail);
     __syncthreads();
     if (threadIdx.x == 0) {
-        p.item_off[n_rows] = carry[0];
-        p.mc_off[n_rows] = carry[1];
-        p.counts[0] = carry[0];
-        p.counts[1] = carry[1];
+        int32_t items = carry[0];
+        for (int q = 0; q < kSingleClasses; ++q) { p.counts[4 + q] = carry[1 + q]; items += carry[1 + q]; }
+        p.mc_off[n_rows] = carry[0];
+        p.counts[0] = items;
+        p.counts[1] = carry[0];
         p.counts[2] = 0;
         p.counts[3] = fail_s;                         // rows left to the whole-row kernel (the seam kernel may add some)
     }
 }
 
-// item_row / mc_row of the chunked rows: one thread per row, a row of many chunks by its wave.
-__global__ __launch_bounds__(256) void bpe_expand_kernel(int64_t n_rows, BpePlan p)
+// The entries of the chunks of the chunked rows: one thread per row, a row of many chunks by its wave.
+__global__ __launch_bounds__(256) void bpe_expand_kernel(const int64_t *__restrict__ offsets, int64_t n_rows,
+                                                         BpePlan p)
 {
     const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int lane = threadIdx.x & 63;
-    int32_t io = 0, mo = 0, nc = 0;
+    int32_t mo = 0, nc = 0, len = 0;
     if (row < n_rows) {
-        io = p.item_off[row];
         mo = p.mc_off[row];
         nc = p.mc_off[row + 1] - mo;                 // 0 for a row that is a single item
+        len = (int32_t)(offsets[row + 1] - offsets[row]);
     }
     const bool big = nc > 8;
     if (!big)
-        for (int32_t k = 0; k < nc; ++k) { p.item_row[io + k] = (int32_t)row; p.mc_row[mo + k] = (int32_t)row; }
+        for (int32_t k = 0; k < nc; ++k) p.rec[mo + k] = make_int4((int32_t)row, k, nc, len);
     uint64_t todo = __ballot(big);
     while (todo) {
         const int src = __builtin_amdgcn_readfirstlane(__builtin_ctzll(todo));
         todo &= todo - 1;
         const int32_t b_row = __builtin_amdgcn_readlane((int32_t)row, src);
-        const int32_t b_io = __builtin_amdgcn_readlane(io, src), b_mo = __builtin_amdgcn_readlane(mo, src);
-        const int32_t b_nc = __builtin_amdgcn_readlane(nc, src);
-        for (int32_t k = lane; k < b_nc; k += 64) { p.item_row[b_io + k] = b_row; p.mc_row[b_mo + k] = b_row; }
+        const int32_t b_mo = __builtin_amdgcn_readlane(mo, src), b_nc = __builtin_amdgcn_readlane(nc, src);
+        const int32_t b_len = __builtin_amdgcn_readlane(len, src);
+        for (int32_t k = lane; k < b_nc; k += 64) p.rec[b_mo + k] = make_int4(b_row, k, b_nc, b_len);
     }
 }
 
@@ -726,6 +751,8 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     __syncthreads();
 
     const int32_t n_items = PLANNED ? p.counts[0] : n_rows;
+    const int32_t n_mc = PLANNED ? p.counts[1] : 0;
+    const int32_t n_single0 = PLANNED ? p.counts[4] : 0, n_single1 = PLANNED ? p.counts[5] : 0;
     // A team's first item is its own number; only the items beyond one per team are handed out
     // through the counter.  (Every team asking the counter at the start of the kernel is a
     // thousand atomics on one address, about 12 ns each, before the last team has its row.)
@@ -746,9 +773,18 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
         if (item >= n_items) break;
         int32_t row = item, k = 0, nc = 1;
         if (PLANNED) {
-            row = p.item_row[item];
-            k = item - p.item_off[row];
-            nc = p.item_off[row + 1] - p.item_off[row];
+            if (item < n_mc) {
+                const int4 rc = p.rec[item];
+                row = rc.x; k = rc.y; nc = rc.z;
+            } else {
+                int32_t j = item - n_mc;
+                const int32_t *list = p.single[0];
+                if (j >= n_single0) {
+                    j -= n_single0; list = p.single[1];
+                    if (j >= n_single1) { j -= n_single1; list = p.single[2]; }
+                }
+                row = list[j];
+            }
         }
         const int64_t start = offsets[row];
         const int64_t len = offsets[row + 1] - start;
@@ -765,7 +801,7 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
             const int64_t e0 = (int64_t)k * p.core - p.overlap < 0 ? 0 : (int64_t)k * p.core - p.overlap;
             int64_t e1 = (int64_t)(k + 1) * p.core + p.overlap;
             if (e1 > len) e1 = len;
-            const int32_t m = p.mc_off[row] + k;
+            const int32_t m = item;                  // chunk items come first in the list
             uint16_t *raw = p.chunk_sym + (size_t)m * p.ext;
             // what the chunk shares with no other: from the end of the left overlap to the start of the right one
             int64_t mid_lo = k > 0 ? (int64_t)k * p.core + p.overlap : 0;
@@ -792,11 +828,10 @@ __global__ __launch_bounds__(256) void bpe_seam_kernel(const int64_t *__restrict
     __shared__ uint16_t sa_s[kSeamStage], sb_s[kSeamStage];
     const int32_t n_mc = p.counts[1];
     for (int32_t m = blockIdx.x; m < n_mc; m += gridDim.x) {
-        const int32_t row = p.mc_row[m];
-        const int32_t k = m - p.mc_off[row];
-        const int32_t nc = p.mc_off[row + 1] - p.mc_off[row];
+        const int4 rc = p.rec[m];
+        const int32_t row = rc.x, k = rc.y, nc = rc.z;
         if (k + 1 >= nc) continue;                                   // last chunk: no seam to the right
-        const int64_t len = offsets[row + 1] - offsets[row];
+        const int64_t len = rc.w;
         const int64_t ea0 = (int64_t)k * p.core - p.overlap < 0 ? 0 : (int64_t)k * p.core - p.overlap;
         int64_t ea1 = (int64_t)(k + 1) * p.core + p.overlap;
         if (ea1 > len) ea1 = len;
@@ -858,10 +893,9 @@ struct ChunkSpan {
 __device__ __forceinline__ ChunkSpan chunk_span(const int64_t *offsets, const BpePlan &p, int32_t m)
 {
     ChunkSpan c;
-    c.row = p.mc_row[m];
-    c.k = m - p.mc_off[c.row];
-    c.nc = p.mc_off[c.row + 1] - p.mc_off[c.row];
-    const int64_t len = offsets[c.row + 1] - offsets[c.row];
+    const int4 rc = p.rec[m];
+    c.row = rc.x; c.k = rc.y; c.nc = rc.z;
+    const int64_t len = rc.w;
     c.e0 = (int64_t)c.k * p.core - p.overlap < 0 ? 0 : (int64_t)c.k * p.core - p.overlap;
     c.lo = c.k > 0 ? p.seam[m - 1] : 0;
     c.hi = c.k + 1 < c.nc ? p.seam[m] : len;
@@ -1136,7 +1170,7 @@ int run_lds(bool long_rows, int chunking, const BpeArgs &a, const uint8_t *bytes
         bpe_plan_kernel<<<1, 1024, 0, s>>>(offsets, n_rows, chunking, p);
         DNATOK_HIP_TRY(hipGetLastError());
         if (chunking) {
-            bpe_expand_kernel<<<(int)((n_rows + 255) / 256), 256, 0, s>>>(n_rows, p);
+            bpe_expand_kernel<<<(int)((n_rows + 255) / 256), 256, 0, s>>>(offsets, n_rows, p);
             DNATOK_HIP_TRY(hipGetLastError());
         }
         return launch_lds_as<NT, TEAMS, CAP, true>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
