@@ -341,26 +341,39 @@ __device__ __forceinline__ void bpe_row(
             }
             team_sync<NT>();
             const int ncand = (int)*cn;
-            for (int c = tid; c < ncand; c += NT) {
-                const int i = (int)C[c];
-                const PosRec<IT> x = P[i];
-                const uint32_t r = x.r;
-                // both neighbours' records are requested together
-                PosRec<IT> yl = P[x.pv != NIL ? x.pv : (IT)i];
-                PosRec<IT> yr = P[x.nx != NIL ? x.nx : (IT)i];
-                uint32_t chain = 0, rp = r;
-                IT q = x.pv;
-                while (q != NIL && yl.r <= rp) {          // candidates to the left with key <= ours
-                    ++chain; rp = yl.r; q = yl.pv;
-                    if (q != NIL) yl = P[q];
+            for (int c0 = 0; c0 < ncand; c0 += NT) {      // the same trip count for every lane
+                const int c = c0 + tid;
+                bool merges = false;
+                int i = 0;
+                if (c < ncand) {
+                    i = (int)C[c];
+                    const PosRec<IT> x = P[i];
+                    const uint32_t r = x.r;
+                    // both neighbours' records are requested together
+                    PosRec<IT> yl = P[x.pv != NIL ? x.pv : (IT)i];
+                    PosRec<IT> yr = P[x.nx != NIL ? x.nx : (IT)i];
+                    uint32_t chain = 0, rp = r;
+                    IT q = x.pv;
+                    while (q != NIL && yl.r <= rp) {      // candidates to the left with key <= ours
+                        ++chain; rp = yl.r; q = yl.pv;
+                        if (q != NIL) yl = P[q];
+                    }
+                    uint32_t chain_r = 0;
+                    rp = r; q = x.nx;
+                    while (q != NIL && yr.r < rp) {       // candidates to the right with key < ours
+                        ++chain_r; rp = yr.r; q = yr.nx;
+                        if (q != NIL) yr = P[q];
+                    }
+                    merges = ((chain | chain_r) & 1u) == 0;
                 }
-                uint32_t chain_r = 0;
-                rp = r; q = x.nx;
-                while (q != NIL && yr.r < rp) {           // candidates to the right with key < ours
-                    ++chain_r; rp = yr.r; q = yr.nx;
-                    if (q != NIL) yr = P[q];
+                // one queue atomic per wave (64 atomics on one LDS word take their turns)
+                const uint64_t bal = __ballot(merges);
+                if (bal != 0) {                           // (uniform over the wave)
+                    uint32_t at = 0;
+                    if (lane == 0) at = atomicAdd(qn, (uint32_t)__builtin_popcountll(bal));
+                    at = (uint32_t)__builtin_amdgcn_readfirstlane((int)at);
+                    if (merges) Q[at + (uint32_t)__builtin_popcountll(bal & ((1ull << lane) - 1ull))] = (IT)i;
                 }
-                if (((chain | chain_r) & 1u) == 0) Q[atomicAdd(qn, 1u)] = (IT)i;
             }
         }
         team_sync<NT>();
