@@ -491,6 +491,29 @@ def test_bpe_repeated_pair_keeps_its_first_rank():
         np.testing.assert_array_equal(r1, r2)
 
 
+def test_bpe_table_near_the_size_limit():
+    """60,000 rules (the 16-bit state allows 65,534): the hashed rule table at its largest."""
+    say("bpe table with 60,000 rules")
+    rng = random.Random(23)
+    short, merges, seen = list("ACGT"), [], set()          # tokens of at most 7 letters
+    while len(merges) < 60000:
+        a, b2 = rng.choice(short), rng.choice(short)
+        if (a, b2) in seen:
+            continue
+        seen.add((a, b2))
+        merges.append((a, b2))
+        if len(a + b2) <= 7:
+            short.append(a + b2)
+    kv = bpe_vocab.KernelVocab(merges)
+    assert len(kv) <= 65535
+    enc = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv))
+    bo = O.BpeOracle(merges)
+    seqs = ["".join(rng.choice("ACGT") for _ in range(rng.randint(1, 1500))) for _ in range(96)]
+    b = util.batch_from_strings(seqs)
+    for s, r, e in zip(seqs, bpe_rows(enc, b), bo.encode_batch(b.data, b.offsets, remap=False)):
+        np.testing.assert_array_equal(r, e, err_msg=s[:40])
+
+
 # ---------------------------------------------------------------- packer
 
 def test_c5_ragged_bpe_and_char_packed(char_enc):
