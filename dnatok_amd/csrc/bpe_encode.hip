@@ -839,9 +839,12 @@ __global__ __launch_bounds__(256) void bpe_seam_kernel(const int64_t *__restrict
 {
     __shared__ uint32_t best[4], red[8];
     __shared__ uint16_t sa_s[kSeamStage], sb_s[kSeamStage];
+    // (the first record is requested beside the count, not behind it; the slot exists either way)
+    int4 rc_first = make_int4(0, 0, 0, 0);
+    if ((int64_t)blockIdx.x < p.max_mc) rc_first = p.rec[blockIdx.x];
     const int32_t n_mc = p.counts[1];
     for (int32_t m = blockIdx.x; m < n_mc; m += gridDim.x) {
-        const int4 rc = p.rec[m];
+        const int4 rc = m == (int32_t)blockIdx.x ? rc_first : p.rec[m];
         const int32_t row = rc.x, k = rc.y, nc = rc.z;
         if (k + 1 >= nc) continue;                                   // last chunk: no seam to the right
         const int64_t len = rc.w;
@@ -889,10 +892,12 @@ __global__ __launch_bounds__(256) void bpe_seam_kernel(const int64_t *__restrict
                 else head += b_at(i) != kNone;
             }
         }
-        uint32_t tail_all, head_all;
-        (void)team_exclusive_sum<256>(tail, red, threadIdx.x >> 6, tail_all);
-        (void)team_exclusive_sum<256>(head, red + 4, threadIdx.x >> 6, head_all);
-        if (threadIdx.x == 0) { p.cnt[4 * (size_t)m + 2] = (int32_t)tail_all; p.cnt[4 * (size_t)(m + 1) + 1] = (int32_t)head_all; }
+        uint32_t both;                                   // (each count is below 2^16: one sum for the two)
+        (void)team_exclusive_sum<256>(tail | (head << 16), red, threadIdx.x >> 6, both);
+        if (threadIdx.x == 0) {
+            p.cnt[4 * (size_t)m + 2] = (int32_t)(both & 0xFFFFu);
+            p.cnt[4 * (size_t)(m + 1) + 1] = (int32_t)(both >> 16);
+        }
         __syncthreads();
     }
 }
@@ -903,7 +908,7 @@ struct ChunkSpan {
     int64_t lo, hi, e0;       // owned row positions [lo, hi); e0 = row position of the chunk's first symbol
 };
 
-__device__ __forceinline__ ChunkSpan chunk_span(const int64_t *offsets, const BpePlan &p, int32_t m)
+__device__ __forceinline__ ChunkSpan chunk_span(const BpePlan &p, int32_t m)
 {
     ChunkSpan c;
     const int4 rc = p.rec[m];
@@ -931,9 +936,11 @@ __global__ __launch_bounds__(256) void bpe_gather_kernel(
     const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int32_t n_mc = p.counts[1];
     for (int32_t m = blockIdx.x; m < n_mc; m += gridDim.x) {
-        const ChunkSpan c = chunk_span(offsets, p, m);
+        const ChunkSpan c = chunk_span(p, m);
         if (p.row_fail[c.row]) continue;
-        // tokens of the row's chunks before this one
+        // tokens of the row's chunks before this one.  (Summing them behind the first block's
+        // loads instead of in front of them made the kernel 10 % slower; requesting the chunk's
+        // record beside the chunk count, and both seams beside the record, 5 %.)
         uint32_t before = 0;
         for (int32_t j = threadIdx.x; j < c.k; j += 256) {
             const int32_t *part = p.cnt + 4 * (size_t)(m - c.k + j);       // {unshared, after left seam, before right seam}
