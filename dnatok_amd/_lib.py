@@ -18,7 +18,7 @@ EXPORTS = [
     "dnatok_char_table_create", "dnatok_char_table_destroy",
     "dnatok_char_encode_padded", "dnatok_char_encode_padded_as", "dnatok_char_encode_packed",
     "dnatok_char_embed_packed",
-    "dnatok_char_unpack_2bit", "dnatok_host_clean_ascii", "dnatok_host_pack_2bit",
+    "dnatok_char_unpack_2bit", "dnatok_host_clean_ascii", "dnatok_host_pack_2bit", "dnatok_host_fasta_scan",
     "dnatok_kmer_table_create", "dnatok_kmer_table_destroy", "dnatok_kmer_encode_padded",
     "dnatok_bpe_table_create", "dnatok_bpe_table_destroy", "dnatok_bpe_scratch_bytes",
     "dnatok_bpe_encode", "dnatok_pack_ragged", "dnatok_pad_rows",
@@ -82,6 +82,8 @@ def lib() -> ctypes.CDLL:
     L.dnatok_char_unpack_2bit.argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int32, c_void_p]
     L.dnatok_host_clean_ascii.argtypes = [c_void_p, c_int64, c_int, c_int, POINTER(c_int64)]
     L.dnatok_host_pack_2bit.argtypes = [c_void_p, c_int64, c_int64, c_void_p]
+    L.dnatok_host_fasta_scan.argtypes = [c_void_p, c_int64, c_int, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
+                                         POINTER(c_int64), POINTER(c_int64)]
     L.dnatok_kmer_table_create.argtypes = [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                            c_int64, c_void_p, c_int32, c_int32, POINTER(c_void_p)]
     L.dnatok_kmer_table_destroy.argtypes = [c_void_p]

@@ -374,6 +374,43 @@ class DNATok:
             width = int(self.token_len)
         return self._char_enc.encode_padded(data, offsets, width, pad_left=(self.padding_side == "left"))
 
+    def encode_fasta_device(self, source, device="cuda"):
+        """FASTA file (path) or FASTA text (bytes) -> (ids int32 [B, T], mask uint8 [B, T], names),
+        one row per record, on the GPU.  The text is scanned once on the host
+        (``encoders.fasta_to_bytes``: no Python string per record), the sequences cross the bus as
+        bytes, and the same kernels run as for ``encode_batch_device``.  Not in the reference,
+        whose callers read their files into Python strings first (src/dna_tokenizer.py:2594-2651)."""
+        self._require_ready()
+        host, off_h, names = encoders.fasta_to_bytes(source, upper_case=bool(self.normalize_case))
+        if not names:
+            raise ValueError("No sequences provided for encoding.")
+        lens = (off_h[1:] - off_h[:-1]).numpy()
+        data, offsets = host.to(device, non_blocking=True), off_h.to(device)
+
+        class _Rows:                                     # strings of single rows, made only when asked for
+            def __getitem__(self, i):
+                return bytes(host[int(off_h[i]):int(off_h[i + 1])].numpy()).decode("ascii", errors="replace")
+
+            def __len__(self):
+                return len(names)
+
+        rows = _Rows()
+        if self.bpe_backend is not None:
+            if getattr(self.bpe_backend, "_normalize", None) is not None:
+                ids, mask = self.bpe_backend.encode_batch([rows[i] for i in range(len(names))], device=device)
+                return ids.to(torch.int32), mask, names
+            ids, mask, _, longest = self.bpe_backend.encode_device(data, offsets, int(lens.max()))
+            width = max(int(longest.item()), 1)
+            return ids[:, :width], mask[:, :width], names
+        if self._kmer_enc is not None:
+            ids, mask = self._encode_kmer_device(rows, data, offsets, lens)
+            return ids, mask, names
+        width = int(lens.max())
+        if self.token_len is not None and self.token_len > width:
+            width = int(self.token_len)
+        ids, mask = self._char_enc.encode_padded(data, offsets, width, pad_left=(self.padding_side == "left"))
+        return ids, mask, names
+
     def _encode_kmer_device(self, seqs, data, offsets, lens) -> Tuple[torch.Tensor, torch.Tensor]:
         from ._lib import lib  # noqa: F401  (fail early if the library is missing)
         k = int(self.kmer_k)

@@ -90,6 +90,41 @@ def pack_2bit_host(ascii_rows: torch.Tensor, out: Optional[torch.Tensor] = None)
     return out
 
 
+def fasta_to_bytes(source, device=None, *, upper_case: bool = False):
+    """FASTA text -> (data uint8 [total], offsets int64 [n + 1], names) in the layout the encoders take.
+
+    ``source``: a path, or the text itself as bytes / bytearray / memoryview / a host uint8 array.
+    A path is memory-mapped, so the file is read once, by the scan.  The sequences land in pinned
+    host memory when a GPU is present and are copied to ``device`` (default: stay on the host).
+    ``names`` is a list of the header lines (without '>'); bases in front of the first header
+    form a record named "" (C ABI: dnatok_host_fasta_scan)."""
+    if isinstance(source, (str, bytes, bytearray, memoryview, np.ndarray)) and not isinstance(source, str):
+        text = np.frombuffer(source, dtype=np.uint8) if not isinstance(source, np.ndarray) else source
+    else:
+        import os
+        text = np.memmap(os.fspath(source), dtype=np.uint8, mode="r") if os.path.getsize(os.fspath(source)) else \
+            np.empty(0, dtype=np.uint8)
+    text = np.ascontiguousarray(text, dtype=np.uint8)
+    n_rec, n_bases = ctypes.c_int64(0), ctypes.c_int64(0)
+    L = _lib.lib()
+    ptr = ctypes.c_void_p(text.ctypes.data) if text.size else None
+    _lib.check(L.dnatok_host_fasta_scan(ptr, text.size, int(upper_case), None, 0, None, None, 0,
+                                        ctypes.byref(n_rec), ctypes.byref(n_bases)), "dnatok_host_fasta_scan")
+    n, total = int(n_rec.value), int(n_bases.value)
+    room = torch.empty(max(total, 1), dtype=torch.uint8, pin_memory=torch.cuda.is_available())
+    offsets = np.zeros(n + 1, dtype=np.int64)
+    spans = np.zeros((max(n, 1), 2), dtype=np.int64)
+    _lib.check(L.dnatok_host_fasta_scan(ptr, text.size, int(upper_case), ctypes.c_void_p(room.data_ptr()), total,
+                                        ctypes.c_void_p(offsets.ctypes.data), ctypes.c_void_p(spans.ctypes.data), n,
+                                        ctypes.byref(n_rec), ctypes.byref(n_bases)), "dnatok_host_fasta_scan")
+    host = room[:total]
+    names = [bytes(text[lo:hi]).decode("utf-8", errors="replace") for lo, hi in spans[:n]]
+    off_t = torch.from_numpy(offsets)
+    if device is not None:
+        host, off_t = host.to(device, non_blocking=True), off_t.to(device)
+    return host, off_t, names
+
+
 class RowNormalizer:
     """A tokenizer normalizer as a device program over ragged rows of bytes
     (C ABI: dnatok_normalize_rows).  ``steps`` are ``_lib.NormStep`` records."""

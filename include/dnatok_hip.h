@@ -108,6 +108,19 @@ int dnatok_host_clean_ascii(uint8_t *bytes_h, int64_t n, int upper_case, int inv
  * DNATok.encode_batch_to_packed_2bit (src/dna_tokenizer.py:3143-3210). */
 int dnatok_host_pack_2bit(const uint8_t *ascii_h, int64_t n_rows, int64_t row_len, uint8_t *packed_h);
 
+/* FASTA text (n bytes in host memory, e.g. a memory-mapped file) -> the sequences of all records laid
+ * end to end in seq_out, offsets_out[n_records + 1] (the layout every encoder here takes) and, when
+ * name_spans_out is not NULL, the byte span [lo, hi) of each record's header line in the text (without
+ * the '>').  Line ends, blanks and tabs inside sequence lines are dropped, lines that start with ';'
+ * are skipped, bases in front of the first header form a record of their own (name span 0, 0),
+ * a-z -> A-Z when upper_case.  Called with seq_out = NULL it only counts: *n_records and *n_bases are
+ * the sizes the second call needs (seq_capacity bases, max_records records).  The reference has no
+ * reader of its own: its callers bring Python strings (src/dna_tokenizer.py:2594-2651, one
+ * str.encode per row); this is the same hand-over for callers that start from a file. */
+int dnatok_host_fasta_scan(const uint8_t *text_h, int64_t n, int upper_case, uint8_t *seq_out,
+                           int64_t seq_capacity, int64_t *offsets_out, int64_t *name_spans_out,
+                           int64_t max_records, int64_t *n_records, int64_t *n_bases);
+
 /* ---------------------------------------------------------------------------------------
  * Non-overlapping k-mer encoder (grid-aligned windows, per-window fallback, tail as single
  * characters).  Replaces DNATok._encode_batch_kmer_numpy_partial (src/dna_tokenizer.py:

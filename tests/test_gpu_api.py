@@ -493,6 +493,55 @@ def test_dnatok_routes_bpe_tokenizers_to_the_backend():
         assert got[i, :len(r)].tolist() == r and bool((got[i, len(r):] == 3).all())
 
 
+def _write_fasta(path, seqs, width=70):
+    with open(path, "w") as fh:
+        for i, s in enumerate(seqs):
+            fh.write(f">rec{i}\n")
+            for j in range(0, len(s), width):
+                fh.write(s[j:j + width] + "\n")
+
+
+def test_fasta_file_encodes_like_the_same_strings(tmp_path):
+    """File -> ids through the host scan, for each of the three kernel families."""
+    rng = random.Random(8)
+    seqs = ["".join(rng.choice("ACGTACGTN") for _ in range(rng.randint(1, 700))) for _ in range(50)]
+    path = tmp_path / "reads.fa"
+    _write_fasta(path, seqs)
+    names = [f"rec{i}" for i in range(len(seqs))]
+
+    h = DNATok(RecordingEmbedder(SimpleCharTokenizer()))
+    h.discover()
+    ids, mask, got_names = h.encode_fasta_device(str(path))
+    want_ids, want_mask = h.encode_batch_device(seqs)
+    assert got_names == names and torch.equal(ids, want_ids) and torch.equal(mask, want_mask)
+
+    hk = DNATok(RecordingEmbedder(MockKmerTokenizer(4)))
+    hk.discover()
+    ids, mask, _ = hk.encode_fasta_device(str(path))
+    want_ids, want_mask = hk.encode_batch_device(seqs)
+    assert torch.equal(ids, want_ids) and torch.equal(mask, want_mask)
+
+    tk = hf.load_bpe_tokenizer("4096")
+
+    class Wrapped:
+        pad_token_id, unk_token_id, padding_side = 3, 0, "right"
+        backend_tokenizer = tk
+
+        def __call__(self, texts, add_special_tokens=False, **kw):
+            return {"input_ids": [e.ids for e in tk.encode_batch(list(texts), add_special_tokens=False)]}
+
+        def get_vocab(self):
+            return tk.get_vocab()
+
+    hb = DNATok(RecordingEmbedder(Wrapped()))
+    hb.discover()
+    ids, mask, _ = hb.encode_fasta_device(path.read_bytes())
+    for i, e in enumerate(tk.encode_batch(seqs, add_special_tokens=False)):
+        assert ids[i, :len(e.ids)].tolist() == e.ids and int(mask[i].sum()) == len(e.ids)
+    with pytest.raises(ValueError, match="No sequences"):
+        h.encode_fasta_device(b"")
+
+
 def test_bpe_kernel_wrapper_contract(tmp_path):
     cfg = util.tokenizer_json("4096")
     p = tmp_path / "merges.txt"

@@ -164,3 +164,51 @@ def test_device_normalizer_compile_and_validation():
     t, m, sc = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_size_t()
     assert L.dnatok_normalize_bounds(run, 2, 4, 100, 30, ctypes.byref(t), ctypes.byref(m), ctypes.byref(sc)) == 0
     assert (t.value, m.value) == (33 * 10 + 1 + 8, 100 + 2) and sc.value >= 2 * t.value
+
+
+def test_fasta_scan_layout_names_and_edge_cases(tmp_path):
+    """Records end to end + offsets; CR LF, blanks inside lines, ';' lines, an empty record, bases in
+    front of the first header, no line feed at the end."""
+    from dnatok_amd import encoders
+    text = b"; comment\nACG T\n>chr1 first\nACGT\nacgtn\r\n\n>empty\n>chr2\nTT\tTT\nGG"
+    data, off, names = encoders.fasta_to_bytes(text)
+    assert bytes(data.numpy()) == b"ACGTACGTacgtnTTTTGG"
+    assert off.tolist() == [0, 4, 13, 13, 19]
+    assert names == ["", "chr1 first", "empty", "chr2"]
+    data, off, _ = encoders.fasta_to_bytes(text, upper_case=True)
+    assert bytes(data.numpy()) == b"ACGTACGTACGTNTTTTGG"
+    # from a file, against a plain Python reading of the same text
+    rng = np.random.default_rng(4)
+    seqs = ["".join(rng.choice(list("ACGTN"), size=int(n))) for n in rng.integers(0, 500, size=40)]
+    path = tmp_path / "reads.fa"
+    with open(path, "w") as fh:
+        for i, s in enumerate(seqs):
+            fh.write(f">read{i} len={len(s)}\n")
+            for j in range(0, len(s), 60):
+                fh.write(s[j:j + 60] + "\n")
+    data, off, names = encoders.fasta_to_bytes(str(path))
+    assert names == [f"read{i} len={len(s)}" for i, s in enumerate(seqs)]
+    assert off.tolist() == np.concatenate([[0], np.cumsum([len(s) for s in seqs])]).tolist()
+    assert bytes(data.numpy()).decode() == "".join(seqs)
+    empty = encoders.fasta_to_bytes(b"")
+    assert empty[0].numel() == 0 and empty[1].tolist() == [0] and empty[2] == []
+
+
+def test_fasta_scan_rejects_too_small_outputs():
+    import ctypes
+    from dnatok_amd import _lib
+    L = _lib.lib()
+    text = np.frombuffer(b">a\nACGT\n>b\nAC\n", dtype=np.uint8)
+    seq = np.zeros(16, dtype=np.uint8)
+    off = np.zeros(4, dtype=np.int64)
+    n_rec, n_bases = ctypes.c_int64(0), ctypes.c_int64(0)
+    args = (ctypes.c_void_p(text.ctypes.data), text.size, 0, ctypes.c_void_p(seq.ctypes.data))
+    rc = L.dnatok_host_fasta_scan(*args, 16, ctypes.c_void_p(off.ctypes.data), None, 1,
+                                  ctypes.byref(n_rec), ctypes.byref(n_bases))
+    assert rc == -3 and b"records" in L.dnatok_last_error()
+    rc = L.dnatok_host_fasta_scan(*args, 5, ctypes.c_void_p(off.ctypes.data), None, 2,
+                                  ctypes.byref(n_rec), ctypes.byref(n_bases))
+    assert rc == -3 and b"bases" in L.dnatok_last_error()
+    rc = L.dnatok_host_fasta_scan(*args, 6, ctypes.c_void_p(off.ctypes.data), None, 2,
+                                  ctypes.byref(n_rec), ctypes.byref(n_bases))
+    assert rc == 0 and (n_rec.value, n_bases.value) == (2, 6) and off[:3].tolist() == [0, 4, 6]
