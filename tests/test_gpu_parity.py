@@ -473,6 +473,59 @@ def test_bpe_nonmonotone_random_tables():
             np.testing.assert_array_equal(r, e, err_msg=f"trial {trial} {s} {merges}")
 
 
+def test_bpe_encode_and_pad_replayed_from_a_graph(bpe):
+    """The engine (work list, chunked rows, seams, gather) and the padder captured once and replayed
+    over changing bytes of the same shape: every replay matches the oracle, i.e. nothing a call
+    leaves behind in the scratch buffer (counters, lists, flags) leaks into the next."""
+    which, enc, bo = bpe
+    say(f"bpe{which} graph replay")
+    lens = [5000, 300, 2048, 2049, 1, 9000, 700, 1500]
+    off_h = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    total, n = int(off_h[-1]), len(lens)
+
+    def batch(seed):
+        rng = np.random.default_rng(seed)
+        d = np.frombuffer(b"ACGT", dtype=np.uint8)[rng.integers(0, 4, size=total)].copy()
+        if seed % 2:                                  # a tandem repeat across a chunk border of row 0
+            d[1500:2300] = np.frombuffer(b"AC" * 400, dtype=np.uint8)
+        return d
+
+    data = torch.from_numpy(batch(0)).to(DEV)
+    off = torch.from_numpy(off_h).to(DEV)
+    t_cap = max(lens)
+    tok_tmp = torch.empty(total, dtype=torch.int32, device=DEV)
+    lengths = torch.empty(n, dtype=torch.int32, device=DEV)
+    out = (torch.empty((n, t_cap), dtype=torch.int32, device=DEV), torch.empty((n, t_cap), dtype=torch.uint8, device=DEV),
+           torch.empty(1, dtype=torch.int32, device=DEV))
+
+    def call():
+        enc.encode(data, off, t_cap, tok_tmp=tok_tmp, lengths=lengths)
+        encoders.pad_rows(tok_tmp, off, lengths, 0, t_cap, fill_to=0, out=out)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()                                        # warm-up outside the capture (scratch, attributes)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for seed in (1, 2, 3, 1):
+        host = batch(seed)
+        data.copy_(torch.from_numpy(host))
+        graph.replay()
+        torch.cuda.synchronize()
+        ref = bo.encode_batch(host, off_h)
+        width = int(out[2].item())
+        assert width == max(len(r) for r in ref)
+        ids, mask, ln = out[0].cpu().numpy(), out[1].cpu().numpy(), lengths.cpu().numpy()
+        for i, r in enumerate(ref):
+            assert ln[i] == len(r)
+            np.testing.assert_array_equal(ids[i, :len(r)], r, err_msg=f"seed {seed} row {i}")
+            assert (ids[i, len(r):width] == 0).all() and mask[i, :len(r)].all() and not mask[i, len(r):width].any()
+
+
 def test_bpe_repeated_pair_keeps_its_first_rank():
     """A pair listed twice: the later entry (another rank, another product) must never be used."""
     say("bpe table with a repeated pair")
