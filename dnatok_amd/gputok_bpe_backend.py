@@ -356,8 +356,9 @@ class GPUTokBPEBackend:
         b = len(seqs)
         t_cap = max(t_cap, 1)
         ids32, mask, lengths, longest = self.encode_device(data, offsets, t_cap)
-        width = int(longest.item())                       # the one host sync: the output shape
-        if int(lengths.min().item()) < 0:
+        # the one host sync: the output shape, and with it the smallest length (negative = failed row)
+        width, shortest = torch.stack((longest[0], lengths.min())).tolist()
+        if shortest < 0:
             raise RuntimeError("BPE engine reported a failed row (negative length)")
         if width == 0:
             return (torch.empty((b, 0), dtype=torch.long, device=dev),
