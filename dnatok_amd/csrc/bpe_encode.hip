@@ -13,9 +13,11 @@
 //     key merges.  Overlaps form chains of strictly decreasing key, along which the decision
 //     alternates, so each candidate walks its left and right chain and merges iff both have
 //     even length (for a run x x x x this is "every other one from the left", HF's tie rule);
-//   * the pairs that merge go onto a per-round queue; the queue deals the apply work (one merge
-//     per thread) and the re-rank work (two table probes per merge) evenly to the team, whatever
-//     positions the merges sit at.  Merges are applied in a doubly linked list over the original
+//   * the candidates of a round go onto a queue and are dealt one per thread for these walks (the
+//     threads find them among their own positions from ranks they keep in registers); the pairs
+//     that merge go onto a second queue, which deals the apply work (one merge per thread) and the
+//     re-rank work (two table lookups per merge) evenly to the team, whatever positions the merges
+//     sit at.  Merges are applied in a doubly linked list over the original
 //     positions (a merge keeps the left position); rank, links and symbol of a position sit in one
 //     record, so a step along a chain is one read; the two neighbour pairs of each new symbol are
 //     re-ranked through the hashed merge table, and only the threads whose positions changed
