@@ -1,7 +1,7 @@
 """``python -m dnatok_amd.dnatok_cli``: info / encode / validate / bench from a shell.
 
 The four commands of the reference's command line (src/dnatok_cli.py:162-307) with the same
-options and the same output fields.  ``--model`` names a tokenizer that can be had without a
+options and the same output fields (plus ``encode --fasta FILE``).  ``--model`` names a tokenizer that can be had without a
 network: a directory or ``tokenizer.json`` on disk (loaded with ``tokenizers.Tokenizer.from_file``
 and, for directories, ``transformers.AutoTokenizer`` when that works offline), or one of the
 built-in synthetic tokenizers of the benchmark configurations:
@@ -169,6 +169,21 @@ def cmd_info(args) -> int:
 def cmd_encode(args) -> int:
     device = args.device or _default_device()
     _, dn = _build_dnatok(args.model, device)
+    if args.fasta:
+        # every record of a FASTA file (not in the reference's command line, which takes --seq only)
+        ids, mask, names = dn.encode_fasta_device(args.fasta, device=device)
+        counts = mask.sum(dim=1).tolist()
+        _emit({
+            "model": args.model,
+            "fasta": args.fasta,
+            "n_records": len(names),
+            "n_tokens_total": int(sum(counts)),
+            "records": [{"name": n, "n_tokens": int(c)} for n, c in zip(names, counts)][: None if args.json else 8],
+            "selected_path": _detect_path(dn),
+        }, args.json)
+        return 0
+    if not args.seq:
+        raise SystemExit("encode: give --seq or --fasta")
     ids = _strip_pad(dn.encode_batch_to_ids([args.seq])[0].tolist(), int(dn.id_pad), dn.padding_side)
     _emit({
         "model": args.model,
@@ -265,7 +280,8 @@ def main(argv: Optional[list] = None) -> int:
     p.set_defaults(fn=cmd_info)
     p = sub.add_parser("encode", help="encode one sequence")
     common(p)
-    p.add_argument("--seq", required=True, help="DNA sequence (ACGT[N])")
+    p.add_argument("--seq", default=None, help="DNA sequence (ACGT[N])")
+    p.add_argument("--fasta", default=None, help="encode every record of this FASTA file instead")
     p.set_defaults(fn=cmd_encode)
     p = sub.add_parser("validate", help="bit identity with the tokenizer on random sequences")
     common(p)

@@ -571,9 +571,15 @@ def test_bpe_kernel_wrapper_contract(tmp_path):
 
 @pytest.mark.parametrize("model,path", [("char", "ascii-lut"), ("ntv3", "ascii-lut"), ("evo2", "ascii-lut"),
                                         ("kmer6", "kmer-6"), ("bpe4096", "gpu-bpe-kernel")])
-def test_cli_info_encode_validate(model, path, capsys):
+def test_cli_info_encode_validate(model, path, capsys, tmp_path):
     import json
     from dnatok_amd import dnatok_cli
+    fa = tmp_path / "two.fa"
+    fa.write_text(">first\nACGTACGTTTGACCA\n>second\nACGT\nTTGA\n")
+    assert dnatok_cli.main(["encode", "--model", model, "--fasta", str(fa), "--json"]) == 0
+    rec = json.loads(capsys.readouterr().out)
+    assert rec["n_records"] == 2 and [r["name"] for r in rec["records"]] == ["first", "second"]
+    assert rec["n_tokens_total"] == sum(r["n_tokens"] for r in rec["records"]) > 0
     assert dnatok_cli.main(["info", "--model", model, "--json"]) == 0
     info = json.loads(capsys.readouterr().out)
     assert info["selected_path"] == path and info["device"] == "cuda"
