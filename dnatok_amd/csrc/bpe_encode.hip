@@ -584,7 +584,10 @@ static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
     const bool chunks = max_len > p.ext;
     p.max_items = n_rows + (chunks ? total / p.core + 1 : 0);
-    p.max_mc = chunks ? 2 * (total / p.core) + 2 : 0;
+    // chunk slots: a chunked row of len bytes takes ceil(len / core) <= len / core + 1 of them, and
+    // there are fewer chunked rows than rows, and than total / core (each is longer than a chunk)
+    const int64_t by_rows = total / p.core + n_rows + 1, by_bytes = 2 * (total / p.core) + 2;
+    p.max_mc = chunks ? (by_rows < by_bytes ? by_rows : by_bytes) : 0;
     size_t o = 0;
     auto take = [&](size_t bytes) { size_t at = o; o = up(o + bytes); return at; };
     const size_t o_counts = take(64);
