@@ -473,6 +473,37 @@ def test_bpe_nonmonotone_random_tables():
             np.testing.assert_array_equal(r, e, err_msg=f"trial {trial} {s} {merges}")
 
 
+def test_bpe_nonmonotone_tables_with_rows_above_the_lds_capacity():
+    """Tables with two rules for one string are not chunked: rows above 2048 bytes go to the whole-row
+    kernel (state in global memory), including its rounds that merge a single pair."""
+    say("bpe non-monotone tables, long rows")
+    rng = random.Random(29)
+    n_nonmonotone = 0
+    for trial in range(6):
+        # "ACG" is made by two rules, and used (rank 3) before the second of them (rank 4)
+        merges = [("A", "C"), ("C", "G"), ("AC", "G"), ("ACG", "T"), ("A", "CG")]
+        toks, seen = list("ACGT") + ["AC", "CG", "ACG", "ACGT"], set(merges)
+        for _ in range(rng.randint(20, 80)):
+            a, b2 = rng.choice(toks), rng.choice(toks)
+            if (a, b2) in seen or len(a + b2) > 10:
+                continue
+            seen.add((a, b2))
+            merges.append((a, b2))
+            if a + b2 not in toks:
+                toks.append(a + b2)
+        strings = [a + b2 for a, b2 in merges]
+        n_nonmonotone += len(set(strings)) < len(strings)
+        kv = bpe_vocab.KernelVocab(merges)
+        enc = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv))
+        bo = O.BpeOracle(merges)
+        seqs = ["".join(rng.choice("ACGT") for _ in range(n)) for n in (2049, 3000, 5000, 700, 1)]
+        seqs.append("AC" * 1500 + "".join(rng.choice("ACGT") for _ in range(500)))
+        b = util.batch_from_strings(seqs)
+        for s, r, e in zip(seqs, bpe_rows(enc, b), bo.encode_batch(b.data, b.offsets, remap=False)):
+            np.testing.assert_array_equal(r, e, err_msg=f"trial {trial} len {len(s)} {merges}")
+    assert n_nonmonotone == 6
+
+
 def test_bpe_encode_and_pad_replayed_from_a_graph(bpe):
     """The engine (work list, chunked rows, seams, gather) and the padder captured once and replayed
     over changing bytes of the same shape: every replay matches the oracle, i.e. nothing a call
