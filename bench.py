@@ -69,7 +69,8 @@ class CharDense(Workload):
     """C1: 64 x 8192 bp char tokenizer; ids int32 + mask uint8, dense [B, T]."""
 
     def __init__(self, n_batches: int):
-        from dnatok_amd import encoders, hf_tokenizers as hf, workloads as wl
+        from dnatok_amd import encoders
+        from tests.support import hf_tokenizers as hf, workloads as wl
         vocab = hf.char_vocab()
         lut = np.zeros(256, dtype=np.int32)
         for ch in "ACGTN":
@@ -124,7 +125,8 @@ class KmerPadded(Workload):
     6000 bp row spelled on its own), rounded up to whole 128-byte lines for ids and mask."""
 
     def __init__(self, n_batches: int, t_cap: int = 6016):
-        from dnatok_amd import encoders, hf_tokenizers as hf, kmer_tables, workloads as wl
+        from dnatok_amd import encoders, kmer_tables
+        from tests.support import hf_tokenizers as hf, workloads as wl
         import torch
         vocab = hf.kmer_vocab(6)
         self.vocab = vocab
@@ -205,7 +207,8 @@ class BpePadded(Workload):
     """C3 / C4: BPE encode, then fused remap + pad-to-longest + mask."""
 
     def __init__(self, which: str, n_batches: int):
-        from dnatok_amd import bpe_vocab, encoders, hf_tokenizers as hf, workloads as wl
+        from dnatok_amd import bpe_vocab, encoders
+        from tests.support import hf_tokenizers as hf, workloads as wl
         import torch
         with open(hf.bpe_tokenizer_path(which)) as fh:
             cfg = json.load(fh)
@@ -280,7 +283,8 @@ class RaggedBoth(Workload):
     pass over the same device buffer; packed ids + offsets + masks stay on the device."""
 
     def __init__(self, n_batches: int = 1):
-        from dnatok_amd import bpe_vocab, encoders, hf_tokenizers as hf, workloads as wl
+        from dnatok_amd import bpe_vocab, encoders
+        from tests.support import hf_tokenizers as hf, workloads as wl
         import torch
         with open(hf.bpe_tokenizer_path("4096")) as fh:
             cfg = json.load(fh)
@@ -382,7 +386,7 @@ def time_steps(w: Workload, steps: int, warmup: int):
 
 def hf_cpu(config: str, threads: int, max_bases: int) -> dict | None:
     env = dict(os.environ, RAYON_NUM_THREADS=str(threads), TOKENIZERS_PARALLELISM="true")
-    cmd = [sys.executable, "-m", "dnatok_amd.hf_baseline", "--config", config, "--budget", "12"]
+    cmd = [sys.executable, "-m", "tests.support.hf_baseline", "--config", config, "--budget", "12"]
     if max_bases:
         cmd += ["--max-bases", str(max_bases)]
     try:
@@ -397,7 +401,8 @@ def fused_embed_extra():
     """Fused byte -> id -> embedding row kernel on one C1 batch (64 x 8192 bases), bf16 rows of 512:
     1 byte read and 1 KiB written per base; checked against the two-step torch form."""
     import torch
-    from dnatok_amd import encoders, hf_tokenizers as hf, workloads as wl
+    from dnatok_amd import encoders
+        from tests.support import hf_tokenizers as hf, workloads as wl
     vocab = hf.char_vocab()
     lut = np.zeros(256, dtype=np.int32)
     for ch in "ACGTN":
@@ -425,7 +430,8 @@ def unpack_2bit_extra():
     the host by the library, one launch; 0.25 byte read and 4 bytes written per base; checked
     against the byte path's ids wherever the text is ACGT (N travels as A)."""
     import torch
-    from dnatok_amd import encoders, hf_tokenizers as hf
+    from dnatok_amd import encoders
+    from tests.support import hf_tokenizers as hf
     vocab = hf.char_vocab()
     lut = np.zeros(256, dtype=np.int32)
     for ch in "ACGTN":
@@ -459,7 +465,8 @@ def device_normalizer_extra():
     N{10,} -> "-", prepend "_", lowercase (four steps, fused into one compaction pass), beside the
     same steps as Python callables string by string on one host core; results compared row by row."""
     import torch
-    from dnatok_amd import encoders, workloads as wl
+    from dnatok_amd import encoders
+    from tests.support import workloads as wl
     from dnatok_amd.gputok_bpe_backend import _compile_normalizer_step, _device_steps_of
     spec = {"type": "Sequence", "normalizers": [
         {"type": "Strip", "strip_left": True, "strip_right": True},

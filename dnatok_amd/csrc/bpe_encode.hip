@@ -34,6 +34,8 @@
 
 #include <stdlib.h>
 #include <string.h>
+#include <atomic>
+#include <unordered_map>
 #include <vector>
 
 struct dnatok_bpe_table {
@@ -562,18 +564,15 @@ static size_t long_slab_bytes(int64_t max_len)
     return ((n * 26) + 255) & ~(size_t)255;     // 16 (records) + 2 + 2 (product, gate) + 2 + 4 (queues)
 }
 
-// chunk geometry: DNATOK_BPE_CHUNK="core,overlap" overrides the default (for experiments)
+// Chunk geometry of the calls that follow (process-wide).  The shipped values are the constants
+// above; dnatok_bpe_set_chunk_geometry lets a test run the chunk / seam / fallback machinery with
+// chunks so small that every few hundred bytes of a row hold a seam.
+static std::atomic<int> g_chunk_core{kChunkCore}, g_chunk_overlap{kChunkOverlap};
+
 static void chunk_geometry(int *core, int *overlap)
 {
-    static int c = 0, v = 0;
-    if (c == 0) {
-        c = kChunkCore; v = kChunkOverlap;
-        const char *env = getenv("DNATOK_BPE_CHUNK");
-        int ec = 0, ev = 0;
-        if (env && sscanf(env, "%d,%d", &ec, &ev) == 2 && ec >= 256 && ev >= 32 && ec > 2 * ev &&
-            ec + 2 * ev <= kLdsCap) { c = ec; v = ev; }
-    }
-    *core = c; *overlap = v;
+    *core = g_chunk_core.load(std::memory_order_relaxed);
+    *overlap = g_chunk_overlap.load(std::memory_order_relaxed);
 }
 
 static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t total)
@@ -1060,6 +1059,12 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
     while (slots < (uint32_t)n_merges * 4u + 2u) { slots <<= 1; --shift; }
     std::vector<uint4> tab;
     std::vector<uint32_t> first_use;                           // lowest rank using a symbol
+    // A pair listed more than once counts with its last entry: HF collects the merges into a map
+    // in list order, so a later entry replaces the rank and product of an earlier one.
+    std::unordered_map<uint32_t, int32_t> last_entry;
+    last_entry.reserve((size_t)n_merges * 2);
+    for (int32_t i = 0; i < n_merges; ++i)
+        last_entry[((uint32_t)pair_a_h[i] << 16) | (uint32_t)pair_b_h[i]] = i;
     for (int attempt = 0;; ++attempt) {
         DNATOK_REQUIRE(shift > 4, DNATOK_E_INVALID, "dnatok_bpe_table_create: the merge table could not be hashed");
         mul1 = kMul[(2 * attempt) & 7]; mul2 = kMul[(2 * attempt + 1) & 7];
@@ -1069,8 +1074,7 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
         for (int32_t i = 0; i < n_merges && placed; ++i) {
             const uint32_t pa = (uint32_t)pair_a_h[i], pb = (uint32_t)pair_b_h[i];
             const uint32_t key = (pa << 16) | pb;
-            if (tab[pair_slot(key, mul1, shift)].x == key || tab[pair_slot(key, mul2, shift)].x == key)
-                continue;                       // a repeated pair keeps its first rank
+            if (last_entry[key] != i) continue;        // replaced by a later entry of the same pair
             if (first_use[pa] == 0xFFFFFFFFu) first_use[pa] = (uint32_t)i;
             if (first_use[pb] == 0xFFFFFFFFu) first_use[pb] = (uint32_t)i;
             uint4 e{key, (uint32_t)i, (uint32_t)new_id_h[i], 0};
@@ -1089,8 +1093,10 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
         if ((attempt & 3) == 3) { slots <<= 1; --shift; }
     }
     int monotone = 1;
-    for (int32_t i = 0; i < n_merges; ++i)
-        if (first_use[new_id_h[i]] <= (uint32_t)i) monotone = 0;
+    for (int32_t i = 0; i < n_merges; ++i) {
+        const uint32_t key = ((uint32_t)pair_a_h[i] << 16) | (uint32_t)pair_b_h[i];
+        if (last_entry[key] == i && first_use[new_id_h[i]] <= (uint32_t)i) monotone = 0;
+    }
     for (uint4 &e : tab)
         if (e.x != kEmptyKey) {
             const uint32_t fu = first_use[e.z];
@@ -1124,6 +1130,18 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
     t->byte_to_sym = (uint16_t *)(b + o_b2s);
     t->out_remap = out_remap_h ? (int32_t *)(b + o_remap) : nullptr;
     *out = t;
+    return DNATOK_OK;
+}
+
+extern "C" int dnatok_bpe_set_chunk_geometry(int32_t core, int32_t overlap)
+{
+    if (core == 0 && overlap == 0) { core = kChunkCore; overlap = kChunkOverlap; }
+    DNATOK_REQUIRE(core >= 256 && overlap >= 32 && core > 2 * overlap && core + 2 * overlap <= kLdsCap,
+                   DNATOK_E_INVALID,
+                   "dnatok_bpe_set_chunk_geometry: need core >= 256, overlap >= 32, core > 2 * overlap, "
+                   "core + 2 * overlap <= %d", kLdsCap);
+    g_chunk_core.store(core, std::memory_order_relaxed);
+    g_chunk_overlap.store(overlap, std::memory_order_relaxed);
     return DNATOK_OK;
 }
 

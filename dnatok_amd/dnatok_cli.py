@@ -10,8 +10,8 @@ built-in synthetic tokenizers of the benchmark configurations:
     ntv3      the NTv3 compat tokenizer class                (kernel: char)
     evo2      byte-level ids, id = ord(c)                    (kernel: char)
     kmer6     non-overlapping 6-mers, grid-aligned fallback  (kernel: k-mer)
-    bpe4096   BPE trained on the synthetic corpus            (kernel: BPE engine)
-    bpe32000  BPE with the 32000 vocabulary                  (kernel: BPE engine)
+
+A BPE tokenizer is named by the path of its ``tokenizer.json`` (kernel: BPE engine).
 
 All encoding runs on the GPU through libdnatok_hip.so; the reference tokenizer it is compared
 with runs on the host.
@@ -26,7 +26,7 @@ import sys
 import time
 from typing import Any, List, Optional, Tuple
 
-BUILTIN = ("char", "ntv3", "evo2", "kmer6", "bpe4096", "bpe32000")
+BUILTIN = ("char", "ntv3", "evo2", "kmer6")
 
 
 class _TokenizerCall:
@@ -53,7 +53,7 @@ class _TokenizerCall:
 
 
 def _load_tokenizer(model: str):
-    from . import dnatok_compat, hf_tokenizers as hf
+    from . import builtin_tokenizers as hf, dnatok_compat
     if model == "char":
         return _TokenizerCall(hf.build_char_tokenizer(), pad_id=hf.char_vocab()["<pad>"])
     if model == "ntv3":
@@ -62,9 +62,6 @@ def _load_tokenizer(model: str):
         return dnatok_compat.Evo2ByteTokenizer()
     if model == "kmer6":
         return _TokenizerCall(hf.build_kmer_tokenizer(6), pad_id=hf.kmer_vocab(6)["<pad>"])
-    if model in ("bpe4096", "bpe32000"):
-        tk = hf.load_bpe_tokenizer(model[3:])
-        return _TokenizerCall(tk, pad_id=tk.token_to_id("[PAD]"))
     path = model
     if os.path.isdir(path):
         try:

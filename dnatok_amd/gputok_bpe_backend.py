@@ -200,19 +200,61 @@ def _extract_merges(cfg: Dict[str, Any]) -> List[str]:
     return out
 
 
+_SPLIT_WHITESPACE_REGEX = {r"\s+", r"\s", " +", " ", r"\n", r"\n+", r"[ \t\n]+", r"[\s]+"}
+
+
+def _pre_tokenizer_reason(pre: Any, model: Dict[str, Any]) -> Optional[str]:
+    """None when the pre-tokenizer leaves a row without white space in one piece (or in pieces the
+    merges never join anyway), else why not."""
+    if pre is None:
+        return None
+    kind = pre.get("type") if isinstance(pre, dict) else None
+    if kind in (None, "WhitespaceSplit"):
+        return None
+    if kind == "Whitespace":
+        # \w+|[^\w\s]+ also cuts between word characters and punctuation: the same as no cut only
+        # when no merge rule spans such a border
+        for m in model.get("merges", []):
+            a, b = (m.split() + ["", ""])[:2] if isinstance(m, str) else (str(m[0]), str(m[1]))
+            word = [bool(_re.match(r"\w", c)) for c in a + b]
+            if any(x != word[0] for x in word):
+                return "pre_tokenizer='Whitespace' with a merge rule across a word / punctuation border"
+        return None
+    if kind == "Split":
+        pattern = pre.get("pattern") or {}
+        if pre.get("invert", False):
+            return "pre_tokenizer='Split' with invert"
+        if "String" in pattern and pattern["String"] and pattern["String"].isspace():
+            return None
+        if pattern.get("Regex") in _SPLIT_WHITESPACE_REGEX:
+            return None
+        return f"pre_tokenizer='Split' on {pattern!r} (only white-space patterns are reproduced)"
+    return f"pre_tokenizer={kind!r}"
+
+
 def _supported_tokenizer(cfg: Optional[Dict[str, Any]]) -> Tuple[bool, str]:
-    """(ok, reason): BPE model, whitespace-type or no pre-tokenizer, reproducible normalizer
-    (reference: 265-295)."""
+    """(ok, reason): a BPE model whose ids this engine reproduces bit for bit.  Refused: another
+    model type; a pre-tokenizer that can cut a row without white space; a normalizer that is not
+    reproduced; and the BPE options that change the ids -- dropout, byte_fallback, ignore_merges,
+    fuse_unk, a continuing_subword_prefix or end_of_word_suffix.  (The reference's gate looks at
+    model type, pre-tokenizer type and normalizer only, src/gputok_bpe_backend.py:265-295, and
+    encodes such a tokenizer as if the options were off.)"""
     if cfg is None:
         return False, "tokenizer.json not found"
     model = cfg.get("model") or {}
     if model.get("type") != "BPE":
         return False, f"model.type={model.get('type')!r} (only BPE supported)"
-    pre = cfg.get("pre_tokenizer")
-    if pre is not None:
-        kind = pre.get("type") if isinstance(pre, dict) else None
-        if kind not in (None, "Whitespace", "Split", "WhitespaceSplit"):
-            return False, f"pre_tokenizer={kind!r}"
+    if model.get("dropout"):
+        return False, f"model.dropout={model.get('dropout')!r} (merges are skipped at random)"
+    for flag in ("byte_fallback", "ignore_merges", "fuse_unk"):
+        if model.get(flag):
+            return False, f"model.{flag}=true changes the ids"
+    for affix in ("continuing_subword_prefix", "end_of_word_suffix"):
+        if model.get(affix):
+            return False, f"model.{affix}={model.get(affix)!r} changes the symbols"
+    reason = _pre_tokenizer_reason(cfg.get("pre_tokenizer"), model)
+    if reason is not None:
+        return False, reason
     norm = cfg.get("normalizer")
     if norm is not None and _compile_normalizer_step(norm) is None:
         return False, f"unsupported normalizer={norm.get('type')!r}"
@@ -259,6 +301,19 @@ class GPUTokBPEBackend:
         self._normalize = _compile_normalizer(cfg)
         # the same steps as a device program, used for all-ASCII batches; None: host callables
         self._normalize_device = _compile_device_normalizer(cfg) if self._normalize is not None else None
+        # What the engine cannot reproduce depends on the input for two kinds of tokenizer: with a
+        # pre-tokenizer, white space inside a row cuts it into words (and is dropped); without an
+        # unk_token, characters outside the vocabulary are dropped.  Such input raises ValueError
+        # (DNATok then takes the row to the tokenizer itself).
+        self._input_guard: Optional[_re.Pattern] = None
+        guard = []
+        if cfg.get("pre_tokenizer") is not None:
+            guard.append(r"\s")
+        if (cfg.get("model") or {}).get("unk_token") is None:
+            singles = "".join(_re.escape(t) for t in (cfg.get("model") or {}).get("vocab", {}) if len(t) == 1)
+            guard.append(f"[^{singles}]" if singles else ".")
+        if guard:
+            self._input_guard = _re.compile("|".join(guard), _re.S)
         self._merges: List[str] = _extract_merges(cfg)
         if not self._merges:
             raise RuntimeError("Tokenizer has no merges; nothing to accelerate.")
@@ -341,7 +396,14 @@ class GPUTokBPEBackend:
         dev = torch.device(device) if not isinstance(device, torch.device) else device
         if dev.type != "cuda":
             raise RuntimeError("GPUTokBPEBackend.encode_batch runs on the GPU only (device='cuda')")
-        if self._normalize is None:
+        if self._input_guard is not None:
+            if self._normalize is not None:
+                seqs = [self._normalize(s) for s in seqs]
+            hit = self._input_guard.search("".join(seqs))
+            if hit is not None:
+                raise ValueError(f"character {hit.group(0)!r} is cut or dropped by this tokenizer "
+                                 "(pre-tokenizer / no unk_token); not reproduced by the GPU engine")
+        if self._normalize is None or self._input_guard is not None:
             data, offsets, lens = encoders.bytes_from_strings(seqs, dev, encoding="utf-8")
             t_cap = int(lens.max())
         elif self._normalize_device is not None and self.normalize_on_device and "".join(seqs).isascii():

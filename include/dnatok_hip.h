@@ -190,6 +190,14 @@ int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t
                       void *scratch, size_t scratch_bytes,
                       int32_t *tok_tmp, int32_t *lengths, void *stream);
 
+/* Test hook, no counterpart in the reference: sets the geometry the calls that follow (in this
+ * process) cut rows longer than core + 2 * overlap bytes with: chunks of `core` bytes, extended by
+ * `overlap` bytes on both sides, joined at seams inside the overlaps.  The shipped geometry is
+ * (1792, 128); (0, 0) restores it.  Tests pass small chunks so that rows of a few kilobytes go
+ * through thousands of seams and whole-row fallbacks.  Results never depend on the geometry.
+ * Not synchronised with encode calls in flight on other threads. */
+int dnatok_bpe_set_chunk_geometry(int32_t core, int32_t overlap);
+
 /* ---------------------------------------------------------------------------------------
  * Ragged-batch packer: turns per-row token runs (tok_tmp + in_offsets + lengths, as the BPE
  * engine leaves them) into the tensors a model consumes, without a host round trip.

@@ -165,7 +165,8 @@ static inline uint64_t mix64(uint64_t x)
 }
 
 /* Merge rule i: (pair_a[i], pair_b[i]) -> new_id[i], rank i.  A pair listed twice keeps
- * its first (lowest) rank, as a dictionary built in rank order would. */
+ * its LAST entry (rank and product): HF collects the merges into a map in list order, so a
+ * later entry replaces an earlier one (checked against the library in tests/test_oracle.py). */
 oracle_bpe_table *oracle_bpe_table_create(const int32_t *pair_a, const int32_t *pair_b,
                                           const int32_t *new_id, int32_t n_merges)
 {
@@ -182,7 +183,6 @@ oracle_bpe_table *oracle_bpe_table_create(const int32_t *pair_a, const int32_t *
         uint64_t key = ((uint64_t)(uint32_t)pair_a[i] << 32) | (uint32_t)pair_b[i];
         uint64_t h = mix64(key) & t->mask;
         while (t->keys[h] != ORACLE_EMPTY && t->keys[h] != key) h = (h + 1) & t->mask;
-        if (t->keys[h] == key) continue;
         t->keys[h] = key;
         t->rank[h] = (uint32_t)i;
         t->new_id[h] = new_id[i];

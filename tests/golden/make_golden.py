@@ -8,7 +8,7 @@
 (add_special_tokens=False) and stores, per configuration and tokenizer: the per-row token
 counts, a SHA-256 over all ids (int32 little endian, rows back to back), and the ids of the
 first row (first 2048).  It also stores a few small hand-sized cases in full.  The inputs
-are regenerated from their seeds by dnatok_amd.workloads, so only outputs are stored.
+are regenerated from their seeds by tests.support.workloads, so only outputs are stored.
 """
 from __future__ import annotations
 
@@ -21,8 +21,8 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 
-from dnatok_amd import hf_tokenizers as hf   # noqa: E402
-from dnatok_amd import workloads as wl       # noqa: E402
+from tests.support import hf_tokenizers as hf   # noqa: E402
+from tests.support import workloads as wl       # noqa: E402
 
 SMALL_CASES = [
     "", "A", "N", "ACGT", "AAAAAAAAAAAAAAAAAAAAAAAAAAAAAAAAA", "ACACACACACACACACACACACACAC",

@@ -2,7 +2,7 @@
 
 Run as its own process (rayon sizes its thread pool once per process):
 
-    RAYON_NUM_THREADS=N TOKENIZERS_PARALLELISM=true python -m dnatok_amd.hf_baseline --config C2
+    RAYON_NUM_THREADS=N TOKENIZERS_PARALLELISM=true python -m tests.support.hf_baseline --config C2
 
 Prints one JSON line: Mbp/s = input bases / median wall time / 1e6, the definition the
 reference's CLI bench uses (src/dnatok_cli.py:272,299-301).  bytes -> str conversion

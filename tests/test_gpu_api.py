@@ -8,7 +8,8 @@ import numpy as np
 import pytest
 import torch
 
-from dnatok_amd import dnatok_compat, hf_tokenizers as hf
+from dnatok_amd import dnatok_compat
+from tests.support import hf_tokenizers as hf
 from dnatok_amd.dna_tokenizer import DNATok
 from dnatok_amd.dnatok_bpe_kernel import DnatokBpeKernel
 from dnatok_amd.gputok_bpe_backend import GPUTokBPEBackend
@@ -329,6 +330,34 @@ def test_bpe_backend_with_normalizer():
         assert ids[i, :len(e.ids)].tolist() == e.ids and int(mask[i].sum()) == len(e.ids)
 
 
+def test_bpe_backend_guards_input_it_cannot_reproduce():
+    """Without an unk_token the library drops characters outside the vocabulary; with a
+    pre-tokenizer it cuts rows at white space.  Rows without such characters are identical, rows
+    with them raise ValueError (DNATok then takes the batch to the tokenizer itself)."""
+    import json
+    from tokenizers import Tokenizer
+    cfg = json.loads(json.dumps(util.tokenizer_json("4096")))
+    cfg["model"]["unk_token"] = None
+    tk = Tokenizer.from_str(json.dumps(cfg))
+    assert [e.ids for e in tk.encode_batch(["ACXGT"])] == [e.ids for e in tk.encode_batch(["ACGT"])]
+    be = GPUTokBPEBackend(tk)
+    seqs = random_seqs(12, 500, alphabet="ACGTN", seed=3)
+    ids, mask = be.encode_batch(seqs)
+    for i, e in enumerate(tk.encode_batch(seqs, add_special_tokens=False)):
+        assert ids[i, :len(e.ids)].tolist() == e.ids and int(mask[i].sum()) == len(e.ids)
+    with pytest.raises(ValueError):
+        be.encode_batch(seqs + ["ACXGT"])
+    cfg = json.loads(json.dumps(util.tokenizer_json("4096")))
+    cfg["pre_tokenizer"] = {"type": "Whitespace"}
+    tk = Tokenizer.from_str(json.dumps(cfg))
+    be = GPUTokBPEBackend(tk)
+    ids, mask = be.encode_batch(seqs)
+    for i, e in enumerate(tk.encode_batch(seqs, add_special_tokens=False)):
+        assert ids[i, :len(e.ids)].tolist() == e.ids and int(mask[i].sum()) == len(e.ids)
+    with pytest.raises(ValueError):
+        be.encode_batch(["ACGT ACGT"])
+
+
 def _rows_to_device(rows):
     from dnatok_amd import encoders
     return encoders.bytes_from_strings(rows, "cuda", encoding="utf-8")
@@ -574,6 +603,8 @@ def test_bpe_kernel_wrapper_contract(tmp_path):
 def test_cli_info_encode_validate(model, path, capsys, tmp_path):
     import json
     from dnatok_amd import dnatok_cli
+    if model == "bpe4096":                       # a BPE tokenizer is named by the path of its tokenizer.json
+        model = hf.bpe_tokenizer_path("4096")
     fa = tmp_path / "two.fa"
     fa.write_text(">first\nACGTACGTTTGACCA\n>second\nACGT\nTTGA\n")
     assert dnatok_cli.main(["encode", "--model", model, "--fasta", str(fa), "--json"]) == 0

@@ -6,8 +6,9 @@ import numpy as np
 import pytest
 import torch
 
-from dnatok_amd import bpe_vocab, encoders, hf_tokenizers as hf, kmer_tables
-from dnatok_amd import workloads as wl
+from dnatok_amd import bpe_vocab, encoders, kmer_tables
+from tests.support import hf_tokenizers as hf
+from tests.support import workloads as wl
 from oracle import oracle as O
 from tests import util
 
@@ -438,6 +439,43 @@ def test_bpe_rows_without_a_seam_fall_back_to_the_whole_row_kernel(bpe):
         np.testing.assert_array_equal(r, e, err_msg=s[:20])
 
 
+@pytest.mark.parametrize("core,overlap", [(256, 32), (512, 96)])
+def test_bpe_small_chunks_many_seams_and_fallbacks(bpe, core, overlap):
+    """The chunk / seam / gather / whole-row-fallback machinery with chunks far smaller than the
+    shipped ones: a few thousand ragged, random and tandem-repeat rows per vocabulary go through tens
+    of thousands of seams, many of which find no position and send their row to the whole-row
+    kernel.  Every row is compared with the oracle."""
+    which, enc, bo = bpe
+    say(f"bpe{which} chunks of {core} + 2 x {overlap}")
+    from dnatok_amd import _lib
+    L = _lib.lib()
+    ext = core + 2 * overlap
+    _lib.check(L.dnatok_bpe_set_chunk_geometry(core, overlap), "dnatok_bpe_set_chunk_geometry")
+    try:
+        rng = random.Random(int(which) + core)
+        n_rows = n_chunked = n_failed = 0
+        for trial in range(5):
+            strings = wl.config5_ragged(300, seed=100 + trial).strings()
+            strings += ["".join(rng.choice("ACGT") for _ in range(rng.randint(1, 6000))) for _ in range(100)]
+            strings += [rng.choice(["A", "AC", "ACG", "AATT", "ACGTC"]) * rng.randint(1, 900) +
+                        "".join(rng.choice("ACGTN") for _ in range(rng.randint(0, 3000))) for _ in range(30)]
+            rng.shuffle(strings)
+            b = util.batch_from_strings(strings)
+            rows = bpe_rows(enc, b)
+            # the plan's counters sit at the start of the scratch buffer: [1] chunk items, [3] rows redone whole
+            counts = enc._scratch[:16].view(torch.int32).cpu().numpy()
+            assert counts[1] > 0
+            n_failed += int(counts[3])
+            n_chunked += int((b.lengths() > ext).sum())
+            n_rows += b.n_seqs
+            for i, (r, e) in enumerate(zip(rows, bo.encode_batch(b.data, b.offsets))):
+                np.testing.assert_array_equal(r, e, err_msg=f"trial {trial} row {i} len {len(strings[i])}")
+        say(f"  {n_rows} rows, {n_chunked} chunked, {n_failed} redone by the whole-row kernel")
+        assert n_rows >= 2000 and 0 < n_failed < n_chunked       # seams accepted and seams refused
+    finally:
+        _lib.check(L.dnatok_bpe_set_chunk_geometry(0, 0), "dnatok_bpe_set_chunk_geometry")
+
+
 def test_bpe_c4_golden():
     say("bpe32000 C4 32x100k")
     cfg = util.tokenizer_json("32000")
@@ -557,22 +595,27 @@ def test_bpe_encode_and_pad_replayed_from_a_graph(bpe):
             assert (ids[i, len(r):width] == 0).all() and mask[i, :len(r)].all() and not mask[i, len(r):width].any()
 
 
-def test_bpe_repeated_pair_keeps_its_first_rank():
-    """A pair listed twice: the later entry (another rank, another product) must never be used."""
-    say("bpe table with a repeated pair")
-    merges = [("A", "C"), ("AC", "G"), ("T", "T"), ("ACG", "TT"), ("G", "A")]
-    kv = bpe_vocab.KernelVocab(merges)
-    a, b2, n = list(kv.pair_a), list(kv.pair_b), list(kv.new_id)
-    a.insert(3, a[0]); b2.insert(3, b2[0]); n.insert(3, n[2])          # (A, C) again, giving TT's id
-    plain = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv))
-    twice = encoders.BpeEncoder(np.array(a, dtype=np.int32), np.array(b2, dtype=np.int32),
-                                np.array(n, dtype=np.int32), len(kv))
+def test_bpe_repeated_pair_takes_its_last_entry():
+    """A pair listed twice counts with its later rank, as in the HF library (the oracle's rule is
+    pinned against the library by tests/test_oracle.py); known case first, then random lists."""
+    say("bpe tables with repeated pairs")
+    from tests.test_oracle import random_merge_list
+    known = [("A", "C"), ("C", "G"), ("A", "C")]
+    kv = bpe_vocab.KernelVocab(known)
+    enc = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv))
+    (row,) = bpe_rows(enc, util.batch_from_strings(["ACG"]))
+    assert [kv.id_to_token[i] for i in row] == ["A", "CG"]
     rng = random.Random(5)
-    seqs = ["".join(rng.choice("ACGT") for _ in range(rng.randint(1, 400))) for _ in range(50)]
-    b = util.batch_from_strings(seqs)
-    # ranks above the inserted entry shift by one, the ids produced do not
-    for r1, r2 in zip(bpe_rows(plain, b), bpe_rows(twice, b)):
-        np.testing.assert_array_equal(r1, r2)
+    for trial in range(25):
+        merges = random_merge_list(rng, rng.randint(3, 40), duplicates=rng.randint(1, 6))
+        kv = bpe_vocab.KernelVocab(merges)
+        enc = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv))
+        bo = O.BpeOracle(merges)
+        seqs = ["".join(rng.choice("ACGT") for _ in range(rng.randint(1, 400))) for _ in range(30)]
+        seqs.append("".join(rng.choice("ACGT") for _ in range(5000)))        # chunked or whole-row path
+        b = util.batch_from_strings(seqs)
+        for sq, r, e in zip(seqs, bpe_rows(enc, b), bo.encode_batch(b.data, b.offsets, remap=False)):
+            np.testing.assert_array_equal(r, e, err_msg=f"trial {trial} {sq[:60]} {merges}")
 
 
 def test_bpe_table_near_the_size_limit():

@@ -1,11 +1,14 @@
 """Host-side logic of the drop-in API that needs no GPU: normalizer compiler truth tables
 (the reference's own CPU unit tests, tests/test_gputok_bpe_backend.py:319-425), tokenizer.json
 handling, and the compat tokenizer classes."""
+import json
+
 import numpy as np
 import pytest
 
-from dnatok_amd import dnatok_compat, hf_tokenizers as hf
-from dnatok_amd.gputok_bpe_backend import (_compile_normalizer, _compile_normalizer_step, _extract_merges,
+from dnatok_amd import dnatok_compat
+from tests.support import hf_tokenizers as hf
+from dnatok_amd.gputok_bpe_backend import (GPUTokBPEBackend, _compile_normalizer, _compile_normalizer_step, _extract_merges,
                                            _read_tokenizer_json, _reconstruct_gputok_vocab,
                                            _supported_tokenizer)
 
@@ -54,6 +57,48 @@ def test_supported_tokenizer_gate():
     assert not _supported_tokenizer({"model": {"type": "WordLevel"}})[0]
     assert not _supported_tokenizer({"model": {"type": "BPE"}, "pre_tokenizer": {"type": "ByteLevel"}})[0]
     assert _supported_tokenizer({"model": {"type": "BPE"}, "pre_tokenizer": None})[0]
+
+
+def test_gate_refuses_bpe_options_that_change_the_ids():
+    """Live HF tokenizers built with each BPE option: the option changes what the library returns
+    (so a backend that ignores it would be wrong), and the gate refuses the tokenizer."""
+    from tokenizers import Tokenizer, models, pre_tokenizers
+    vocab = {"[UNK]": 0, "A": 1, "C": 2, "G": 3, "T": 4, "AC": 5, "ACG": 6, "##C": 7, "##G": 8, "T</w>": 9,
+             "<0x4E>": 10, "ACGT": 11, "GT": 12}
+    merges = [("A", "C"), ("AC", "G"), ("G", "T")]
+    plain = Tokenizer(models.BPE(vocab=vocab, merges=merges, unk_token="[UNK]"))
+    assert plain.encode("ACGT").ids == [6, 4] and plain.encode("ANNC").ids == [1, 0, 0, 2]
+    assert _supported_tokenizer(json.loads(plain.to_str())) == (True, "ok")
+    variants = {
+        "dropout": (dict(dropout=0.5), None),
+        "fuse_unk": (dict(fuse_unk=True), ("ANNC", [1, 0, 2])),
+        "byte_fallback": (dict(byte_fallback=True), ("ANC", [1, 10, 2])),
+        "ignore_merges": (dict(ignore_merges=True), ("ACGT", [11])),
+        "continuing_subword_prefix": (dict(continuing_subword_prefix="##", merges=[("A", "##C")]), ("AG", [1, 8])),
+        "end_of_word_suffix": (dict(end_of_word_suffix="</w>"), ("AT", [1, 9])),
+    }
+    for name, (kwargs, known) in variants.items():
+        tk = Tokenizer(models.BPE(vocab=vocab, unk_token="[UNK]", **dict(dict(merges=merges), **kwargs)))
+        if known is not None:
+            text, ids = known
+            assert tk.encode(text).ids == ids and plain.encode(text).ids != ids, name
+        ok, reason = _supported_tokenizer(json.loads(tk.to_str()))
+        assert not ok and name in reason, (name, reason)
+        assert not GPUTokBPEBackend.is_supported(tk)
+    # pre-tokenizers: white-space cuts are fine (rows hold none), other cuts are not
+    for pre, want in ((pre_tokenizers.WhitespaceSplit(), True), (pre_tokenizers.Whitespace(), True),
+                      (pre_tokenizers.Split(" ", "removed"), True), (pre_tokenizers.Split("C", "isolated"), False),
+                      (pre_tokenizers.ByteLevel(), False), (pre_tokenizers.Digits(), False)):
+        tk = Tokenizer(models.BPE(vocab=vocab, merges=merges, unk_token="[UNK]"))
+        tk.pre_tokenizer = pre
+        assert _supported_tokenizer(json.loads(tk.to_str()))[0] is want, pre
+    # "Whitespace" also cuts between letters and punctuation: refused when a merge spans such a border
+    v2 = dict(vocab, **{"-": 13, "A-": 14})
+    tk = Tokenizer(models.BPE(vocab=v2, merges=merges + [("A", "-")], unk_token="[UNK]"))
+    tk.pre_tokenizer = pre_tokenizers.Whitespace()
+    assert tk.encode("A-C").ids == [1, 13, 2]                   # the library does not apply A + -
+    ok, reason = _supported_tokenizer(json.loads(tk.to_str()))
+    assert not ok and "border" in reason
 
 
 def test_tokenizer_json_from_live_object_and_merges():

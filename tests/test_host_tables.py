@@ -1,7 +1,8 @@
 """Host-side table builders of the product against the oracle's independent restatement."""
 import numpy as np
 
-from dnatok_amd import bpe_vocab, hf_tokenizers as hf, kmer_tables
+from dnatok_amd import bpe_vocab, kmer_tables
+from tests.support import hf_tokenizers as hf
 from oracle import oracle as O
 from tests import util
 

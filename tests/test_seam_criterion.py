@@ -8,7 +8,7 @@ import random
 
 import numpy as np
 
-from dnatok_amd import workloads as wl
+from tests.support import workloads as wl
 from oracle import oracle as O
 from tests import util
 

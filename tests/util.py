@@ -7,8 +7,8 @@ from functools import lru_cache
 
 import numpy as np
 
-from dnatok_amd import hf_tokenizers as hf
-from dnatok_amd import workloads as wl
+from tests.support import hf_tokenizers as hf
+from tests.support import workloads as wl
 from oracle import oracle as O
 
 from tests.golden.check import GOLDEN_DIR, check_against_golden, golden, sha_of_rows  # noqa: F401
