@@ -556,6 +556,7 @@ struct BpePlan {                          // device arrays inside the scratch bu
     size_t slab_bytes, total_bytes;
     int64_t max_items, max_mc;
     int core, overlap, ext;   // chunk core, overlap on each side, core + 2 * overlap
+    int n_slabs;              // workgroups of the whole-row fallback kernel (one slab of state each)
 };
 
 static size_t long_slab_bytes(int64_t max_len)
@@ -575,7 +576,8 @@ static void chunk_geometry(int *core, int *overlap)
     *overlap = g_chunk_overlap.load(std::memory_order_relaxed);
 }
 
-static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t total)
+static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t total,
+                         int64_t max_slabs = kLongGrid)
 {
     BpePlan p{};
     chunk_geometry(&p.core, &p.overlap);
@@ -599,8 +601,9 @@ static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t
     const size_t o_fail = take(4 * (size_t)n_rows);
     const size_t o_sym = take(2 * (size_t)p.ext * (size_t)p.max_mc);
     p.slab_bytes = chunks ? long_slab_bytes(max_len) : 0;
-    const int64_t slabs = n_rows < kLongGrid ? n_rows : kLongGrid;
-    const size_t o_slabs = take(chunks ? p.slab_bytes * (size_t)slabs : 0);
+    const int64_t slabs = n_rows < max_slabs ? n_rows : max_slabs;
+    p.n_slabs = (int)(slabs < 1 ? 1 : slabs);
+    const size_t o_slabs = take(chunks ? p.slab_bytes * (size_t)p.n_slabs : 0);
     p.total_bytes = o + 256;
     if (base) {
         p.counts = (int32_t *)(base + o_counts);
@@ -1223,23 +1226,10 @@ int run_lds(bool long_rows, int chunking, const BpeArgs &a, const uint8_t *bytes
 
 }  // namespace
 
-extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets,
-                                 int64_t n_rows, int64_t max_len, int64_t total, void *scratch,
-                                 size_t scratch_bytes, int32_t *tok_tmp, int32_t *lengths, void *stream)
+// The launches of one encode call; p lies inside a scratch buffer that holds p.total_bytes.
+static int bpe_encode_launch(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets, int64_t n_rows,
+                             int64_t max_len, const BpePlan &p, int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
 {
-    DNATOK_REQUIRE(t && offsets && lengths, DNATOK_E_INVALID, "dnatok_bpe_encode: null argument");
-    DNATOK_REQUIRE(n_rows >= 0 && max_len >= 0 && total >= 0, DNATOK_E_INVALID,
-                   "dnatok_bpe_encode: negative size");
-    DNATOK_REQUIRE(max_len < (int64_t)1 << 31 && total / 256 + n_rows < (int64_t)1 << 30, DNATOK_E_TOO_LARGE,
-                   "dnatok_bpe_encode: batch too large for 32-bit work indices");
-    if (n_rows == 0) return DNATOK_OK;
-    DNATOK_REQUIRE(total == 0 || (bytes && tok_tmp), DNATOK_E_INVALID, "dnatok_bpe_encode: null buffer");
-    const BpePlan need = make_plan(nullptr, n_rows, max_len, total);
-    DNATOK_REQUIRE(scratch && scratch_bytes >= need.total_bytes, DNATOK_E_SCRATCH,
-                   "dnatok_bpe_encode: scratch holds %zu bytes, %zu needed", scratch_bytes, need.total_bytes);
-    DNATOK_REQUIRE(((uintptr_t)scratch & 255) == 0, DNATOK_E_INVALID, "dnatok_bpe_encode: scratch must be 256-byte aligned");
-    const BpePlan p = make_plan((uint8_t *)scratch, n_rows, max_len, total);
-    hipStream_t s = (hipStream_t)stream;
     BpeArgs a{t->tab, t->byte_to_sym, t->out_remap, t->shift, t->mul1, t->mul2, t->n_merges};
 
     const bool long_rows = max_len > p.ext;
@@ -1262,10 +1252,94 @@ extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, co
             bpe_gather_kernel<<<(int)(g < 1 ? 1 : g), 256, 0, s>>>(a, offsets, p, tok_tmp, lengths);
             DNATOK_HIP_TRY(hipGetLastError());
         }
-        const int64_t slabs = n_rows < kLongGrid ? n_rows : kLongGrid;
-        bpe_long_kernel<kLongThreads><<<(int)slabs, kLongThreads, 0, s>>>(a, bytes, offsets, n_rows, max_len, p,
-                                                                         tok_tmp, lengths);
+        bpe_long_kernel<kLongThreads><<<p.n_slabs, kLongThreads, 0, s>>>(a, bytes, offsets, n_rows, max_len, p,
+                                                                        tok_tmp, lengths);
         DNATOK_HIP_TRY(hipGetLastError());
     }
     return DNATOK_OK;
+}
+
+static int bpe_encode_check(const char *who, const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets,
+                            int64_t n_rows, int64_t max_len, int64_t total, const int32_t *tok_tmp,
+                            const int32_t *lengths)
+{
+    DNATOK_REQUIRE(t && offsets && lengths, DNATOK_E_INVALID, "%s: null argument", who);
+    DNATOK_REQUIRE(n_rows >= 0 && max_len >= 0 && total >= 0, DNATOK_E_INVALID, "%s: negative size", who);
+    DNATOK_REQUIRE(max_len < (int64_t)1 << 31 && total / 256 + n_rows < (int64_t)1 << 30, DNATOK_E_TOO_LARGE,
+                   "%s: batch too large for 32-bit work indices", who);
+    DNATOK_REQUIRE(n_rows == 0 || total == 0 || (bytes && tok_tmp), DNATOK_E_INVALID, "%s: null buffer", who);
+    return DNATOK_OK;
+}
+
+extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets,
+                                 int64_t n_rows, int64_t max_len, int64_t total, void *scratch,
+                                 size_t scratch_bytes, int32_t *tok_tmp, int32_t *lengths, void *stream)
+{
+    const int bad = bpe_encode_check("dnatok_bpe_encode", t, bytes, offsets, n_rows, max_len, total, tok_tmp, lengths);
+    if (bad) return bad;
+    if (n_rows == 0) return DNATOK_OK;
+    const BpePlan need = make_plan(nullptr, n_rows, max_len, total);
+    DNATOK_REQUIRE(scratch && scratch_bytes >= need.total_bytes, DNATOK_E_SCRATCH,
+                   "dnatok_bpe_encode: scratch holds %zu bytes, %zu needed", scratch_bytes, need.total_bytes);
+    DNATOK_REQUIRE(((uintptr_t)scratch & 255) == 0, DNATOK_E_INVALID, "dnatok_bpe_encode: scratch must be 256-byte aligned");
+    const BpePlan p = make_plan((uint8_t *)scratch, n_rows, max_len, total);
+    return bpe_encode_launch(t, bytes, offsets, n_rows, max_len, p, tok_tmp, lengths, (hipStream_t)stream);
+}
+
+// ---- the entry point that allocates nothing -------------------------------------------------
+//
+// The work buffer of dnatok_bpe_encode_static: one array in the code object's own device memory
+// (each GPU the library runs on holds its copy until the process ends).  Host code never uses the
+// array's name as an address: the address on the current device is asked for once per device.
+constexpr size_t kStaticScratchBytes = DNATOK_BPE_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) uint8_t scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<uint8_t *> g_static_scratch[kMaxDevices];
+
+static int static_scratch_ptr(uint8_t **out)
+{
+    int dev = 0;
+    DNATOK_HIP_TRY(hipGetDevice(&dev));
+    DNATOK_REQUIRE(dev >= 0 && dev < kMaxDevices, DNATOK_E_INVALID,
+                   "dnatok_bpe_encode_static: device index %d beyond %d", dev, kMaxDevices);
+    uint8_t *ptr = g_static_scratch[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        // (two threads asking at once get the same answer; the address of a device's copy is fixed)
+        void *sym = nullptr;
+        DNATOK_HIP_TRY(hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)));
+        DNATOK_REQUIRE(sym != nullptr, DNATOK_E_HIP, "dnatok_bpe_encode_static: no address for the work buffer");
+        ptr = (uint8_t *)sym;
+        g_static_scratch[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return DNATOK_OK;
+}
+
+extern "C" size_t dnatok_bpe_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int dnatok_bpe_encode_static(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets,
+                                        int64_t n_rows, int64_t max_len, int64_t total,
+                                        int32_t *tok_tmp, int32_t *lengths, void *stream)
+{
+    const int bad = bpe_encode_check("dnatok_bpe_encode_static", t, bytes, offsets, n_rows, max_len, total, tok_tmp,
+                                     lengths);
+    if (bad) return bad;
+    if (n_rows == 0) return DNATOK_OK;
+    // Fewer slabs for the whole-row fallback kernel (fewer rows redone at once) before giving up:
+    // the slabs are what grows with the longest row.
+    int64_t slabs = kLongGrid;
+    BpePlan need = make_plan(nullptr, n_rows, max_len, total, slabs);
+    while (need.total_bytes > kStaticScratchBytes && slabs > 1) {
+        slabs /= 2;
+        need = make_plan(nullptr, n_rows, max_len, total, slabs);
+    }
+    DNATOK_REQUIRE(need.total_bytes <= kStaticScratchBytes, DNATOK_E_TOO_LARGE,
+                   "dnatok_bpe_encode_static: this batch needs %zu bytes of work space, the built-in buffer holds "
+                   "%zu (use dnatok_bpe_encode with a caller-provided buffer)", need.total_bytes, kStaticScratchBytes);
+    uint8_t *base = nullptr;
+    const int rc = static_scratch_ptr(&base);
+    if (rc) return rc;
+    const BpePlan p = make_plan(base, n_rows, max_len, total, slabs);
+    return bpe_encode_launch(t, bytes, offsets, n_rows, max_len, p, tok_tmp, lengths, (hipStream_t)stream);
 }

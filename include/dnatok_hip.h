@@ -190,6 +190,24 @@ int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t
                       void *scratch, size_t scratch_bytes,
                       int32_t *tok_tmp, int32_t *lengths, void *stream);
 
+/* The same encode for callers that cannot allocate device memory or hand over a work buffer: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference (whose tokenize_batch grows torch tensors on demand,
+ * src/dnatok_bpe_kernel/dnatok_bpe.cu:956-1015).  The work space is an array of
+ * DNATOK_BPE_STATIC_SCRATCH_BYTES bytes inside the library's own device image, one copy per GPU,
+ * held until the process ends; the call allocates and frees nothing.  A batch that needs more
+ * (dnatok_bpe_scratch_bytes grows with the row count, the number of 1792-byte chunks of the rows
+ * above 2048 bytes, and the longest row) is refused with DNATOK_E_TOO_LARGE; rows that have to be
+ * redone whole are then redone fewer at a time before that happens.  All calls on one GPU share
+ * the array: two calls whose device work overlaps (different streams, or another thread) race;
+ * calls on one stream, and replays of a captured call, are fine.  Inputs, outputs and results as
+ * for dnatok_bpe_encode. */
+#define DNATOK_BPE_STATIC_SCRATCH_BYTES (32u << 20)
+size_t dnatok_bpe_static_scratch_bytes(void);
+int dnatok_bpe_encode_static(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets,
+                             int64_t n_rows, int64_t max_len, int64_t total,
+                             int32_t *tok_tmp, int32_t *lengths, void *stream);
+
 /* Test hook, no counterpart in the reference: sets the geometry the calls that follow (in this
  * process) cut rows longer than core + 2 * overlap bytes with: chunks of `core` bytes, extended by
  * `overlap` bytes on both sides, joined at seams inside the overlaps.  The shipped geometry is
