@@ -402,7 +402,7 @@ def fused_embed_extra():
     1 byte read and 1 KiB written per base; checked against the two-step torch form."""
     import torch
     from dnatok_amd import encoders
-        from tests.support import hf_tokenizers as hf, workloads as wl
+    from tests.support import hf_tokenizers as hf, workloads as wl
     vocab = hf.char_vocab()
     lut = np.zeros(256, dtype=np.int32)
     for ch in "ACGTN":
