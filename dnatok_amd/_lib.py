@@ -22,7 +22,7 @@ EXPORTS = [
     "dnatok_kmer_table_create", "dnatok_kmer_table_destroy", "dnatok_kmer_encode_padded",
     "dnatok_bpe_table_create", "dnatok_bpe_table_destroy", "dnatok_bpe_scratch_bytes",
     "dnatok_bpe_encode", "dnatok_bpe_static_scratch_bytes", "dnatok_bpe_encode_static",
-    "dnatok_bpe_set_chunk_geometry", "dnatok_pack_ragged", "dnatok_pad_rows",
+    "dnatok_bpe_set_chunk_geometry", "dnatok_pack_ragged", "dnatok_pad_rows", "dnatok_pad_rows_as",
     "dnatok_normalize_bounds", "dnatok_normalize_rows",
 ]
 
@@ -107,6 +107,8 @@ def lib() -> ctypes.CDLL:
                                      c_void_p, c_void_p, c_void_p]
     L.dnatok_pad_rows.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int32, c_int64,
                                   c_int64, c_void_p, c_void_p, c_void_p, c_void_p]
+    L.dnatok_pad_rows_as.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int32, c_int64, c_int64,
+                                     c_int64, c_int64, c_int, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]
     L.dnatok_normalize_bounds.argtypes = [c_void_p, c_int32, c_int64, c_int64, c_int64, POINTER(c_int64),
                                           POINTER(c_int64), POINTER(c_size_t)]
     L.dnatok_normalize_rows.argtypes = [c_void_p, c_int32, c_void_p, c_void_p, c_int64, c_int64, c_int64,

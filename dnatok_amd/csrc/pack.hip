@@ -112,17 +112,20 @@ __global__ __launch_bounds__(1024) void rows_max_kernel(const int32_t *__restric
     if (threadIdx.x == 0) *max_len = m;
 }
 
-// Padded layout: workgroup (row, tile) copies the row's tokens that fall into its tile of
-// columns and pads the rest of the tile up to the width: fill_to, or with fill_to = 0 the longest
-// row of the batch.  That one is found by every workgroup for itself while the batch is small
-// (FUSED_MAX: the lengths are a few KB in L2, and no launch, atomic or second pass over the rows
-// is needed), and read from max_len, where rows_max_kernel has put it, otherwise.
-template <bool FUSED_MAX>
+// Padded layout: workgroup (row, tile) writes one tile of columns of a row: the row's tokens that
+// fall into it and the pad id elsewhere, up to the width.  The width is fill_to, or with
+// fill_to = 0 the longest row of the batch, raised to min_width and rounded up to a multiple of
+// pad_multiple (never beyond t_cap).  The longest row is found by every workgroup for itself while
+// the batch is small (FUSED_MAX: the lengths are a few KB in L2, and no launch, atomic or second
+// pass over the rows is needed), and read from max_len, where rows_max_kernel has put it,
+// otherwise.  pad_left puts a row's tokens at the right end of the width.  OUT is the id type.
+template <bool FUSED_MAX, typename OUT>
 __global__ __launch_bounds__(256) void pad_rows_kernel(
     const int32_t *__restrict__ tok_tmp, const int64_t *__restrict__ in_offsets,
     const int32_t *__restrict__ lengths, int64_t n_rows, int64_t tiles_per_row,
-    const int32_t *__restrict__ remap, int32_t pad_id, int64_t t_cap, int64_t fill_to,
-    int32_t *__restrict__ ids, uint8_t *__restrict__ mask, int32_t *__restrict__ max_len)
+    const int32_t *__restrict__ remap, int32_t pad_id, int64_t t_cap, int64_t fill_to, int64_t min_width,
+    int64_t pad_multiple, int pad_left, OUT *__restrict__ ids, uint8_t *__restrict__ mask,
+    int32_t *__restrict__ max_len, int32_t *__restrict__ width_out)
 {
     __shared__ uint32_t red[4];
     int64_t width = fill_to;
@@ -135,6 +138,10 @@ __global__ __launch_bounds__(256) void pad_rows_kernel(
     } else if (fill_to == 0) {
         width = *max_len;
     }
+    if (width < min_width) width = min_width;
+    if (pad_multiple > 1 && width % pad_multiple) width += pad_multiple - width % pad_multiple;
+    if (width > t_cap) width = t_cap;
+    if (width_out && blockIdx.x == 0 && threadIdx.x == 0) *width_out = (int32_t)width;
     const int64_t n_tiles = n_rows * tiles_per_row;
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const int64_t row = tile / tiles_per_row;
@@ -142,20 +149,25 @@ __global__ __launch_bounds__(256) void pad_rows_kernel(
         int64_t len = lengths[row];
         if (len < 0) len = 0;
         if (len > t_cap) len = t_cap;
-        const int64_t end = len > width ? len : width;                // cells of the row that get written
+        // with padding on the left a row longer than the width keeps its first `width` tokens
+        const int64_t shift = pad_left ? (width > len ? width - len : 0) : 0;
+        const int64_t kept = pad_left && len > width ? width : len;
+        const int64_t end = pad_left ? width : (len > width ? len : width);    // cells of the row that get written
         if (c0 >= end) continue;
         const int64_t c1 = c0 + kPadTile < end ? c0 + kPadTile : end;
         const int32_t *src = tok_tmp + in_offsets[row];
-        int32_t *o = ids + row * t_cap;
+        OUT *o = ids + row * t_cap;
         uint8_t *m = mask ? mask + row * t_cap : nullptr;
         for (int64_t j = c0 + threadIdx.x; j < c1; j += 256) {
             int32_t v = pad_id;
-            if (j < len) {
-                v = src[j];
+            const int64_t k = j - shift;
+            const bool tok = k >= 0 && k < kept;
+            if (tok) {
+                v = src[k];
                 if (remap) v = remap[v];
             }
-            o[j] = v;
-            if (m) m[j] = j < len ? 1 : 0;
+            o[j] = (OUT)v;
+            if (m) m[j] = tok ? 1 : 0;
         }
     }
 }
@@ -191,6 +203,28 @@ extern "C" int dnatok_pack_ragged(const int32_t *tok_tmp, const int64_t *in_offs
     return DNATOK_OK;
 }
 
+template <typename OUT>
+static int launch_pad_rows(const int32_t *tok_tmp, const int64_t *in_offsets, const int32_t *lengths, int64_t n_rows,
+                           const int32_t *remap, int32_t pad_id, int64_t t_cap, int64_t fill_to, int64_t min_width,
+                           int64_t pad_multiple, int pad_left, OUT *ids, uint8_t *mask, int32_t *max_len,
+                           int32_t *width_out, hipStream_t s)
+{
+    const int64_t tiles_per_row = t_cap > 0 ? (t_cap + kPadTile - 1) / kPadTile : 1;
+    const int grid = capped_grid(n_rows * tiles_per_row);
+    if (n_rows <= kPadFuseRows) {
+        pad_rows_kernel<true, OUT><<<grid, 256, 0, s>>>(tok_tmp, in_offsets, lengths, n_rows, tiles_per_row, remap, pad_id,
+                                                        t_cap, fill_to, min_width, pad_multiple, pad_left, ids, mask,
+                                                        max_len, width_out);
+    } else {
+        if (max_len) rows_max_kernel<<<1, 1024, 0, s>>>(lengths, n_rows, t_cap, max_len);
+        pad_rows_kernel<false, OUT><<<grid, 256, 0, s>>>(tok_tmp, in_offsets, lengths, n_rows, tiles_per_row, remap,
+                                                         pad_id, t_cap, fill_to, min_width, pad_multiple, pad_left, ids,
+                                                         mask, max_len, width_out);
+    }
+    DNATOK_HIP_TRY(hipGetLastError());
+    return DNATOK_OK;
+}
+
 extern "C" int dnatok_pad_rows(const int32_t *tok_tmp, const int64_t *in_offsets,
                                const int32_t *lengths, int64_t n_rows, const int32_t *remap,
                                int32_t pad_id, int64_t t_cap, int64_t fill_to, int32_t *ids,
@@ -201,17 +235,32 @@ extern "C" int dnatok_pad_rows(const int32_t *tok_tmp, const int64_t *in_offsets
                    "dnatok_pad_rows: need 0 <= fill_to <= t_cap");
     DNATOK_REQUIRE(fill_to > 0 || max_len, DNATOK_E_INVALID, "dnatok_pad_rows: fill_to = 0 needs max_len");
     if (n_rows == 0) return DNATOK_OK;
+    return launch_pad_rows<int32_t>(tok_tmp, in_offsets, lengths, n_rows, remap, pad_id, t_cap, fill_to, 0, 1, 0, ids,
+                                    mask, max_len, nullptr, (hipStream_t)stream);
+}
+
+extern "C" int dnatok_pad_rows_as(const int32_t *tok_tmp, const int64_t *in_offsets, const int32_t *lengths,
+                                  int64_t n_rows, const int32_t *remap, int32_t pad_id, int64_t t_cap,
+                                  int64_t fill_to, int64_t min_width, int64_t pad_multiple, int pad_left,
+                                  void *ids, int32_t id_bytes, uint8_t *mask, int32_t *max_len,
+                                  int32_t *width_out, void *stream)
+{
+    DNATOK_REQUIRE(in_offsets && lengths && ids, DNATOK_E_INVALID, "dnatok_pad_rows_as: null argument");
+    DNATOK_REQUIRE(n_rows >= 0 && t_cap >= 0 && fill_to >= 0 && fill_to <= t_cap && min_width >= 0 && min_width <= t_cap &&
+                       pad_multiple >= 0,
+                   DNATOK_E_INVALID, "dnatok_pad_rows_as: need 0 <= fill_to, min_width <= t_cap and pad_multiple >= 0");
+    DNATOK_REQUIRE(fill_to > 0 || max_len, DNATOK_E_INVALID, "dnatok_pad_rows_as: fill_to = 0 needs max_len");
+    DNATOK_REQUIRE(id_bytes == 1 || id_bytes == 2 || id_bytes == 4 || id_bytes == 8, DNATOK_E_INVALID,
+                   "dnatok_pad_rows_as: id_bytes must be 1, 2, 4 or 8");
+    if (n_rows == 0) return DNATOK_OK;
     hipStream_t s = (hipStream_t)stream;
-    const int64_t tiles_per_row = t_cap > 0 ? (t_cap + kPadTile - 1) / kPadTile : 1;
-    const int grid = capped_grid(n_rows * tiles_per_row);
-    if (n_rows <= kPadFuseRows) {
-        pad_rows_kernel<true><<<grid, 256, 0, s>>>(tok_tmp, in_offsets, lengths, n_rows, tiles_per_row, remap, pad_id,
-                                                   t_cap, fill_to, ids, mask, max_len);
-    } else {
-        if (max_len) rows_max_kernel<<<1, 1024, 0, s>>>(lengths, n_rows, t_cap, max_len);
-        pad_rows_kernel<false><<<grid, 256, 0, s>>>(tok_tmp, in_offsets, lengths, n_rows, tiles_per_row, remap, pad_id,
-                                                    t_cap, fill_to, ids, mask, max_len);
+#define GO(T) launch_pad_rows<T>(tok_tmp, in_offsets, lengths, n_rows, remap, pad_id, t_cap, fill_to, min_width, pad_multiple, \
+                                 pad_left ? 1 : 0, (T *)ids, mask, max_len, width_out, s)
+    switch (id_bytes) {
+        case 1: return GO(uint8_t);
+        case 2: return GO(int16_t);
+        case 4: return GO(int32_t);
+        default: return GO(int64_t);
     }
-    DNATOK_HIP_TRY(hipGetLastError());
-    return DNATOK_OK;
+#undef GO
 }

@@ -350,6 +350,18 @@ class DNATok:
         want = self._tokenize_batch_cpu(seqs)
         if got.shape != want.shape or not torch.equal(got.cpu(), want):
             raise RuntimeError("DNATok.discover(): table encode disagrees with the tokenizer")
+        if k > 1:
+            # A trailing remainder of fewer than k characters is spelled with the single-character
+            # table; a tokenizer that does something else with it (drops it, one <unk> for all of it)
+            # gets such rows back from the tokenizer itself.
+            self._kmer_tail_ok = True
+            tails = ["".join(rng.choice(list(_DNA_UPPER), size=m)) for m in (8 * k + 1, 3 * k + k - 1, 2 * k + 1)]
+            got = self.encode_batch_to_ids(tails)
+            want = self._tokenize_batch_cpu(tails)
+            if got.shape != want.shape or not torch.equal(got.cpu(), want):
+                self._kmer_tail_ok = False
+                self.log.info("trailing characters are not tokenized one by one; rows whose length is "
+                              "no multiple of %d go to the tokenizer", k)
 
     # ------------------------------------------------------------------- encode
 
@@ -358,21 +370,46 @@ class DNATok:
             raise RuntimeError("DNATok.discover() must be called before encoding.")
 
     def encode_batch_device(self, seqs: Sequence[str], device="cuda") -> Tuple[torch.Tensor, torch.Tensor]:
-        """Device-resident encode: (ids int32 [B, T], mask uint8 [B, T]) on the GPU, padded on
-        ``padding_side`` (char) or on the right (k-mer, BPE) to the longest row."""
+        """Device-resident encode: (ids int32 [B, T], mask uint8 [B, T]) on the GPU, every row
+        padded on ``padding_side`` to the longest row, or to ``token_len`` when that is larger
+        (reference: _pad_id_list, src/dna_tokenizer.py:1878-1894)."""
+        return self._encode_rows_device(seqs, device, dtype=torch.int32,
+                                        min_width=int(self.token_len or 0), pad_multiple=1)
+
+    def _encode_rows_device(self, seqs: Sequence[str], device, *, dtype: torch.dtype, min_width: int,
+                            pad_multiple: int) -> Tuple[torch.Tensor, torch.Tensor]:
         self._require_ready()
         if not seqs:
             raise ValueError("No sequences provided for encoding.")
+        left = self.padding_side == "left"
         if self.bpe_backend is not None:
-            ids, mask = self.bpe_backend.encode_batch(list(seqs), device=device)
-            return ids.to(torch.int32), mask
+            tok, offsets, lengths, t_cap = self.bpe_backend.tokens_device(list(seqs), device=device)
+            return self._pad_bpe_runs(tok, offsets, lengths, t_cap, dtype=dtype, min_width=min_width,
+                                      pad_multiple=pad_multiple)
         data, offsets, lens = encoders.bytes_from_strings(seqs, device)
         if self._kmer_enc is not None:
-            return self._encode_kmer_device(seqs, data, offsets, lens)
-        width = int(lens.max())
-        if self.token_len is not None and self.token_len > width:
-            width = int(self.token_len)
-        return self._char_enc.encode_padded(data, offsets, width, pad_left=(self.padding_side == "left"))
+            return self._encode_kmer_device(seqs, data, offsets, lens, dtype=dtype, min_width=min_width,
+                                            pad_multiple=pad_multiple)
+        width = max(int(lens.max()), int(min_width))
+        if pad_multiple > 1 and width % pad_multiple:
+            width += pad_multiple - width % pad_multiple
+        return self._char_enc.encode_padded(data, offsets, width, pad_left=left, dtype=dtype)
+
+    def _pad_bpe_runs(self, tok, offsets, lengths, t_cap: int, *, dtype, min_width: int, pad_multiple: int):
+        """The engine's token runs -> padded rows: remap, padding side, least width, multiple and
+        id type in one launch; one host read for the shape (and the smallest length: a negative
+        one is a failed row)."""
+        be = self.bpe_backend
+        cap = max(int(t_cap), int(min_width), 1)
+        if pad_multiple > 1 and cap % pad_multiple:
+            cap += pad_multiple - cap % pad_multiple
+        ids, mask, stats = encoders.pad_rows_as(tok, offsets, lengths, int(be.pad_id), cap, min_width=min_width,
+                                                pad_multiple=pad_multiple, pad_left=(self.padding_side == "left"),
+                                                dtype=dtype, remap=be._remap_on(tok.device))
+        _, width, shortest = torch.cat((stats, lengths.min()[None])).tolist()
+        if shortest < 0:
+            raise RuntimeError("BPE engine reported a failed row (negative length)")
+        return ids[:, :width], mask[:, :width]
 
     def encode_fasta_device(self, source, device="cuda"):
         """FASTA file (path) or FASTA text (bytes) -> (ids int32 [B, T], mask uint8 [B, T], names),
@@ -386,6 +423,7 @@ class DNATok:
             raise ValueError("No sequences provided for encoding.")
         lens = (off_h[1:] - off_h[:-1]).numpy()
         data, offsets = host.to(device, non_blocking=True), off_h.to(device)
+        min_width = int(self.token_len or 0)
 
         class _Rows:                                     # strings of single rows, made only when asked for
             def __getitem__(self, i):
@@ -396,60 +434,90 @@ class DNATok:
 
         rows = _Rows()
         if self.bpe_backend is not None:
-            if getattr(self.bpe_backend, "_normalize", None) is not None:
-                ids, mask = self.bpe_backend.encode_batch([rows[i] for i in range(len(names))], device=device)
-                return ids.to(torch.int32), mask, names
-            ids, mask, _, longest = self.bpe_backend.encode_device(data, offsets, int(lens.max()))
-            width = max(int(longest.item()), 1)
-            return ids[:, :width], mask[:, :width], names
-        if self._kmer_enc is not None:
-            ids, mask = self._encode_kmer_device(rows, data, offsets, lens)
+            be = self.bpe_backend
+            if getattr(be, "_normalize", None) is not None or getattr(be, "_input_guard", None) is not None:
+                ids, mask = self.encode_batch_device([rows[i] for i in range(len(names))], device=device)
+                return ids, mask, names
+            t_cap = max(int(lens.max()), 1)
+            tok, lengths = be._dnatok.tokenize_device(data, offsets, t_cap)
+            ids, mask = self._pad_bpe_runs(tok, offsets, lengths, t_cap, dtype=torch.int32, min_width=min_width,
+                                           pad_multiple=1)
             return ids, mask, names
-        width = int(lens.max())
-        if self.token_len is not None and self.token_len > width:
-            width = int(self.token_len)
+        if self._kmer_enc is not None:
+            ids, mask = self._encode_kmer_device(rows, data, offsets, lens, dtype=torch.int32, min_width=min_width,
+                                                 pad_multiple=1)
+            return ids, mask, names
+        width = max(int(lens.max()), min_width)
         ids, mask = self._char_enc.encode_padded(data, offsets, width, pad_left=(self.padding_side == "left"))
         return ids, mask, names
 
-    def _encode_kmer_device(self, seqs, data, offsets, lens) -> Tuple[torch.Tensor, torch.Tensor]:
-        from ._lib import lib  # noqa: F401  (fail early if the library is missing)
+    def _encode_kmer_device(self, seqs, data, offsets, lens, *, dtype=torch.int32, min_width: int = 0,
+                            pad_multiple: int = 1) -> Tuple[torch.Tensor, torch.Tensor]:
+        """k-mer rows on the device.  Right padding to the longest row with int32 ids comes straight
+        out of the encoder; any other layout (left padding, a least width, a multiple, a narrower id
+        type) is one more launch of the packer over the encoder's rows.  Rows the tables cannot
+        express (a window without tokens of its own, more tokens than the row's room, a foreign byte
+        when those are not accepted, a row shorter than one window, which the reference hands to the
+        tokenizer as well, src/dna_tokenizer.py:1389-1398) get the tokenizer's own answer."""
         k = int(self.kmer_k)
-        # row stride of the output buffers: a multiple of 128 cells keeps every row of ids and of
-        # the mask on cache-line boundaries, which the store path of the kernel is built around
-        t_cap = int(lens.max()) + 4
+        left = self.padding_side == "left"
+        n = len(lens)
+        longest_in = int(lens.max())
+        # room per row: every window may expand to the longest expansion of the table
+        grow = max(int(self._kmer_tables.exp_len.max(initial=0)), 1)
+        t_cap = (longest_in // k) * grow + k
+        # a stride of whole 128-byte lines keeps every row of ids and of the mask on line boundaries
         t_cap += (-t_cap) % 128
+        plain = (not left) and dtype == torch.int32 and pad_multiple <= 1
         # the width of the previous batch is a good guess of this one's in a stream of batches
         ids, mask, lengths, status, longest = self._kmer_enc.encode_padded(
-            data, offsets, t_cap, fill_to=0, width_guess=getattr(self, "_kmer_width_guess", 0))
-        width = int(longest.item())                      # one scalar: the output shape
-        self._kmer_width_guess = width
-        if self.token_len is not None and self.token_len > width:
-            extra = int(self.token_len)
-            ids, mask, lengths, status, longest = self._kmer_enc.encode_padded(
-                data, offsets, max(t_cap, extra + (-extra) % 128), fill_to=extra)
-            width = extra
+            data, offsets, t_cap, fill_to=0, width_guess=getattr(self, "_kmer_width_guess", 0) if plain else 0)
+        if plain:
+            width = int(longest.item())                  # one scalar: the output shape
+            self._kmer_width_guess = width
+            plain = width >= min_width
+        if not plain:
+            cap = max(t_cap, int(min_width))
+            if pad_multiple > 1 and cap % pad_multiple:
+                cap += pad_multiple - cap % pad_multiple
+            row_at = torch.arange(n, dtype=torch.int64, device=ids.device) * t_cap
+            ids, mask, stats = encoders.pad_rows_as(ids.view(-1), row_at, lengths, int(self.id_pad), cap,
+                                                    min_width=min_width, pad_multiple=pad_multiple, pad_left=left,
+                                                    dtype=dtype)
+            width = int(stats[1].item())
         ids, mask = ids[:, :width], mask[:, :width]
         bad = status.cpu().numpy()
-        need = (bad & 2) != 0
+        need = (bad & (2 | 4)) != 0
         if self.require_valid_chars or not self.handle_invalid_chars:
             need |= (bad & 1) != 0
+        need |= np.asarray(lens) < k
+        if not getattr(self, "_kmer_tail_ok", True):
+            need |= (np.asarray(lens) % k) != 0
         if need.any() and not self.allow_incomplete_kmer_lut:
-            # rows the tables cannot express: the tokenizer's own answer, spliced in
             rows = np.nonzero(need)[0].tolist()
             fixed = self._tok_ids([seqs[i] for i in rows])
             new_w = max(width, max(len(r) for r in fixed))
+            if pad_multiple > 1 and new_w % pad_multiple:
+                new_w += pad_multiple - new_w % pad_multiple
             if new_w > width:
-                pad_i = torch.full((ids.shape[0], new_w - width), int(self.id_pad), dtype=ids.dtype, device=ids.device)
-                ids = torch.cat([ids, pad_i], dim=1)
-                mask = torch.cat([mask, torch.zeros_like(pad_i, dtype=torch.uint8)], dim=1)
+                extra = new_w - width
+                pad_i = torch.full((n, extra), int(self.id_pad), dtype=ids.dtype, device=ids.device)
+                pad_m = torch.zeros((n, extra), dtype=torch.uint8, device=ids.device)
+                ids = torch.cat([pad_i, ids], dim=1) if left else torch.cat([ids, pad_i], dim=1)
+                mask = torch.cat([pad_m, mask], dim=1) if left else torch.cat([mask, pad_m], dim=1)
             else:
                 ids, mask = ids.clone(), mask.clone()
             for i, r in zip(rows, fixed):
                 ids[i] = int(self.id_pad)
                 mask[i] = 0
                 if r:
-                    ids[i, :len(r)] = torch.as_tensor(r, dtype=ids.dtype, device=ids.device)
-                    mask[i, :len(r)] = 1
+                    cur = torch.as_tensor(r, dtype=ids.dtype, device=ids.device)
+                    if left:
+                        ids[i, new_w - len(r):] = cur
+                        mask[i, new_w - len(r):] = 1
+                    else:
+                        ids[i, :len(r)] = cur
+                        mask[i, :len(r)] = 1
         return ids, mask
 
     def encode_batch_to_ids(self, seqs: List[str]) -> torch.Tensor:
@@ -486,24 +554,10 @@ class DNATok:
                 target += pad_multiple - target % pad_multiple
             return self._char_enc.encode_padded(data, offsets, target, pad_left=(self.padding_side == "left"),
                                                 dtype=narrow)
-        old = self.token_len
-        self.token_len = None
-        try:
-            ids, mask = self.encode_batch_device(seqs)
-        finally:
-            self.token_len = old
-        target = ids.shape[1]
-        if pad_to_max:
-            target = max(target, int(max_tokens))
-        if pad_multiple > 1 and target % pad_multiple:
-            target += pad_multiple - target % pad_multiple
-        if target > ids.shape[1]:
-            extra = target - ids.shape[1]
-            pad_i = torch.full((ids.shape[0], extra), int(self.id_pad), dtype=ids.dtype, device=ids.device)
-            pad_m = torch.zeros((ids.shape[0], extra), dtype=torch.uint8, device=ids.device)
-            ids = torch.cat([ids, pad_i], dim=1)
-            mask = torch.cat([mask, pad_m], dim=1)
-        return ids.to(narrow), mask
+        # k-mer and BPE: side, width and id type come out of the packer's launch
+        return self._encode_rows_device(seqs, "cuda", dtype=narrow,
+                                        min_width=int(max_tokens) if pad_to_max else 0,
+                                        pad_multiple=int(pad_multiple))
 
     # ------------------------------------------------------------------ bytes path
 
@@ -579,7 +633,7 @@ class DNATok:
         if self._kmer_enc is not None:
             t_cap = t + 4 + (-(t + 4)) % 128
             ids, mask, lengths, status, longest = self._kmer_enc.encode_padded(data, offsets, t_cap, fill_to=0)
-            if int(status.abs().max().item()) & 3:
+            if bool((status & 7).any().item()):
                 raise RuntimeError("k-mer bytes path: a row needs the tokenizer's own answer")
             return ids[:, :int(longest.item())].to(torch.int64)
         ids, _ = self._char_enc.encode_packed(data, row_len=t)

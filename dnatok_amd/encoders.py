@@ -417,3 +417,25 @@ def pad_rows(tok_tmp: torch.Tensor, in_offsets: torch.Tensor, lengths: torch.Ten
                                           _ptr(ids), _ptr(mask), _ptr(max_len), _stream()),
                "dnatok_pad_rows")
     return ids, mask, max_len
+
+
+def pad_rows_as(tok_tmp: torch.Tensor, in_offsets: torch.Tensor, lengths: torch.Tensor, pad_id: int,
+                t_cap: int, *, fill_to: int = 0, min_width: int = 0, pad_multiple: int = 1,
+                pad_left: bool = False, dtype: torch.dtype = torch.int32,
+                remap: Optional[torch.Tensor] = None, want_mask: bool = True):
+    """The padded layout with the choices of DNATok's padding: side, a least width (``token_len``),
+    a multiple, the id type.  Returns (ids[B, t_cap] of ``dtype``, mask, stats int32[2] =
+    {longest row, width}); view ``ids[:, :width]`` (C ABI: dnatok_pad_rows_as)."""
+    if dtype not in (torch.uint8, torch.int16, torch.int32, torch.int64):
+        raise ValueError("dtype must be uint8, int16, int32 or int64")
+    n_rows = lengths.numel()
+    dev = tok_tmp.device
+    ids = torch.empty((n_rows, t_cap), dtype=dtype, device=dev)
+    mask = torch.empty((n_rows, t_cap), dtype=torch.uint8, device=dev) if want_mask else None
+    stats = torch.zeros(2, dtype=torch.int32, device=dev)
+    _lib.check(_lib.lib().dnatok_pad_rows_as(
+        _ptr(tok_tmp), _ptr(in_offsets), _ptr(lengths), n_rows, _ptr(remap), int(pad_id), int(t_cap),
+        int(fill_to), min(int(min_width), int(t_cap)), int(pad_multiple), int(bool(pad_left)), _ptr(ids),
+        ids.element_size(), _ptr(mask), ctypes.c_void_p(stats.data_ptr()),
+        ctypes.c_void_p(stats.data_ptr() + 4), _stream()), "dnatok_pad_rows_as")
+    return ids, mask, stats

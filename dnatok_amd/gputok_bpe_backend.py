@@ -389,8 +389,11 @@ class GPUTokBPEBackend:
 
     # ------------------------------------------------------------------- reference API
 
-    def encode_batch(self, seqs: List[str], *, device: object = "cuda"
-                     ) -> Tuple[torch.Tensor, torch.Tensor]:
+    def tokens_device(self, seqs: List[str], *, device: object = "cuda"):
+        """Strings -> the engine's token runs on the device: ``(tok_tmp int32, offsets int64 [B+1],
+        lengths int32 [B], t_cap)`` with row b's kernel-space tokens at
+        ``tok_tmp[offsets[b] : offsets[b] + lengths[b]]`` and t_cap a host-known bound of the row
+        lengths.  What ``encode_batch`` pads; DNATok pads the same runs its own way."""
         if not seqs:
             raise ValueError("No sequences provided.")
         dev = torch.device(device) if not isinstance(device, torch.device) else device
@@ -415,9 +418,16 @@ class GPUTokBPEBackend:
             norm = [self._normalize(s) for s in seqs]
             data, offsets, lens = encoders.bytes_from_strings(norm, dev, encoding="utf-8")
             t_cap = int(lens.max())
-        b = len(seqs)
         t_cap = max(t_cap, 1)
-        ids32, mask, lengths, longest = self.encode_device(data, offsets, t_cap)
+        tok, lengths = self._dnatok.tokenize_device(data, offsets, t_cap)
+        return tok, offsets, lengths, t_cap
+
+    def encode_batch(self, seqs: List[str], *, device: object = "cuda"
+                     ) -> Tuple[torch.Tensor, torch.Tensor]:
+        tok, offsets, lengths, t_cap = self.tokens_device(seqs, device=device)
+        dev, b = tok.device, len(seqs)
+        ids32, mask, longest = encoders.pad_rows(tok, offsets, lengths, self.pad_id, t_cap, fill_to=0,
+                                                 remap=self._remap_on(dev))
         # the one host sync: the output shape, and with it the smallest length (negative = failed row)
         width, shortest = torch.stack((longest[0], lengths.min())).tolist()
         if shortest < 0:

@@ -236,6 +236,21 @@ int dnatok_pad_rows(const int32_t *tok_tmp, const int64_t *in_offsets, const int
                     int64_t n_rows, const int32_t *remap, int32_t pad_id, int64_t t_cap,
                     int64_t fill_to, int32_t *ids, uint8_t *mask, int32_t *max_len, void *stream);
 
+/* The same with everything DNATok.encode_batch_to_ids / encode_batch_with_padding do to token rows
+ * after the encode (src/dna_tokenizer.py:1878-1894 _pad_id_list: padding side and token_len;
+ * 2150-2236: pad_multiple and the narrowest id type), in the one launch:
+ *   width     = fill_to, or with fill_to = 0 the longest row; then at least min_width, rounded up
+ *               to a multiple of pad_multiple (0 or 1: none), at most t_cap; written to width_out
+ *               (int32[1], NULL allowed), while max_len still receives the longest row;
+ *   pad_left  = 1: a row's tokens end at column width - 1 (a row longer than the width keeps its
+ *               first `width` tokens), 0: they start at column 0;
+ *   ids       = [n_rows, t_cap] of id_bytes-wide integers (1: uint8, 2: int16, 4: int32, 8: int64). */
+int dnatok_pad_rows_as(const int32_t *tok_tmp, const int64_t *in_offsets, const int32_t *lengths,
+                       int64_t n_rows, const int32_t *remap, int32_t pad_id, int64_t t_cap,
+                       int64_t fill_to, int64_t min_width, int64_t pad_multiple, int pad_left,
+                       void *ids, int32_t id_bytes, uint8_t *mask, int32_t *max_len,
+                       int32_t *width_out, void *stream);
+
 /* ---------------------------------------------------------------------------------------
  * Tokenizer normalizer on the device: the steps GPUTokBPEBackend compiles from a
  * tokenizer.json "normalizer" and applies string by string on the host before the kernel

@@ -208,17 +208,28 @@ def kmer_encode_batch(t: KmerTables, data: np.ndarray, offsets: np.ndarray, t_ca
     return ids, mask, lengths
 
 
-def pad_rows(rows: Sequence[np.ndarray], pad_id: int, t_out: int | None = None
-             ) -> Tuple[np.ndarray, np.ndarray]:
-    """Right-pad to the longest row: ids int32 [B,T], mask uint8 [B,T]
-    (mask[b,j] = j < len_b, reference: src/gputok_bpe_backend.py:593-600)."""
+def pad_rows(rows: Sequence[np.ndarray], pad_id: int, t_out: int | None = None, *, pad_left: bool = False,
+             min_width: int = 0, pad_multiple: int = 1, dtype=np.int32) -> Tuple[np.ndarray, np.ndarray]:
+    """Pad to the longest row (or t_out): ids [B,T], mask uint8 [B,T].  Right padding:
+    mask[b,j] = j < len_b (reference: src/gputok_bpe_backend.py:593-600).  pad_left, min_width
+    (token_len) and pad_multiple as DNATok pads rows: a row's tokens end at the last column, the
+    width is at least min_width and a multiple of pad_multiple (src/dna_tokenizer.py:1878-1894
+    _pad_id_list, 2150-2236 encode_batch_with_padding); a row longer than the width keeps its
+    first tokens."""
     t = max((r.size for r in rows), default=0) if t_out is None else t_out
-    ids = np.full((len(rows), t), pad_id, dtype=np.int32)
+    t = max(t, int(min_width))
+    if pad_multiple > 1 and t % pad_multiple:
+        t += pad_multiple - t % pad_multiple
+    ids = np.full((len(rows), t), pad_id, dtype=dtype)
     mask = np.zeros((len(rows), t), dtype=np.uint8)
     for b, r in enumerate(rows):
         n = min(t, r.size)
-        ids[b, :n] = r[:n]
-        mask[b, :n] = 1
+        if pad_left:
+            ids[b, t - n:] = r[:n]
+            mask[b, t - n:] = 1
+        else:
+            ids[b, :n] = r[:n]
+            mask[b, :n] = 1
     return ids, mask
 
 

@@ -522,6 +522,73 @@ def test_dnatok_routes_bpe_tokenizers_to_the_backend():
         assert got[i, :len(r)].tolist() == r and bool((got[i, len(r):] == 3).all())
 
 
+def _bpe_wrapped(side):
+    tk = hf.load_bpe_tokenizer("4096")
+
+    class Wrapped:                       # the attributes DNATok reads from an HF tokenizer
+        pad_token_id, unk_token_id, padding_side = 3, 0, side
+        backend_tokenizer = tk
+
+        def __call__(self, texts, add_special_tokens=False, **kw):
+            return {"input_ids": [e.ids for e in tk.encode_batch(list(texts), add_special_tokens=False)]}
+
+        def get_vocab(self):
+            return tk.get_vocab()
+
+    return Wrapped()
+
+
+@pytest.mark.parametrize("side", ["left", "right"])
+@pytest.mark.parametrize("family", ["kmer", "bpe"])
+def test_ragged_rows_follow_padding_side_and_token_len(family, side):
+    """Ragged batches through a k-mer and a BPE tokenizer: every row padded on the tokenizer's side to
+    the longest row or to token_len, as the reference pads token rows (_pad_id_list,
+    src/dna_tokenizer.py:1878-1894; BPE rows 2063-2078).  Expected: the tokenizer's own rows, padded in
+    plain Python."""
+    if family == "kmer":
+        tok = MockKmerTokenizer(k=4)
+        tok.padding_side = side
+        alphabet = "ACGTN"
+    else:
+        tok, alphabet = _bpe_wrapped(side), "ACGT"
+    h = DNATok(RecordingEmbedder(tok, vocab=8192), padding_side=side)
+    h.discover()
+    assert h.padding_side == side
+    assert (h.kmer_k == 4) if family == "kmer" else (h.bpe_backend is not None)
+    random.seed(3)
+    seqs = ["".join(random.choice(alphabet) for _ in range(n)) for n in (40, 7, 400, 1, 123, 4, 399, 64)]
+    rows = h._tok_ids(seqs)
+    for token_len in (None, max(len(r) for r in rows) + 9, 3):
+        h.token_len = token_len
+        got = h.encode_batch_to_ids(seqs)
+        want = h._tokenize_batch_cpu(seqs)
+        assert got.shape == want.shape and torch.equal(got, want), (family, side, token_len)
+        ids, mask = h.encode_batch_device(seqs)
+        assert ids.dtype == torch.int32 and torch.equal(ids.cpu().long(), want)
+        lens = torch.tensor([len(r) for r in rows])
+        assert torch.equal(mask.cpu().sum(1).long(), lens)
+        col = torch.arange(want.shape[1])[None, :]
+        inside = (col >= want.shape[1] - lens[:, None]) if side == "left" else (col < lens[:, None])
+        assert torch.equal(mask.cpu().bool(), inside)
+    h.token_len = None
+    # encode_batch_with_padding: cut to max_tokens, a multiple of pad_multiple, the narrowest id type
+    k = 4 if family == "kmer" else 1
+    for max_tokens, to_max, mult in ((50, False, 16), (50, True, 8), (500, True, 1)):
+        ids, mask = h.encode_batch_with_padding(seqs, max_tokens, pad_to_max=to_max, pad_multiple=mult)
+        cut = h._tok_ids([q[:max_tokens * k] for q in seqs])
+        width = max(len(r) for r in cut)
+        if to_max:
+            width = max(width, max_tokens)
+        if mult > 1 and width % mult:
+            width += mult - width % mult
+        assert tuple(ids.shape) == (len(seqs), width) and ids.dtype in (torch.uint8, torch.int16)
+        for i, r in enumerate(cut):
+            row, m = ids[i].cpu().long(), mask[i].cpu()
+            sl = slice(width - len(r), width) if side == "left" else slice(0, len(r))
+            assert row[sl].tolist() == r and int(m.sum()) == len(r) and bool(m[sl].all())
+            assert int((row != h.id_pad).sum()) <= len(r)
+
+
 def _write_fasta(path, seqs, width=70):
     with open(path, "w") as fh:
         for i, s in enumerate(seqs):

@@ -684,3 +684,46 @@ def test_pad_rows_matches_reference_semantics():
         eids, emask = O.pad_rows(erows, 3, width)
         np.testing.assert_array_equal(ids[:, :width].cpu().numpy(), eids)
         np.testing.assert_array_equal(mask[:, :width].cpu().numpy(), emask)
+
+
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.int16, torch.int32, torch.int64])
+@pytest.mark.parametrize("pad_left", [False, True])
+def test_pad_rows_side_width_multiple_and_id_type(dtype, pad_left):
+    """dnatok_pad_rows_as against the oracle's padding rules (pinned by hand-written cases): ragged token
+    runs, empty rows, a least width above and below the longest row, multiples, a fixed width that cuts
+    rows, and both the small-batch and the large-batch form of the kernel."""
+    say(f"pad_rows_as {dtype} left={pad_left}")
+    rng = np.random.default_rng(17)
+    hi = 200 if dtype == torch.uint8 else 30000
+    np_dtype = {torch.uint8: np.uint8, torch.int16: np.int16, torch.int32: np.int32, torch.int64: np.int64}[dtype]
+    for n_rows in (1, 37, 2500):
+        lens = rng.integers(0, 300, size=n_rows)
+        lens[0] = 0
+        rows = [rng.integers(0, hi, size=n, dtype=np.int32) for n in lens]
+        room = lens + rng.integers(0, 5, size=n_rows)               # runs lie apart in the source buffer
+        off_h = np.concatenate([[0], np.cumsum(room)]).astype(np.int64)
+        flat = np.full(int(off_h[-1]) + 1, -1, dtype=np.int32)
+        for r, o in zip(rows, off_h):
+            flat[o:o + r.size] = r
+        remap_h = rng.permutation(hi).astype(np.int32)
+        tok, off = torch.from_numpy(flat).to(DEV), torch.from_numpy(off_h).to(DEV)
+        lengths = torch.from_numpy(lens.astype(np.int32)).to(DEV)
+        remap = torch.from_numpy(remap_h).to(DEV)
+        longest = int(lens.max())
+        for fill_to, min_width, mult in ((0, 0, 1), (0, longest + 13, 1), (0, 5, 16), (0, 0, 64), (longest // 2 + 1, 0, 1),
+                                         (longest + 7, 0, 8)):
+            t_cap = max(longest, fill_to, min_width) + 70
+            ids, mask, stats = encoders.pad_rows_as(tok, off, lengths, 3, t_cap, fill_to=fill_to, min_width=min_width,
+                                                    pad_multiple=mult, pad_left=pad_left, dtype=dtype, remap=remap)
+            torch.cuda.synchronize()
+            got_longest, width = stats.cpu().tolist()
+            assert got_longest == longest
+            want_rows = [remap_h[r] for r in rows]
+            e_ids, e_mask = O.pad_rows(want_rows, 3, fill_to if fill_to else None, pad_left=pad_left, min_width=min_width,
+                                       pad_multiple=mult, dtype=np_dtype)
+            if fill_to and not pad_left:
+                # right padding writes a row longer than the fixed width in full; compare the width's columns
+                e_ids, e_mask = e_ids[:, :width], e_mask[:, :width]
+            assert width == e_ids.shape[1], (n_rows, fill_to, min_width, mult, width, e_ids.shape)
+            np.testing.assert_array_equal(ids[:, :width].cpu().numpy(), e_ids)
+            np.testing.assert_array_equal(mask[:, :width].cpu().numpy(), e_mask)

@@ -132,6 +132,27 @@ def test_kmer_encode_batch_equals_rows_plus_padding():
     np.testing.assert_array_equal(mask[3], [1, 1, 0, 0])
 
 
+def test_pad_rows_sides_width_and_multiple_by_hand():
+    """The padding rules of DNATok (side, token_len as a least width, a multiple) on cases written
+    out by hand."""
+    rows = [np.array([5, 6, 7], np.int32), np.array([], np.int32), np.array([9], np.int32)]
+    ids, mask = O.pad_rows(rows, 0)
+    np.testing.assert_array_equal(ids, [[5, 6, 7], [0, 0, 0], [9, 0, 0]])
+    np.testing.assert_array_equal(mask, [[1, 1, 1], [0, 0, 0], [1, 0, 0]])
+    ids, mask = O.pad_rows(rows, 0, pad_left=True)
+    np.testing.assert_array_equal(ids, [[5, 6, 7], [0, 0, 0], [0, 0, 9]])
+    np.testing.assert_array_equal(mask, [[1, 1, 1], [0, 0, 0], [0, 0, 1]])
+    ids, mask = O.pad_rows(rows, 2, pad_left=True, min_width=5)
+    np.testing.assert_array_equal(ids, [[2, 2, 5, 6, 7], [2, 2, 2, 2, 2], [2, 2, 2, 2, 9]])
+    np.testing.assert_array_equal(mask, [[0, 0, 1, 1, 1], [0, 0, 0, 0, 0], [0, 0, 0, 0, 1]])
+    ids, mask = O.pad_rows(rows, 1, min_width=2, pad_multiple=4, dtype=np.uint8)
+    assert ids.dtype == np.uint8
+    np.testing.assert_array_equal(ids, [[5, 6, 7, 1], [1, 1, 1, 1], [9, 1, 1, 1]])
+    ids, mask = O.pad_rows(rows, 1, 2, pad_left=True)             # a fixed width below the longest row
+    np.testing.assert_array_equal(ids, [[5, 6], [1, 1], [1, 9]])
+    np.testing.assert_array_equal(mask, [[1, 1], [0, 0], [0, 1]])
+
+
 # ------------------------------------------------------------------- BPE
 
 @pytest.mark.parametrize("which,name,maker", [
