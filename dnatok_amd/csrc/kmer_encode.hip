@@ -28,7 +28,8 @@
 
 #include <limits.h>
 #include <string.h>
-#include <atomic>
+#include <mutex>
+#include <unordered_map>
 #include <vector>
 
 struct dnatok_kmer_table {
@@ -42,17 +43,20 @@ struct dnatok_kmer_table {
     int32_t *lut4;           // [4^k]  id of an ACGT-only window, or -1
     int2 *entry;             // [5^k]  {id, 0} | {-len, offset into flat} | {INT_MIN, 0} = nothing known
     int32_t *flat;           // expansion lists
-    // Running maxima of pad-to-longest calls.  A call takes the next of kMaxSlots slots (calls in
-    // flight on different streams use different slots).  A slot is two 64-bit words: the running
-    // maximum, tagged in its upper half with the slot's generation, and the generation itself,
-    // which the padding pass of a call bumps when it is done with the maximum.  A maximum of a
-    // later call is therefore larger than anything an earlier call left behind, and the slot
-    // never has to be cleared (a launch saved per call; replays of a captured call stay exact).
+    // Running maxima of pad-to-longest calls.  Every stream that encodes with this table gets a
+    // slot of its own (calls on one stream are ordered, calls on different streams may overlap and
+    // must not share one); a stream beyond the kMaxSlots-th is served without a slot, by a clearing
+    // launch on the caller's max_len.  A slot is two 64-bit words: the running maximum, tagged in
+    // its upper half with the slot's generation, and the generation itself, which the padding pass
+    // of a call bumps when it is done with the maximum.  A maximum of a later call is therefore
+    // larger than anything an earlier call left behind, and the slot never has to be cleared (a
+    // launch saved per call; replays of a captured call stay exact).
     unsigned long long *max_slots;
-    mutable std::atomic<uint32_t> call_seq;
+    mutable std::mutex slot_lock;
+    mutable std::unordered_map<void *, int> slot_of_stream;
 };
 
-constexpr int kMaxSlots = 16;
+constexpr int kMaxSlots = 64;
 constexpr int kMaxSlotStride = 32;       // 64-bit words between two slots (one 256-byte line each)
 
 namespace dnatok {
@@ -680,7 +684,6 @@ extern "C" int dnatok_kmer_table_create(int k, const int8_t *digit_h, const int3
     t->entry = (int2 *)(b + o_entry);
     t->flat = (int32_t *)(b + o_flat);
     t->max_slots = (unsigned long long *)(b + o_slots);
-    t->call_seq.store(0);
     *out = t;
     return DNATOK_OK;
 }
@@ -717,9 +720,13 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
     KmerArgs a{t->digit, t->single, t->lut4, t->entry, t->flat, t->pad_id, t->missing_id};
     MaxRef mref{nullptr};
     if (to_longest) {
-        const uint32_t seq = t->call_seq.fetch_add(1, std::memory_order_relaxed);
-        mref.slot = t->max_slots + (size_t)(seq % kMaxSlots) * kMaxSlotStride;
-    } else if (max_len) {
+        std::lock_guard<std::mutex> hold(t->slot_lock);
+        auto it = t->slot_of_stream.find(stream);
+        if (it == t->slot_of_stream.end() && (int)t->slot_of_stream.size() < kMaxSlots)
+            it = t->slot_of_stream.emplace(stream, (int)t->slot_of_stream.size()).first;
+        if (it != t->slot_of_stream.end()) mref.slot = t->max_slots + (size_t)it->second * kMaxSlotStride;
+    }
+    if (!mref.slot && max_len) {
         kmer_init_kernel<<<1, 1, 0, s>>>(max_len);
         DNATOK_HIP_TRY(hipGetLastError());
     }

@@ -153,7 +153,10 @@ void dnatok_kmer_table_destroy(dnatok_kmer_t *t);
  * fill_to < 0: as fill_to = 0, with -fill_to as the caller's guess of that longest row (say,
  *              the width of the previous batch of a stream).  Rows are padded to the guess while
  *              they are written and only what is missing afterwards; a guess that is too small
- *              or too large costs time, never correctness (cells past max_len are unspecified). */
+ *              or too large costs time, never correctness (cells past max_len are unspecified).
+ * Calls on one table may overlap on different streams (fill_to <= 0 keeps its running maximum in
+ * a device word per stream); calls issued from several host threads are serialised only for the
+ * moment that word is looked up. */
 int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *bytes, const int64_t *offsets,
                               int64_t n_rows, int64_t t_cap, int64_t fill_to,
                               int32_t *ids, uint8_t *mask, int32_t *lengths, int32_t *status,

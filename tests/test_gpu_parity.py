@@ -305,6 +305,37 @@ def test_kmer_pad_to_longest_replayed_from_a_graph(kmer_enc):
     assert widths[1] == length // 6 and widths[0] > widths[1] and widths[3] > widths[2] > widths[1]
 
 
+def test_kmer_pad_to_longest_calls_on_many_streams_do_not_share_a_maximum(kmer_enc):
+    """Pad-to-longest calls queued on several streams at once, nothing synchronised in between:
+    every call reports the longest row of its own batch.  70 streams is more than the table keeps
+    running maxima for, so the last ones take the path that clears the caller's max_len instead."""
+    say("kmer pad-to-longest on many streams")
+    n, length, t_cap = 256, 6000, 6016
+    batches = [wl.config2_kmer(n, length, seed=40 + i, n_fraction=f) for i, f in enumerate((0.0, 0.05, 0.01, 0.1))]
+    dev = [to_dev(b) for b in batches]
+    want = []
+    for data, off in dev:
+        r = kmer_enc.encode_padded(data, off, t_cap, fill_to=0)
+        torch.cuda.synchronize()
+        want.append((int(r[4].item()), r[0].cpu().numpy(), r[2].cpu().numpy()))
+    assert len({w[0] for w in want}) == len(want)
+    streams = [torch.cuda.Stream() for _ in range(70)]
+    torch.cuda.synchronize()
+    got = []
+    for rnd in range(2):
+        for i, st in enumerate(streams):
+            which = (i + rnd) % len(dev)
+            with torch.cuda.stream(st):
+                got.append((which, kmer_enc.encode_padded(dev[which][0], dev[which][1], t_cap, fill_to=0,
+                                                          width_guess=length // 6 if i % 3 else 0)))
+    torch.cuda.synchronize()
+    for which, r in got:
+        width, ids, lengths = want[which]
+        assert int(r[4].item()) == width
+        np.testing.assert_array_equal(r[2].cpu().numpy(), lengths)
+        np.testing.assert_array_equal(r[0][:, :width].cpu().numpy(), ids[:, :width])
+
+
 def test_kmer_general_tables_not_spelled():
     """Tables whose N windows are not spelled character by character: N windows that have an
     id of their own, expansions of other lengths, and windows with nothing at all."""
