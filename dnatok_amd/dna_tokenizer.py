@@ -469,12 +469,12 @@ class DNATok:
         # a stride of whole 128-byte lines keeps every row of ids and of the mask on line boundaries
         t_cap += (-t_cap) % 128
         plain = (not left) and dtype == torch.int32 and pad_multiple <= 1
-        # the width of the previous batch is a good guess of this one's in a stream of batches
+        # the width of the previous batch (plus a margin) is a good guess of this one's in a stream of batches
         ids, mask, lengths, status, longest = self._kmer_enc.encode_padded(
             data, offsets, t_cap, fill_to=0, width_guess=getattr(self, "_kmer_width_guess", 0) if plain else 0)
         if plain:
             width = int(longest.item())                  # one scalar: the output shape
-            self._kmer_width_guess = width
+            self._kmer_width_guess = encoders.width_guess_after(width)
             plain = width >= min_width
         if not plain:
             cap = max(t_cap, int(min_width))

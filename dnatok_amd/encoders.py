@@ -272,6 +272,19 @@ class CharEncoder:
         return out
 
 
+def width_guess_after(previous_width: int) -> int:
+    """The ``width_guess`` to pass for the next batch of a stream whose last batch came out
+    ``previous_width`` tokens wide.  A guess above the true width costs the few extra pad cells
+    (written next to the row's own cells); a guess below it costs a second visit to every row, so
+    the guess carries a margin: 1/64 of the width, at least 8 tokens, up to a whole 128-byte line of
+    ids."""
+    w = int(previous_width)
+    if w <= 0:
+        return 0
+    w += max(8, w >> 6)
+    return w + (-w) % 32
+
+
 class KmerEncoder:
     """Grid-aligned k-mer windows with per-window fallback (C ABI: dnatok_kmer_*)."""
 
