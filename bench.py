@@ -163,7 +163,7 @@ class KmerPadded(Workload):
     selects the policy: "previous" (the library's: previous width plus a margin), "stale"
     (the previous width as it is, which is too small every other call) or "none"."""
 
-    def __init__(self, n_batches: int, t_cap: int = 6016, guess: str = "previous"):
+    def __init__(self, n_batches: int, t_cap: int = 0, guess: str = "previous"):
         from dnatok_amd import encoders, kmer_tables
         from tests.support import hf_tokenizers as hf, workloads as wl
         import torch
@@ -173,7 +173,6 @@ class KmerPadded(Workload):
         self.enc = encoders.KmerEncoder(6, t.digit, t.kmer_lut, t.single, vocab["<pad>"], vocab["<unk>"],
                                         t.exp_off, t.exp_len, t.exp_flat)
         self.n_rows = 256 * n_batches
-        self.t_cap = t_cap
         self.guess = guess
         self.off = _dev(np.arange(self.n_rows + 1, dtype=np.int64) * 6000)
         self.hosts, self.sets = [], []
@@ -185,6 +184,32 @@ class KmerPadded(Workload):
             self.hosts.append(host)
             self.sets.append(_dev(host))
         dev = "cuda"
+        # the widths of the two data sets, from a first pass with room for the worst case
+        self.t_cap = 6016
+        scratch = tuple(torch.empty(shape, dtype=dt, device=dev) for shape, dt in (
+            ((self.n_rows, 6016), torch.int32), ((self.n_rows, 6016), torch.uint8), ((self.n_rows,), torch.int32),
+            ((self.n_rows,), torch.int32), ((1,), torch.int32)))
+        self.widths = []
+        for which in (0, 1):
+            self.out = scratch
+            self.run(which, 0)
+            torch.cuda.synchronize()
+            t_max = int(scratch[4].item())
+            assert t_max == int(scratch[2].max().item())
+            self.widths.append(t_max)
+        del scratch
+        self.out = None
+        torch.cuda.empty_cache()
+        # The stride of the rows: as the library does it in a stream of batches, the guess of the
+        # width rounded up to whole 128-byte lines (a batch wider than that would come out cut
+        # and be encoded again with the worst-case stride; check() sees that none is).  Without
+        # a usable guess the rows lie the worst case apart.
+        if not t_cap:
+            t_cap = 6016
+            if guess == "previous":
+                g = max(encoders.width_guess_after(wd) for wd in self.widths)
+                t_cap = g + (-g) % 128
+        self.t_cap = t_cap
         self.out = (torch.empty((self.n_rows, t_cap), dtype=torch.int32, device=dev),
                     torch.empty((self.n_rows, t_cap), dtype=torch.uint8, device=dev),
                     torch.empty(self.n_rows, dtype=torch.int32, device=dev),
@@ -196,14 +221,7 @@ class KmerPadded(Workload):
                "stale": "width of the previous call, which ran on different data, passed as the guess as it is",
                "none": "no width guess"}[guess]
         self.name = (f"C2 non-overlapping 6-mer vocab-4106, 256x6000 bp batches, {n_batches} distinct batch(es) "
-                     f"per call, two data sets taking turns, pad to longest row ({how})")
-        self.widths = []
-        for which in (0, 1):
-            self.run(which, 0)
-            torch.cuda.synchronize()
-            t_max = int(self.out[4].item())
-            assert t_max == int(self.out[2].max().item())
-            self.widths.append(t_max)
+                     f"per call, two data sets taking turns, pad to longest row ({how}), rows {t_cap} cells apart")
         # 1 B/base read; int32 id + uint8 mask for every cell of [rows, T_max]; int32 length per row;
         # the mean over the two data sets, which take turns
         self.algorithmic_bytes = self.bases + 5 * self.n_rows * sum(self.widths) // 2 + 4 * self.n_rows

@@ -469,11 +469,24 @@ class DNATok:
         # a stride of whole 128-byte lines keeps every row of ids and of the mask on line boundaries
         t_cap += (-t_cap) % 128
         plain = (not left) and dtype == torch.int32 and pad_multiple <= 1
-        # the width of the previous batch (plus a margin) is a good guess of this one's in a stream of batches
+        # The width of the previous batch (plus a margin) is a good guess of this one's in a stream
+        # of batches: rows are padded that far while they are written, and the rows are laid out
+        # that far apart (whole 128-byte lines), which makes the output nearly dense in memory
+        # instead of a fifth of a worst-case buffer.  A batch that turns out wider than the guess
+        # fills the stride to the last cell; it is then encoded again with room for the worst case.
+        guess = getattr(self, "_kmer_width_guess", 0) if plain else 0
+        worst = t_cap
+        if guess:
+            t_cap = min(worst, guess + (-guess) % 128)
         ids, mask, lengths, status, longest = self._kmer_enc.encode_padded(
-            data, offsets, t_cap, fill_to=0, width_guess=getattr(self, "_kmer_width_guess", 0) if plain else 0)
+            data, offsets, t_cap, fill_to=0, width_guess=guess)
         if plain:
             width = int(longest.item())                  # one scalar: the output shape
+            if width >= t_cap and t_cap < worst:
+                t_cap = worst
+                ids, mask, lengths, status, longest = self._kmer_enc.encode_padded(
+                    data, offsets, t_cap, fill_to=0, width_guess=0)
+                width = int(longest.item())
             self._kmer_width_guess = encoders.width_guess_after(width)
             plain = width >= min_width
         if not plain:

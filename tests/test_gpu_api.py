@@ -273,6 +273,23 @@ def test_kmer_discover_and_encode():
     assert bool((ids[:, short.shape[1]:] == 0).all()) and bool((mask[:, short.shape[1]:] == 0).all())
 
 
+def test_kmer_stream_of_batches_with_a_much_wider_one_in_between():
+    """In a stream of batches the rows are laid out only as far apart as the previous batch was
+    wide (plus a margin); a batch that needs more room than that is encoded again with room for
+    the worst case, and every batch equals the tokenizer's own answer."""
+    tok = MockKmerTokenizer(4)
+    h = DNATok(RecordingEmbedder(tok))
+    h.discover()
+    narrow = random_seqs(48, 2000, alphabet="ACGT", seed=11)
+    few_n = random_seqs(48, 2000, alphabet="ACGT" * 30 + "N", seed=12)
+    wide = random_seqs(48, 2000, alphabet="ACGTN", seed=13)            # most windows are spelled
+    for seqs in (narrow, few_n, narrow, wide, wide, narrow, few_n):
+        want = tok(seqs, padding=True, return_tensors="pt")["input_ids"]
+        ids, mask = h.encode_batch_device(seqs)
+        assert torch.equal(ids.cpu().long(), want)
+        assert torch.equal(mask.cpu().bool(), want != tok.pad_token_id)
+
+
 def test_kmer_multi_token_windows_follow_the_tokenizer():
     tok = FakeKmerTokenizer(3)
     emb = RecordingEmbedder(tok, 256)
