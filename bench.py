@@ -628,6 +628,48 @@ def device_normalizer_extra():
             "kernels": "norm_rows_kernel + norm_count_kernel + norm_emit_kernel"}
 
 
+def pathological_extra():
+    """BPE on rows made of long runs of equal pairs (a homopolymer, tandem repeats), beside random rows
+    of the same size: a run makes every pair's rank equal to its neighbour's, the case in which a
+    candidate's walk along its left chain would be as long as the run.  Every row is checked against
+    the Hugging Face tokenizer run here."""
+    import random
+    import torch
+    from dnatok_amd import bpe_vocab, encoders
+    from tests.support import hf_tokenizers as hf
+    rng = random.Random(3)
+    rnd = lambda n: "".join(rng.choices("ACGT", k=n))
+    out = {}
+    for which in ("4096", "32000"):
+        with open(hf.bpe_tokenizer_path(which)) as fh:
+            cfg = json.load(fh)
+        kv = bpe_vocab.KernelVocab(bpe_vocab.split_merges(cfg["model"]["merges"]))
+        vocab = cfg["model"]["vocab"]
+        enc = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv), out_remap=kv.remap_to(vocab, vocab["[UNK]"]))
+        tk = hf.load_bpe_tokenizer(which)
+        rows = {}
+        for name, text in (("random_2kb", rnd(2048)), ("poly_a_2kb", "A" * 2048), ("ac_repeat_2kb", "AC" * 1024),
+                           ("random_100kb", rnd(100_000)), ("poly_a_100kb", "A" * 100_000),
+                           ("aaat_repeat_100kb", "AAAT" * 25_000)):
+            host = np.frombuffer(text.encode("ascii"), dtype=np.uint8)
+            data, off = _dev(host), _dev(np.array([0, host.size], dtype=np.int64))
+            tok = torch.empty(host.size, dtype=torch.int32, device="cuda")
+            lengths = torch.empty(1, dtype=torch.int32, device="cuda")
+            enc.encode(data, off, host.size, tok_tmp=tok, lengths=lengths)
+            torch.cuda.synchronize()
+            got = tok[:int(lengths.item())].cpu().numpy()
+            same_rows([got], hf_live_rows(tk, host, [0, host.size]), f"BPE vocab-{which} {name}")
+
+            class W:
+                def step(self):
+                    enc.encode(data, off, host.size, tok_tmp=tok, lengths=lengths)
+            _, dm = time_steps(W(), 10, 2)
+            rows[name] = {"device_us_per_call": dm * 1e3}
+        rows["poly_a_2kb_over_random_2kb"] = rows["poly_a_2kb"]["device_us_per_call"] / rows["random_2kb"]["device_us_per_call"]
+        out[f"vocab_{which}"] = rows
+    return out
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -761,6 +803,7 @@ def main() -> None:
         result["fused_embedding_gather"] = fused_embed_extra()
         result["unpack_2bit"] = unpack_2bit_extra()
         result["device_normalizer"] = device_normalizer_extra()
+        result["pathological"] = pathological_extra()
 
     print(json.dumps(result), flush=True)
 

@@ -191,13 +191,19 @@ __device__ __forceinline__ void bpe_row(
     const int wv = (NT == 64) ? 0 : (tid >> 6);
     uint32_t *qn = red + 4 * (NT / 64);        // number of merges queued in the current round
     uint32_t *cn = qn + 1;                     // number of candidates queued in the current round
+    uint32_t *capf = qn + 2;                   // some walk of the current round gave up (see kWalkCap)
+    // Steps a candidate walks along its left chain before it gives up.  Chains are a few steps
+    // long, except inside a run of equal pairs (x x x x ..., every pair has the rank of its left
+    // neighbour), where position i would walk i steps: a round with such a run decides all its
+    // candidates again by a scan over the positions instead (exact_decide below).
+    constexpr int kWalkCap = 24;
     // position i belongs to thread i % NT: in every pass the lanes of a wave touch consecutive
     // positions, so the LDS state arrays are read and written without bank conflicts
 
     // symbols, links and the initial pair of every position, kProbes pairs of table reads in flight at a time
     uint32_t cmin = kEmptyKey, cgate = kEmptyKey;
     D[tid] = 0;
-    if (tid == 0) { *qn = 0; *cn = 0; }
+    if (tid == 0) { *qn = 0; *cn = 0; *capf = 0; }
     // With PER > 0 the row's bytes come into LDS first (the candidate queue is free until the first
     // round), 8 aligned bytes per thread: one trip to memory for the whole row instead of one per
     // batch of table reads.  Only a word that reaches over the row's first or last byte is put
@@ -345,6 +351,7 @@ __device__ __forceinline__ void bpe_row(
             }
             team_sync<NT>();
             const int ncand = (int)*cn;
+            bool gave_up = false;
             for (int c0 = 0; c0 < ncand; c0 += NT) {      // the same trip count for every lane
                 const int c = c0 + tid;
                 bool merges = false;
@@ -359,6 +366,7 @@ __device__ __forceinline__ void bpe_row(
                     uint32_t chain = 0, rp = r;
                     IT q = x.pv;
                     while (q != NIL && yl.r <= rp) {      // candidates to the left with key <= ours
+                        if (chain == (uint32_t)kWalkCap) { gave_up = true; break; }
                         ++chain; rp = yl.r; q = yl.pv;
                         if (q != NIL) yl = P[q];
                     }
@@ -379,8 +387,81 @@ __device__ __forceinline__ void bpe_row(
                     if (merges) Q[at + (uint32_t)__builtin_popcountll(bal & ((1ull << lane) - 1ull))] = (IT)i;
                 }
             }
+            if (gave_up) *capf = 1;
         }
         team_sync<NT>();
+        if (!single && *capf) {
+            // Exact decision for every candidate of the round without walking to the left.  The
+            // left chain of candidate i has even length iff x(i) = 0, where x runs over the live
+            // positions from left to right: x(i) = x(left neighbour) ^ 1 if that neighbour is a
+            // candidate with a rank <= ours, else 0.  Every position is a function on that one
+            // bit (keep: a dead position; flip; set to 0), functions compose, so the positions
+            // are taken NT at a time in index order (which is the list's order), a wave at a time
+            // from two ballots, with the bit carried from wave to wave and from block to block.
+            constexpr int NW = NT / 64;
+            const int lane = tid & 63;
+            team_sync<NT>();                            // everyone has read the flag
+            if (tid == 0) { *qn = 0; *capf = 0; }
+            team_sync<NT>();
+            uint32_t carry = 0;                         // x of the last live position before the block
+            int blk = 0;
+            for (int b0 = 0; b0 < n0; b0 += NT, blk ^= 1) {      // the same trip count for every lane
+                const int i = b0 + tid;
+                bool keep = true, flips = false, cand = false;
+                PosRec<IT> x;
+                x.r = DEAD; x.nx = NIL; x.pv = NIL; x.s = DEAD;
+                if (i < n0) x = P[i];
+                if (x.s != DEAD) {
+                    cand = (uint32_t)x.r < limit;
+                    bool link = false;
+                    if (cand && x.pv != NIL) link = (uint32_t)P[x.pv].r <= (uint32_t)x.r;
+                    keep = link; flips = link;
+                }
+                const uint64_t kp = __ballot(keep), fl = __ballot(flips);
+                const uint64_t upto = lane == 63 ? ~0ull : ((2ull << lane) - 1ull);     // lanes 0 .. lane
+                const uint64_t resets = ~kp & upto;
+                uint64_t seg = upto;
+                if (resets != 0) seg &= ~((1ull << (63 - __builtin_clzll(resets))) - 1ull);    // from the last reset on
+                uint32_t xi = (uint32_t)__builtin_popcountll(fl & seg) & 1u;              // with 0 coming in
+                const bool w_keep = kp == ~0ull;
+                const uint32_t w_bit = (uint32_t)__builtin_amdgcn_readlane((int)xi, 63);
+                uint32_t into_wave = carry;
+                if (NW > 1) {
+                    if (lane == 0) red[blk * NW + wv] = (w_keep ? 2u : 0u) | w_bit;
+                    team_sync<NT>();
+                    uint32_t c = carry;
+#pragma unroll
+                    for (int w = 0; w < NW; ++w) {
+                        if (w == wv) into_wave = c;
+                        const uint32_t e = red[blk * NW + w];
+                        c = (e & 2u) ? (c ^ (e & 1u)) : (e & 1u);
+                    }
+                    carry = c;
+                } else {
+                    carry = w_keep ? (carry ^ w_bit) : w_bit;
+                }
+                if (resets == 0) xi ^= into_wave;
+                bool merges = false;
+                if (cand && xi == 0) {
+                    uint32_t chain_r = 0, rp = x.r;
+                    IT q = x.nx;
+                    PosRec<IT> yr = P[q != NIL ? q : (IT)i];
+                    while (q != NIL && yr.r < rp) {       // candidates to the right with key < ours
+                        ++chain_r; rp = yr.r; q = yr.nx;
+                        if (q != NIL) yr = P[q];
+                    }
+                    merges = (chain_r & 1u) == 0;
+                }
+                const uint64_t bal = __ballot(merges);
+                if (bal != 0) {                           // (uniform over the wave)
+                    uint32_t at = 0;
+                    if (lane == 0) at = atomicAdd(qn, (uint32_t)__builtin_popcountll(bal));
+                    at = (uint32_t)__builtin_amdgcn_readfirstlane((int)at);
+                    if (merges) Q[at + (uint32_t)__builtin_popcountll(bal & ((1ull << lane) - 1ull))] = (IT)i;
+                }
+            }
+            team_sync<NT>();
+        }
         const int nm = (int)*qn;                   // merges of this round (they do not overlap)
 
         // apply: position i absorbs its right neighbour j; one merge per thread and pass

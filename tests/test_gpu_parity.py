@@ -470,6 +470,24 @@ def test_bpe_rows_without_a_seam_fall_back_to_the_whole_row_kernel(bpe):
         np.testing.assert_array_equal(r, e, err_msg=s[:20])
 
 
+def test_bpe_long_runs_of_equal_pairs(bpe):
+    """Rows in which every pair has the rank of its neighbour for thousands of positions (a
+    homopolymer, a tandem repeat after its first merges): the left chain of a candidate would be
+    as long as the run, so such rounds decide by a scan over the positions instead of walking.
+    100 kbp rows go through chunks, seams and, where no seam is accepted, the whole-row kernel."""
+    which, enc, bo = bpe
+    say(f"bpe{which} long runs of equal pairs")
+    rng = random.Random(17)
+    rnd = lambda n: "".join(rng.choices("ACGT", k=n))
+    seqs = ["A" * 100_000, "AC" * 50_000, "AAAT" * 25_000,
+            rnd(3000) + "A" * 2000 + rnd(3000),                   # a 2 kbp run inside random sequence
+            rnd(500) + "T" * 700 + rnd(100) + "GA" * 400 + rnd(200),
+            "A" * 25, "A" * 26, "C" * 49, "AC" * 25, "A" * 23 + "C" + "A" * 30, "G" * 2047, "G" * 2048]
+    b = util.batch_from_strings(seqs)
+    for s, r, e in zip(seqs, bpe_rows(enc, b), bo.encode_batch(b.data, b.offsets)):
+        np.testing.assert_array_equal(r, e, err_msg=f"{s[:24]}... ({len(s)} bp)")
+
+
 @pytest.mark.parametrize("core,overlap", [(256, 32), (512, 96)])
 def test_bpe_small_chunks_many_seams_and_fallbacks(bpe, core, overlap):
     """The chunk / seam / gather / whole-row-fallback machinery with chunks far smaller than the
