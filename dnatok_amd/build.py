@@ -17,6 +17,23 @@ HIPCC_FLAGS = [
 ]
 
 
+def hostpack_path() -> str:
+    import sysconfig
+    return os.path.join(_HERE, "_hostpack" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
+
+
+def build_hostpack(verbose: bool = False) -> str:
+    """The small CPython module that packs a list of str into a byte buffer (host code only)."""
+    import sysconfig
+    cc = os.environ.get("CC", "gcc")
+    cmd = [cc, "-O2", "-shared", "-fPIC", "-Wall", "-I" + sysconfig.get_paths()["include"],
+           os.path.join(CSRC, "hostpack.c"), "-o", hostpack_path()]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return hostpack_path()
+
+
 def hipcc() -> str:
     for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
         if cand and (os.path.isabs(cand) and os.path.exists(cand) or not os.path.isabs(cand)):
@@ -50,6 +67,7 @@ def build_extension(verbose: bool = False) -> str:
         raise RuntimeError("hipcc failed")
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]
     subprocess.check_call(cmd)
+    build_hostpack(verbose)
     return LIB_PATH
 
 

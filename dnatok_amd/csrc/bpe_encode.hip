@@ -651,17 +651,27 @@ static size_t long_slab_bytes(int64_t max_len)
 // chunks so small that every few hundred bytes of a row hold a seam.
 static std::atomic<int> g_chunk_core{kChunkCore}, g_chunk_overlap{kChunkOverlap};
 
-static void chunk_geometry(int *core, int *overlap)
+// A batch whose long rows make far fewer chunks than teams fit the chip (a few rows of a few
+// thousand bytes each) is cut finer, down to a core of 512 bytes: more, shorter items run side by
+// side, and the batch is latency-bound either way (one row of 100 kbp: 48 -> 38 us per call).
+// Only with the shipped geometry, and only when the batch has long rows at all.
+static void chunk_geometry(int *core, int *overlap, int64_t max_len, int64_t total)
 {
     *core = g_chunk_core.load(std::memory_order_relaxed);
     *overlap = g_chunk_overlap.load(std::memory_order_relaxed);
+    if (*core == kChunkCore && *overlap == kChunkOverlap && max_len > kChunkCore + 2 * kChunkOverlap) {
+        constexpr int64_t kTeams = 1024;                 // about what is resident at once
+        int64_t c = (total / kTeams + 127) & ~(int64_t)127;
+        if (c < 512) c = 512;
+        if (c < kChunkCore) *core = (int)c;
+    }
 }
 
 static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t total,
                          int64_t max_slabs = kLongGrid)
 {
     BpePlan p{};
-    chunk_geometry(&p.core, &p.overlap);
+    chunk_geometry(&p.core, &p.overlap, max_len, total);
     p.ext = p.core + 2 * p.overlap;
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
     const bool chunks = max_len > p.ext;
@@ -707,7 +717,7 @@ constexpr int kPlanRows = 4;
 constexpr int kPlanScans = 1 + kSingleClasses;
 
 __global__ __launch_bounds__(1024) void bpe_plan_kernel(
-    const int64_t *__restrict__ offsets, int64_t n_rows, int chunking, BpePlan p)
+    const int64_t *__restrict__ offsets, int64_t n_rows, int chunking, int expand_here, BpePlan p)
 {
     __shared__ uint32_t wt[kPlanScans][16];
     __shared__ int32_t carry[kPlanScans];
@@ -771,7 +781,12 @@ __global__ __launch_bounds__(1024) void bpe_plan_kernel(
             const int32_t row = (int32_t)(row0 + r);
             p.mc_off[row] = at[0];
             // the entries of the chunks are written by bpe_expand_kernel (a single workgroup
-            // writing tens of thousands of scattered words is bound by its one CU's store path)
+            // writing tens of thousands of scattered words is bound by its one CU's store path),
+            // except for a small batch of rows of few chunks each, which saves that launch
+            if (expand_here && add[r][0]) {
+                const int32_t nc = (int32_t)add[r][0], len = (int32_t)(off[r + 1] - off[r]);
+                for (int32_t k = 0; k < nc; ++k) p.rec[at[0] + k] = make_int4(row, k, nc, len);
+            }
 #pragma unroll
             for (int q = 0; q < kSingleClasses; ++q)
                 if (add[r][1 + q]) p.single[q][at[1 + q]] = row;
@@ -1294,9 +1309,10 @@ int run_lds(bool long_rows, int chunking, const BpeArgs &a, const uint8_t *bytes
 {
     const bool planned = long_rows || n_rows > lds_resident_teams<NT, TEAMS, CAP>();
     if (planned) {
-        bpe_plan_kernel<<<1, 1024, 0, s>>>(offsets, n_rows, chunking, p);
+        const int expand_here = chunking >> 1;
+        bpe_plan_kernel<<<1, 1024, 0, s>>>(offsets, n_rows, chunking & 1, expand_here, p);
         DNATOK_HIP_TRY(hipGetLastError());
-        if (chunking) {
+        if ((chunking & 1) && !expand_here) {
             bpe_expand_kernel<<<(int)((n_rows + 255) / 256), 256, 0, s>>>(offsets, n_rows, p);
             DNATOK_HIP_TRY(hipGetLastError());
         }
@@ -1314,7 +1330,10 @@ static int bpe_encode_launch(const dnatok_bpe_t *t, const uint8_t *bytes, const 
     BpeArgs a{t->tab, t->byte_to_sym, t->out_remap, t->shift, t->mul1, t->mul2, t->n_merges};
 
     const bool long_rows = max_len > p.ext;
-    const int chunking = (long_rows && t->monotone) ? 1 : 0;
+    int chunking = (long_rows && t->monotone) ? 1 : 0;
+    // bit 1: the plan kernel writes the chunk entries itself (a small batch of rows of at most 16
+    // chunks each: a few stores per thread, and one launch less)
+    if (chunking && n_rows <= 4096 && max_len <= 16 * (int64_t)p.core) chunking |= 2;
     // the LDS capacity variant follows the longest row (or the chunk size for longer rows):
     // less LDS per workgroup means more workgroups per CU
     int rc;

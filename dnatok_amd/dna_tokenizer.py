@@ -377,38 +377,73 @@ class DNATok:
                                         min_width=int(self.token_len or 0), pad_multiple=1)
 
     def _encode_rows_device(self, seqs: Sequence[str], device, *, dtype: torch.dtype, min_width: int,
-                            pad_multiple: int) -> Tuple[torch.Tensor, torch.Tensor]:
+                            pad_multiple: int, host_ids: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+        """``host_ids``: the caller wants the ids on the host; where the layout allows it they are
+        copied down inside the call, under its one wait, and left in ``_staged_host_ids`` (a view
+        of the tokenizer's pinned buffer, valid until the next call)."""
         self._require_ready()
         if not seqs:
             raise ValueError("No sequences provided for encoding.")
         left = self.padding_side == "left"
+        self._staged_host_ids = None
         if self.bpe_backend is not None:
-            tok, offsets, lengths, t_cap = self.bpe_backend.tokens_device(list(seqs), device=device)
+            tok, offsets, lengths, t_cap = self.bpe_backend.tokens_device(list(seqs), device=device, meta_tail=2)
             return self._pad_bpe_runs(tok, offsets, lengths, t_cap, dtype=dtype, min_width=min_width,
-                                      pad_multiple=pad_multiple)
+                                      pad_multiple=pad_multiple, host_ids=host_ids, stats_behind_lengths=True)
         data, offsets, lens = encoders.bytes_from_strings(seqs, device)
         if self._kmer_enc is not None:
             return self._encode_kmer_device(seqs, data, offsets, lens, dtype=dtype, min_width=min_width,
-                                            pad_multiple=pad_multiple)
+                                            pad_multiple=pad_multiple, host_ids=host_ids)
         width = max(int(lens.max()), int(min_width))
         if pad_multiple > 1 and width % pad_multiple:
             width += pad_multiple - width % pad_multiple
         return self._char_enc.encode_padded(data, offsets, width, pad_left=left, dtype=dtype)
 
-    def _pad_bpe_runs(self, tok, offsets, lengths, t_cap: int, *, dtype, min_width: int, pad_multiple: int):
+    def _pad_bpe_runs(self, tok, offsets, lengths, t_cap: int, *, dtype, min_width: int, pad_multiple: int,
+                      host_ids: bool = False, stats_behind_lengths: bool = False):
         """The engine's token runs -> padded rows: remap, padding side, least width, multiple and
         id type in one launch; one host read for the shape (and the smallest length: a negative
         one is a failed row)."""
         be = self.bpe_backend
-        cap = max(int(t_cap), int(min_width), 1)
-        if pad_multiple > 1 and cap % pad_multiple:
-            cap += pad_multiple - cap % pad_multiple
-        ids, mask, stats = encoders.pad_rows_as(tok, offsets, lengths, int(be.pad_id), cap, min_width=min_width,
-                                                pad_multiple=pad_multiple, pad_left=(self.padding_side == "left"),
-                                                dtype=dtype, remap=be._remap_on(tok.device))
-        _, width, shortest = torch.cat((stats, lengths.min()[None])).tolist()
-        if shortest < 0:
-            raise RuntimeError("BPE engine reported a failed row (negative length)")
+        worst = max(int(t_cap), int(min_width), 1)
+        if pad_multiple > 1 and worst % pad_multiple:
+            worst += pad_multiple - worst % pad_multiple
+        # In a stream of batches the rows are laid out only as far apart as the previous batch was
+        # wide (plus a margin): a token run is several times shorter than its row of bytes.  A
+        # batch that needs more room than that is padded again with room for the worst case.
+        guess = getattr(self, "_bpe_width_guess", 0)
+        cap = worst
+        if guess:
+            cap = max(guess + (-guess) % 128, int(min_width))
+            if pad_multiple > 1 and cap % pad_multiple:
+                cap += pad_multiple - cap % pad_multiple
+            cap = min(cap, worst)
+        n = lengths.numel()
+        # lengths and the padding's two statistics in one allocation: one copy brings them down
+        # (with stats_behind_lengths the caller got the lengths as the head of an allocation of n + 2)
+        meta = torch.as_strided(lengths, (n + 2,), (1,)) if stats_behind_lengths else None
+        while True:
+            ids, mask, stats = encoders.pad_rows_as(tok, offsets, lengths, int(be.pad_id), cap, min_width=min_width,
+                                                    pad_multiple=pad_multiple, pad_left=(self.padding_side == "left"),
+                                                    dtype=dtype, remap=be._remap_on(tok.device),
+                                                    stats=None if meta is None else meta[n:])
+            staged = None
+            if host_ids and cap < worst:
+                nbytes = n * cap * ids.element_size()
+                staged = self._pinned(nbytes)[:nbytes].view(ids.dtype).view(n, cap)
+                staged.copy_(ids, non_blocking=True)
+            if meta is not None:
+                meta_h = meta.cpu().numpy()                                  # (the one wait)
+                longest, width, shortest = int(meta_h[n]), int(meta_h[n + 1]), int(meta_h[:n].min())
+            else:
+                longest, width, shortest = torch.cat((stats, lengths.min()[None])).tolist()
+            if shortest < 0:
+                raise RuntimeError("BPE engine reported a failed row (negative length)")
+            if longest < cap or cap >= worst:            # (the packer reports lengths cut to the stride)
+                break
+            cap = worst                                  # a row may have been cut: once more, with room for all
+        self._bpe_width_guess = encoders.width_guess_after(longest)
+        self._staged_host_ids = staged[:, :width] if staged is not None else None
         return ids[:, :width], mask[:, :width]
 
     def encode_fasta_device(self, source, device="cuda"):
@@ -451,8 +486,19 @@ class DNATok:
         ids, mask = self._char_enc.encode_padded(data, offsets, width, pad_left=(self.padding_side == "left"))
         return ids, mask, names
 
+    def _pinned(self, nbytes: int) -> torch.Tensor:
+        """The tokenizer's pinned host buffer for results on their way down (grown as needed; its
+        content is copied out before the call that filled it returns)."""
+        buf = getattr(self, "_pinned_buf", None)
+        if buf is None or buf.numel() < nbytes:
+            size = 1 << 20
+            while size < nbytes:
+                size *= 2
+            buf = self._pinned_buf = torch.empty(size, dtype=torch.uint8, pin_memory=True)
+        return buf
+
     def _encode_kmer_device(self, seqs, data, offsets, lens, *, dtype=torch.int32, min_width: int = 0,
-                            pad_multiple: int = 1) -> Tuple[torch.Tensor, torch.Tensor]:
+                            pad_multiple: int = 1, host_ids: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
         """k-mer rows on the device.  Right padding to the longest row with int32 ids comes straight
         out of the encoder; any other layout (left padding, a least width, a multiple, a narrower id
         type) is one more launch of the packer over the encoder's rows.  Rows the tables cannot
@@ -478,15 +524,30 @@ class DNATok:
         worst = t_cap
         if guess:
             t_cap = min(worst, guess + (-guess) % 128)
-        ids, mask, lengths, status, longest = self._kmer_enc.encode_padded(
-            data, offsets, t_cap, fill_to=0, width_guess=guess)
+        # lengths, status and the longest row share one allocation: one copy brings them to the host
+        meta = torch.empty(2 * n + 1, dtype=torch.int32, device=data.device)
+
+        def run(cap: int, guess: int):
+            out = (torch.empty((n, cap), dtype=torch.int32, device=data.device),
+                   torch.empty((n, cap), dtype=torch.uint8, device=data.device), meta[:n], meta[n:2 * n], meta[2 * n:])
+            return self._kmer_enc.encode_padded(data, offsets, cap, fill_to=0, width_guess=guess, out=out)
+
+        ids, mask, lengths, status, longest = run(t_cap, guess)
+        staged = None
+        if host_ids and plain and guess:
+            # the ids start their way down before the width is known (the rows lie only the guess
+            # apart, so little more than the answer is copied); the wait below covers both copies
+            staged = self._pinned(n * t_cap * 4)[:n * t_cap * 4].view(torch.int32).view(n, t_cap)
+            staged.copy_(ids, non_blocking=True)
+        meta_h = meta.cpu().numpy()                      # (the one wait of the call)
         if plain:
-            width = int(longest.item())                  # one scalar: the output shape
+            width = int(meta_h[2 * n])                   # the output shape
             if width >= t_cap and t_cap < worst:
                 t_cap = worst
-                ids, mask, lengths, status, longest = self._kmer_enc.encode_padded(
-                    data, offsets, t_cap, fill_to=0, width_guess=0)
-                width = int(longest.item())
+                staged = None
+                ids, mask, lengths, status, longest = run(t_cap, 0)
+                meta_h = meta.cpu().numpy()
+                width = int(meta_h[2 * n])
             self._kmer_width_guess = encoders.width_guess_after(width)
             plain = width >= min_width
         if not plain:
@@ -499,7 +560,8 @@ class DNATok:
                                                     dtype=dtype)
             width = int(stats[1].item())
         ids, mask = ids[:, :width], mask[:, :width]
-        bad = status.cpu().numpy()
+        self._staged_host_ids = staged[:, :width] if staged is not None and plain else None
+        bad = meta_h[n:2 * n]
         need = (bad & (2 | 4)) != 0
         if self.require_valid_chars or not self.handle_invalid_chars:
             need |= (bad & 1) != 0
@@ -507,6 +569,7 @@ class DNATok:
         if not getattr(self, "_kmer_tail_ok", True):
             need |= (np.asarray(lens) % k) != 0
         if need.any() and not self.allow_incomplete_kmer_lut:
+            self._staged_host_ids = None
             rows = np.nonzero(need)[0].tolist()
             fixed = self._tok_ids([seqs[i] for i in rows])
             new_w = max(width, max(len(r) for r in fixed))
@@ -535,9 +598,14 @@ class DNATok:
 
     def encode_batch_to_ids(self, seqs: List[str]) -> torch.Tensor:
         """CPU pinned int64 [B, T] (reference: 2049-2148)."""
-        ids, _ = self.encode_batch_device(seqs)
+        single = self.bpe_backend is None and self._kmer_enc is None
+        ids, _ = self._encode_rows_device(seqs, "cuda", dtype=torch.int64 if single else torch.int32,
+                                          min_width=int(self.token_len or 0), pad_multiple=1, host_ids=True)
         out = torch.empty(ids.shape, dtype=torch.int64, pin_memory=True)
-        out.copy_(ids)                                   # int32 -> int64 on the way down
+        staged = self._staged_host_ids
+        # k-mer and BPE ids came down inside the call (int32 -> int64 on the host); the character
+        # tables write int64 themselves and are copied as they are
+        out.copy_(staged if staged is not None else ids)
         return out
 
     def encode_batch_to_ids_staging(self, seqs: List[str], *, dtype: Optional[torch.dtype] = None) -> torch.Tensor:

@@ -9,7 +9,7 @@ tokenizer's ids is the caller's remap table, as in ``GPUTokBPEBackend``.
 """
 from __future__ import annotations
 
-from typing import Dict, List, Optional, Sequence, Tuple
+from typing import Optional, Dict, List, Optional, Sequence, Tuple
 
 import torch
 
@@ -57,11 +57,12 @@ class DnatokBpeKernel:
             raise IndexError("id out of range")
         return self._impl.vocab.id_to_token[idx]
 
-    def tokenize_device(self, data: torch.Tensor, offsets: torch.Tensor, max_len: int
-                        ) -> Tuple[torch.Tensor, torch.Tensor]:
+    def tokenize_device(self, data: torch.Tensor, offsets: torch.Tensor, max_len: int, *,
+                        lengths: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
         """Device-resident entry: uint8 bytes + int64 offsets -> (tok_tmp, lengths); row b's
-        tokens are tok_tmp[offsets[b] : offsets[b] + lengths[b]]."""
-        return self._impl.encoder.encode(data, offsets, max_len)
+        tokens are tok_tmp[offsets[b] : offsets[b] + lengths[b]].  ``lengths`` (int32 [B] on the
+        device) may be given by the caller."""
+        return self._impl.encoder.encode(data, offsets, max_len, lengths=lengths)
 
     def tokenize_batch(self, texts: Sequence[str], *, clone: bool = False
                        ) -> Tuple[torch.Tensor, torch.Tensor]:

@@ -9,6 +9,7 @@ and uint8 masks that stay on the device.
 from __future__ import annotations
 
 import ctypes
+import threading
 from typing import Optional, Sequence, Tuple
 
 import numpy as np
@@ -41,16 +42,61 @@ def _require_cuda(t: torch.Tensor, dtype: torch.dtype, name: str) -> None:
         raise ValueError(f"{name} must be a contiguous {dtype} tensor on the GPU")
 
 
+try:                                    # the C packer is host code; without it the strings are joined in Python
+    from . import _hostpack
+except ImportError:                     # pragma: no cover
+    _hostpack = None
+
+
+class _PinnedStage(threading.local):
+    """Per thread: a pinned host buffer the packer writes into, and the event that says when the
+    last copy out of it has finished."""
+    buf: Optional[torch.Tensor] = None
+    event = None
+
+
+_stage = _PinnedStage()
+
+
+def _pack_to_device(seqs: Sequence[str], device, utf8: bool):
+    """Strings -> pinned buffer (offsets, then bytes, written by the C packer) -> one copy to the
+    device.  Returns (data, offsets, host_lengths) as views of one device allocation."""
+    st = _stage
+    if st.event is not None:
+        st.event.synchronize()                   # the previous batch has left the buffer
+    if st.buf is None:
+        st.buf = torch.empty(1 << 20, dtype=torch.uint8, pin_memory=True)
+    r = _hostpack.pack_strings(seqs, st.buf.data_ptr(), st.buf.numel(), int(utf8))
+    if isinstance(r, int):                       # too small: -r bytes are needed
+        size = 1 << 20
+        while size < -r:
+            size *= 2
+        st.buf = torch.empty(size, dtype=torch.uint8, pin_memory=True)
+        r = _hostpack.pack_strings(seqs, st.buf.data_ptr(), st.buf.numel(), int(utf8))
+    n, total, _, bytes_at = r
+    used = bytes_at + total
+    dev = torch.empty(used, dtype=torch.uint8, device=device)
+    dev.copy_(st.buf[:used], non_blocking=True)
+    if st.event is None:
+        st.event = torch.cuda.Event()
+    st.event.record()
+    lens = np.diff(st.buf[:8 * (n + 1)].view(torch.int64).numpy())
+    return dev[bytes_at:used], dev[:8 * (n + 1)].view(torch.int64), lens
+
+
 def bytes_from_strings(seqs: Sequence[str], device="cuda", encoding: str = "ascii"
                        ) -> Tuple[torch.Tensor, torch.Tensor, np.ndarray]:
     """Concatenate strings into one device uint8 buffer + device int64 offsets.
 
-    Returns (data, offsets, host_lengths).  One join and one H2D copy per call
+    Returns (data, offsets, host_lengths).  The rows' bytes and their offsets are written into a
+    pinned buffer by one pass in C and cross the bus in one copy
     (reference: DNATokBPE::tokenize_batch, src/dnatok_bpe_kernel/dnatok_bpe.cu:872-887).
     ``encoding`` = "ascii": one byte per character, non-ASCII characters become ``?`` (what the
     table paths of the reference do, src/dna_tokenizer.py:1793); "utf-8": the bytes the
     reference's BPE kernel sees, since its binding receives ``std::string``.
     """
+    if _hostpack is not None and torch.device(device).type == "cuda":
+        return _pack_to_device(seqs, device, encoding == "utf-8")
     joined = "".join(seqs)
     if encoding == "utf-8" and not joined.isascii():
         parts = [s.encode("utf-8") for s in seqs]
@@ -435,17 +481,20 @@ def pad_rows(tok_tmp: torch.Tensor, in_offsets: torch.Tensor, lengths: torch.Ten
 def pad_rows_as(tok_tmp: torch.Tensor, in_offsets: torch.Tensor, lengths: torch.Tensor, pad_id: int,
                 t_cap: int, *, fill_to: int = 0, min_width: int = 0, pad_multiple: int = 1,
                 pad_left: bool = False, dtype: torch.dtype = torch.int32,
-                remap: Optional[torch.Tensor] = None, want_mask: bool = True):
+                remap: Optional[torch.Tensor] = None, want_mask: bool = True,
+                stats: Optional[torch.Tensor] = None):
     """The padded layout with the choices of DNATok's padding: side, a least width (``token_len``),
     a multiple, the id type.  Returns (ids[B, t_cap] of ``dtype``, mask, stats int32[2] =
-    {longest row, width}); view ``ids[:, :width]`` (C ABI: dnatok_pad_rows_as)."""
+    {longest row, width}); view ``ids[:, :width]`` (C ABI: dnatok_pad_rows_as).  ``stats`` may be
+    given (two int32 on the device, e.g. next to the lengths, so that one copy brings both down)."""
     if dtype not in (torch.uint8, torch.int16, torch.int32, torch.int64):
         raise ValueError("dtype must be uint8, int16, int32 or int64")
     n_rows = lengths.numel()
     dev = tok_tmp.device
     ids = torch.empty((n_rows, t_cap), dtype=dtype, device=dev)
     mask = torch.empty((n_rows, t_cap), dtype=torch.uint8, device=dev) if want_mask else None
-    stats = torch.zeros(2, dtype=torch.int32, device=dev)
+    if stats is None:
+        stats = torch.empty(2, dtype=torch.int32, device=dev)
     _lib.check(_lib.lib().dnatok_pad_rows_as(
         _ptr(tok_tmp), _ptr(in_offsets), _ptr(lengths), n_rows, _ptr(remap), int(pad_id), int(t_cap),
         int(fill_to), min(int(min_width), int(t_cap)), int(pad_multiple), int(bool(pad_left)), _ptr(ids),

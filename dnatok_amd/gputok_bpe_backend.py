@@ -389,11 +389,13 @@ class GPUTokBPEBackend:
 
     # ------------------------------------------------------------------- reference API
 
-    def tokens_device(self, seqs: List[str], *, device: object = "cuda"):
+    def tokens_device(self, seqs: List[str], *, device: object = "cuda", meta_tail: int = 0):
         """Strings -> the engine's token runs on the device: ``(tok_tmp int32, offsets int64 [B+1],
         lengths int32 [B], t_cap)`` with row b's kernel-space tokens at
         ``tok_tmp[offsets[b] : offsets[b] + lengths[b]]`` and t_cap a host-known bound of the row
-        lengths.  What ``encode_batch`` pads; DNATok pads the same runs its own way."""
+        lengths.  What ``encode_batch`` pads; DNATok pads the same runs its own way.  With
+        ``meta_tail`` > 0 the lengths are the head of an int32 allocation with that many more
+        entries behind them (for the padding's statistics: one copy then brings both to the host)."""
         if not seqs:
             raise ValueError("No sequences provided.")
         dev = torch.device(device) if not isinstance(device, torch.device) else device
@@ -419,7 +421,9 @@ class GPUTokBPEBackend:
             data, offsets, lens = encoders.bytes_from_strings(norm, dev, encoding="utf-8")
             t_cap = int(lens.max())
         t_cap = max(t_cap, 1)
-        tok, lengths = self._dnatok.tokenize_device(data, offsets, t_cap)
+        n = offsets.numel() - 1
+        lengths = torch.empty(n + int(meta_tail), dtype=torch.int32, device=data.device)[:n] if meta_tail else None
+        tok, lengths = self._dnatok.tokenize_device(data, offsets, t_cap, lengths=lengths)
         return tok, offsets, lengths, t_cap
 
     def encode_batch(self, seqs: List[str], *, device: object = "cuda"

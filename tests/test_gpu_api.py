@@ -288,6 +288,7 @@ def test_kmer_stream_of_batches_with_a_much_wider_one_in_between():
         ids, mask = h.encode_batch_device(seqs)
         assert torch.equal(ids.cpu().long(), want)
         assert torch.equal(mask.cpu().bool(), want != tok.pad_token_id)
+        assert torch.equal(h.encode_batch_to_ids(seqs), want)
 
 
 def test_kmer_multi_token_windows_follow_the_tokenizer():
@@ -553,6 +554,26 @@ def _bpe_wrapped(side):
             return tk.get_vocab()
 
     return Wrapped()
+
+
+@pytest.mark.parametrize("side", ["left", "right"])
+def test_bpe_stream_of_batches_with_longer_rows_in_between(side):
+    """As for the k-mer rows: in a stream of batches BPE rows are laid out only as far apart as the
+    previous batch was wide; a batch with longer token rows than that is padded again with room for
+    the worst case.  Ids on the host and on the device equal the tokenizer's own rows."""
+    tok = _bpe_wrapped(side)
+    h = DNATok(RecordingEmbedder(tok, vocab=8192), padding_side=side)
+    h.discover()
+    short = random_seqs(24, 600, alphabet="ACGT", seed=21)
+    long_ = random_seqs(24, 5000, alphabet="ACGT", seed=22)
+    ragged = [s[:n] for s, n in zip(random_seqs(24, 3000, alphabet="ACGT", seed=23), range(1, 3000, 120))]
+    for seqs in (short, short, long_, short, ragged, long_, long_, short):
+        want = h._tokenize_batch_cpu(seqs)
+        got = h.encode_batch_to_ids(seqs)
+        assert got.dtype == torch.int64 and got.shape == want.shape and torch.equal(got, want)
+        ids, mask = h.encode_batch_device(seqs)
+        assert torch.equal(ids.cpu().long(), want)
+        assert torch.equal(mask.cpu().bool(), want != 3)
 
 
 @pytest.mark.parametrize("side", ["left", "right"])

@@ -257,3 +257,23 @@ def test_fasta_scan_rejects_too_small_outputs():
     rc = L.dnatok_host_fasta_scan(*args, 6, ctypes.c_void_p(off.ctypes.data), None, 2,
                                   ctypes.byref(n_rec), ctypes.byref(n_bases))
     assert rc == 0 and (n_rec.value, n_bases.value) == (2, 6) and off[:3].tolist() == [0, 4, 6]
+
+
+def test_hostpack_writes_offsets_and_bytes_as_the_python_path_does():
+    """The C packer against plain Python: offsets, bytes, the two encodings, the size it asks for."""
+    import torch
+    from dnatok_amd import _hostpack
+    rows = ["ACGT", "", "h\u00e9llo\u4e16", "N" * 300, "acgt"]
+    for utf8 in (0, 1):
+        want = [r.encode("utf-8") if utf8 else r.encode("ascii", errors="replace") for r in rows]
+        buf = torch.zeros(4096, dtype=torch.uint8)
+        n, total, longest, at = _hostpack.pack_strings(rows, buf.data_ptr(), buf.numel(), utf8)
+        assert (n, total, longest) == (len(rows), sum(map(len, want)), max(map(len, want))) and at % 256 == 0
+        offsets = buf[:8 * (n + 1)].view(torch.int64).tolist()
+        assert offsets == [sum(map(len, want[:i])) for i in range(n + 1)]
+        assert bytes(buf[at:at + total].numpy()) == b"".join(want)
+        assert _hostpack.pack_strings(rows, buf.data_ptr(), at + total - 1, utf8) == -(at + total)
+        assert _hostpack.pack_strings(tuple(rows), buf.data_ptr(), buf.numel(), utf8)[1] == total
+    assert _hostpack.pack_strings([], buf.data_ptr(), buf.numel(), 0) == (0, 0, 0, 256)
+    with pytest.raises(TypeError):
+        _hostpack.pack_strings(["A", b"C"], buf.data_ptr(), buf.numel(), 0)
