@@ -191,12 +191,16 @@ __device__ __forceinline__ void bpe_row(
     const int wv = (NT == 64) ? 0 : (tid >> 6);
     uint32_t *qn = red + 4 * (NT / 64);        // number of merges queued in the current round
     uint32_t *cn = qn + 1;                     // number of candidates queued in the current round
-    uint32_t *capf = qn + 2;                   // some walk of the current round gave up (see kWalkCap)
+    uint32_t *capf = qn + 2;                   // walks of the current round that gave up (see kWalkCap)
     // Steps a candidate walks along its left chain before it gives up.  Chains are a few steps
     // long, except inside a run of equal pairs (x x x x ..., every pair has the rank of its left
-    // neighbour), where position i would walk i steps: a round with such a run decides all its
-    // candidates again by a scan over the positions instead (exact_decide below).
+    // neighbour), where position i would walk i steps.  A candidate that gives up goes onto a list
+    // (the far end of the candidate queue).  Up to kLateMax of them (a homopolymer or microsatellite
+    // of some dozen copies) then finish their walks, one per thread; with more, the round decides
+    // all its candidates again by a scan over the positions instead (below), which costs about as
+    // much as a round.
     constexpr int kWalkCap = 24;
+    constexpr uint32_t kLateMax = 64;
     // position i belongs to thread i % NT: in every pass the lanes of a wave touch consecutive
     // positions, so the LDS state arrays are read and written without bank conflicts
 
@@ -300,6 +304,7 @@ __device__ __forceinline__ void bpe_row(
         // unevenly over the threads) are first collected on a queue of their own and then dealt out
         // one per thread: every thread walks one candidate's chains at a time, with all lanes of a
         // wave busy, instead of its own positions one after the other with most lanes idle.
+        int ncand = 0;
         if (single) {
             if (tid == 0) { Q[0] = (IT)leftmost; *qn = 1; }
         } else {
@@ -350,8 +355,7 @@ __device__ __forceinline__ void bpe_row(
                 }
             }
             team_sync<NT>();
-            const int ncand = (int)*cn;
-            bool gave_up = false;
+            ncand = (int)*cn;
             for (int c0 = 0; c0 < ncand; c0 += NT) {      // the same trip count for every lane
                 const int c = c0 + tid;
                 bool merges = false;
@@ -365,6 +369,7 @@ __device__ __forceinline__ void bpe_row(
                     PosRec<IT> yr = P[x.nx != NIL ? x.nx : (IT)i];
                     uint32_t chain = 0, rp = r;
                     IT q = x.pv;
+                    bool gave_up = false;
                     while (q != NIL && yl.r <= rp) {      // candidates to the left with key <= ours
                         if (chain == (uint32_t)kWalkCap) { gave_up = true; break; }
                         ++chain; rp = yl.r; q = yl.pv;
@@ -376,7 +381,11 @@ __device__ __forceinline__ void bpe_row(
                         ++chain_r; rp = yr.r; q = yr.nx;
                         if (q != NIL) yr = P[q];
                     }
-                    merges = ((chain | chain_r) & 1u) == 0;
+                    merges = !gave_up && ((chain | chain_r) & 1u) == 0;
+                    if (gave_up) {
+                        const uint32_t k = atomicAdd(capf, 1u);
+                        if (k < kLateMax && n0 - 1 - (int)k >= ncand) C[n0 - 1 - (int)k] = (IT)i;
+                    }
                 }
                 // one queue atomic per wave (64 atomics on one LDS word take their turns)
                 const uint64_t bal = __ballot(merges);
@@ -387,10 +396,44 @@ __device__ __forceinline__ void bpe_row(
                     if (merges) Q[at + (uint32_t)__builtin_popcountll(bal & ((1ull << lane) - 1ull))] = (IT)i;
                 }
             }
-            if (gave_up) *capf = 1;
         }
         team_sync<NT>();
-        if (!single && *capf) {
+        const uint32_t late = single ? 0u : *capf;
+        const bool by_scan = late > kLateMax || ncand + (int)late > n0;
+        if (late != 0 && !by_scan) {
+            // the few walks that gave up, in full, one per thread
+            const int lane = tid & 63;
+            bool merges = false;
+            int i = 0;
+            if ((uint32_t)tid < late) {
+                i = (int)C[n0 - 1 - tid];
+                const PosRec<IT> x = P[i];
+                uint32_t chain = 0, rp = x.r;
+                IT q = x.pv;
+                PosRec<IT> y = P[q != NIL ? q : (IT)i];
+                while (q != NIL && y.r <= rp) {
+                    ++chain; rp = y.r; q = y.pv;
+                    if (q != NIL) y = P[q];
+                }
+                uint32_t chain_r = 0;
+                rp = x.r; q = x.nx;
+                y = P[q != NIL ? q : (IT)i];
+                while (q != NIL && y.r < rp) {
+                    ++chain_r; rp = y.r; q = y.nx;
+                    if (q != NIL) y = P[q];
+                }
+                merges = ((chain | chain_r) & 1u) == 0;
+            }
+            const uint64_t bal = __ballot(merges);
+            if (bal != 0) {                               // (uniform over the wave)
+                uint32_t at = 0;
+                if (lane == 0) at = atomicAdd(qn, (uint32_t)__builtin_popcountll(bal));
+                at = (uint32_t)__builtin_amdgcn_readfirstlane((int)at);
+                if (merges) Q[at + (uint32_t)__builtin_popcountll(bal & ((1ull << lane) - 1ull))] = (IT)i;
+            }
+            team_sync<NT>();
+        }
+        if (late != 0 && by_scan) {
             // Exact decision for every candidate of the round without walking to the left.  The
             // left chain of candidate i has even length iff x(i) = 0, where x runs over the live
             // positions from left to right: x(i) = x(left neighbour) ^ 1 if that neighbour is a
@@ -400,8 +443,8 @@ __device__ __forceinline__ void bpe_row(
             // from two ballots, with the bit carried from wave to wave and from block to block.
             constexpr int NW = NT / 64;
             const int lane = tid & 63;
-            team_sync<NT>();                            // everyone has read the flag
-            if (tid == 0) { *qn = 0; *capf = 0; }
+            team_sync<NT>();                            // everyone has read the count
+            if (tid == 0) *qn = 0;
             team_sync<NT>();
             uint32_t carry = 0;                         // x of the last live position before the block
             int blk = 0;
@@ -514,7 +557,7 @@ __device__ __forceinline__ void bpe_row(
             }
         }
         team_sync<NT>();
-        if (tid == 0) { *qn = 0; *cn = 0; }        // seen by the next round's decide (a sync lies between)
+        if (tid == 0) { *qn = 0; *cn = 0; *capf = 0; }   // seen by the next round's decide (a sync lies between)
 
         if (D[tid]) {
             D[tid] = 0;
