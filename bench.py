@@ -670,6 +670,51 @@ def pathological_extra():
     return out
 
 
+def merge_table_placement_extra():
+    """The BPE merge table of the 4096 vocabulary in global memory (L2; the default) against its compact
+    48 KB form kept in LDS by every workgroup (`dnatok_bpe_set_table_placement`), on batches of 1 KB rows:
+    512 rows (one per workgroup resident with the table in LDS) and the C3 batch of 1024 rows (two rounds
+    of workgroups with the table in LDS).  Tokens compared between the placements and, for C3, with the
+    golden vectors."""
+    import torch
+    from dnatok_amd import _lib, bpe_vocab, encoders
+    from tests.golden import check as util
+    from tests.support import hf_tokenizers as hf, workloads as wl
+    with open(hf.bpe_tokenizer_path("4096")) as fh:
+        cfg = json.load(fh)
+    kv = bpe_vocab.KernelVocab(bpe_vocab.split_merges(cfg["model"]["merges"]))
+    vocab = cfg["model"]["vocab"]
+    enc = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv), out_remap=kv.remap_to(vocab, vocab["[UNK]"]))
+    place = _lib.lib().dnatok_bpe_set_table_placement
+    out = {}
+    try:
+        for rows in (512, 1024):
+            b = wl.config3_bpe4096() if rows == 1024 else wl.config3_bpe4096(rows, 1024, seed=wl.SEEDS["C3"] + 7)
+            data, off = _dev(b.data), _dev(b.offsets)
+            tok = torch.empty(b.total, dtype=torch.int32, device="cuda")
+            lengths = torch.empty(rows, dtype=torch.int32, device="cuda")
+            seen = {}
+            for name, mode in (("global_memory", 0), ("lds", 2)):
+                assert place(mode) == 0
+                enc.encode(data, off, 1024, tok_tmp=tok, lengths=lengths)
+                torch.cuda.synchronize()
+                ln = lengths.cpu().numpy()
+                flat = tok.cpu().numpy()
+                seen[name] = [flat[b.offsets[i]:b.offsets[i] + ln[i]].copy() for i in range(rows)]
+
+                class W:
+                    def step(self):
+                        enc.encode(data, off, 1024, tok_tmp=tok, lengths=lengths)
+                _, dm = time_steps(W(), 20, 3)
+                out[f"{rows}_rows_{name}_us"] = dm * 1e3
+            same_rows(seen["lds"], seen["global_memory"], f"merge table placement, {rows} rows")
+            if rows == 1024:
+                util.check_against_golden("C3_bpe4096", seen["lds"])
+    finally:
+        place(0)
+    return out
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -678,6 +723,8 @@ def main() -> None:
     ap.add_argument("--config", default="C2", choices=["C1", "C2", "C3", "C4", "C5"])
     ap.add_argument("--per-call", action="store_true", help="time one exact batch instead of the sustained form")
     ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--only-extra", default="", choices=["", "merge_table_placement", "pathological"],
+                    help="run only this extra after the headline (for profiling it)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, the known-size kernel that the "
@@ -754,7 +801,10 @@ def main() -> None:
         result["oracle_port_cpu"] = {"value": v, "unit": "Mbp/s", "cores": 1, "kind": "port",
                                      "sample": sample + " (C restatement used by the tests, one thread)"}
 
-    if not args.no_extras:
+    if args.only_extra:
+        result[args.only_extra] = {"merge_table_placement": merge_table_placement_extra,
+                                   "pathological": pathological_extra}[args.only_extra]()
+    elif not args.no_extras:
         per_call = {}
         for cfg in ["C1", "C2", "C3", "C4", "C5"]:
             ww = make_workload(cfg, sustained=False)
@@ -804,6 +854,7 @@ def main() -> None:
         result["unpack_2bit"] = unpack_2bit_extra()
         result["device_normalizer"] = device_normalizer_extra()
         result["pathological"] = pathological_extra()
+        result["merge_table_placement"] = merge_table_placement_extra()
 
     print(json.dumps(result), flush=True)
 

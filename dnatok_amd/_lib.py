@@ -22,7 +22,7 @@ EXPORTS = [
     "dnatok_kmer_table_create", "dnatok_kmer_table_destroy", "dnatok_kmer_encode_padded",
     "dnatok_bpe_table_create", "dnatok_bpe_table_destroy", "dnatok_bpe_scratch_bytes",
     "dnatok_bpe_encode", "dnatok_bpe_static_scratch_bytes", "dnatok_bpe_encode_static",
-    "dnatok_bpe_set_chunk_geometry", "dnatok_pack_ragged", "dnatok_pad_rows", "dnatok_pad_rows_as",
+    "dnatok_bpe_set_chunk_geometry", "dnatok_bpe_set_table_placement", "dnatok_pack_ragged", "dnatok_pad_rows", "dnatok_pad_rows_as",
     "dnatok_normalize_bounds", "dnatok_normalize_rows",
 ]
 
@@ -103,6 +103,7 @@ def lib() -> ctypes.CDLL:
     L.dnatok_bpe_encode_static.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                            c_void_p, c_void_p, c_void_p]
     L.dnatok_bpe_set_chunk_geometry.argtypes = [c_int32, c_int32]
+    L.dnatok_bpe_set_table_placement.argtypes = [c_int32]
     L.dnatok_pack_ragged.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_void_p]
     L.dnatok_pad_rows.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int32, c_int64,

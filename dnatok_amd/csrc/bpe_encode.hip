@@ -47,6 +47,8 @@ struct dnatok_bpe_table {
     uint4 *tab;                  // [slots]  {key = a << 16 | b, rank, product | gate << 16, 0}
     uint16_t *byte_to_sym;       // [256]
     int32_t *out_remap;          // [n_symbols] or nullptr
+    uint32_t *ltab;              // the compact form of the table that fits LDS (kLdsTabWords words), or nullptr
+    uint32_t lmul1, lmul2;       // its two multipliers
 };
 
 namespace dnatok {
@@ -60,6 +62,8 @@ struct BpeArgs {
     const int32_t *out_remap;
     uint32_t shift, mul1, mul2;
     int32_t n_merges;
+    const uint32_t *ltab;
+    uint32_t lmul1, lmul2;
 };
 
 // What a position keeps about the pair it starts: the rule's rank (kNone = no rule), the
@@ -108,6 +112,58 @@ __device__ __forceinline__ PairInfo pair_finish(uint32_t a, uint32_t b, const Pa
     const uint32_t y = first ? pr.e1.y : pr.e2.y, z = first ? pr.e1.z : pr.e2.z;
     if (!first && pr.e2.x != key) return PairInfo{kNone, kNone, kNone};
     return PairInfo{y, z & 0xFFFFu, z >> 16};
+}
+
+// The compact form of the merge table, for tables of at most 8192 symbols and 4095 rules: small
+// enough (48 KB) for a workgroup to keep in LDS when a batch leaves that much room.  A pair's key has
+// 26 bits (two 13-bit symbols); key * odd multiplier mod 2^26 is a bijection, whose upper 13 bits are
+// the slot and whose lower 13 bits are kept in the slot, together with which of the two functions
+// placed the rule there: slot number, remainder and function give the key back, so a matching
+// remainder is a matching key.  Slot word: rank << 15 | remainder << 2 | function << 1 | 1 (0 = empty).
+// Product and gate of a rule are looked up by its rank in a second array.
+constexpr int kLdsTabSlots = 8192;
+constexpr int kLdsTabRanks = 4096;
+constexpr int kLdsTabWords = kLdsTabSlots + kLdsTabRanks;      // 48 KB
+
+struct LdsPairTable {
+    const uint32_t *tab;         // [kLdsTabSlots], in LDS
+    const uint32_t *pg;          // [kLdsTabRanks] product | gate << 16, in LDS
+    uint32_t mul1, mul2;
+};
+
+struct LdsPairProbe {
+    uint32_t e1, e2, want1, want2;
+};
+
+__host__ __device__ __forceinline__ uint32_t lds_pair_hash(uint32_t key24, uint32_t mul)
+{
+    return (key24 * mul) & 0x3FFFFFFu;
+}
+
+__device__ __forceinline__ LdsPairProbe pair_probe(const LdsPairTable &t, uint32_t a, uint32_t b)
+{
+    const uint32_t key = ((a & 0x1FFFu) << 13) | (b & 0x1FFFu);
+    const uint32_t h1 = lds_pair_hash(key, t.mul1), h2 = lds_pair_hash(key, t.mul2);
+    LdsPairProbe pr;
+    pr.e1 = t.tab[h1 >> 13];
+    pr.e2 = t.tab[h2 >> 13];
+    pr.want1 = ((h1 & 0x1FFFu) << 2) | 1u;
+    pr.want2 = ((h2 & 0x1FFFu) << 2) | 3u;
+    return pr;
+}
+
+__device__ __forceinline__ PairInfo pair_finish(const LdsPairTable &t, uint32_t, uint32_t, const LdsPairProbe &pr)
+{
+    const bool first = (pr.e1 & 0x7FFFu) == pr.want1;
+    if (!first && (pr.e2 & 0x7FFFu) != pr.want2) return PairInfo{kNone, kNone, kNone};
+    const uint32_t rank = (first ? pr.e1 : pr.e2) >> 15;
+    const uint32_t pg = t.pg[rank];
+    return PairInfo{rank, pg & 0xFFFFu, pg >> 16};
+}
+
+__device__ __forceinline__ PairInfo pair_finish(const PairTable &, uint32_t a, uint32_t b, const PairProbe &pr)
+{
+    return pair_finish(a, b, pr);
 }
 
 template <int NT>
@@ -174,9 +230,9 @@ struct alignas(4 * sizeof(IT)) PosRec {
 // One row.  tid = index in the team; P/NS/MC hold n0 entries, Q (the merges of the current round)
 // n0 / 2, C (its candidates) n0; D holds NT bytes; PER > 0 says that n0 <= PER * NT, and every thread
 // then keeps the ranks of its own positions in registers as well; red holds 4 * (NT / 64) + 4 words.  Tokens go to out[0 .. *out_len).
-template <int NT, typename IT, int PER>
+template <int NT, typename IT, int PER, typename PT>
 __device__ __forceinline__ void bpe_row(
-    const PairTable pt, const uint16_t *byte_to_sym,
+    const PT pt, const uint16_t *byte_to_sym,
     const int32_t *out_remap, const uint8_t *__restrict__ src, const int n0, PosRec<IT> *P,
     uint16_t *NS, uint16_t *MC, IT *Q, IT *C, uint8_t *D, uint32_t *red, const int tid,
     int32_t *__restrict__ out, int32_t *__restrict__ out_len, uint16_t *__restrict__ raw_out = nullptr,
@@ -238,7 +294,7 @@ __device__ __forceinline__ void bpe_row(
     }
     auto byte_at = [&](int i) -> uint32_t { return PER > 0 ? stage[head + i] : src[i]; };
     for (int i0 = tid; i0 < n0; i0 += kProbes * NT) {
-        PairProbe e[kProbes];
+        decltype(pair_probe(pt, 0u, 0u)) e[kProbes];
         uint32_t sa[kProbes], sb[kProbes];
 #pragma unroll
         for (int j = 0; j < kProbes; ++j) {
@@ -253,7 +309,7 @@ __device__ __forceinline__ void bpe_row(
             const int i = i0 + j * NT;
             if (i >= n0) continue;
             PairInfo pi{kNone, kNone, kNone};
-            if (i + 1 < n0) pi = pair_finish(sa[j], sb[j], e[j]);
+            if (i + 1 < n0) pi = pair_finish(pt, sa[j], sb[j], e[j]);
             PosRec<IT> x;
             x.r = (IT)pi.rank;
             x.nx = (i + 1 < n0) ? (IT)(i + 1) : NIL;
@@ -525,7 +581,7 @@ __device__ __forceinline__ void bpe_row(
         // neighbour), probe 2m + 1 the pair (left neighbour, new).  The probes are dealt evenly to
         // the threads, kProbes pairs of table reads in flight per thread.
         for (int p0 = tid; p0 < 2 * nm; p0 += kProbes * NT) {
-            PairProbe e[kProbes];
+            decltype(pair_probe(pt, 0u, 0u)) e[kProbes];
             uint32_t sa[kProbes], sb[kProbes];
             IT target[kProbes];
             bool valid[kProbes];
@@ -550,7 +606,7 @@ __device__ __forceinline__ void bpe_row(
             for (int j = 0; j < kProbes; ++j) {
                 if (target[j] == NIL) continue;       // no probe, or no left neighbour
                 PairInfo pi{kNone, kNone, kNone};
-                if (valid[j]) pi = pair_finish(sa[j], sb[j], e[j]);
+                if (valid[j]) pi = pair_finish(pt, sa[j], sb[j], e[j]);
                 const int q = (int)target[j];
                 P[q].r = (IT)pi.rank; NS[q] = (uint16_t)pi.product; MC[q] = (uint16_t)pi.gate;
                 D[q % NT] = 1;
@@ -693,6 +749,7 @@ static size_t long_slab_bytes(int64_t max_len)
 // above; dnatok_bpe_set_chunk_geometry lets a test run the chunk / seam / fallback machinery with
 // chunks so small that every few hundred bytes of a row hold a seam.
 static std::atomic<int> g_chunk_core{kChunkCore}, g_chunk_overlap{kChunkOverlap};
+static std::atomic<int> g_table_placement{0};      // dnatok_bpe_set_table_placement
 
 // A batch whose long rows make far fewer chunks than teams fit the chip (a few rows of a few
 // thousand bytes each) is cut finer, down to a core of 512 bytes: more, shorter items run side by
@@ -888,7 +945,7 @@ __global__ __launch_bounds__(256) void bpe_expand_kernel(const int64_t *__restri
 // workgroup shares an item.  PLANNED: the items are those of the work list (rows and chunks of
 // long rows), handed out through an atomic counter.  Otherwise (no row of the batch is longer
 // than CAP) an item is a row, teams take rows round robin, and no work list is built at all.
-template <int NT, int TEAMS, int CAP, bool PLANNED>
+template <int NT, int TEAMS, int CAP, bool PLANNED, bool LTAB = false>
 __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     BpeArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
     BpePlan p, int32_t n_rows, int32_t *__restrict__ tok_tmp, int32_t *__restrict__ lengths)
@@ -906,7 +963,17 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     uint16_t *MC = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
     uint16_t *Q = reinterpret_cast<uint16_t *>(sp) + (size_t)team * (CAP / 2); sp += (size_t)TEAMS * CAP;
     uint16_t *C = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
-    uint8_t *D = sp + (size_t)team * NT;
+    uint8_t *D = sp + (size_t)team * NT; sp += (size_t)TEAMS * NT;
+    // LTAB: the workgroup keeps the compact form of the merge table in LDS (a copy per workgroup,
+    // brought in with 16-byte loads before the first row)
+    uint32_t *ltab = nullptr;
+    if (LTAB) {
+        ltab = reinterpret_cast<uint32_t *>(smem + ((sp - smem + 15) & ~(ptrdiff_t)15));
+        const uint4 *src4 = reinterpret_cast<const uint4 *>(a.ltab);
+        uint4 *dst4 = reinterpret_cast<uint4 *>(ltab);
+        for (int i = threadIdx.x; i < kLdsTabWords / 4; i += NT * TEAMS) dst4[i] = src4[i];
+    }
+    const LdsPairTable lpt{ltab, ltab + kLdsTabSlots, a.lmul1, a.lmul2};
     __syncthreads();
 
     const int32_t n_items = PLANNED ? p.counts[0] : n_rows;
@@ -954,8 +1021,12 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
             // too long: left to the whole-row kernel (row_fail is set); empty: no tokens
             if (tid == 0) lengths[row] = len > CAP ? -1 : 0;
         } else if (nc == 1) {
-            bpe_row<NT, uint16_t, (CAP + NT - 1) / NT>(pt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC,
-                                  Q, C, D, red, tid, tok_tmp + start, lengths + row);
+            if (LTAB)
+                bpe_row<NT, uint16_t, (CAP + NT - 1) / NT>(lpt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC,
+                                      Q, C, D, red, tid, tok_tmp + start, lengths + row);
+            else
+                bpe_row<NT, uint16_t, (CAP + NT - 1) / NT>(pt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC,
+                                      Q, C, D, red, tid, tok_tmp + start, lengths + row);
         } else {
             const int64_t e0 = (int64_t)k * p.core - p.overlap < 0 ? 0 : (int64_t)k * p.core - p.overlap;
             int64_t e1 = (int64_t)(k + 1) * p.core + p.overlap;
@@ -1247,15 +1318,52 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
     std::vector<uint16_t> b2s(256);
     for (int i = 0; i < 256; ++i) b2s[i] = (uint16_t)byte_to_id_h[i];
 
+    // the compact form for LDS (see LdsPairTable), when symbols and ranks fit 12 bits
+    std::vector<uint32_t> ltab;
+    uint32_t lmul1 = 0, lmul2 = 0;
+    if (n_symbols <= 8192 && n_merges <= kLdsTabRanks - 1 && n_merges > 0) {
+        static const uint32_t kMul24[6] = {0x29E3779u, 0x185EBCBu, 0x3C2B2AFu, 0x227D4EBu, 0x1165667u, 0x2D3A265u};   // odd, 26 bits
+        for (int attempt = 0; attempt < 3 && ltab.empty(); ++attempt) {
+            lmul1 = kMul24[2 * attempt]; lmul2 = kMul24[2 * attempt + 1];
+            std::vector<uint32_t> slot(kLdsTabSlots, 0), key_of(kLdsTabSlots, 0), pg(kLdsTabRanks, kNone | (kNone << 16));
+            bool placed = true;
+            for (int32_t i = 0; i < n_merges && placed; ++i) {
+                const uint32_t pa = (uint32_t)pair_a_h[i], pb = (uint32_t)pair_b_h[i];
+                if (last_entry[(pa << 16) | pb] != i) continue;
+                const uint32_t fu = first_use[new_id_h[i]];
+                pg[i] = (uint32_t)new_id_h[i] | ((fu == 0xFFFFFFFFu ? kNone : fu) << 16);
+                uint32_t key = (pa << 13) | pb, rank = (uint32_t)i, came_from = 0xFFFFFFFFu;
+                placed = false;
+                for (int kick = 0; kick < 512; ++kick) {
+                    const uint32_t h1 = lds_pair_hash(key, lmul1), h2 = lds_pair_hash(key, lmul2);
+                    const uint32_t s1 = h1 >> 13, s2 = h2 >> 13;
+                    const uint32_t w1 = (rank << 15) | ((h1 & 0x1FFFu) << 2) | 1u, w2 = (rank << 15) | ((h2 & 0x1FFFu) << 2) | 3u;
+                    if (slot[s1] == 0) { slot[s1] = w1; key_of[s1] = key; placed = true; break; }
+                    if (slot[s2] == 0) { slot[s2] = w2; key_of[s2] = key; placed = true; break; }
+                    const uint32_t v = (s1 == came_from) ? s2 : s1;        // push out the rule of the other slot
+                    const uint32_t out_key = key_of[v], out_rank = slot[v] >> 15;
+                    slot[v] = v == s1 ? w1 : w2; key_of[v] = key;
+                    key = out_key; rank = out_rank; came_from = v;
+                }
+            }
+            if (placed) {
+                ltab = slot;
+                ltab.insert(ltab.end(), pg.begin(), pg.end());
+            }
+        }
+    }
+
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
     const size_t o_tab = 0;
     const size_t o_b2s = up(o_tab + (size_t)slots * sizeof(uint4));
     const size_t o_remap = up(o_b2s + 512);
-    const size_t total = up(o_remap + (out_remap_h ? (size_t)n_symbols * 4 : 0)) + 256;
+    const size_t o_ltab = up(o_remap + (out_remap_h ? (size_t)n_symbols * 4 : 0));
+    const size_t total = up(o_ltab + ltab.size() * 4) + 256;
     std::vector<uint8_t> host(total, 0);
     memcpy(&host[o_tab], tab.data(), (size_t)slots * sizeof(uint4));
     memcpy(&host[o_b2s], b2s.data(), 512);
     if (out_remap_h) memcpy(&host[o_remap], out_remap_h, (size_t)n_symbols * 4);
+    if (!ltab.empty()) memcpy(&host[o_ltab], ltab.data(), ltab.size() * 4);
     void *blob = nullptr;
     hipError_t e = hipMalloc(&blob, total);
     if (e == hipSuccess) e = hipMemcpy(blob, host.data(), total, hipMemcpyHostToDevice);
@@ -1271,6 +1379,8 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
     t->tab = (uint4 *)(b + o_tab);
     t->byte_to_sym = (uint16_t *)(b + o_b2s);
     t->out_remap = out_remap_h ? (int32_t *)(b + o_remap) : nullptr;
+    t->ltab = ltab.empty() ? nullptr : (uint32_t *)(b + o_ltab);
+    t->lmul1 = lmul1; t->lmul2 = lmul2;
     *out = t;
     return DNATOK_OK;
 }
@@ -1284,6 +1394,13 @@ extern "C" int dnatok_bpe_set_chunk_geometry(int32_t core, int32_t overlap)
                    "core + 2 * overlap <= %d", kLdsCap);
     g_chunk_core.store(core, std::memory_order_relaxed);
     g_chunk_overlap.store(overlap, std::memory_order_relaxed);
+    return DNATOK_OK;
+}
+
+extern "C" int dnatok_bpe_set_table_placement(int32_t mode)
+{
+    DNATOK_REQUIRE(mode >= 0 && mode <= 2, DNATOK_E_INVALID, "dnatok_bpe_set_table_placement: mode is 0, 1 or 2");
+    g_table_placement.store(mode, std::memory_order_relaxed);
     return DNATOK_OK;
 }
 
@@ -1341,6 +1458,43 @@ int launch_lds_as(const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets
     return DNATOK_OK;
 }
 
+// Where the merge table is kept (dnatok_bpe_set_table_placement): 0 = in global memory (L2), always;
+// 1 = the compact form in LDS when the table has one, no row is longer than 1024 bytes and the batch
+// leaves the room for it (at most one row per team resident with the table's 48 KB added to every
+// workgroup); 2 = the compact form for every such batch, whatever its size.  0 is the default because
+// it measured faster: bringing 48 KB into every workgroup costs more than the lookups save (256 rows
+// of 1 KB: 23.8 us against 25.1 us with the table in LDS, 512 rows: 25.7 against 26.7; 1024 rows, which
+// then need two rounds of workgroups: 30.4 against 49.4).
+// The unplanned 1 KB form of the LDS kernel with the compact table in LDS.
+template <int NT, int TEAMS, int CAP>
+int64_t ltab_resident_teams()
+{
+    static const int resident = resident_workgroups(bpe_lds_kernel<NT, TEAMS, CAP, false, true>, NT * TEAMS,
+                                                    lds_bytes<NT, TEAMS, CAP>() + kLdsTabWords * 4 + 16, 1);
+    return (int64_t)resident * TEAMS;
+}
+
+template <int NT, int TEAMS, int CAP>
+int launch_lds_ltab(const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets, const BpePlan &p,
+                    int64_t n_rows, int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
+{
+    const size_t lds = lds_bytes<NT, TEAMS, CAP>() + kLdsTabWords * 4 + 16;
+    auto kern = bpe_lds_kernel<NT, TEAMS, CAP, false, true>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        DNATOK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_set = true;
+    }
+    int64_t grid = (n_rows + TEAMS - 1) / TEAMS;
+    const int64_t resident = ltab_resident_teams<NT, TEAMS, CAP>() / TEAMS;
+    if (grid > resident) grid = resident;
+    if (grid < 1) grid = 1;
+    kern<<<(int)grid, NT * TEAMS, lds, s>>>(a, bytes, offsets, p, (int32_t)n_rows, tok_tmp, lengths);
+    DNATOK_HIP_TRY(hipGetLastError());
+    return DNATOK_OK;
+}
+
 // The work list (plan) is needed when rows are cut into chunks or left to the whole-row kernel,
 // and when there are more rows than resident teams: rows then are dealt through the list's
 // counter, since rows take different times and a fixed share per team ends in a long tail
@@ -1350,6 +1504,11 @@ template <int NT, int TEAMS, int CAP>
 int run_lds(bool long_rows, int chunking, const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets,
             const BpePlan &p, int64_t n_rows, int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
 {
+    if (CAP == 1024 && !long_rows && a.ltab) {
+        const int mode = g_table_placement.load(std::memory_order_relaxed);
+        if (mode == 2 || (mode == 1 && n_rows <= ltab_resident_teams<NT, TEAMS, 1024>()))
+            return launch_lds_ltab<NT, TEAMS, 1024>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    }
     const bool planned = long_rows || n_rows > lds_resident_teams<NT, TEAMS, CAP>();
     if (planned) {
         const int expand_here = chunking >> 1;
@@ -1370,7 +1529,7 @@ int run_lds(bool long_rows, int chunking, const BpeArgs &a, const uint8_t *bytes
 static int bpe_encode_launch(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets, int64_t n_rows,
                              int64_t max_len, const BpePlan &p, int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
 {
-    BpeArgs a{t->tab, t->byte_to_sym, t->out_remap, t->shift, t->mul1, t->mul2, t->n_merges};
+    BpeArgs a{t->tab, t->byte_to_sym, t->out_remap, t->shift, t->mul1, t->mul2, t->n_merges, t->ltab, t->lmul1, t->lmul2};
 
     const bool long_rows = max_len > p.ext;
     int chunking = (long_rows && t->monotone) ? 1 : 0;

@@ -219,6 +219,15 @@ int dnatok_bpe_encode_static(const dnatok_bpe_t *t, const uint8_t *bytes, const 
  * Not synchronised with encode calls in flight on other threads. */
 int dnatok_bpe_set_chunk_geometry(int32_t core, int32_t overlap);
 
+/* Where the merge table of the calls that follow is kept (process-wide; no counterpart in the
+ * reference, whose kernel reads its hash table from global memory, dnatok_bpe.cu:822-837).  A table
+ * of at most 8192 symbols and 4095 rules also has a compact form of 48 KB.  mode 0 (default): every
+ * batch reads the table from global memory (L2), which measured faster.  mode 1: a batch of rows of
+ * at most 1024 bytes, few enough for one row per resident workgroup with those 48 KB added to each,
+ * is encoded by workgroups that keep the compact form in LDS.  mode 2: the compact form for every
+ * batch of rows of at most 1024 bytes (for measurements).  Results are identical in all modes. */
+int dnatok_bpe_set_table_placement(int32_t mode);
+
 /* ---------------------------------------------------------------------------------------
  * Ragged-batch packer: turns per-row token runs (tok_tmp + in_offsets + lengths, as the BPE
  * engine leaves them) into the tensors a model consumes, without a host round trip.

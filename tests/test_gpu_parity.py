@@ -525,6 +525,34 @@ def test_bpe_small_chunks_many_seams_and_fallbacks(bpe, core, overlap):
         _lib.check(L.dnatok_bpe_set_chunk_geometry(0, 0), "dnatok_bpe_set_chunk_geometry")
 
 
+def test_bpe_compact_table_in_lds_gives_the_same_tokens():
+    """The 4096 vocabulary has a compact form that workgroups keep in LDS for batches of short rows
+    that leave the room (not the default: it measured slower).  Same tokens as with the table in
+    global memory and as the oracle: a batch small enough for one row per resident workgroup, and the C3
+    batch with the compact form forced."""
+    from dnatok_amd import _lib
+    say("bpe4096 compact table in LDS")
+    cfg = util.tokenizer_json("4096")
+    kv = bpe_vocab.KernelVocab(bpe_vocab.split_merges(cfg["model"]["merges"]))
+    enc = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv), out_remap=kv.remap_to(cfg["model"]["vocab"], 0))
+    bo = util.bpe_oracle("4096")
+    rng = random.Random(5)
+    seqs = ["".join(rng.choices("ACGTN", weights=[24, 24, 24, 24, 1], k=rng.choice([1, 2, 7, 64, 500, 1000, 1023, 1024])))
+            for _ in range(300)] + ["A" * 1024, "AC" * 512, ""]
+    small = util.batch_from_strings(seqs)
+    want = [np.asarray(r) for r in bo.encode_batch(small.data, small.offsets)]
+    place = _lib.lib().dnatok_bpe_set_table_placement
+    try:
+        for mode in (0, 1, 2):
+            assert place(mode) == 0
+            for s, r, e in zip(seqs, bpe_rows(enc, small), want):
+                np.testing.assert_array_equal(r, e, err_msg=f"mode {mode}: {s[:20]}")
+            util.check_against_golden("C3_bpe4096", bpe_rows(enc, wl.config3_bpe4096()))
+        assert place(3) != 0
+    finally:
+        place(0)
+
+
 def test_bpe_c4_golden():
     say("bpe32000 C4 32x100k")
     cfg = util.tokenizer_json("32000")
