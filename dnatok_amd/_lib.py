@@ -19,7 +19,7 @@ EXPORTS = [
     "dnatok_char_encode_padded", "dnatok_char_encode_padded_as", "dnatok_char_encode_packed",
     "dnatok_char_embed_packed",
     "dnatok_char_unpack_2bit", "dnatok_host_clean_ascii", "dnatok_host_pack_2bit", "dnatok_host_fasta_scan",
-    "dnatok_kmer_table_create", "dnatok_kmer_table_destroy", "dnatok_kmer_encode_padded",
+    "dnatok_kmer_table_create", "dnatok_kmer_table_destroy", "dnatok_kmer_set_team_rows", "dnatok_kmer_encode_padded",
     "dnatok_bpe_table_create", "dnatok_bpe_table_destroy", "dnatok_bpe_scratch_bytes",
     "dnatok_bpe_encode", "dnatok_bpe_static_scratch_bytes", "dnatok_bpe_encode_static",
     "dnatok_bpe_set_chunk_geometry", "dnatok_bpe_set_table_placement", "dnatok_pack_ragged", "dnatok_pad_rows", "dnatok_pad_rows_as",
@@ -89,6 +89,7 @@ def lib() -> ctypes.CDLL:
                                            c_int64, c_void_p, c_int32, c_int32, POINTER(c_void_p)]
     L.dnatok_kmer_table_destroy.argtypes = [c_void_p]
     L.dnatok_kmer_table_destroy.restype = None
+    L.dnatok_kmer_set_team_rows.argtypes = [c_int32]
     L.dnatok_kmer_encode_padded.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
     L.dnatok_bpe_table_create.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32,

@@ -28,7 +28,9 @@
 
 #include <limits.h>
 #include <string.h>
+#include <atomic>
 #include <mutex>
+#include <stdlib.h>
 #include <unordered_map>
 #include <vector>
 
@@ -57,6 +59,10 @@ struct dnatok_kmer_table {
 };
 
 constexpr int kMaxSlots = 64;
+
+// Batches of up to this many rows are encoded by kmer_team_kernel (a workgroup per row); -1: as
+// many rows as workgroups of that kernel fit the chip at once.  (dnatok_kmer_set_team_rows)
+static std::atomic<int> g_team_rows{-1};
 constexpr int kMaxSlotStride = 32;       // 64-bit words between two slots (one 256-byte line each)
 
 namespace dnatok {
@@ -535,6 +541,347 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
     }
 }
 
+// ---- few rows: a workgroup per row ---------------------------------------------------------------
+//
+// With fewer rows than workgroups fit the chip (one 256-row batch), a wave per row leaves most of
+// the chip idle while every wave walks its row step by step.  Here the four waves of a workgroup
+// share a row: wave w takes steps w, w + 4, ...; the token counts of the four steps of a round go
+// through LDS, so that every wave knows where its tokens start.  A wave writes its run by itself,
+// whole 16-byte groups and single cells at both ends (no waiting for whole lines as in
+// kmer_rows_kernel: this kernel is for batches that are bound by latency, not by bandwidth).
+// The padding pass stays a launch of its own: letting the workgroup that finishes last do it
+// (a ticket counter behind a device-scope fence) measured 39 us per call instead of 15, because
+// such a fence writes back the L2 of the workgroup's XCD.
+template <int K, bool LUT4_LDS, bool CHARS, bool HAS_MASK>
+__global__ __launch_bounds__(kKmerThreads) void kmer_team_kernel(
+    KmerArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
+    int64_t n_rows, int64_t t_cap, int64_t fill_to, int32_t *__restrict__ ids,
+    uint8_t *__restrict__ mask, int32_t *__restrict__ lengths, int32_t *__restrict__ status,
+    int32_t *__restrict__ max_len, MaxRef mref)
+{
+    constexpr uint32_t POW4 = 1u << (2 * K);
+    constexpr int NWV = kKmerThreads / 64;
+    __shared__ uint32_t s_dig[256];
+    __shared__ int32_t s_single[256];
+    __shared__ __attribute__((aligned(16))) int32_t s_lut4[LUT4_LDS ? POW4 : 4];
+    __shared__ int32_t s_spell[256];
+    __shared__ __attribute__((aligned(16))) int32_t s_stage[NWV][kStageWords];
+    __shared__ uint32_t s_tot[2][NWV];
+    __shared__ int32_t s_stat[NWV];
+
+    const int lane = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    // The kernel's life is a few trips to memory, so they are made to overlap: the bytes of the
+    // workgroup's first row are requested first, then the tables (the id table with 16-byte loads,
+    // all in flight together), and only then does anyone wait.
+    uint32_t w_first[K];
+#pragma unroll
+    for (int i = 0; i < K; ++i) w_first[i] = 0;
+    if ((int64_t)blockIdx.x < n_rows) {
+        const int64_t row_start = offsets[blockIdx.x];
+        const int len = (int)(offsets[blockIdx.x + 1] - row_start);
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint8_t *>(bytes + row_start), (short)0, len, 0x00020000);
+        const int off = (wv * kWaveUnits + lane * kUnitsPerLane) * K;
+        int i = 0;
+#pragma unroll
+        for (; i + 4 <= K; i += 4) {
+            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, off + 4 * i, 0, 0);
+            w_first[i] = v.x; w_first[i + 1] = v.y; w_first[i + 2] = v.z; w_first[i + 3] = v.w;
+        }
+        if (i + 2 <= K) {
+            const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rs, off + 4 * i, 0, 0);
+            w_first[i] = v.x; w_first[i + 1] = v.y;
+            i += 2;
+        }
+        if (i < K) w_first[i] = __builtin_amdgcn_raw_buffer_load_b32(rs, off + 4 * i, 0, 0);
+    }
+    if (LUT4_LDS) {
+        constexpr int kVec = POW4 / 4;                               // 16-byte pieces of the id table
+        constexpr int kPer = (kVec + kKmerThreads - 1) / kKmerThreads;
+        const uint4 *src4 = reinterpret_cast<const uint4 *>(a.lut4);
+        uint4 v[kPer];
+#pragma unroll
+        for (int q = 0; q < kPer; ++q) {
+            const int at = (int)threadIdx.x + q * kKmerThreads;
+            v[q] = at < kVec ? src4[at] : uint4{0, 0, 0, 0};
+        }
+        uint4 *dst4 = reinterpret_cast<uint4 *>(s_lut4);
+#pragma unroll
+        for (int q = 0; q < kPer; ++q) {
+            const int at = (int)threadIdx.x + q * kKmerThreads;
+            if (at < kVec) dst4[at] = v[q];
+        }
+    }
+    for (int i = threadIdx.x; i < 256; i += kKmerThreads) {
+        const int d = a.digit[i];
+        s_dig[i] = d < 0 ? kDigBad : (d >= 4 ? kDigN : (uint32_t)d);
+        s_single[i] = a.single[i];
+        s_spell[i] = a.single[(int)"ACGTN"[d < 0 || d > 4 ? 4 : d]];
+    }
+    __syncthreads();
+
+    int32_t *const buf = s_stage[wv];
+    const int cap = t_cap > INT_MAX - 16 ? INT_MAX - 16 : (int)t_cap;
+    const int fill = fill_to > cap ? cap : (int)fill_to;
+    int64_t wg_max = 0;
+    const unsigned long long slot_gen = mref.slot ? mref.slot[1] : 0ull;
+
+    for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
+        const int64_t row_start = offsets[row];
+        const int len = (int)(offsets[row + 1] - row_start);
+        const int full = len / K;
+        const int n_units = full + (len - full * K);
+        const uint8_t *src = bytes + row_start;
+        int32_t *out = ids + row * t_cap;
+        const int mis = (int)((reinterpret_cast<uintptr_t>(out) >> 2) & 3);
+        int32_t *outA = out - mis;
+        uint8_t *moutA = HAS_MASK ? mask + row * t_cap - mis : nullptr;
+        const int hi_cap = mis + cap;
+        int running = 0;
+        int32_t my_status = 0;
+        const __amdgpu_buffer_rsrc_t rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(src), (short)0, len, 0x00020000);
+
+        int par = 0;
+        for (int r0 = 0; r0 < n_units; r0 += NWV * kWaveUnits, par ^= 1) {     // the same rounds for every wave
+            const int u0 = r0 + wv * kWaveUnits;
+            const int ub = u0 + lane * kUnitsPerLane;
+            const bool lane_full = ub + kUnitsPerLane <= full;     // 4 whole windows
+            const bool empty = ub >= n_units;
+            uint32_t w[K];
+            if (row == (int64_t)blockIdx.x && r0 == 0) {
+#pragma unroll
+                for (int i = 0; i < K; ++i) w[i] = w_first[i];
+            } else {
+                const int off = ub * K;                            // reads past the row's end return 0
+                int i = 0;
+#pragma unroll
+                for (; i + 4 <= K; i += 4) {
+                    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off + 4 * i, 0, 0);
+                    w[i] = v.x; w[i + 1] = v.y; w[i + 2] = v.z; w[i + 3] = v.w;
+                }
+                if (i + 2 <= K) {
+                    const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, off + 4 * i, 0, 0);
+                    w[i] = v.x; w[i + 1] = v.y;
+                    i += 2;
+                }
+                if (i < K) w[i] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, off + 4 * i, 0, 0);
+            }
+            auto digit_of = [&](int bi) -> uint32_t { return s_dig[(w[bi >> 2] >> (8 * (bi & 3))) & 255u]; };
+            uint32_t code[kUnitsPerLane];
+            int32_t t[kUnitsPerLane];
+#pragma unroll
+            for (int j = 0; j < kUnitsPerLane; ++j) {
+                uint32_t c = 0;
+#pragma unroll
+                for (int i = 0; i < K; ++i) c = (c << 2) + digit_of(j * K + i);
+                code[j] = c;
+                const uint32_t idx = c & (POW4 - 1);
+                t[j] = LUT4_LDS ? s_lut4[idx] : a.lut4[idx];
+            }
+            const uint32_t any_flag = code[0] | code[1] | code[2] | code[3];
+            const bool fast = lane_full && any_flag < POW4 && (t[0] | t[1] | t[2] | t[3]) >= 0;
+
+            // tokens per unit and per lane (as in kmer_rows_kernel)
+            int32_t cnt[kUnitsPerLane], ex[kUnitsPerLane], ey[kUnitsPerLane];
+            uint32_t lane_cnt = 0;
+            if (fast) {
+                lane_cnt = kUnitsPerLane;
+            } else if (lane_full) {
+#pragma unroll
+                for (int j = 0; j < kUnitsPerLane; ++j) {
+                    ex[j] = 0; ey[j] = 0;
+                    if (code[j] < POW4 && t[j] >= 0) {
+                        cnt[j] = 1;
+                    } else if (CHARS) {
+                        cnt[j] = K;
+                    } else {
+                        int c5 = 0;
+#pragma unroll
+                        for (int i = 0; i < K; ++i) {
+                            const uint32_t v = digit_of(j * K + i);
+                            c5 = c5 * 5 + ((v & (kDigN | kDigBad)) ? 4 : (int)v);
+                        }
+                        const int2 e = a.entry[c5];
+                        ex[j] = e.x; ey[j] = e.y;
+                        cnt[j] = e.x >= 0 ? 1 : (e.x == INT_MIN ? 1 : -e.x);
+                        if (e.x == INT_MIN) my_status |= DNATOK_ROW_MISSING_KMER;
+                    }
+                    if ((code[j] >> 17) != 0) {
+                        bool bad = false;
+#pragma unroll
+                        for (int i = 0; i < K; ++i) bad = bad || (digit_of(j * K + i) & kDigBad);
+                        if (bad) my_status |= DNATOK_ROW_INVALID_BYTE;
+                    }
+                    lane_cnt += (uint32_t)cnt[j];
+                }
+            } else if (!empty) {
+#pragma unroll 1
+                for (int j = 0; j < kUnitsPerLane; ++j) {
+                    const int u = ub + j;
+                    int n = 0;
+                    if (u < full) {
+                        uint32_t c = 0;
+                        int c5 = 0;
+#pragma unroll
+                        for (int i = 0; i < K; ++i) {
+                            const uint32_t v = s_dig[src[u * K + i]];
+                            c = (c << 2) + v;
+                            if (v & kDigBad) my_status |= DNATOK_ROW_INVALID_BYTE;
+                            c5 = c5 * 5 + ((v & (kDigN | kDigBad)) ? 4 : (int)v);
+                        }
+                        int32_t id = -1;
+                        if (c < POW4) id = LUT4_LDS ? s_lut4[c] : a.lut4[c];
+                        if (id >= 0) {
+                            n = 1;
+                        } else {
+                            const int2 e = a.entry[c5];
+                            n = e.x >= 0 ? 1 : (e.x == INT_MIN ? 1 : -e.x);
+                            if (e.x == INT_MIN) my_status |= DNATOK_ROW_MISSING_KMER;
+                        }
+                    } else if (u < n_units) {
+                        n = 1;
+                    }
+                    lane_cnt += (uint32_t)n;
+                }
+            }
+            const uint32_t inc = wave_inclusive_sum_u32(lane_cnt);
+            const uint32_t step_total = __builtin_amdgcn_readlane(inc, 63);
+
+            // where the wave's run starts: the steps of the waves before it in this round
+            if (lane == 0) s_tot[par][wv] = step_total;
+            __syncthreads();
+            uint32_t before = 0, round_total = 0;
+#pragma unroll
+            for (int q = 0; q < NWV; ++q) {
+                const uint32_t v = s_tot[par][q];
+                before += q < wv ? v : 0u;
+                round_total += v;
+            }
+            const int A = mis + running + (int)before;             // cell the step's first token goes to
+            const int A_end = A + (int)step_total;
+            const int lo = A, hi = A_end < hi_cap ? A_end : hi_cap;
+            const uint32_t carry = (uint32_t)A & 3u;
+            const uint32_t n_avail = carry + step_total;
+            const uint32_t s0 = carry + (inc - lane_cnt);
+            const int e0 = A & ~3;
+
+            auto produce = [&](auto put) {
+                uint32_t s = s0;
+                if (fast) {
+#pragma unroll
+                    for (int j = 0; j < kUnitsPerLane; ++j) put(s + j, t[j]);
+                } else if (lane_full) {
+#pragma unroll
+                    for (int j = 0; j < kUnitsPerLane; ++j) {
+                        if (code[j] < POW4 && t[j] >= 0) {
+                            put(s, t[j]);
+                            ++s;
+                        } else if (CHARS) {
+#pragma unroll
+                            for (int i = 0; i < K; ++i) {
+                                const int bi = j * K + i;
+                                put(s + i, s_spell[(w[bi >> 2] >> (8 * (bi & 3))) & 255u]);
+                            }
+                            s += K;
+                        } else if (ex[j] >= 0) {
+                            put(s, ex[j]);
+                            ++s;
+                        } else if (ex[j] == INT_MIN) {
+                            put(s, a.missing_id);
+                            ++s;
+                        } else {
+                            for (int e = 0; e < -ex[j]; ++e) put(s + e, a.flat[ey[j] + e]);
+                            s += -ex[j];
+                        }
+                    }
+                } else if (!empty) {
+#pragma unroll 1
+                    for (int j = 0; j < kUnitsPerLane; ++j) {
+                        const int u = ub + j;
+                        if (u < full) {
+                            uint32_t c = 0;
+                            int c5 = 0;
+#pragma unroll
+                            for (int i = 0; i < K; ++i) {
+                                const uint32_t v = s_dig[src[u * K + i]];
+                                c = (c << 2) + v;
+                                c5 = c5 * 5 + ((v & (kDigN | kDigBad)) ? 4 : (int)v);
+                            }
+                            int32_t id = -1;
+                            if (c < POW4) id = LUT4_LDS ? s_lut4[c] : a.lut4[c];
+                            if (id >= 0) {
+                                put(s, id);
+                                ++s;
+                            } else {
+                                const int2 e = a.entry[c5];
+                                if (e.x >= 0 || e.x == INT_MIN) {
+                                    put(s, e.x >= 0 ? e.x : a.missing_id);
+                                    ++s;
+                                } else {
+                                    for (int q = 0; q < -e.x; ++q) put(s + q, a.flat[e.y + q]);
+                                    s += -e.x;
+                                }
+                            }
+                        } else if (u < n_units) {
+                            put(s, s_single[src[full * K + (u - full)]]);
+                            ++s;
+                        }
+                    }
+                }
+            };
+            // the staged run, written out in passes of kStageCap tokens (one pass unless a step
+            // expands to more than that)
+            for (uint32_t pass = 0; pass < n_avail; pass += kStageCap) {
+                produce([&](uint32_t s, int32_t tok) {
+                    const uint32_t rel = s - pass;
+                    if (rel < (uint32_t)kStageCap) buf[rel] = tok;
+                });
+                wave_sync();
+                const uint32_t count = pass + kStageCap >= n_avail ? n_avail - pass : (uint32_t)kStageCap;
+                const uint32_t n_groups = (count + 3) >> 2;
+                for (uint32_t g = lane; g < n_groups; g += 64) {
+                    const int4v x = *reinterpret_cast<const int4v *>(buf + 4 * g);
+                    const int32_t v[4] = {x.x, x.y, x.z, x.w};
+                    store_group(outA, moutA, e0 + (int)pass + 4 * (int)g, lo, hi, v, 1u);
+                }
+                wave_sync();
+            }
+            running += (int)round_total;
+        }
+
+        // the row's end: length, status, padding (by the first wave)
+        const bool any_bad = __ballot(my_status & DNATOK_ROW_INVALID_BYTE) != 0;
+        const bool any_missing = __ballot(my_status & DNATOK_ROW_MISSING_KMER) != 0;
+        if (lane == 0) s_stat[wv] = (any_bad ? DNATOK_ROW_INVALID_BYTE : 0) | (any_missing ? DNATOK_ROW_MISSING_KMER : 0);
+        __syncthreads();
+        const int stored = running < cap ? running : cap;
+        if (wv == 0) {
+            int32_t st = 0;
+#pragma unroll
+            for (int q = 0; q < NWV; ++q) st |= s_stat[q];
+            if (running > t_cap) st |= DNATOK_ROW_TRUNCATED;
+            if (lane == 0) {
+                lengths[row] = (int32_t)running;
+                if (status) status[row] = st;
+            }
+            if (fill > stored) pad_cells(outA, moutA, mis, stored, fill, a.pad_id, lane);
+        }
+        if (stored > wg_max) wg_max = stored;
+        __syncthreads();                      // s_stat and s_tot are written again by the next row
+    }
+    if (wv == 0) {
+        if (mref.slot) {
+            const unsigned long long v = (slot_gen << 32) | (unsigned long long)wg_max;
+            if (lane == 0 && (wg_max > 0 || blockIdx.x == 0) && __builtin_nontemporal_load(mref.slot) < v)
+                atomicMax(mref.slot, v);
+        } else if (max_len && lane == 0 && wg_max > 0 && (int64_t)__builtin_nontemporal_load(max_len) < wg_max) {
+            atomicMax(max_len, (int32_t)wg_max);
+        }
+    }
+}
+
 // Pads every row from its stored length up to the batch maximum found on the device.  A wave
 // reads the lengths of kPadRows rows at once, then pads the rows that fall short one after
 // the other, so that the stores of all of them are in flight together.
@@ -688,6 +1035,13 @@ extern "C" int dnatok_kmer_table_create(int k, const int8_t *digit_h, const int3
     return DNATOK_OK;
 }
 
+extern "C" int dnatok_kmer_set_team_rows(int32_t max_rows)
+{
+    DNATOK_REQUIRE(max_rows >= -1, DNATOK_E_INVALID, "dnatok_kmer_set_team_rows: -1 (automatic), 0 (never) or a row count");
+    g_team_rows.store(max_rows, std::memory_order_relaxed);
+    return DNATOK_OK;
+}
+
 extern "C" void dnatok_kmer_table_destroy(dnatok_kmer_t *t)
 {
     if (!t) return;
@@ -732,9 +1086,17 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
     }
     // persistent waves: the tables are staged into LDS once per workgroup
     const int64_t want = (n_rows + kKmerThreads / 64 - 1) / (kKmerThreads / 64);
+    // few rows (a workgroup for every row at once): the four waves of a workgroup share a row
 #define LAUNCH3(KK, L, C, M)                                                                      \
     do {                                                                                          \
         static const int resident = resident_workgroups(kmer_rows_kernel<KK, L, C, M>, kKmerThreads, 0, 4); \
+        static const int team_resident = resident_workgroups(kmer_team_kernel<KK, L, C, M>, kKmerThreads, 0, 4); \
+        const int team_rows = g_team_rows.load(std::memory_order_relaxed);                       \
+        if (n_rows <= (team_rows < 0 ? team_resident : team_rows)) {                              \
+            kmer_team_kernel<KK, L, C, M><<<(int)n_rows, kKmerThreads, 0, s>>>(                   \
+                a, bytes, offsets, n_rows, t_cap, fill_to, ids, mask, lengths, status, max_len, mref); \
+            break;                                                                                \
+        }                                                                                         \
         const int64_t grid = want < resident ? want : resident;                                   \
         kmer_rows_kernel<KK, L, C, M><<<(int)grid, kKmerThreads, 0, s>>>(                         \
             a, bytes, offsets, n_rows, t_cap, fill_to, ids, mask, lengths, status, max_len, mref); \

@@ -143,6 +143,13 @@ int  dnatok_kmer_table_create(int k, const int8_t *digit_h, const int32_t *kmer_
                               dnatok_kmer_t **out);
 void dnatok_kmer_table_destroy(dnatok_kmer_t *t);
 
+/* Which of the two k-mer kernels the calls that follow use (process-wide; no counterpart in the
+ * reference; a switch for tests and measurements, results are identical).  A batch of up to
+ * max_rows rows is encoded with a workgroup per row (four waves share a row: the latency of a small
+ * batch), a larger one with a wave per row (the bandwidth of a large one).  -1 (default): as many
+ * rows as workgroups fit the chip at once; 0: always a wave per row. */
+int dnatok_kmer_set_team_rows(int32_t max_rows);
+
 /* ids int32[n_rows, t_cap], mask uint8[n_rows, t_cap] (NULL allowed): t_cap is the row stride.
  * lengths int32[n_rows] receives each row's token count (also when it exceeds t_cap),
  * status int32[n_rows] the DNATOK_ROW_* bits (NULL allowed), max_len int32[1] the largest

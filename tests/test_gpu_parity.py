@@ -175,6 +175,21 @@ def test_char_c5_packed(char_enc):
 
 # ----------------------------------------------------------------- k-mer
 
+@pytest.fixture(autouse=True, params=["rows_by_wave", "rows_by_workgroup"])
+def kmer_kernel_choice(request):
+    """Every test runs with both k-mer kernels: a wave per row (forced for all batches) and the
+    automatic choice, which gives the batches of these tests a workgroup per row."""
+    from dnatok_amd import _lib
+    if "kmer" not in request.node.name:
+        if request.param == "rows_by_workgroup":
+            pytest.skip("not a k-mer test")
+        yield
+        return
+    _lib.lib().dnatok_kmer_set_team_rows(0 if request.param == "rows_by_wave" else -1)
+    yield
+    _lib.lib().dnatok_kmer_set_team_rows(-1)
+
+
 @pytest.fixture(scope="module")
 def kmer_enc():
     t = kmer_tables.tables_from_vocab(hf.kmer_vocab(6), 6, 0)
