@@ -815,6 +815,8 @@ static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t
 // round of loads and one scan (the kernel is a chain of load latencies and barriers, not work).
 constexpr int kPlanRows = 4;
 constexpr int kPlanScans = 1 + kSingleClasses;
+constexpr int kPlanInlineRows = 4096;      // the plan kernel writes the chunk entries itself up to this
+constexpr int kPlanInlineChunks = 8192;    // many rows and this many chunks (a bound known on the host)
 
 __global__ __launch_bounds__(1024) void bpe_plan_kernel(
     const int64_t *__restrict__ offsets, int64_t n_rows, int chunking, int expand_here, BpePlan p)
@@ -822,6 +824,7 @@ __global__ __launch_bounds__(1024) void bpe_plan_kernel(
     __shared__ uint32_t wt[kPlanScans][16];
     __shared__ int32_t carry[kPlanScans];
     __shared__ int32_t fail_s;
+    __shared__ int32_t s_mc[kPlanInlineRows], s_len[kPlanInlineRows];   // first chunk and length of every row (expand_here)
     if (threadIdx.x < kPlanScans) carry[threadIdx.x] = 0;
     if (threadIdx.x == 0) fail_s = 0;
     __syncthreads();
@@ -882,11 +885,8 @@ __global__ __launch_bounds__(1024) void bpe_plan_kernel(
             p.mc_off[row] = at[0];
             // the entries of the chunks are written by bpe_expand_kernel (a single workgroup
             // writing tens of thousands of scattered words is bound by its one CU's store path),
-            // except for a small batch of rows of few chunks each, which saves that launch
-            if (expand_here && add[r][0]) {
-                const int32_t nc = (int32_t)add[r][0], len = (int32_t)(off[r + 1] - off[r]);
-                for (int32_t k = 0; k < nc; ++k) p.rec[at[0] + k] = make_int4(row, k, nc, len);
-            }
+            // except for a batch of few chunks, whose entries are written below (a launch less)
+            if (expand_here) { s_mc[row] = at[0]; s_len[row] = (int32_t)(off[r + 1] - off[r]); }
 #pragma unroll
             for (int q = 0; q < kSingleClasses; ++q)
                 if (add[r][1 + q]) p.single[q][at[1 + q]] = row;
@@ -902,6 +902,23 @@ __global__ __launch_bounds__(1024) void bpe_plan_kernel(
     }
     if (n_fail) atomicAdd(&fail_s, n_fail);
     __syncthreads();
+    if (expand_here) {
+        // chunk c belongs to the last row whose first chunk is at or before c
+        const int32_t total = carry[0];
+        for (int32_t c = threadIdx.x; c < total; c += 1024) {
+            int32_t lo = 0, hi = (int32_t)n_rows;             // first row whose first chunk lies beyond c
+            while (lo < hi) {
+                const int32_t mid = (lo + hi) >> 1;
+                if (s_mc[mid] <= c) lo = mid + 1; else hi = mid;
+            }
+            // rows without chunks share their first-chunk number with the next row: step back to the
+            // row that owns c (the last one at or before c that has chunks is the one found: a row
+            // without chunks has the same number as its successor, so the search ends behind them)
+            const int32_t row = lo - 1;
+            const int32_t first = s_mc[row], next = row + 1 < (int32_t)n_rows ? s_mc[row + 1] : total;
+            p.rec[c] = make_int4(row, c - first, next - first, s_len[row]);
+        }
+    }
     if (threadIdx.x == 0) {
         int32_t items = carry[0];
         for (int q = 0; q < kSingleClasses; ++q) { p.counts[4 + q] = carry[1 + q]; items += carry[1 + q]; }
@@ -1533,9 +1550,8 @@ static int bpe_encode_launch(const dnatok_bpe_t *t, const uint8_t *bytes, const 
 
     const bool long_rows = max_len > p.ext;
     int chunking = (long_rows && t->monotone) ? 1 : 0;
-    // bit 1: the plan kernel writes the chunk entries itself (a small batch of rows of at most 16
-    // chunks each: a few stores per thread, and one launch less)
-    if (chunking && n_rows <= 4096 && max_len <= 16 * (int64_t)p.core) chunking |= 2;
+    // bit 1: the plan kernel writes the chunk entries itself (few rows, few chunks: one launch less)
+    if (chunking && n_rows <= kPlanInlineRows && p.max_mc <= kPlanInlineChunks) chunking |= 2;
     // the LDS capacity variant follows the longest row (or the chunk size for longer rows):
     // less LDS per workgroup means more workgroups per CU
     int rc;

@@ -175,19 +175,17 @@ def test_char_c5_packed(char_enc):
 
 # ----------------------------------------------------------------- k-mer
 
-@pytest.fixture(autouse=True, params=["rows_by_wave", "rows_by_workgroup"])
+@pytest.fixture
 def kmer_kernel_choice(request):
-    """Every test runs with both k-mer kernels: a wave per row (forced for all batches) and the
+    """Which k-mer kernel the test's batches get: a wave per row (forced for all batches) or the
     automatic choice, which gives the batches of these tests a workgroup per row."""
     from dnatok_amd import _lib
-    if "kmer" not in request.node.name:
-        if request.param == "rows_by_workgroup":
-            pytest.skip("not a k-mer test")
-        yield
-        return
     _lib.lib().dnatok_kmer_set_team_rows(0 if request.param == "rows_by_wave" else -1)
-    yield
+    yield request.param
     _lib.lib().dnatok_kmer_set_team_rows(-1)
+
+
+both_kmer_kernels = pytest.mark.parametrize("kmer_kernel_choice", ["rows_by_wave", "rows_by_workgroup"], indirect=True)
 
 
 @pytest.fixture(scope="module")
@@ -202,7 +200,8 @@ def rows_from_padded(ids, lengths):
     return [ids[r, :lengths[r]] for r in range(ids.shape[0])]
 
 
-def test_kmer_c2(kmer_enc):
+@both_kmer_kernels
+def test_kmer_c2(kmer_enc, kmer_kernel_choice):
     say("kmer C2 256x6000")
     b = wl.config2_kmer()
     data, off = to_dev(b)
@@ -218,8 +217,9 @@ def test_kmer_c2(kmer_enc):
     assert int(status.abs().sum().item()) == 0
 
 
+@both_kmer_kernels
 @pytest.mark.parametrize("k", [2, 3, 4, 5, 6, 7, 8])
-def test_kmer_ragged_all_k(k):
+def test_kmer_ragged_all_k(k, kmer_kernel_choice):
     say(f"kmer ragged k={k}")
     vocab = hf.kmer_vocab(k)
     t = kmer_tables.tables_from_vocab(vocab, k, 0)
@@ -251,7 +251,8 @@ def test_kmer_ragged_all_k(k):
         np.testing.assert_array_equal(mask[:, :width].cpu().numpy(), emask)
 
 
-def test_kmer_pad_to_longest_with_width_guess():
+@both_kmer_kernels
+def test_kmer_pad_to_longest_with_width_guess(kmer_kernel_choice):
     """fill_to = 0 with a guess of the longest row: a guess below, at or above the true width
     gives the same ids / mask / lengths / max_len inside [:, :max_len]."""
     say("kmer width guess")
@@ -278,7 +279,8 @@ def test_kmer_pad_to_longest_with_width_guess():
         np.testing.assert_array_equal(got[3].cpu().numpy(), ref[3].cpu().numpy())
 
 
-def test_kmer_pad_to_longest_replayed_from_a_graph(kmer_enc):
+@both_kmer_kernels
+def test_kmer_pad_to_longest_replayed_from_a_graph(kmer_enc, kmer_kernel_choice):
     """A captured pad-to-longest call, replayed over changing input: every replay reports the
     longest row of its own input (first a batch with long rows, then shorter ones, then long
     again), and matches the eager call."""
@@ -320,7 +322,8 @@ def test_kmer_pad_to_longest_replayed_from_a_graph(kmer_enc):
     assert widths[1] == length // 6 and widths[0] > widths[1] and widths[3] > widths[2] > widths[1]
 
 
-def test_kmer_pad_to_longest_calls_on_many_streams_do_not_share_a_maximum(kmer_enc):
+@both_kmer_kernels
+def test_kmer_pad_to_longest_calls_on_many_streams_do_not_share_a_maximum(kmer_enc, kmer_kernel_choice):
     """Pad-to-longest calls queued on several streams at once, nothing synchronised in between:
     every call reports the longest row of its own batch.  70 streams is more than the table keeps
     running maxima for, so the last ones take the path that clears the caller's max_len instead."""
@@ -351,7 +354,8 @@ def test_kmer_pad_to_longest_calls_on_many_streams_do_not_share_a_maximum(kmer_e
         np.testing.assert_array_equal(r[0][:, :width].cpu().numpy(), ids[:, :width])
 
 
-def test_kmer_general_tables_not_spelled():
+@both_kmer_kernels
+def test_kmer_general_tables_not_spelled(kmer_kernel_choice):
     """Tables whose N windows are not spelled character by character: N windows that have an
     id of their own, expansions of other lengths, and windows with nothing at all."""
     say("kmer general (non-spelled) tables")
@@ -392,7 +396,8 @@ def test_kmer_general_tables_not_spelled():
     np.testing.assert_array_equal(mask[:, :m].cpu().numpy(), emask)
 
 
-def test_kmer_missing_windows_without_expansion():
+@both_kmer_kernels
+def test_kmer_missing_windows_without_expansion(kmer_kernel_choice):
     say("kmer missing windows")
     t = kmer_tables.tables_from_vocab(hf.kmer_vocab(4), 4, 0)
     enc = encoders.KmerEncoder(4, t.digit, t.kmer_lut, t.single, pad_id=1, missing_id=3)
