@@ -54,6 +54,7 @@ struct dnatok_kmer_table {
     // larger than anything an earlier call left behind, and the slot never has to be cleared (a
     // launch saved per call; replays of a captured call stay exact).
     unsigned long long *max_slots;
+    unsigned long long *max_trees;       // kTreeWords words per slot (see kmer_team_kernel)
     mutable std::mutex slot_lock;
     mutable std::unordered_map<void *, int> slot_of_stream;
 };
@@ -64,6 +65,10 @@ constexpr int kMaxSlots = 64;
 // many rows as workgroups of that kernel fit the chip at once.  (dnatok_kmer_set_team_rows)
 static std::atomic<int> g_team_rows{-1};
 constexpr int kMaxSlotStride = 32;       // 64-bit words between two slots (one 256-byte line each)
+// A call whose kernel reports the maximum itself (kmer_team_kernel, publish) gathers it up a tree
+// of 64-bit words with four 16-bit fields each: kTreeRows leaves, four children per word.
+constexpr int kTreeRows = 1024;
+constexpr int kTreeWords = 512;          // 256 + 64 + 16 + 4 + 1 words used, 4 KB per slot
 
 namespace dnatok {
 
@@ -110,6 +115,7 @@ __global__ void kmer_init_kernel(int32_t *max_len) { *max_len = 0; }
 // slot[1] = generation.
 struct MaxRef {
     unsigned long long *slot;
+    unsigned long long *tree;      // kTreeWords words of the slot's stream, all zero between calls
 };
 
 // Stores the group of 4 cells [e, e + 4) of a row whose cells are addressed from the
@@ -549,15 +555,17 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
 // through LDS, so that every wave knows where its tokens start.  A wave writes its run by itself,
 // whole 16-byte groups and single cells at both ends (no waiting for whole lines as in
 // kmer_rows_kernel: this kernel is for batches that are bound by latency, not by bandwidth).
-// The padding pass stays a launch of its own: letting the workgroup that finishes last do it
-// (a ticket counter behind a device-scope fence) measured 39 us per call instead of 15, because
-// such a fence writes back the L2 of the workgroup's XCD.
+// Padding up to a maximum that only the whole batch knows stays a launch of its own: letting the
+// workgroup that finishes last do it (a ticket counter behind a device-scope fence) measured 39 us
+// per call instead of 15, because such a fence writes back the L2 of the workgroup's XCD.  With
+// `publish` there is nothing to pad afterwards (the rows are as far apart as the caller's guess,
+// and padded that far here), and the maximum alone travels on atomics, with no fence: 8.8 us.
 template <int K, bool LUT4_LDS, bool CHARS, bool HAS_MASK>
 __global__ __launch_bounds__(kKmerThreads) void kmer_team_kernel(
     KmerArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
     int64_t n_rows, int64_t t_cap, int64_t fill_to, int32_t *__restrict__ ids,
     uint8_t *__restrict__ mask, int32_t *__restrict__ lengths, int32_t *__restrict__ status,
-    int32_t *__restrict__ max_len, MaxRef mref)
+    int32_t *__restrict__ max_len, MaxRef mref, int publish)
 {
     constexpr uint32_t POW4 = 1u << (2 * K);
     constexpr int NWV = kKmerThreads / 64;
@@ -626,6 +634,7 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_team_kernel(
     const int fill = fill_to > cap ? cap : (int)fill_to;
     int64_t wg_max = 0;
     const unsigned long long slot_gen = mref.slot ? mref.slot[1] : 0ull;
+    unsigned long long sent = 0, sent_val = 0;       // publish: the row's length + 1 and what its tree word held before
 
     for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
         const int64_t row_start = offsets[row];
@@ -642,6 +651,10 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_team_kernel(
         int32_t my_status = 0;
         const __amdgpu_buffer_rsrc_t rsrc =
             __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(src), (short)0, len, 0x00020000);
+        if (publish && n_units == 0 && wv == 0 && lane == 0) {
+            sent_val = 1;
+            sent = atomicAdd(mref.tree + (blockIdx.x >> 2), 1ull << (16 * (blockIdx.x & 3)));
+        }
 
         int par = 0;
         for (int r0 = 0; r0 < n_units; r0 += NWV * kWaveUnits, par ^= 1) {     // the same rounds for every wave
@@ -762,6 +775,14 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_team_kernel(
             const int A = mis + running + (int)before;             // cell the step's first token goes to
             const int A_end = A + (int)step_total;
             const int lo = A, hi = A_end < hi_cap ? A_end : hi_cap;
+            if (publish && wv == 0 && lane == 0 && r0 + NWV * kWaveUnits >= n_units) {
+                // the row's length is known here, before its last tokens are written: the
+                // maximum travels while they are (see the end of the kernel)
+                const int total = running + (int)round_total;
+                const int kept = total < cap ? total : cap;
+                sent_val = (unsigned long long)kept + 1;
+                sent = atomicAdd(mref.tree + (blockIdx.x >> 2), sent_val << (16 * (blockIdx.x & 3)));
+            }
             const uint32_t carry = (uint32_t)A & 3u;
             const uint32_t n_avail = carry + step_total;
             const uint32_t s0 = carry + (inc - lane_cnt);
@@ -872,7 +893,45 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_team_kernel(
         __syncthreads();                      // s_stat and s_tot are written again by the next row
     }
     if (wv == 0) {
-        if (mref.slot) {
+        if (mref.slot && publish) {
+            // No padding pass follows (every row is padded as far as any row can reach), so the
+            // kernel reports the batch's maximum itself, and without a fence: nothing but atomics
+            // carries it.  A workgroup (it has one row: the grid is the batch) added its length + 1
+            // into its 16-bit field of a tree word as soon as the length was known; the atomic
+            // returns the fields of those that came before, so the one that completes a word
+            // knows the maximum of its four, clears the word for the next call and carries the
+            // maximum one level up in the same way.  Who completes the root writes max_len.
+            // (One counter and one atomicMax for all workgroups cost 3 us here, two of them spent
+            // queueing at that one address.)
+            if (lane == 0) {
+                unsigned long long *level = mref.tree;
+                unsigned idx = blockIdx.x, n_here = gridDim.x;
+                unsigned long long mine = sent_val, before = sent;
+                for (;;) {
+                    const unsigned long long all = before + (mine << (16 * (idx & 3)));
+                    const unsigned members = n_here - (idx & ~3u) < 4u ? n_here - (idx & ~3u) : 4u;
+                    unsigned arrived = 0;
+                    unsigned long long best = 0;
+#pragma unroll
+                    for (int f = 0; f < 4; ++f) {
+                        const unsigned long long v = (all >> (16 * f)) & 0xFFFFull;
+                        arrived += v != 0;
+                        best = v > best ? v : best;
+                    }
+                    if (arrived < members) break;
+                    atomicExch(level + (idx >> 2), 0ull);
+                    if (n_here <= 4) {
+                        *max_len = (int32_t)best - 1;
+                        break;
+                    }
+                    level += (n_here + 3) >> 2;
+                    n_here = (n_here + 3) >> 2;
+                    idx >>= 2;
+                    mine = best;
+                    before = atomicAdd(level + (idx >> 2), mine << (16 * (idx & 3)));
+                }
+            }
+        } else if (mref.slot) {
             const unsigned long long v = (slot_gen << 32) | (unsigned long long)wg_max;
             if (lane == 0 && (wg_max > 0 || blockIdx.x == 0) && __builtin_nontemporal_load(mref.slot) < v)
                 atomicMax(mref.slot, v);
@@ -941,7 +1000,7 @@ static int launch_pad(int32_t *ids, uint8_t *mask, const int32_t *lengths, int64
 int launch_pad_to_max(int32_t *ids, uint8_t *mask, const int32_t *lengths, int64_t n_rows,
                       int64_t t_cap, int32_t *max_len, int32_t pad_id, int32_t already, hipStream_t s)
 {
-    return launch_pad(ids, mask, lengths, n_rows, t_cap, max_len, pad_id, already, MaxRef{nullptr}, s);
+    return launch_pad(ids, mask, lengths, n_rows, t_cap, max_len, pad_id, already, MaxRef{nullptr, nullptr}, s);
 }
 
 }  // namespace dnatok
@@ -1006,7 +1065,8 @@ extern "C" int dnatok_kmer_table_create(int k, const int8_t *digit_h, const int3
     const size_t o_entry = up(o_lut4 + pow4 * 4);
     const size_t o_flat = up(o_entry + pow5 * sizeof(int2));
     const size_t o_slots = up(o_flat + (has_exp ? n_flat * 4 : 0));
-    const size_t bytes = up(o_slots + (size_t)kMaxSlots * kMaxSlotStride * 8) + 256;
+    const size_t o_trees = up(o_slots + (size_t)kMaxSlots * kMaxSlotStride * 8);
+    const size_t bytes = up(o_trees + (size_t)kMaxSlots * kTreeWords * 8) + 256;
     std::vector<uint8_t> host(bytes, 0);
     memcpy(&host[o_digit], digit_h, 256);
     memcpy(&host[o_single], single_h, 256 * 4);
@@ -1031,6 +1091,7 @@ extern "C" int dnatok_kmer_table_create(int k, const int8_t *digit_h, const int3
     t->entry = (int2 *)(b + o_entry);
     t->flat = (int32_t *)(b + o_flat);
     t->max_slots = (unsigned long long *)(b + o_slots);
+    t->max_trees = (unsigned long long *)(b + o_trees);
     *out = t;
     return DNATOK_OK;
 }
@@ -1072,13 +1133,16 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
     if (n_rows == 0) return DNATOK_OK;
     hipStream_t s = (hipStream_t)stream;
     KmerArgs a{t->digit, t->single, t->lut4, t->entry, t->flat, t->pad_id, t->missing_id};
-    MaxRef mref{nullptr};
+    MaxRef mref{nullptr, nullptr};
     if (to_longest) {
         std::lock_guard<std::mutex> hold(t->slot_lock);
         auto it = t->slot_of_stream.find(stream);
         if (it == t->slot_of_stream.end() && (int)t->slot_of_stream.size() < kMaxSlots)
             it = t->slot_of_stream.emplace(stream, (int)t->slot_of_stream.size()).first;
-        if (it != t->slot_of_stream.end()) mref.slot = t->max_slots + (size_t)it->second * kMaxSlotStride;
+        if (it != t->slot_of_stream.end()) {
+            mref.slot = t->max_slots + (size_t)it->second * kMaxSlotStride;
+            mref.tree = t->max_trees + (size_t)it->second * kTreeWords;
+        }
     }
     if (!mref.slot && max_len) {
         kmer_init_kernel<<<1, 1, 0, s>>>(max_len);
@@ -1086,15 +1150,23 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
     }
     // persistent waves: the tables are staged into LDS once per workgroup
     const int64_t want = (n_rows + kKmerThreads / 64 - 1) / (kKmerThreads / 64);
-    // few rows (a workgroup for every row at once): the four waves of a workgroup share a row
+    // few rows (a workgroup for every row at once): the four waves of a workgroup share a row.
+    // When the row stride is already cut to the guess (at most kTightStride cells beyond it), those
+    // rows are padded to the whole stride while they are written, which covers every possible
+    // maximum: the kernel then reports the maximum itself and the padding launch is left out.
+    constexpr int64_t kTightStride = 256;
+    bool padded_in_kernel = false;
 #define LAUNCH3(KK, L, C, M)                                                                      \
     do {                                                                                          \
         static const int resident = resident_workgroups(kmer_rows_kernel<KK, L, C, M>, kKmerThreads, 0, 4); \
         static const int team_resident = resident_workgroups(kmer_team_kernel<KK, L, C, M>, kKmerThreads, 0, 4); \
         const int team_rows = g_team_rows.load(std::memory_order_relaxed);                       \
         if (n_rows <= (team_rows < 0 ? team_resident : team_rows)) {                              \
+            padded_in_kernel = to_longest && mref.slot && guess > 0 && t_cap - guess <= kTightStride && \
+                               n_rows <= kTreeRows && t_cap < 0xFFFF;                            \
             kmer_team_kernel<KK, L, C, M><<<(int)n_rows, kKmerThreads, 0, s>>>(                   \
-                a, bytes, offsets, n_rows, t_cap, fill_to, ids, mask, lengths, status, max_len, mref); \
+                a, bytes, offsets, n_rows, t_cap, padded_in_kernel ? t_cap : fill_to, ids, mask,  \
+                lengths, status, max_len, mref, padded_in_kernel ? 1 : 0);                        \
             break;                                                                                \
         }                                                                                         \
         const int64_t grid = want < resident ? want : resident;                                   \
@@ -1122,7 +1194,7 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
 #undef LAUNCH2
 #undef LAUNCH3
     DNATOK_HIP_TRY(hipGetLastError());
-    if (to_longest)
+    if (to_longest && !padded_in_kernel)
         return launch_pad(ids, mask, lengths, n_rows, t_cap, max_len, t->pad_id, (int32_t)guess, mref, s);
     return DNATOK_OK;
 }

@@ -280,6 +280,80 @@ def test_kmer_pad_to_longest_with_width_guess(kmer_kernel_choice):
 
 
 @both_kmer_kernels
+def test_kmer_pad_to_longest_with_row_stride_cut_to_the_guess(kmer_enc, kmer_kernel_choice):
+    """Rows only a little further apart than the guessed width (the layout a stream of batches
+    uses): the workgroup-per-row kernel then pads to the stride and reports the maximum itself,
+    with no padding launch.  Guesses below, at and above the true width, strides that cut rows
+    off, eager calls and calls with a wide stride in between (they share the running maximum's
+    slot), and a captured call replayed over changing input."""
+    say("kmer tight stride")
+    n, length = 48, 3000
+    batches = [wl.config2_kmer(n, length, seed=s, n_fraction=f) for s, f in ((91, 0.02), (92, 0.0), (93, 0.06))]
+    want = []
+    for b in batches:
+        data, off = to_dev(b)
+        r = kmer_enc.encode_padded(data, off, 3008, fill_to=0)
+        torch.cuda.synchronize()
+        want.append((int(r[4].item()), r[0].cpu().numpy(), r[1].cpu().numpy(), r[2].cpu().numpy()))
+    for rnd in range(2):
+        for b, (width, ids, mask, lengths) in zip(batches, want):
+            data, off = to_dev(b)
+            for guess, t_cap in ((width - 40, width + 24), (width, width), (width + 3, width + 131), (width + 3, width + 259),
+                                 (width - 100, width - 36), (8, 200)):
+                got = kmer_enc.encode_padded(data, off, t_cap, fill_to=0, width_guess=guess)
+                torch.cuda.synchronize()
+                w = min(width, t_cap)
+                assert int(got[4].item()) == w, (guess, t_cap)
+                np.testing.assert_array_equal(got[0][:, :w].cpu().numpy(), ids[:, :w])
+                np.testing.assert_array_equal(got[1][:, :w].cpu().numpy(), mask[:, :w])
+                np.testing.assert_array_equal(got[2].cpu().numpy(), lengths)
+                np.testing.assert_array_equal((got[3].cpu().numpy() & 4) != 0, lengths > t_cap)
+    # every shape of the tree the maximum is gathered on: 1 .. 1024 rows, the longest row anywhere
+    for n_rows in (1, 2, 3, 4, 5, 7, 16, 17, 63, 64, 65, 255, 256, 257, 1023, 1024, 1025):
+        rng = np.random.default_rng(n_rows)
+        lens = rng.integers(0, 240, size=n_rows)
+        lens[rng.integers(0, n_rows)] = 300 + n_rows % 7
+        b = util.batch_from_strings(["".join(rng.choice(list("ACGTN"), p=[.245, .245, .245, .245, .02], size=m)) for m in lens])
+        data, off = to_dev(b)
+        ref = kmer_enc.encode_padded(data, off, 320, fill_to=0)
+        torch.cuda.synchronize()
+        width = int(ref[4].item())
+        assert width == int(ref[2].max().item())
+        for rep in range(2):
+            got = kmer_enc.encode_padded(data, off, width + 8, fill_to=0, width_guess=width - 3 + 5 * rep)
+            torch.cuda.synchronize()
+            assert int(got[4].item()) == width, n_rows
+            np.testing.assert_array_equal(got[0][:, :width].cpu().numpy(), ref[0][:, :width].cpu().numpy())
+            np.testing.assert_array_equal(got[1][:, :width].cpu().numpy(), ref[1][:, :width].cpu().numpy())
+            np.testing.assert_array_equal(got[2].cpu().numpy(), ref[2].cpu().numpy())
+    # a captured call with a tight stride, replayed over the three batches
+    t_cap, guess = max(w[0] for w in want) + 16, max(w[0] for w in want) - 8
+    data = torch.zeros(n * length, dtype=torch.uint8, device=DEV)
+    off = torch.arange(n + 1, dtype=torch.int64, device=DEV) * length
+    out = (torch.empty((n, t_cap), dtype=torch.int32, device=DEV), torch.empty((n, t_cap), dtype=torch.uint8, device=DEV),
+           torch.empty(n, dtype=torch.int32, device=DEV), torch.empty(n, dtype=torch.int32, device=DEV),
+           torch.empty(1, dtype=torch.int32, device=DEV))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        kmer_enc.encode_padded(data, off, t_cap, fill_to=0, width_guess=guess, out=out)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        kmer_enc.encode_padded(data, off, t_cap, fill_to=0, width_guess=guess, out=out)
+    for i in (0, 1, 2, 1, 0, 2):
+        data.copy_(torch.from_numpy(batches[i].data))
+        graph.replay()
+        torch.cuda.synchronize()
+        width, ids, mask, lengths = want[i]
+        assert int(out[4].item()) == width
+        np.testing.assert_array_equal(out[0][:, :width].cpu().numpy(), ids[:, :width])
+        np.testing.assert_array_equal(out[1][:, :width].cpu().numpy(), mask[:, :width])
+        np.testing.assert_array_equal(out[2].cpu().numpy(), lengths)
+
+
+@both_kmer_kernels
 def test_kmer_pad_to_longest_replayed_from_a_graph(kmer_enc, kmer_kernel_choice):
     """A captured pad-to-longest call, replayed over changing input: every replay reports the
     longest row of its own input (first a batch with long rows, then shorter ones, then long
