@@ -96,6 +96,10 @@ constexpr uint32_t kFlushMask = kFlushCells - 1;
 // for a byte outside the alphabet, so that "window code < 4^k" means "k plain bases".
 constexpr uint32_t kDigN = 1u << 16;
 constexpr uint32_t kDigBad = 1u << 17;
+// In a window code c = sum of digit_i << 2 (K - 1 - i) the flags of the digits do not meet (the
+// digits' own two bits stay below bit 16 for K <= 8): N flags land on even bits from 16 up,
+// foreign-byte flags on odd bits from 17 up.
+constexpr uint32_t kCodeBadBits = 0xAAAA0000u;
 // byte offset past the end of every row descriptor (its stores are dropped), and the cache
 // policy bits of the buffer stores (streaming: the output is not read again by the kernel)
 constexpr uint32_t kDropOffset = 0x80000000u;
@@ -318,13 +322,9 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
                         cnt[j] = e.x >= 0 ? 1 : (e.x == INT_MIN ? 1 : -e.x);
                         if (e.x == INT_MIN) my_status |= DNATOK_ROW_MISSING_KMER;
                     }
-                    if ((code[j] >> 17) != 0) {
-                        // some digit may carry the foreign-byte flag (bit 17, shifted left by 0..2(K-1))
-                        bool bad = false;
-#pragma unroll
-                        for (int i = 0; i < K; ++i) bad = bad || (digit_of(j * K + i) & kDigBad);
-                        if (bad) my_status |= DNATOK_ROW_INVALID_BYTE;
-                    }
+                    // the foreign-byte flag of digit i sits at bit 17 + 2 (K - 1 - i) of the window's
+                    // code, the N flag one below it: an odd bit above 16 is a foreign byte
+                    if (code[j] & kCodeBadBits) my_status |= DNATOK_ROW_INVALID_BYTE;
                     lane_cnt += (uint32_t)cnt[j];
                 }
             } else if (!empty) {
@@ -398,6 +398,17 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
     #pragma unroll
                     for (int j = 0; j < kUnitsPerLane; ++j) put(s + j, t[j]);
                 } else if (lane_full) {
+                    // The tokens the lane's bytes are spelled with: all lookups on their way together
+                    // (a window at a time they are four trips to LDS in a row, on the step that
+                    // takes longest anyway), where the registers allow it (k <= 6: more would
+                    // cost the kernel a wave per SIMD).
+                    constexpr bool kSpellAhead = CHARS && K <= 6;
+                    int32_t sp[kSpellAhead ? kUnitsPerLane * K : 1];
+                    if (kSpellAhead) {
+    #pragma unroll
+                        for (int bi = 0; bi < kUnitsPerLane * K; ++bi)
+                            sp[bi] = s_spell[(w[bi >> 2] >> (8 * (bi & 3))) & 255u];
+                    }
     #pragma unroll
                     for (int j = 0; j < kUnitsPerLane; ++j) {
                         if (code[j] < POW4 && t[j] >= 0) {
@@ -407,7 +418,7 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
     #pragma unroll
                             for (int i = 0; i < K; ++i) {
                                 const int bi = j * K + i;
-                                put(s + i, s_spell[(w[bi >> 2] >> (8 * (bi & 3))) & 255u]);
+                                put(s + i, kSpellAhead ? sp[kSpellAhead ? bi : 0] : s_spell[(w[bi >> 2] >> (8 * (bi & 3))) & 255u]);
                             }
                             s += K;
                         } else if (ex[j] >= 0) {
@@ -721,12 +732,7 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_team_kernel(
                         cnt[j] = e.x >= 0 ? 1 : (e.x == INT_MIN ? 1 : -e.x);
                         if (e.x == INT_MIN) my_status |= DNATOK_ROW_MISSING_KMER;
                     }
-                    if ((code[j] >> 17) != 0) {
-                        bool bad = false;
-#pragma unroll
-                        for (int i = 0; i < K; ++i) bad = bad || (digit_of(j * K + i) & kDigBad);
-                        if (bad) my_status |= DNATOK_ROW_INVALID_BYTE;
-                    }
+                    if (code[j] & kCodeBadBits) my_status |= DNATOK_ROW_INVALID_BYTE;
                     lane_cnt += (uint32_t)cnt[j];
                 }
             } else if (!empty) {
