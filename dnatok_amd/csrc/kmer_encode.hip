@@ -391,6 +391,42 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
             const int A_end = A + (int)step_total;
             const int hi = last_step && A_end < hi_cap ? A_end : hi_cap;
 
+            // the tokens of a lane's units one unit at a time, from the row's bytes in memory (the
+            // ragged end of a row: whole windows first, then single characters); put(s, tok)
+            auto emit_units = [&](auto put, uint32_t s) {
+    #pragma unroll 1
+                for (int j = 0; j < kUnitsPerLane; ++j) {
+                    const int u = ub + j;
+                    if (u < full) {
+                        uint32_t c = 0;
+                        int c5 = 0;
+    #pragma unroll
+                        for (int i = 0; i < K; ++i) {
+                            const uint32_t v = s_dig[src[u * K + i]];
+                            c = (c << 2) + v;
+                            c5 = c5 * 5 + ((v & (kDigN | kDigBad)) ? 4 : (int)v);
+                        }
+                        int32_t id = -1;
+                        if (c < POW4) id = LUT4_LDS ? s_lut4[c] : a.lut4[c];
+                        if (id >= 0) {
+                            put(s, id);
+                            ++s;
+                        } else {
+                            const int2 e = a.entry[c5];
+                            if (e.x >= 0 || e.x == INT_MIN) {
+                                put(s, e.x >= 0 ? e.x : a.missing_id);
+                                ++s;
+                            } else {
+                                for (int q = 0; q < -e.x; ++q) put(s + q, a.flat[e.y + q]);
+                                s += -e.x;
+                            }
+                        }
+                    } else if (u < n_units) {
+                        put(s, s_single[src[full * K + (u - full)]]);
+                        ++s;
+                    }
+                }
+            };
             // the lanes' tokens in scanned order; put(s, tok) places token s of the staged run
             auto produce = [&](auto put) {
                 uint32_t s = s0;
@@ -433,38 +469,7 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
                         }
                     }
                 } else if (!empty) {
-    #pragma unroll 1
-                    for (int j = 0; j < kUnitsPerLane; ++j) {
-                        const int u = ub + j;
-                        if (u < full) {
-                            uint32_t c = 0;
-                            int c5 = 0;
-    #pragma unroll
-                            for (int i = 0; i < K; ++i) {
-                                const uint32_t v = s_dig[src[u * K + i]];
-                                c = (c << 2) + v;
-                                c5 = c5 * 5 + ((v & (kDigN | kDigBad)) ? 4 : (int)v);
-                            }
-                            int32_t id = -1;
-                            if (c < POW4) id = LUT4_LDS ? s_lut4[c] : a.lut4[c];
-                            if (id >= 0) {
-                                put(s, id);
-                                ++s;
-                            } else {
-                                const int2 e = a.entry[c5];
-                                if (e.x >= 0 || e.x == INT_MIN) {
-                                    put(s, e.x >= 0 ? e.x : a.missing_id);
-                                    ++s;
-                                } else {
-                                    for (int q = 0; q < -e.x; ++q) put(s + q, a.flat[e.y + q]);
-                                    s += -e.x;
-                                }
-                            }
-                        } else if (u < n_units) {
-                            put(s, s_single[src[full * K + (u - full)]]);
-                            ++s;
-                        }
-                    }
+                    emit_units(put, s);
                 }
             };
             auto group_at = [&](uint32_t g, int32_t *v) {
@@ -472,6 +477,12 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
                 v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
             };
 
+            // How a step with more tokens than the staging area holds is written out.  In passes
+            // for k <= 6: that kernel has 123 registers either way (4 waves per SIMD), and measured
+            // 1-3 % faster on the 6-mer workload than the same kernel with 78 registers and the
+            // cell-by-cell form (at 4 and at 5 waves per SIMD).  Cell by cell for k = 7, 8, where
+            // the passes push the kernel beyond 128 registers (3 waves per SIMD).
+            constexpr bool kStageInPasses = K <= 6;
             if (n_avail <= (uint32_t)kStageCap) {
                 produce([&](uint32_t s, int32_t tok) { buf[s] = tok; });
                 wave_sync();
@@ -503,7 +514,7 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
                 if ((uint32_t)lane < left) keep = buf[(n_avail & ~kFlushMask) + lane];
                 wave_sync();
                 if ((uint32_t)lane < left) buf[lane] = keep;
-            } else {
+            } else if (kStageInPasses) {
                 // more than kStageCap tokens in one step: staged and written out in several passes
                 settle();
                 for (uint32_t pass = 0; pass < n_avail; pass += kStageCap) {
@@ -528,6 +539,30 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
                     if ((uint32_t)lane < left) buf[lane] = keep;
                     wave_sync();
                 }
+            } else {
+                // More than kStageCap tokens in one step, k >= 7: every lane writes its own tokens
+                // cell by cell, reading the row's bytes from memory as the lanes of a ragged end
+                // do.  Rare and slow on purpose: the passes above keep everything a step computes
+                // alive across a loop, which for these k costs the kernel a wave per SIMD.  The
+                // tokens past the last whole unit also go to the staging area, where the next
+                // step looks for them.
+                settle();
+                const int e0 = A & ~(int)kFlushMask;
+                const uint32_t keep_from = last_step ? 0xFFFFFFFFu : (n_avail & ~kFlushMask);
+                int32_t left_over = 0;
+                if ((uint32_t)lane < carry) left_over = buf[lane];
+                wave_sync();
+                auto put_cell = [&](uint32_t s, int32_t tok) {
+                    const int e = e0 + (int)s;
+                    if (e >= lo && e < hi) {
+                        outA[e] = tok;
+                        if (HAS_MASK) moutA[e] = 1;
+                    }
+                    if (s >= keep_from) buf[s - keep_from] = tok;
+                };
+                if ((uint32_t)lane < carry) put_cell((uint32_t)lane, left_over);
+                if (!empty) emit_units(put_cell, s0);
+                wave_sync();
             }
             }
             store_vec(sv_whole, sv_r, sv_v);

@@ -252,6 +252,51 @@ def test_kmer_ragged_all_k(k, kmer_kernel_choice):
 
 
 @both_kmer_kernels
+@pytest.mark.parametrize("k", [3, 6, 8])
+def test_kmer_steps_with_more_tokens_than_the_staging_area(kmer_kernel_choice, k):
+    """Long stretches of N (every window of a step spelled out: up to k times 256 tokens where a
+    wave stages 512) between plain stretches of every length, so that such a step is entered and
+    left at every alignment, follows and precedes staged and plain steps, ends a row, and is cut
+    by the row stride."""
+    say(f"kmer steps beyond the staging area k={k}")
+    vocab = hf.kmer_vocab(k)
+    t = kmer_tables.tables_from_vocab(vocab, k, 0)
+    enc = encoders.KmerEncoder(k, t.digit, t.kmer_lut, t.single, pad_id=1, missing_id=0,
+                               exp_off=t.exp_off, exp_len=t.exp_len, exp_flat=t.exp_flat)
+    ot = O.kmer_tables_from_vocab(vocab, k, 0)
+    rng = np.random.default_rng(100 + k)
+    strings = []
+    for r in range(96):
+        parts = []
+        for _ in range(rng.integers(1, 6)):
+            parts.append("".join(rng.choice(list("ACGT"), size=rng.integers(0, 2500))))
+            parts.append("N" * int(rng.integers(1, 4000)))
+            if rng.random() < 0.3:
+                parts.append("".join(rng.choice(list("ACGTN"), p=[.2, .2, .2, .2, .2], size=rng.integers(0, 900))))
+        if r % 3 == 0:
+            parts.append("".join(rng.choice(list("ACGT"), size=rng.integers(0, 2000))))
+        strings.append("".join(parts))
+    strings[5] = "N" * 20000
+    strings[6] = "ACGT" * 100 + "N" * (256 * k * 3) + "ACGT" * 700
+    b = util.batch_from_strings(strings)
+    data, off = to_dev(b)
+    erows, estatus = O.kmer_encode(ot, b.data, b.offsets)
+    longest = max(r.size for r in erows)
+    for cap in (longest + 5, longest // 2 + 3, 2048):
+        ids, mask, lengths, status, max_len = enc.encode_padded(data, off, cap, fill_to=0)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(lengths.cpu().numpy(), [r.size for r in erows])
+        st = status.cpu().numpy()
+        np.testing.assert_array_equal(st & 3, estatus)
+        np.testing.assert_array_equal((st & 4) != 0, np.array([r.size > cap for r in erows]))
+        width = min(cap, longest)
+        assert int(max_len.item()) == width
+        eids, emask = O.pad_rows(erows, 1, width)
+        np.testing.assert_array_equal(ids[:, :width].cpu().numpy(), eids)
+        np.testing.assert_array_equal(mask[:, :width].cpu().numpy(), emask)
+
+
+@both_kmer_kernels
 def test_kmer_pad_to_longest_with_width_guess(kmer_kernel_choice):
     """fill_to = 0 with a guess of the longest row: a guess below, at or above the true width
     gives the same ids / mask / lengths / max_len inside [:, :max_len]."""
