@@ -670,6 +670,75 @@ def pathological_extra():
     return out
 
 
+def kmer_rows_with_n_extra():
+    """The 6-mer encoder on 65,536 rows of 6000 bp that differ only in where they hold N: none, one
+    per row (anywhere / at the start: every later step of the row is then written shifted), 32
+    windows of N at the start (160 extra cells: later steps fall on whole lines again) and the
+    workload's 0.5 % in runs of 1-50.  Every data set is checked against the Hugging Face tokenizer
+    run here on a sample of rows; the stride and the guess follow the library's policy for a stream
+    of batches."""
+    import torch
+    from dnatok_amd import encoders, kmer_tables
+    from tests.support import hf_tokenizers as hf
+    n_rows, length = 65536, 6000
+    vocab = hf.kmer_vocab(6)
+    t = kmer_tables.tables_from_vocab(vocab, 6, vocab["<unk>"])
+    enc = encoders.KmerEncoder(6, t.digit, t.kmer_lut, t.single, vocab["<pad>"], vocab["<unk>"],
+                               t.exp_off, t.exp_len, t.exp_flat)
+    tk = hf.build_kmer_tokenizer(6)
+    off = _dev(np.arange(n_rows + 1, dtype=np.int64) * length)
+    rng = np.random.default_rng(5)
+
+    def free():
+        return many_batches_uniform(n_rows, length, 7002)
+
+    def one_anywhere():
+        a = free().reshape(n_rows, length)
+        a[np.arange(n_rows), rng.integers(0, length, n_rows)] = ord("N")
+        return a.reshape(-1)
+
+    def at_start(n_windows):
+        a = free().reshape(n_rows, length)
+        a[:, :max(1, 6 * n_windows)] = ord("N")
+        return a.reshape(-1)
+
+    out = {}
+    for name, make in (("no_n", free), ("one_n_per_row_anywhere", one_anywhere),
+                       ("one_n_at_row_start", lambda: at_start(0)), ("32_n_windows_at_row_start", lambda: at_start(32)),
+                       ("workload_runs_of_n", lambda: many_batches_uniform(n_rows, length, 7002, n_run_fraction=0.005))):
+        host = make()
+        data = _dev(host)
+        r = enc.encode_padded(data, off, 6016, fill_to=0)
+        torch.cuda.synchronize()
+        width = int(r[4].item())
+        del r
+        guess = encoders.width_guess_after(width)
+        t_cap = guess + (-guess) % 128
+        buf = (torch.empty((n_rows, t_cap), dtype=torch.int32, device="cuda"),
+               torch.empty((n_rows, t_cap), dtype=torch.uint8, device="cuda"),
+               torch.empty(n_rows, dtype=torch.int32, device="cuda"), torch.empty(n_rows, dtype=torch.int32, device="cuda"),
+               torch.empty(1, dtype=torch.int32, device="cuda"))
+
+        class W:
+            def step(self):
+                enc.encode_padded(data, off, t_cap, fill_to=0, width_guess=guess, out=buf)
+        W().step()
+        torch.cuda.synchronize()
+        assert int(buf[4].item()) == width
+        rows = np.concatenate([np.arange(64), rng.integers(0, n_rows, 64)])
+        want = hf_live_rows(tk, np.concatenate([host[r * length:(r + 1) * length] for r in rows]),
+                            np.arange(rows.size + 1, dtype=np.int64) * length)
+        ids, ln = buf[0].cpu().numpy(), buf[2].cpu().numpy()
+        same_rows([ids[r, :ln[r]] for r in rows], want, f"6-mer rows, {name}")
+        _, dm = time_steps(W(), 10, 3)
+        by = n_rows * length + 5 * n_rows * width + 4 * n_rows
+        out[name] = {"t_max": width, "rows_apart": t_cap, "device_us_per_call": dm * 1e3,
+                     "hbm_frac": by / (dm * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        del data, buf
+        torch.cuda.empty_cache()
+    return out
+
+
 def merge_table_placement_extra():
     """The BPE merge table of the 4096 vocabulary in global memory (L2; the default) against its compact
     48 KB form kept in LDS by every workgroup (`dnatok_bpe_set_table_placement`), on batches of 1 KB rows:
@@ -723,7 +792,7 @@ def main() -> None:
     ap.add_argument("--config", default="C2", choices=["C1", "C2", "C3", "C4", "C5"])
     ap.add_argument("--per-call", action="store_true", help="time one exact batch instead of the sustained form")
     ap.add_argument("--no-extras", action="store_true")
-    ap.add_argument("--only-extra", default="", choices=["", "merge_table_placement", "pathological"],
+    ap.add_argument("--only-extra", default="", choices=["", "merge_table_placement", "pathological", "kmer_rows_with_n"],
                     help="run only this extra after the headline (for profiling it)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -803,7 +872,8 @@ def main() -> None:
 
     if args.only_extra:
         result[args.only_extra] = {"merge_table_placement": merge_table_placement_extra,
-                                   "pathological": pathological_extra}[args.only_extra]()
+                                   "pathological": pathological_extra,
+                                   "kmer_rows_with_n": kmer_rows_with_n_extra}[args.only_extra]()
     elif not args.no_extras:
         per_call = {}
         for cfg in ["C1", "C2", "C3", "C4", "C5"]:
