@@ -879,7 +879,8 @@ def main() -> None:
         for cfg in ["C1", "C2", "C3", "C4", "C5"]:
             ww = make_workload(cfg, sustained=False)
             ww.check()
-            wm, dm = time_steps(ww, 20, 3)
+            # 200 calls: a call of 10 us is otherwise timed by the host's first, slow launches
+            wm, dm = time_steps(ww, 200, 20)
             per_call[cfg] = {"workload": ww.name, "ms_per_call": wm, "device_ms_per_call": dm,
                              "mbp_per_s": ww.bases / (wm * 1e-3) / 1e6,
                              "hbm_frac": ww.algorithmic_bytes / (dm * 1e-3) / 1e9 / HBM_PEAK_GBS}
