@@ -402,6 +402,8 @@ class RaggedBoth(Workload):
             lut[ord(ch)] = cv[ch]
         self.lut = lut
         self.char = encoders.CharEncoder(lut, pad_id=cv["<pad>"])
+        self.lut_dev = _dev(lut)
+        self.one_pass = True          # False: the char tokenizer as a launch of its own after the BPE engine
         first = wl.config5_ragged()
         self.first = first
         batches = [first] + [wl.config5_ragged(seed=wl.SEEDS["C5"] + 100 + i) for i in range(n_batches - 1)]
@@ -421,7 +423,7 @@ class RaggedBoth(Workload):
         self.cmask = torch.empty(total, dtype=torch.uint8, device="cuda")
         self.bases = total
         self.kernel = "bpe_lds_kernel"
-        self.name = (f"C5 ragged, {n_batches} x 4096 sequences ({total / 1e6:.1f} Mbp) per call: BPE vocab-4096 + char, "
+        self.name = (f"C5 ragged, {n_batches} x 4096 sequences ({total / 1e6:.1f} Mbp) per call: BPE vocab-4096 + char in one pass over the bytes, "
                      f"packed ids/offsets/masks")
         self.step()
         torch.cuda.synchronize()
@@ -431,10 +433,16 @@ class RaggedBoth(Workload):
 
     def step(self):
         from dnatok_amd import encoders
-        self.bpe.encode(self.data, self.off, self.max_len, tok_tmp=self.tok, lengths=self.lengths)
+        if self.one_pass:
+            # BPE tokens and single-character ids from one pass over the bytes
+            self.bpe.encode_with_chars(self.data, self.off, self.max_len, self.lut_dev, tok_tmp=self.tok,
+                                       lengths=self.lengths, char_ids=self.cids, char_mask=self.cmask)
+        else:
+            self.bpe.encode(self.data, self.off, self.max_len, tok_tmp=self.tok, lengths=self.lengths)
         self.pids, self.out_off, self.pmask = encoders.pack_ragged(self.tok, self.off, self.lengths,
                                                                    out=self.pack_out)
-        self.char.encode_packed(self.data, want_mask=True, ids=self.cids, mask=self.cmask)
+        if not self.one_pass:
+            self.char.encode_packed(self.data, want_mask=True, ids=self.cids, mask=self.cmask)
 
     def check(self):
         """The first 4096 sequences against the committed golden vectors; with more batches per call,

@@ -64,7 +64,15 @@ struct BpeArgs {
     int32_t n_merges;
     const uint32_t *ltab;
     uint32_t lmul1, lmul2;
+    // single-character ids of the same bytes, written in the same pass (dnatok_bpe_encode_with_chars):
+    // char_ids[i] = char_lut[bytes[i]], char_mask[i] = 1 (null: no mask)
+    const int32_t *char_lut;
+    int32_t *char_ids;
+    uint8_t *char_mask;
 };
+
+typedef int32_t bpe_int4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t bpe_u32_a1 __attribute__((aligned(1)));
 
 // What a position keeps about the pair it starts: the rule's rank (kNone = no rule), the
 // symbol the rule produces, and the rule's gate (lowest rank of any rule using that product).
@@ -230,14 +238,20 @@ struct alignas(4 * sizeof(IT)) PosRec {
 // One row.  tid = index in the team; P/NS/MC hold n0 entries, Q (the merges of the current round)
 // n0 / 2, C (its candidates) n0; D holds NT bytes; PER > 0 says that n0 <= PER * NT, and every thread
 // then keeps the ranks of its own positions in registers as well; red holds 4 * (NT / 64) + 4 words.  Tokens go to out[0 .. *out_len).
-template <int NT, typename IT, int PER, typename PT>
+// CHARS: while the piece's bytes pass through the registers on their way into LDS, the
+// single-character id of every byte in [char_lo, char_hi) is written to char_ids (and 1 to char_mask,
+// when given); both pointers are those of the piece's byte 0.
+template <int NT, typename IT, int PER, bool CHARS = false, typename PT>
 __device__ __forceinline__ void bpe_row(
     const PT pt, const uint16_t *byte_to_sym,
     const int32_t *out_remap, const uint8_t *__restrict__ src, const int n0, PosRec<IT> *P,
     uint16_t *NS, uint16_t *MC, IT *Q, IT *C, uint8_t *D, uint32_t *red, const int tid,
     int32_t *__restrict__ out, int32_t *__restrict__ out_len, uint16_t *__restrict__ raw_out = nullptr,
-    const int mid_lo = 0, const int mid_hi = 0, int32_t *__restrict__ mid_out = nullptr)
+    const int mid_lo = 0, const int mid_hi = 0, int32_t *__restrict__ mid_out = nullptr,
+    const int32_t *__restrict__ char_lut = nullptr, int32_t *__restrict__ char_ids = nullptr,
+    uint8_t *__restrict__ char_mask = nullptr, const int char_lo = 0, const int char_hi = 0)
 {
+    static_assert(!CHARS || PER > 0, "the single-character ids are written from the staged bytes");
     constexpr IT NIL = (IT)~(IT)0;
     constexpr IT DEAD = (IT)kNone;
     // pairs of table reads in flight per thread.  (Four cost 20 registers and a wave per SIMD; four
@@ -289,6 +303,29 @@ __device__ __forceinline__ void bpe_row(
                 v = uint2{lo, hi};
             }
             *reinterpret_cast<uint2 *>(stage + 8 * wd) = v;
+            if (CHARS) {
+                if (first >= char_lo && first + 8 <= char_hi) {
+                    int32_t c[8];
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) c[q] = char_lut[((q < 4 ? v.x : v.y) >> (8 * (q & 3))) & 255u];
+                    const bpe_int4_a4 x0 = {c[0], c[1], c[2], c[3]}, x1 = {c[4], c[5], c[6], c[7]};
+                    __builtin_nontemporal_store(x0, reinterpret_cast<bpe_int4_a4 *>(char_ids + first));
+                    __builtin_nontemporal_store(x1, reinterpret_cast<bpe_int4_a4 *>(char_ids + first + 4));
+                    if (char_mask) {
+                        __builtin_nontemporal_store((bpe_u32_a1)0x01010101u, reinterpret_cast<bpe_u32_a1 *>(char_mask + first));
+                        __builtin_nontemporal_store((bpe_u32_a1)0x01010101u, reinterpret_cast<bpe_u32_a1 *>(char_mask + first + 4));
+                    }
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) {
+                        const int pos = first + q;
+                        if (pos >= char_lo && pos < char_hi) {
+                            char_ids[pos] = char_lut[((q < 4 ? v.x : v.y) >> (8 * (q & 3))) & 255u];
+                            if (char_mask) char_mask[pos] = 1;
+                        }
+                    }
+                }
+            }
         }
         team_sync<NT>();
     }
@@ -962,7 +999,7 @@ __global__ __launch_bounds__(256) void bpe_expand_kernel(const int64_t *__restri
 // workgroup shares an item.  PLANNED: the items are those of the work list (rows and chunks of
 // long rows), handed out through an atomic counter.  Otherwise (no row of the batch is longer
 // than CAP) an item is a row, teams take rows round robin, and no work list is built at all.
-template <int NT, int TEAMS, int CAP, bool PLANNED, bool LTAB = false>
+template <int NT, int TEAMS, int CAP, bool PLANNED, bool LTAB = false, bool CHARS = false>
 __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     BpeArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
     BpePlan p, int32_t n_rows, int32_t *__restrict__ tok_tmp, int32_t *__restrict__ lengths)
@@ -1037,13 +1074,21 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
         if (nc == 1 && (len > CAP || len <= 0)) {
             // too long: left to the whole-row kernel (row_fail is set); empty: no tokens
             if (tid == 0) lengths[row] = len > CAP ? -1 : 0;
+            if (CHARS) {
+                for (int64_t i = tid; i < len; i += NT) {
+                    a.char_ids[start + i] = a.char_lut[bytes[start + i]];
+                    if (a.char_mask) a.char_mask[start + i] = 1;
+                }
+            }
         } else if (nc == 1) {
             if (LTAB)
                 bpe_row<NT, uint16_t, (CAP + NT - 1) / NT>(lpt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC,
                                       Q, C, D, red, tid, tok_tmp + start, lengths + row);
             else
-                bpe_row<NT, uint16_t, (CAP + NT - 1) / NT>(pt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC,
-                                      Q, C, D, red, tid, tok_tmp + start, lengths + row);
+                bpe_row<NT, uint16_t, (CAP + NT - 1) / NT, CHARS>(
+                    pt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC, Q, C, D, red, tid, tok_tmp + start,
+                    lengths + row, nullptr, 0, 0, nullptr, a.char_lut, CHARS ? a.char_ids + start : nullptr,
+                    CHARS && a.char_mask ? a.char_mask + start : nullptr, 0, (int)len);
         } else {
             const int64_t e0 = (int64_t)k * p.core - p.overlap < 0 ? 0 : (int64_t)k * p.core - p.overlap;
             int64_t e1 = (int64_t)(k + 1) * p.core + p.overlap;
@@ -1054,9 +1099,13 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
             int64_t mid_lo = k > 0 ? (int64_t)k * p.core + p.overlap : 0;
             if (mid_lo > len) mid_lo = len;
             const int64_t mid_hi = k + 1 < nc ? (int64_t)(k + 1) * p.core - p.overlap : len;
-            bpe_row<NT, uint16_t, (CAP + NT - 1) / NT>(pt, b2s, a.out_remap, bytes + start + e0, (int)(e1 - e0),
-                                  P, NS, MC, Q, C, D, red, tid, nullptr, nullptr, raw,
-                                  (int)(mid_lo - e0), (int)(mid_hi - e0), p.cnt + 4 * (size_t)m);
+            // the single-character ids of a long row are written chunk by chunk: every chunk those of its core
+            const int64_t core_hi = (int64_t)(k + 1) * p.core < len ? (int64_t)(k + 1) * p.core : len;
+            bpe_row<NT, uint16_t, (CAP + NT - 1) / NT, CHARS>(
+                pt, b2s, a.out_remap, bytes + start + e0, (int)(e1 - e0), P, NS, MC, Q, C, D, red, tid, nullptr,
+                nullptr, raw, (int)(mid_lo - e0), (int)(mid_hi - e0), p.cnt + 4 * (size_t)m, a.char_lut,
+                CHARS ? a.char_ids + start + e0 : nullptr, CHARS && a.char_mask ? a.char_mask + start + e0 : nullptr,
+                (int)((int64_t)k * p.core - e0), (int)(core_hi - e0));
         }
         team_sync<NT>();
     }
@@ -1453,12 +1502,12 @@ int64_t lds_resident_teams()
     return (int64_t)resident * TEAMS;
 }
 
-template <int NT, int TEAMS, int CAP, bool PLANNED>
+template <int NT, int TEAMS, int CAP, bool PLANNED, bool CHARS = false>
 int launch_lds_as(const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets, const BpePlan &p,
                   int64_t n_rows, int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
 {
     const size_t lds = lds_bytes<NT, TEAMS, CAP>();
-    auto kern = bpe_lds_kernel<NT, TEAMS, CAP, PLANNED>;
+    auto kern = bpe_lds_kernel<NT, TEAMS, CAP, PLANNED, false, CHARS>;
     static bool attr_set = false;
     if (!attr_set) {
         DNATOK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -1521,7 +1570,7 @@ template <int NT, int TEAMS, int CAP>
 int run_lds(bool long_rows, int chunking, const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets,
             const BpePlan &p, int64_t n_rows, int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
 {
-    if (CAP == 1024 && !long_rows && a.ltab) {
+    if (CAP == 1024 && !long_rows && a.ltab && !a.char_ids) {
         const int mode = g_table_placement.load(std::memory_order_relaxed);
         if (mode == 2 || (mode == 1 && n_rows <= ltab_resident_teams<NT, TEAMS, 1024>()))
             return launch_lds_ltab<NT, TEAMS, 1024>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
@@ -1535,8 +1584,10 @@ int run_lds(bool long_rows, int chunking, const BpeArgs &a, const uint8_t *bytes
             bpe_expand_kernel<<<(int)((n_rows + 255) / 256), 256, 0, s>>>(offsets, n_rows, p);
             DNATOK_HIP_TRY(hipGetLastError());
         }
+        if (a.char_ids) return launch_lds_as<NT, TEAMS, CAP, true, true>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
         return launch_lds_as<NT, TEAMS, CAP, true>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
     }
+    if (a.char_ids) return launch_lds_as<NT, TEAMS, CAP, false, true>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
     return launch_lds_as<NT, TEAMS, CAP, false>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
 }
 
@@ -1544,9 +1595,12 @@ int run_lds(bool long_rows, int chunking, const BpeArgs &a, const uint8_t *bytes
 
 // The launches of one encode call; p lies inside a scratch buffer that holds p.total_bytes.
 static int bpe_encode_launch(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets, int64_t n_rows,
-                             int64_t max_len, const BpePlan &p, int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
+                             int64_t max_len, const BpePlan &p, int32_t *tok_tmp, int32_t *lengths, hipStream_t s,
+                             const int32_t *char_lut = nullptr, int32_t *char_ids = nullptr,
+                             uint8_t *char_mask = nullptr)
 {
-    BpeArgs a{t->tab, t->byte_to_sym, t->out_remap, t->shift, t->mul1, t->mul2, t->n_merges, t->ltab, t->lmul1, t->lmul2};
+    BpeArgs a{t->tab, t->byte_to_sym, t->out_remap, t->shift, t->mul1, t->mul2, t->n_merges, t->ltab, t->lmul1, t->lmul2,
+              char_lut, char_ids, char_mask};
 
     const bool long_rows = max_len > p.ext;
     int chunking = (long_rows && t->monotone) ? 1 : 0;
@@ -1602,6 +1656,28 @@ extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, co
     DNATOK_REQUIRE(((uintptr_t)scratch & 255) == 0, DNATOK_E_INVALID, "dnatok_bpe_encode: scratch must be 256-byte aligned");
     const BpePlan p = make_plan((uint8_t *)scratch, n_rows, max_len, total);
     return bpe_encode_launch(t, bytes, offsets, n_rows, max_len, p, tok_tmp, lengths, (hipStream_t)stream);
+}
+
+extern "C" int dnatok_bpe_encode_with_chars(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets,
+                                            int64_t n_rows, int64_t max_len, int64_t total, void *scratch,
+                                            size_t scratch_bytes, int32_t *tok_tmp, int32_t *lengths,
+                                            const int32_t *char_lut, int32_t *char_ids, uint8_t *char_mask,
+                                            void *stream)
+{
+    const int bad = bpe_encode_check("dnatok_bpe_encode_with_chars", t, bytes, offsets, n_rows, max_len, total, tok_tmp,
+                                     lengths);
+    if (bad) return bad;
+    DNATOK_REQUIRE(char_lut && (char_ids || total == 0), DNATOK_E_INVALID,
+                   "dnatok_bpe_encode_with_chars: char_lut and char_ids are required");
+    if (n_rows == 0) return DNATOK_OK;
+    const BpePlan need = make_plan(nullptr, n_rows, max_len, total);
+    DNATOK_REQUIRE(scratch && scratch_bytes >= need.total_bytes, DNATOK_E_SCRATCH,
+                   "dnatok_bpe_encode_with_chars: scratch holds %zu bytes, %zu needed", scratch_bytes, need.total_bytes);
+    DNATOK_REQUIRE(((uintptr_t)scratch & 255) == 0, DNATOK_E_INVALID,
+                   "dnatok_bpe_encode_with_chars: scratch must be 256-byte aligned");
+    const BpePlan p = make_plan((uint8_t *)scratch, n_rows, max_len, total);
+    return bpe_encode_launch(t, bytes, offsets, n_rows, max_len, p, tok_tmp, lengths, (hipStream_t)stream, char_lut,
+                             char_ids, char_mask);
 }
 
 // ---- the entry point that allocates nothing -------------------------------------------------

@@ -439,6 +439,35 @@ class BpeEncoder:
                    "dnatok_bpe_encode")
         return tok_tmp, lengths
 
+    def encode_with_chars(self, data: torch.Tensor, offsets: torch.Tensor, max_len: int, char_lut: torch.Tensor, *,
+                          tok_tmp: Optional[torch.Tensor] = None, lengths: Optional[torch.Tensor] = None,
+                          char_ids: Optional[torch.Tensor] = None, char_mask: Optional[torch.Tensor] = None,
+                          want_char_mask: bool = True):
+        """``encode`` plus the single-character ids of the same bytes from the same pass over them:
+        ``char_ids[i] = char_lut[data[i]]`` (``char_lut``: device int32[256], e.g.
+        ``CharEncoder.lut_device``), ``char_mask[i] = 1``.  Returns (tok_tmp, lengths, char_ids, char_mask)."""
+        _require_cuda(data, torch.uint8, "data")
+        _require_cuda(offsets, torch.int64, "offsets")
+        _require_cuda(char_lut, torch.int32, "char_lut")
+        if char_lut.numel() != 256:
+            raise ValueError("char_lut must hold 256 ids")
+        n_rows = offsets.numel() - 1
+        total = data.numel()
+        if tok_tmp is None:
+            tok_tmp = torch.empty(max(total, 1), dtype=torch.int32, device=data.device)
+        if lengths is None:
+            lengths = torch.empty(n_rows, dtype=torch.int32, device=data.device)
+        if char_ids is None:
+            char_ids = torch.empty(max(total, 1), dtype=torch.int32, device=data.device)
+        if char_mask is None and want_char_mask:
+            char_mask = torch.empty(max(total, 1), dtype=torch.uint8, device=data.device)
+        scratch = self._get_scratch(n_rows, int(max_len), total, data.device)
+        _lib.check(_lib.lib().dnatok_bpe_encode_with_chars(
+            self._h, _ptr(data), _ptr(offsets), n_rows, int(max_len), total, _ptr(scratch), scratch.numel(),
+            _ptr(tok_tmp), _ptr(lengths), _ptr(char_lut), _ptr(char_ids),
+            _ptr(char_mask) if char_mask is not None else None, _stream()), "dnatok_bpe_encode_with_chars")
+        return tok_tmp, lengths, char_ids, char_mask
+
 
 def pack_ragged(tok_tmp: torch.Tensor, in_offsets: torch.Tensor, lengths: torch.Tensor, *,
                 remap: Optional[torch.Tensor] = None, want_mask: bool = True, out=None):

@@ -597,6 +597,47 @@ def test_bpe_long_rows(bpe):
         np.testing.assert_array_equal(r, e)
 
 
+def test_bpe_with_single_character_ids_from_the_same_pass(bpe):
+    """dnatok_bpe_encode_with_chars: the tokens are those of dnatok_bpe_encode and the character ids
+    are lut[byte] for every byte, on every route a row can take: short rows one per team, more rows
+    than teams (the work list), rows cut into chunks (each chunk writes the characters of its
+    core), rows redone by the whole-row kernel, empty rows, a mask or none; buffers start at odd
+    addresses so that no store may assume more than its 4-byte alignment."""
+    which, enc, bo = bpe
+    say(f"bpe{which} + single-character ids in one pass")
+    lut = np.zeros(256, dtype=np.int32)
+    for i, ch in enumerate("ACGTN"):
+        lut[ord(ch)] = 7 + i
+    lut_dev = torch.from_numpy(lut).to(DEV)
+    rng = random.Random(41)
+    rnd = lambda n: "".join(rng.choices("ACGTN", weights=[24, 24, 24, 24, 4], k=n))
+    batches = [
+        [rnd(n) for n in (0, 1, 7, 8, 9, 63, 1000, 1024, 0, 333)],
+        [rnd(rng.randint(0, 900)) for _ in range(3000)],
+        wl.config5_ragged(300, seed=12).strings() + ["", rnd(5000), "A" * 30000, rnd(100_001), "ACGTC" * 4000],
+    ]
+    for seqs in batches:
+        b = util.batch_from_strings(seqs)
+        data, off = to_dev(b)
+        max_len = int(b.lengths().max())
+        total = int(b.data.size)
+        for shift, want_mask in ((0, True), (3, False), (5, True)):
+            # the same bytes at another alignment: outputs that start `shift` elements into their allocation
+            d2 = torch.empty(total + 16, dtype=torch.uint8, device=DEV)[shift:shift + total].copy_(data)
+            cids = torch.full((total + 16,), -1, dtype=torch.int32, device=DEV)[shift:shift + max(total, 1)]
+            cmask = torch.zeros(total + 16, dtype=torch.uint8, device=DEV)[shift:shift + max(total, 1)] if want_mask else None
+            tok, lengths, cids, cmask = enc.encode_with_chars(d2, off, max_len, lut_dev, char_ids=cids, char_mask=cmask,
+                                                              want_char_mask=want_mask)
+            torch.cuda.synchronize()
+            np.testing.assert_array_equal(cids[:total].cpu().numpy(), lut[b.data])
+            if want_mask:
+                assert bool((cmask[:total] == 1).all())
+            tok, lengths = tok.cpu().numpy(), lengths.cpu().numpy()
+            ref = bo.encode_batch(b.data, b.offsets)
+            for i, e in enumerate(ref):
+                np.testing.assert_array_equal(tok[b.offsets[i]:b.offsets[i] + lengths[i]], e, err_msg=f"row {i}")
+
+
 def test_bpe_rows_without_a_seam_fall_back_to_the_whole_row_kernel(bpe):
     """Tandem repeats far longer than the chunk overlap: neighbouring chunk runs can stay out
     of phase, no seam is accepted, and the row is redone by the whole-row kernel."""
@@ -755,6 +796,16 @@ def test_bpe_nonmonotone_tables_with_rows_above_the_lds_capacity():
         b = util.batch_from_strings(seqs)
         for s, r, e in zip(seqs, bpe_rows(enc, b), bo.encode_batch(b.data, b.offsets, remap=False)):
             np.testing.assert_array_equal(r, e, err_msg=f"trial {trial} len {len(s)} {merges}")
+        # the same rows with the single-character ids asked for: rows left to the whole-row kernel get theirs too
+        data, off = to_dev(b)
+        lut = (np.arange(256, dtype=np.int32) * 3 + 1)
+        tok, lengths, cids, cmask = enc.encode_with_chars(data, off, int(b.lengths().max()), torch.from_numpy(lut).to(DEV))
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(cids.cpu().numpy(), lut[b.data])
+        assert bool((cmask == 1).all())
+        tok, lengths = tok.cpu().numpy(), lengths.cpu().numpy()
+        for i, e in enumerate(bo.encode_batch(b.data, b.offsets, remap=False)):
+            np.testing.assert_array_equal(tok[b.offsets[i]:b.offsets[i] + lengths[i]], e)
     assert n_nonmonotone == 6
 
 
