@@ -204,9 +204,9 @@ int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t
  * over them: char_ids[i] = char_lut[bytes[i]] for every byte of every row (int32[total], laid out as
  * the bytes are: row b at offsets[b]), char_mask[i] = 1 (uint8[total], NULL allowed); char_lut is a
  * device int32[256].  This is dnatok_char_encode_packed fused into the merge engine for batches that
- * go through both tokenizers (the reference runs the two tokenizers one after the other,
- * src/dna_tokenizer.py:3143-3210 over src/gputok_bpe_backend.py:531-601); tokens, lengths, scratch
- * and errors as for dnatok_bpe_encode. */
+ * go through both tokenizers (the reference runs the two one after the other: the ASCII table
+ * path, src/dna_tokenizer.py:2594-2651, and GPUTokBPEBackend.encode_batch,
+ * src/gputok_bpe_backend.py:531-601); tokens, lengths, scratch and errors as for dnatok_bpe_encode. */
 int dnatok_bpe_encode_with_chars(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets,
                                  int64_t n_rows, int64_t max_len, int64_t total,
                                  void *scratch, size_t scratch_bytes,
