@@ -67,8 +67,8 @@ static std::atomic<int> g_team_rows{-1};
 constexpr int kMaxSlotStride = 32;       // 64-bit words between two slots (one 256-byte line each)
 // A call whose kernel reports the maximum itself (kmer_team_kernel, publish) gathers it up a tree
 // of 64-bit words with four 16-bit fields each: kTreeRows leaves, four children per word.
-constexpr int kTreeRows = 1024;
-constexpr int kTreeWords = 512;          // 256 + 64 + 16 + 4 + 1 words used, 4 KB per slot
+constexpr int kTreeRows = 2048;          // workgroups of one call (a row each, or the persistent grid)
+constexpr int kTreeWords = 1024;         // 512 + 128 + 32 + 8 + 2 + 1 words used, 8 KB per slot
 
 namespace dnatok {
 
@@ -160,12 +160,52 @@ __device__ __forceinline__ void wave_sync()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// The longest row of a call without a padding pass (every row padded as far as any row can
+// reach), found without a fence: nothing but atomics carries it.  Every workgroup adds its
+// maximum + 1 into its 16-bit field of a 64-bit word shared by four workgroups; the atomic returns
+// the fields of those that came before, so the workgroup that completes a word knows the maximum
+// of its four, clears the word for the next call and carries the maximum one level up in the same
+// way (a 4-ary tree, `tree` holds its words level by level).  Who completes the root writes
+// max_len.  `mine` is the caller's value + 1 and `before` what its own atomicAdd at the lowest
+// level returned (the caller issues that one itself, as early as it knows its value); one lane
+// calls this.  (One counter and one atomicMax for 256 workgroups cost 3 us, two of them spent
+// queueing at that one address.)
+__device__ __forceinline__ void climb_max_tree(unsigned long long *tree, unsigned idx, unsigned n_here,
+                                               unsigned long long mine, unsigned long long before,
+                                               int32_t *__restrict__ max_len)
+{
+    unsigned long long *level = tree;
+    for (;;) {
+        const unsigned long long all = before + (mine << (16 * (idx & 3)));
+        const unsigned members = n_here - (idx & ~3u) < 4u ? n_here - (idx & ~3u) : 4u;
+        unsigned arrived = 0;
+        unsigned long long best = 0;
+#pragma unroll
+        for (int f = 0; f < 4; ++f) {
+            const unsigned long long v = (all >> (16 * f)) & 0xFFFFull;
+            arrived += v != 0;
+            best = v > best ? v : best;
+        }
+        if (arrived < members) break;
+        atomicExch(level + (idx >> 2), 0ull);
+        if (n_here <= 4) {
+            *max_len = (int32_t)best - 1;
+            break;
+        }
+        level += (n_here + 3) >> 2;
+        n_here = (n_here + 3) >> 2;
+        idx >>= 2;
+        mine = best;
+        before = atomicAdd(level + (idx >> 2), mine << (16 * (idx & 3)));
+    }
+}
+
 template <int K, bool LUT4_LDS, bool CHARS, bool HAS_MASK>
 __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
     KmerArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
     int64_t n_rows, int64_t t_cap, int64_t fill_to, int32_t *__restrict__ ids,
     uint8_t *__restrict__ mask, int32_t *__restrict__ lengths, int32_t *__restrict__ status,
-    int32_t *__restrict__ max_len, MaxRef mref)
+    int32_t *__restrict__ max_len, MaxRef mref, int publish)
 {
     constexpr uint32_t POW4 = 1u << (2 * K);
     __shared__ uint32_t s_dig[256];
@@ -183,7 +223,7 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
     }
     if (LUT4_LDS)
         for (uint32_t i = threadIdx.x; i < POW4; i += kKmerThreads) s_lut4[i] = a.lut4[i];
-    __syncthreads();          // the only workgroup barrier: from here on every wave runs alone
+    __syncthreads();          // from here on every wave runs alone (one more barrier at the very end, with `publish`)
 
     const int lane = threadIdx.x & 63;
     int32_t *const buf = s_stage[__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6))];
@@ -581,6 +621,21 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
         if (stored > wave_max) wave_max = stored;
         if (fill > stored) pad_cells(outA, moutA, mis, stored, fill, a.pad_id, lane);
     }
+    if (publish) {
+        // no padding pass follows: the workgroups' maxima go up the tree (climb_max_tree)
+        __shared__ uint32_t s_wave_max[kKmerThreads / 64];
+        if (lane == 0) s_wave_max[wave_in_wg] = (uint32_t)wave_max;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            uint32_t m = 0;
+#pragma unroll
+            for (int q = 0; q < kKmerThreads / 64; ++q) m = s_wave_max[q] > m ? s_wave_max[q] : m;
+            const unsigned long long mine = (unsigned long long)m + 1;
+            const unsigned long long before = atomicAdd(mref.tree + (blockIdx.x >> 2), mine << (16 * (blockIdx.x & 3)));
+            climb_max_tree(mref.tree, blockIdx.x, gridDim.x, mine, before, max_len);
+        }
+        return;
+    }
     // one atomic per wave at most, skipped when another wave already published a larger value
     if (mref.slot) {
         // (the first wave publishes even a maximum of 0: the slot then carries this call's tag)
@@ -935,43 +990,9 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_team_kernel(
     }
     if (wv == 0) {
         if (mref.slot && publish) {
-            // No padding pass follows (every row is padded as far as any row can reach), so the
-            // kernel reports the batch's maximum itself, and without a fence: nothing but atomics
-            // carries it.  A workgroup (it has one row: the grid is the batch) added its length + 1
-            // into its 16-bit field of a tree word as soon as the length was known; the atomic
-            // returns the fields of those that came before, so the one that completes a word
-            // knows the maximum of its four, clears the word for the next call and carries the
-            // maximum one level up in the same way.  Who completes the root writes max_len.
-            // (One counter and one atomicMax for all workgroups cost 3 us here, two of them spent
-            // queueing at that one address.)
-            if (lane == 0) {
-                unsigned long long *level = mref.tree;
-                unsigned idx = blockIdx.x, n_here = gridDim.x;
-                unsigned long long mine = sent_val, before = sent;
-                for (;;) {
-                    const unsigned long long all = before + (mine << (16 * (idx & 3)));
-                    const unsigned members = n_here - (idx & ~3u) < 4u ? n_here - (idx & ~3u) : 4u;
-                    unsigned arrived = 0;
-                    unsigned long long best = 0;
-#pragma unroll
-                    for (int f = 0; f < 4; ++f) {
-                        const unsigned long long v = (all >> (16 * f)) & 0xFFFFull;
-                        arrived += v != 0;
-                        best = v > best ? v : best;
-                    }
-                    if (arrived < members) break;
-                    atomicExch(level + (idx >> 2), 0ull);
-                    if (n_here <= 4) {
-                        *max_len = (int32_t)best - 1;
-                        break;
-                    }
-                    level += (n_here + 3) >> 2;
-                    n_here = (n_here + 3) >> 2;
-                    idx >>= 2;
-                    mine = best;
-                    before = atomicAdd(level + (idx >> 2), mine << (16 * (idx & 3)));
-                }
-            }
+            // the workgroup (it has one row: the grid is the batch) added its length + 1 to its tree
+            // word as soon as the length was known, before the row's last tokens were written
+            if (lane == 0) climb_max_tree(mref.tree, blockIdx.x, gridDim.x, sent_val, sent, max_len);
         } else if (mref.slot) {
             const unsigned long long v = (slot_gen << 32) | (unsigned long long)wg_max;
             if (lane == 0 && (wg_max > 0 || blockIdx.x == 0) && __builtin_nontemporal_load(mref.slot) < v)
@@ -1192,10 +1213,12 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
     // persistent waves: the tables are staged into LDS once per workgroup
     const int64_t want = (n_rows + kKmerThreads / 64 - 1) / (kKmerThreads / 64);
     // few rows (a workgroup for every row at once): the four waves of a workgroup share a row.
-    // When the row stride is already cut to the guess (at most kTightStride cells beyond it), those
+    // When the row stride is already cut to the guess (at most kTightStride cells beyond it), the
     // rows are padded to the whole stride while they are written, which covers every possible
-    // maximum: the kernel then reports the maximum itself and the padding launch is left out.
+    // maximum: the kernel (either of the two) then reports the maximum itself and the padding
+    // launch is left out (4 % of the 6-mer workload's step, 40 % of a single batch's).
     constexpr int64_t kTightStride = 256;
+    const bool tight = to_longest && mref.slot && guess > 0 && t_cap - guess <= kTightStride && t_cap < 0xFFFF;
     bool padded_in_kernel = false;
 #define LAUNCH3(KK, L, C, M)                                                                      \
     do {                                                                                          \
@@ -1203,16 +1226,17 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
         static const int team_resident = resident_workgroups(kmer_team_kernel<KK, L, C, M>, kKmerThreads, 0, 4); \
         const int team_rows = g_team_rows.load(std::memory_order_relaxed);                       \
         if (n_rows <= (team_rows < 0 ? team_resident : team_rows)) {                              \
-            padded_in_kernel = to_longest && mref.slot && guess > 0 && t_cap - guess <= kTightStride && \
-                               n_rows <= kTreeRows && t_cap < 0xFFFF;                            \
+            padded_in_kernel = tight && n_rows <= kTreeRows;                                      \
             kmer_team_kernel<KK, L, C, M><<<(int)n_rows, kKmerThreads, 0, s>>>(                   \
                 a, bytes, offsets, n_rows, t_cap, padded_in_kernel ? t_cap : fill_to, ids, mask,  \
                 lengths, status, max_len, mref, padded_in_kernel ? 1 : 0);                        \
             break;                                                                                \
         }                                                                                         \
         const int64_t grid = want < resident ? want : resident;                                   \
+        padded_in_kernel = tight && grid <= kTreeRows;                                            \
         kmer_rows_kernel<KK, L, C, M><<<(int)grid, kKmerThreads, 0, s>>>(                         \
-            a, bytes, offsets, n_rows, t_cap, fill_to, ids, mask, lengths, status, max_len, mref); \
+            a, bytes, offsets, n_rows, t_cap, padded_in_kernel ? t_cap : fill_to, ids, mask,      \
+            lengths, status, max_len, mref, padded_in_kernel ? 1 : 0);                            \
     } while (0)
 #define LAUNCH2(KK, L, C)                                                                         \
     do {                                                                                          \
