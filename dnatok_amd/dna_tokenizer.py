@@ -408,10 +408,12 @@ class DNATok:
         worst = max(int(t_cap), int(min_width), 1)
         if pad_multiple > 1 and worst % pad_multiple:
             worst += pad_multiple - worst % pad_multiple
-        # In a stream of batches the rows are laid out only as far apart as the previous batch was
-        # wide (plus a margin): a token run is several times shorter than its row of bytes.  A
+        # In a stream of batches the rows are laid out only as far apart as the recent batches were
+        # wide (encoders.WidthGuess, plus a margin): a token run is several times shorter than its row of bytes.  A
         # batch that needs more room than that is padded again with room for the worst case.
-        guess = getattr(self, "_bpe_width_guess", 0)
+        if not hasattr(self, "_bpe_widths"):
+            self._bpe_widths = encoders.WidthGuess()
+        guess = self._bpe_widths.next()
         cap = worst
         if guess:
             cap = max(guess + (-guess) % 128, int(min_width))
@@ -442,7 +444,7 @@ class DNATok:
             if longest < cap or cap >= worst:            # (the packer reports lengths cut to the stride)
                 break
             cap = worst                                  # a row may have been cut: once more, with room for all
-        self._bpe_width_guess = encoders.width_guess_after(longest)
+        self._bpe_widths.update(longest)
         self._staged_host_ids = staged[:, :width] if staged is not None else None
         return ids[:, :width], mask[:, :width]
 
@@ -515,12 +517,14 @@ class DNATok:
         # a stride of whole 128-byte lines keeps every row of ids and of the mask on line boundaries
         t_cap += (-t_cap) % 128
         plain = (not left) and dtype == torch.int32 and pad_multiple <= 1
-        # The width of the previous batch (plus a margin) is a good guess of this one's in a stream
-        # of batches: rows are padded that far while they are written, and the rows are laid out
+        # The width of the recent batches (encoders.WidthGuess, plus a margin) is a good guess of this
+        # one's in a stream of batches: rows are padded that far while they are written, and the rows are laid out
         # that far apart (whole 128-byte lines), which makes the output nearly dense in memory
         # instead of a fifth of a worst-case buffer.  A batch that turns out wider than the guess
         # fills the stride to the last cell; it is then encoded again with room for the worst case.
-        guess = getattr(self, "_kmer_width_guess", 0) if plain else 0
+        if not hasattr(self, "_kmer_widths"):
+            self._kmer_widths = encoders.WidthGuess()
+        guess = self._kmer_widths.next() if plain else 0
         worst = t_cap
         if guess:
             t_cap = min(worst, guess + (-guess) % 128)
@@ -548,7 +552,7 @@ class DNATok:
                 ids, mask, lengths, status, longest = run(t_cap, 0)
                 meta_h = meta.cpu().numpy()
                 width = int(meta_h[2 * n])
-            self._kmer_width_guess = encoders.width_guess_after(width)
+            self._kmer_widths.update(width)
             plain = width >= min_width
         if not plain:
             cap = max(t_cap, int(min_width))

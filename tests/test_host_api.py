@@ -277,3 +277,28 @@ def test_hostpack_writes_offsets_and_bytes_as_the_python_path_does():
     assert _hostpack.pack_strings([], buf.data_ptr(), buf.numel(), 0) == (0, 0, 0, 256)
     with pytest.raises(TypeError):
         _hostpack.pack_strings(["A", b"C"], buf.data_ptr(), buf.numel(), 0)
+
+
+def test_width_guess_of_a_stream_follows_the_recent_peak():
+    """encoders.WidthGuess: the guess of the next batch's width comes from the largest of the recent
+    widths (fading by 1/256 per batch), not from the last batch alone.  On widths that wander as
+    those of small 6-mer batches do (1100 .. 1265 tokens) the row stride derived from it (whole
+    128-byte lines) is then almost never too small, which the previous width plus its margin is for
+    one batch in seven; it still comes down when the stream turns narrower."""
+    from dnatok_amd import encoders
+    rng = np.random.default_rng(3)
+    # widest row of a batch: a base level with an occasional long run of N
+    widths = 1100 + (rng.gamma(1.2, 28, size=4000)).astype(np.int64).clip(0, 165)
+    stride = lambda g: g + (-g) % 128
+    wg, short_peak, short_prev = encoders.WidthGuess(), 0, 0
+    assert not wg and wg.next() == 0
+    for i, w in enumerate(widths[:-1]):
+        wg.update(int(w))
+        assert wg and wg.next() >= int(w) + 8 and wg.next() % 32 == 0
+        short_peak += int(widths[i + 1]) >= stride(wg.next())
+        short_prev += int(widths[i + 1]) >= stride(encoders.width_guess_after(int(w)))
+    assert short_peak * 8 < short_prev and short_peak < 0.015 * widths.size
+    # a stream that turns narrower: the guess follows within a few hundred batches
+    for _ in range(450):
+        wg.update(300)
+    assert wg.next() <= 352
