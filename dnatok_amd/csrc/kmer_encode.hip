@@ -175,6 +175,10 @@ __device__ __forceinline__ void climb_max_tree(unsigned long long *tree, unsigne
                                                int32_t *__restrict__ max_len)
 {
     unsigned long long *level = tree;
+    // words this workgroup completed: cleared when it is done climbing, so that a level costs one
+    // trip to memory (the add, whose answer is waited for) and not two
+    unsigned long long *completed[8];
+    int n_completed = 0;
     for (;;) {
         const unsigned long long all = before + (mine << (16 * (idx & 3)));
         const unsigned members = n_here - (idx & ~3u) < 4u ? n_here - (idx & ~3u) : 4u;
@@ -187,7 +191,7 @@ __device__ __forceinline__ void climb_max_tree(unsigned long long *tree, unsigne
             best = v > best ? v : best;
         }
         if (arrived < members) break;
-        atomicExch(level + (idx >> 2), 0ull);
+        completed[n_completed++] = level + (idx >> 2);
         if (n_here <= 4) {
             *max_len = (int32_t)best - 1;
             break;
@@ -198,6 +202,7 @@ __device__ __forceinline__ void climb_max_tree(unsigned long long *tree, unsigne
         mine = best;
         before = atomicAdd(level + (idx >> 2), mine << (16 * (idx & 3)));
     }
+    for (int i = 0; i < n_completed; ++i) atomicExch(completed[i], 0ull);
 }
 
 template <int K, bool LUT4_LDS, bool CHARS, bool HAS_MASK>
