@@ -206,7 +206,7 @@ class KmerPadded(Workload):
         # a usable guess the rows lie the worst case apart.
         if not t_cap:
             t_cap = 6016
-            if guess == "previous":
+            if guess in ("previous", "fixed"):
                 g = max(encoders.width_guess_after(wd) for wd in self.widths)
                 t_cap = g + (-g) % 128
         self.t_cap = t_cap
@@ -214,28 +214,32 @@ class KmerPadded(Workload):
                     torch.empty((self.n_rows, t_cap), dtype=torch.uint8, device=dev),
                     torch.empty(self.n_rows, dtype=torch.int32, device=dev),
                     torch.empty(self.n_rows, dtype=torch.int32, device=dev),
-                    torch.empty(1, dtype=torch.int32, device=dev))
+                    torch.empty(1, dtype=torch.int32, device=dev) if guess != "fixed" else None)
         self.bases = self.hosts[0].size
         self.kernel = "kmer_rows_kernel"
         how = {"previous": "width of the previous call, which ran on different data, plus the library's margin, passed as the guess",
                "stale": "width of the previous call, which ran on different data, passed as the guess as it is",
-               "none": "no width guess"}[guess]
+               "none": "no width guess", "fixed": ""}[guess]
         self.name = (f"C2 non-overlapping 6-mer vocab-4106, 256x6000 bp batches, {n_batches} distinct batch(es) "
-                     f"per call, two data sets taking turns, pad to longest row ({how}), rows {t_cap} cells apart")
-        # 1 B/base read; int32 id + uint8 mask for every cell of [rows, T_max]; int32 length per row;
-        # the mean over the two data sets, which take turns
-        self.algorithmic_bytes = self.bases + 5 * self.n_rows * sum(self.widths) // 2 + 4 * self.n_rows
+                     f"per call, two data sets taking turns, " +
+                     (f"pad to longest row ({how})" if guess != "fixed" else
+                      f"padded to a fixed width of {t_cap} cells (the reference's token_len; no longest row to find)") +
+                     f", rows {t_cap} cells apart")
+        # 1 B/base read; int32 id + uint8 mask for every cell of [rows, T_max] (the fixed width: of
+        # [rows, t_cap]); int32 length per row; the mean over the two data sets, which take turns
+        cells = self.n_rows * sum(self.widths) // 2 if guess != "fixed" else self.n_rows * t_cap
+        self.algorithmic_bytes = self.bases + 5 * cells + 4 * self.n_rows
         self.turn = 0
 
     def run(self, which: int, width_guess: int):
-        self.enc.encode_padded(self.sets[which], self.off, self.t_cap, fill_to=0, width_guess=width_guess,
-                               out=self.out)
+        self.enc.encode_padded(self.sets[which], self.off, self.t_cap, fill_to=self.t_cap if self.guess == "fixed" else 0,
+                               width_guess=width_guess, out=self.out)
         self.last = which
 
     def step(self):
         from dnatok_amd import encoders
         previous = self.widths[self.turn ^ 1]
-        guess = {"previous": encoders.width_guess_after(previous), "stale": previous, "none": 0}[self.guess]
+        guess = {"previous": encoders.width_guess_after(previous), "stale": previous, "none": 0, "fixed": 0}[self.guess]
         self.run(self.turn, guess)
         self.turn ^= 1
 
@@ -252,8 +256,8 @@ class KmerPadded(Workload):
             self.step()
             torch.cuda.synchronize()
             ln = lengths.cpu().numpy()
-            m = int(max_len.item())
-            assert m == self.widths[which] == int(ln.max())
+            m = int(max_len.item()) if max_len is not None else self.t_cap
+            assert self.widths[which] == int(ln.max()) and (max_len is None or m == self.widths[which])
             assert int(status.abs().sum().item()) == 0
             if which == 0:
                 util.check_against_golden("C2_kmer", [ids[r, :ln[r]].cpu().numpy() for r in range(256)])
@@ -909,9 +913,9 @@ def main() -> None:
             torch.cuda.empty_cache()
         result["sustained"] = sustained
         if args.config == "C2" and not args.per_call:
-            # the same workload under the other width-guess policies
+            # the same workload under the other width-guess policies, and padded to a fixed width instead
             other = {}
-            for guess in ("stale", "none"):
+            for guess in ("stale", "none", "fixed"):
                 ww = make_workload("C2", sustained=True, guess=guess)
                 ww.check()
                 wm, dm = time_steps(ww, args.steps, args.warmup)
