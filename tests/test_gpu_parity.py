@@ -399,6 +399,37 @@ def test_kmer_pad_to_longest_with_row_stride_cut_to_the_guess(kmer_enc, kmer_ker
 
 
 @both_kmer_kernels
+@pytest.mark.parametrize("k", [2, 3, 4, 5, 7, 8])
+def test_kmer_row_stride_cut_to_the_guess_for_every_k(kmer_kernel_choice, k):
+    """The one-launch form of pad-to-longest (rows as far apart as the guess) for the other window
+    lengths, with and without a mask, with strides that are no multiple of four cells: the same
+    ids, mask, lengths and longest row as the call with room for the worst case."""
+    say(f"kmer tight stride k={k}")
+    vocab = hf.kmer_vocab(k)
+    t = kmer_tables.tables_from_vocab(vocab, k, 0)
+    enc = encoders.KmerEncoder(k, t.digit, t.kmer_lut, t.single, pad_id=1, missing_id=0,
+                               exp_off=t.exp_off, exp_len=t.exp_len, exp_flat=t.exp_flat)
+    rng = np.random.default_rng(200 + k)
+    for n_rows in (3, 70, 1300):
+        lens = rng.integers(0, 900, size=n_rows)
+        b = util.batch_from_strings(["".join(rng.choice(list("ACGTN"), p=[.24, .24, .24, .24, .04], size=m)) for m in lens])
+        data, off = to_dev(b)
+        ref = enc.encode_padded(data, off, 904, fill_to=0)
+        torch.cuda.synchronize()
+        width = int(ref[4].item())
+        assert width == int(ref[2].max().item())
+        for t_cap, guess, want_mask in ((width + 1, width - 5, True), (width + 30, width + 2, False), (width + 255, width, True)):
+            got = enc.encode_padded(data, off, t_cap, fill_to=0, width_guess=guess, want_mask=want_mask)
+            torch.cuda.synchronize()
+            assert int(got[4].item()) == width, (n_rows, t_cap)
+            np.testing.assert_array_equal(got[0][:, :width].cpu().numpy(), ref[0][:, :width].cpu().numpy())
+            if want_mask:
+                np.testing.assert_array_equal(got[1][:, :width].cpu().numpy(), ref[1][:, :width].cpu().numpy())
+            np.testing.assert_array_equal(got[2].cpu().numpy(), ref[2].cpu().numpy())
+            np.testing.assert_array_equal(got[3].cpu().numpy(), ref[3].cpu().numpy())
+
+
+@both_kmer_kernels
 def test_kmer_pad_to_longest_replayed_from_a_graph(kmer_enc, kmer_kernel_choice):
     """A captured pad-to-longest call, replayed over changing input: every replay reports the
     longest row of its own input (first a batch with long rows, then shorter ones, then long
