@@ -88,6 +88,15 @@ class NTv3Tokenizer(_SimpleTokenizer):
         unk = self.unk_token_id
         return [self._token_to_id.get(c.upper(), unk) if c.upper() in self._std else unk for c in text]
 
+    def save_vocabulary(self, save_dir: str, prefix: Optional[str] = None):
+        """Writes ``[prefix-]vocab.json`` (token -> id), which the constructor reads back
+        (reference: src/dnatok_compat.py:152-156)."""
+        os.makedirs(save_dir, exist_ok=True)
+        path = os.path.join(save_dir, (f"{prefix}-" if prefix else "") + "vocab.json")
+        with open(path, "w", encoding="utf-8") as fh:
+            json.dump(self._token_to_id, fh, indent=2)
+        return (path,)
+
 
 class Evo2ByteTokenizer(_SimpleTokenizer):
     """Byte-level tokenizer of Evo2: id = ord(c) (reference: src/dnatok_compat.py:181-218)."""
@@ -106,6 +115,15 @@ class Evo2ByteTokenizer(_SimpleTokenizer):
 
     def _encode_one(self, text: str) -> List[int]:
         return [ord(c) if ord(c) < self._vocab_size else self.unk_token_id for c in text]
+
+    def save_vocabulary(self, save_dir: str, prefix: Optional[str] = None):
+        """Writes ``[prefix-]evo2_vocab.json`` holding the vocabulary size, all there is to this
+        tokenizer (reference: src/dnatok_compat.py:213-218)."""
+        os.makedirs(save_dir, exist_ok=True)
+        path = os.path.join(save_dir, (f"{prefix}-" if prefix else "") + "evo2_vocab.json")
+        with open(path, "w", encoding="utf-8") as fh:
+            json.dump({"vocab_size": self._vocab_size}, fh)
+        return (path,)
 
 
 class CharTokenizer(_SimpleTokenizer):

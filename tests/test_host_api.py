@@ -130,6 +130,18 @@ def test_compat_tokenizers():
 
 # ------------------------------------------------------------------ host ingest (C ABI, CPU code)
 
+def test_compat_tokenizers_save_their_vocabulary(tmp_path):
+    """save_vocabulary as the reference's classes have it (src/dnatok_compat.py:152-156, 213-218):
+    the NTv3 file is read back by the constructor, the Evo2 file holds the vocabulary size."""
+    t = dnatok_compat.NTv3Tokenizer()
+    (path,) = t.save_vocabulary(str(tmp_path), "x")
+    assert path.endswith("x-vocab.json")
+    again = dnatok_compat.NTv3Tokenizer(vocab_file=path)
+    assert again.get_vocab() == t.get_vocab() and again.encode("ACGTNacgtx") == t.encode("ACGTNacgtx")
+    (path,) = dnatok_compat.Evo2ByteTokenizer(300).save_vocabulary(str(tmp_path))
+    assert path.endswith("evo2_vocab.json") and json.load(open(path)) == {"vocab_size": 300}
+
+
 def test_host_clean_ascii_matches_oracle():
     import torch
     from dnatok_amd import encoders
