@@ -263,6 +263,58 @@ def cmd_bench(args) -> int:
     return 0
 
 
+def cmd_demo(args) -> int:
+    """info, encode of a sample, bit identity on 50 short sequences, a small benchmark: the
+    reference's end-to-end run (src/dnatok_cli.py:310-348) over a model this build can load."""
+    print("=" * 70)
+    print(f"dnatok demo: model={args.model}")
+    print("=" * 70)
+    args.json = False
+    print("\n[1/4] tokenizer info")
+    cmd_info(args)
+    print("\n[2/4] encode a sample sequence")
+    args.seq, args.fasta = args.sample or "ACGT" * 15, None
+    cmd_encode(args)
+    print("\n[3/4] bit identity with the tokenizer (n=50, random ACGT sequences, 256 bp)")
+    args.n, args.window, args.seed = 50, 256, 42
+    rc = cmd_validate(args)
+    if rc != 0:
+        print("  bit identity FAILED: see first_mismatch above")
+        return rc
+    print("  bit identity holds")
+    print("\n[4/4] small benchmark (n=100, 1024 bp, 32 per call, 4 host threads)")
+    args.n, args.window, args.chunk, args.hf_threads, args.seed = 100, 1024, 32, 4, 11
+    return cmd_bench(args)
+
+
+# What --model accepts.  The reference's registry (src/dnatok_cli.py:55-76) names models on the
+# Hugging Face hub; nothing is downloaded here, so the registry names what is built in and what a
+# local path may be.
+MODEL_REGISTRY = {
+    "char": ("char", "built in", "single-nucleotide ids A C G T N + specials (vocab 11): byte table kernel"),
+    "ntv3": ("ntv3", "built in", "NTv3 single-nucleotide vocabulary (dnatok_compat.NTv3Tokenizer): byte table kernel"),
+    "evo2": ("evo2", "built in", "Evo2 byte tokenizer, id = byte (dnatok_compat.Evo2ByteTokenizer): byte table kernel"),
+    "kmer6": ("kmer6", "built in", "non-overlapping 6-mers, windows with N spelled per character (vocab 4101): k-mer kernel"),
+    "bpe": ("<path>/tokenizer.json", "local file", "Hugging Face BPE tokenizer (DNABERT-2, GENA-LM, METAGENE-1 style files): "
+            "BPE engine when GPUTokBPEBackend.is_supported accepts it, else the tokenizer itself"),
+}
+
+
+def cmd_list_models(args) -> int:
+    rows = [{"family": fam, "model": model, "source": source, "notes": notes}
+            for fam, (model, source, notes) in MODEL_REGISTRY.items()]
+    if args.json:
+        json.dump(rows, sys.stdout, indent=2)
+        print()
+        return 0
+    widths = {k: max(len(k), max(len(str(r[k])) for r in rows)) for k in rows[0]}
+    print("  " + "  ".join(k.ljust(widths[k]) for k in rows[0]))
+    print("  " + "  ".join("-" * widths[k] for k in rows[0]))
+    for r in rows:
+        print("  " + "  ".join(str(r[k]).ljust(widths[k]) for k in rows[0]))
+    return 0
+
+
 def main(argv: Optional[list] = None) -> int:
     ap = argparse.ArgumentParser(prog="dnatok", description="DNA tokenization on the MI355X backend")
     sub = ap.add_subparsers(dest="cmd", required=True)
@@ -294,6 +346,13 @@ def main(argv: Optional[list] = None) -> int:
     p.add_argument("--hf-threads", type=int, default=8)
     p.add_argument("--seed", type=int, default=11)
     p.set_defaults(fn=cmd_bench)
+    p = sub.add_parser("demo", help="info + encode + validate + a small bench, end to end")
+    common(p)
+    p.add_argument("--sample", default=None, help="sample sequence for the encode step")
+    p.set_defaults(fn=cmd_demo)
+    p = sub.add_parser("list-models", help="what --model accepts")
+    p.add_argument("--json", action="store_true")
+    p.set_defaults(fn=cmd_list_models)
     args = ap.parse_args(argv)
     return int(args.fn(args))
 

@@ -729,3 +729,16 @@ def test_cli_info_encode_validate(model, path, capsys, tmp_path):
                             "--hf-threads", "2", "--json"]) == 0
     b = json.loads(capsys.readouterr().out)
     assert b["total_bp"] == 64 * 512 and b["dnatok_mbp_per_s"] > 0
+
+
+def test_cli_demo_and_list_models(capsys):
+    """`demo` runs info, encode, validate and a small bench in a row and returns their verdict;
+    `list-models` prints what --model accepts."""
+    import json
+    from dnatok_amd import dnatok_cli
+    assert dnatok_cli.main(["demo", "--model", "kmer6", "--sample", "ACGTNNACGTACGT"]) == 0
+    out = capsys.readouterr().out
+    assert "[4/4]" in out and "bit identity holds" in out and "kmer-6" in out
+    assert dnatok_cli.main(["list-models", "--json"]) == 0
+    rows = json.loads(capsys.readouterr().out)
+    assert {"char", "kmer6", "bpe"} <= {r["family"] for r in rows}
