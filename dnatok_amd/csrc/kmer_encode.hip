@@ -80,7 +80,11 @@ struct KmerArgs {
     int32_t pad_id, missing_id;
 };
 
-constexpr int kKmerThreads = 256;
+constexpr int kKmerThreads = 256;         // kmer_team_kernel: four waves share a row
+// kmer_rows_kernel: eight waves, a row each, share one copy of the tables.  Measured on the 6-mer
+// workload (one-launch step): 128 threads 181 us, 256 170.9, 384 183 (12 waves per CU), 512 168.6,
+// 768 177 (12 waves), 1024 as 256; N-free input 141.3 -> 137.5 us with 512.
+constexpr int kRowsThreads = 512;
 constexpr int kUnitsPerLane = 4;
 constexpr int kWaveUnits = 64 * kUnitsPerLane;          // units one wave handles per step
 // Staging area of one wave: kStageCap tokens in scanned order (+ room to read the last group whole).
@@ -206,7 +210,7 @@ __device__ __forceinline__ void climb_max_tree(unsigned long long *tree, unsigne
 }
 
 template <int K, bool LUT4_LDS, bool CHARS, bool HAS_MASK>
-__global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
+__global__ __launch_bounds__(kRowsThreads) void kmer_rows_kernel(
     KmerArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
     int64_t n_rows, int64_t t_cap, int64_t fill_to, int32_t *__restrict__ ids,
     uint8_t *__restrict__ mask, int32_t *__restrict__ lengths, int32_t *__restrict__ status,
@@ -217,9 +221,9 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
     __shared__ int32_t s_single[256];
     __shared__ int32_t s_lut4[LUT4_LDS ? POW4 : 1];
     __shared__ int32_t s_spell[256];     // token a byte is spelled with inside a non-plain window
-    __shared__ __attribute__((aligned(16))) int32_t s_stage[kKmerThreads / 64][kStageWords];
+    __shared__ __attribute__((aligned(16))) int32_t s_stage[kRowsThreads / 64][kStageWords];
 
-    for (int i = threadIdx.x; i < 256; i += kKmerThreads) {
+    for (int i = threadIdx.x; i < 256; i += kRowsThreads) {
         const int d = a.digit[i];
         s_dig[i] = d < 0 ? kDigBad : (d >= 4 ? kDigN : (uint32_t)d);
         s_single[i] = a.single[i];
@@ -227,7 +231,7 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
         s_spell[i] = a.single[(int)"ACGTN"[d < 0 || d > 4 ? 4 : d]];
     }
     if (LUT4_LDS)
-        for (uint32_t i = threadIdx.x; i < POW4; i += kKmerThreads) s_lut4[i] = a.lut4[i];
+        for (uint32_t i = threadIdx.x; i < POW4; i += kRowsThreads) s_lut4[i] = a.lut4[i];
     __syncthreads();          // from here on every wave runs alone (one more barrier at the very end, with `publish`)
 
     const int lane = threadIdx.x & 63;
@@ -237,8 +241,8 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
     int64_t wave_max = 0;
     const unsigned long long slot_gen = mref.slot ? mref.slot[1] : 0ull;
     const int wave_in_wg = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const int64_t wave = (int64_t)blockIdx.x * (kKmerThreads / 64) + wave_in_wg;
-    const int64_t n_waves = (int64_t)gridDim.x * (kKmerThreads / 64);
+    const int64_t wave = (int64_t)blockIdx.x * (kRowsThreads / 64) + wave_in_wg;
+    const int64_t n_waves = (int64_t)gridDim.x * (kRowsThreads / 64);
 
     for (int64_t row = wave; row < n_rows; row += n_waves) {
         const int64_t row_start = offsets[row];
@@ -628,13 +632,13 @@ __global__ __launch_bounds__(kKmerThreads) void kmer_rows_kernel(
     }
     if (publish) {
         // no padding pass follows: the workgroups' maxima go up the tree (climb_max_tree)
-        __shared__ uint32_t s_wave_max[kKmerThreads / 64];
+        __shared__ uint32_t s_wave_max[kRowsThreads / 64];
         if (lane == 0) s_wave_max[wave_in_wg] = (uint32_t)wave_max;
         __syncthreads();
         if (threadIdx.x == 0) {
             uint32_t m = 0;
 #pragma unroll
-            for (int q = 0; q < kKmerThreads / 64; ++q) m = s_wave_max[q] > m ? s_wave_max[q] : m;
+            for (int q = 0; q < kRowsThreads / 64; ++q) m = s_wave_max[q] > m ? s_wave_max[q] : m;
             const unsigned long long mine = (unsigned long long)m + 1;
             const unsigned long long before = atomicAdd(mref.tree + (blockIdx.x >> 2), mine << (16 * (blockIdx.x & 3)));
             climb_max_tree(mref.tree, blockIdx.x, gridDim.x, mine, before, max_len);
@@ -1216,7 +1220,7 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
         DNATOK_HIP_TRY(hipGetLastError());
     }
     // persistent waves: the tables are staged into LDS once per workgroup
-    const int64_t want = (n_rows + kKmerThreads / 64 - 1) / (kKmerThreads / 64);
+    const int64_t want = (n_rows + kRowsThreads / 64 - 1) / (kRowsThreads / 64);
     // few rows (a workgroup for every row at once): the four waves of a workgroup share a row.
     // When the row stride is already cut to the guess (at most kTightStride cells beyond it), the
     // rows are padded to the whole stride while they are written, which covers every possible
@@ -1227,7 +1231,7 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
     bool padded_in_kernel = false;
 #define LAUNCH3(KK, L, C, M)                                                                      \
     do {                                                                                          \
-        static const int resident = resident_workgroups(kmer_rows_kernel<KK, L, C, M>, kKmerThreads, 0, 4); \
+        static const int resident = resident_workgroups(kmer_rows_kernel<KK, L, C, M>, kRowsThreads, 0, 2); \
         static const int team_resident = resident_workgroups(kmer_team_kernel<KK, L, C, M>, kKmerThreads, 0, 4); \
         const int team_rows = g_team_rows.load(std::memory_order_relaxed);                       \
         if (n_rows <= (team_rows < 0 ? team_resident : team_rows)) {                              \
@@ -1239,7 +1243,7 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
         }                                                                                         \
         const int64_t grid = want < resident ? want : resident;                                   \
         padded_in_kernel = tight && grid <= kTreeRows;                                            \
-        kmer_rows_kernel<KK, L, C, M><<<(int)grid, kKmerThreads, 0, s>>>(                         \
+        kmer_rows_kernel<KK, L, C, M><<<(int)grid, kRowsThreads, 0, s>>>(                         \
             a, bytes, offsets, n_rows, t_cap, padded_in_kernel ? t_cap : fill_to, ids, mask,      \
             lengths, status, max_len, mref, padded_in_kernel ? 1 : 0);                            \
     } while (0)
