@@ -799,8 +799,10 @@ def merge_table_placement_extra():
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=400,
+                    help="timed steps (the default runs the headline for 70 ms: the first tens of steps after an idle\n"
+                         "period run 2-3 %% slower than the hundreds after them)")
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--config", default="C2", choices=["C1", "C2", "C3", "C4", "C5"])
     ap.add_argument("--per-call", action="store_true", help="time one exact batch instead of the sustained form")
     ap.add_argument("--no-extras", action="store_true")
@@ -905,7 +907,7 @@ def main() -> None:
                 continue
             ww = make_workload(cfg, sustained=True)
             ww.check()
-            wm, dm = time_steps(ww, 10, 2)
+            wm, dm = time_steps(ww, 50, 10)
             sustained[cfg] = {"workload": ww.name, "ms_per_step": wm, "device_ms_per_step": dm,
                               "mbp_per_s": ww.bases / (wm * 1e-3) / 1e6,
                               "hbm_frac": ww.algorithmic_bytes / (dm * 1e-3) / 1e9 / HBM_PEAK_GBS}
