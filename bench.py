@@ -293,7 +293,10 @@ class KmerPadded(Workload):
 
 
 class BpePadded(Workload):
-    """C3 / C4: BPE encode, then fused remap + pad-to-longest + mask."""
+    """C3 / C4: BPE encode, remap, pad to the longest row, mask.  Rows that the engine takes whole
+    (C3) are padded by the engine itself while it writes them out (dnatok_bpe_encode_padded), the
+    rows as far apart as the stream's width guess says (encoders.WidthGuess, fed by the set-up
+    call); rows that are cut into chunks (C4) are assembled first and padded by a launch of its own."""
 
     def __init__(self, which: str, n_batches: int):
         from dnatok_amd import bpe_vocab, encoders
@@ -332,14 +335,28 @@ class BpePadded(Workload):
         self.kernel = "bpe_lds_kernel" if length <= 4096 else "bpe_long_kernel"
         self.name = (f"{'C3' if which == '4096' else 'C4'} BPE vocab-{which}, {rows}x{length} bp batches, "
                      f"{n_batches} distinct batch(es) per call, pad to longest row")
+        self.one_pass = False
         self.step()
         torch.cuda.synchronize()
         t_max = int(self.max_len.item())
         self.t_max = t_max
+        if length <= self.enc.padded_direct_max():
+            widths = encoders.WidthGuess()
+            widths.update(t_max)
+            self.stride = min(widths.next(), length)
+            self.pad_out = (torch.empty((self.n_rows, self.stride), dtype=torch.int32, device="cuda"),
+                            torch.empty((self.n_rows, self.stride), dtype=torch.uint8, device="cuda"),
+                            self.lengths, torch.empty(1, dtype=torch.int32, device="cuda"))
+            self.one_pass = True
+            self.name += f" (one pass, rows {self.stride} cells apart)"
         self.algorithmic_bytes = host.size + 5 * self.n_rows * t_max + 4 * self.n_rows
 
     def step(self):
         from dnatok_amd import encoders
+        if self.one_pass:
+            self.ids, self.mask, _, self.max_len = self.enc.encode_padded(
+                self.data, self.off, self.length, self.stride, self.pad_id, out=self.pad_out)
+            return
         self.enc.encode(self.data, self.off, self.length, tok_tmp=self.tok, lengths=self.lengths)
         self.ids, self.mask, self.max_len = encoders.pad_rows(self.tok, self.off, self.lengths, self.pad_id,
                                                               self.t_cap, fill_to=0, out=self.pad_out)
@@ -356,6 +373,7 @@ class BpePadded(Workload):
         rows = [self.ids[r, :ln[r]].cpu().numpy() for r in range(self.rows_per_batch)]
         util.check_against_golden(self.golden, rows)
         assert (ln > 0).all() and int(self.max_len.item()) == int(ln.max())
+        assert not self.one_pass or int(ln.max()) <= self.stride, "a row was cut by the stride"
         if self.n_rows > self.rows_per_batch:
             n_live = min(self.rows_per_batch, 256)
             first = self.n_rows - n_live

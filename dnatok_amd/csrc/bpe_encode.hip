@@ -35,6 +35,7 @@
 #include <stdlib.h>
 #include <string.h>
 #include <atomic>
+#include <mutex>
 #include <unordered_map>
 #include <vector>
 
@@ -49,7 +50,16 @@ struct dnatok_bpe_table {
     int32_t *out_remap;          // [n_symbols] or nullptr
     uint32_t *ltab;              // the compact form of the table that fits LDS (kLdsTabWords words), or nullptr
     uint32_t lmul1, lmul2;       // its two multipliers
+    // dnatok_bpe_encode_padded: the tree of atomics that carries a call's longest row
+    // (dnatok::publish_max), one per stream that encodes with this table (calls on one stream are
+    // ordered, calls on different streams may overlap); a stream beyond the kMaxTreeSlots-th gets
+    // its maximum from a launch over the lengths instead
+    unsigned long long *max_trees;
+    mutable std::mutex slot_lock;
+    mutable std::unordered_map<void *, int> slot_of_stream;
 };
+
+constexpr int kMaxTreeSlots = 64;
 
 namespace dnatok {
 
@@ -69,6 +79,17 @@ struct BpeArgs {
     const int32_t *char_lut;
     int32_t *char_ids;
     uint8_t *char_mask;
+    // rows padded in the same pass (dnatok_bpe_encode_padded; pad_ids = null: not asked for): row b's
+    // ids go to pad_ids[b * pad_stride ..], through pad_remap when given, pad_id behind them up to
+    // the stride, 1 / 0 to pad_mask (null: no mask); the longest row's token count goes up max_tree
+    // (null: the caller finds it from the lengths) into *longest
+    int32_t *pad_ids;
+    uint8_t *pad_mask;
+    const int32_t *pad_remap;
+    int64_t pad_stride;
+    int32_t pad_id;
+    unsigned long long *max_tree;
+    int32_t *longest;
 };
 
 typedef int32_t bpe_int4_a4 __attribute__((ext_vector_type(4), aligned(4)));
@@ -241,15 +262,21 @@ struct alignas(4 * sizeof(IT)) PosRec {
 // CHARS: while the piece's bytes pass through the registers on their way into LDS, the
 // single-character id of every byte in [char_lo, char_hi) is written to char_ids (and 1 to char_mask,
 // when given); both pointers are those of the piece's byte 0.
-template <int NT, typename IT, int PER, bool CHARS = false, typename PT>
-__device__ __forceinline__ void bpe_row(
+// pad_stride > 0: out is a row of pad_stride cells; tokens beyond it are dropped (the count handed
+// back is that of all tokens), the cells behind the tokens get pad_id, pad_mask (when given) 1 for
+// a token and 0 for padding, and ids pass through remap2 (when given) after out_remap.
+// Returns the row's token count (0 for a chunk).
+template <int NT, typename IT, int PER, bool CHARS = false, bool PAD = false, typename PT>
+__device__ __forceinline__ int32_t bpe_row(
     const PT pt, const uint16_t *byte_to_sym,
     const int32_t *out_remap, const uint8_t *__restrict__ src, const int n0, PosRec<IT> *P,
     uint16_t *NS, uint16_t *MC, IT *Q, IT *C, uint8_t *D, uint32_t *red, const int tid,
     int32_t *__restrict__ out, int32_t *__restrict__ out_len, uint16_t *__restrict__ raw_out = nullptr,
     const int mid_lo = 0, const int mid_hi = 0, int32_t *__restrict__ mid_out = nullptr,
     const int32_t *__restrict__ char_lut = nullptr, int32_t *__restrict__ char_ids = nullptr,
-    uint8_t *__restrict__ char_mask = nullptr, const int char_lo = 0, const int char_hi = 0)
+    uint8_t *__restrict__ char_mask = nullptr, const int char_lo = 0, const int char_hi = 0,
+    const int pad_stride = 0, const int32_t pad_id = 0, uint8_t *__restrict__ pad_mask = nullptr,
+    const int32_t *__restrict__ remap2 = nullptr)
 {
     static_assert(!CHARS || PER > 0, "the single-character ids are written from the staged bytes");
     constexpr IT NIL = (IT)~(IT)0;
@@ -687,7 +714,7 @@ __device__ __forceinline__ void bpe_row(
         team_sync<NT>();                         // red may still be read by the last round's minimum
         (void)team_exclusive_sum<NT>(live, red, wv, total);
         if (tid == 0) *mid_out = (int32_t)total;
-        return;
+        return 0;
     }
     // Compact the live symbols to the output, in position order.  Position i = pass * NT + tid, so a
     // pass is NT consecutive positions: a ballot per wave gives every lane its place among the
@@ -721,12 +748,24 @@ __device__ __forceinline__ void bpe_row(
                 if (w < wv) mine += c;
                 at += c;
             }
-            if (sy[k] != kNone) out[mine + before[k]] = out_remap ? out_remap[sy[k]] : (int32_t)sy[k];
+            const uint32_t cell = mine + before[k];
+            if (sy[k] != kNone && (!PAD || cell < (uint32_t)pad_stride)) {
+                int32_t id = out_remap ? out_remap[sy[k]] : (int32_t)sy[k];
+                if (PAD && remap2) id = remap2[id];
+                out[cell] = id;
+            }
         }
         done = at;
         team_sync<NT>();                                             // wave_cnt is rewritten by the next block
     }
     if (tid == 0) *out_len = stuck ? -2 : (int32_t)done;
+    if (PAD) {
+        const int kept = (int)done < pad_stride ? (int)done : pad_stride;
+        for (int i = kept + tid; i < pad_stride; i += NT) out[i] = pad_id;
+        if (pad_mask)
+            for (int i = tid; i < pad_stride; i += NT) pad_mask[i] = i < kept ? 1 : 0;
+    }
+    return (int32_t)done;
 }
 
 // ---- long rows in chunks -------------------------------------------------------------------
@@ -999,7 +1038,12 @@ __global__ __launch_bounds__(256) void bpe_expand_kernel(const int64_t *__restri
 // workgroup shares an item.  PLANNED: the items are those of the work list (rows and chunks of
 // long rows), handed out through an atomic counter.  Otherwise (no row of the batch is longer
 // than CAP) an item is a row, teams take rows round robin, and no work list is built at all.
-template <int NT, int TEAMS, int CAP, bool PLANNED, bool LTAB = false, bool CHARS = false>
+// CHUNKS = false: the list holds whole rows only (no row of the batch is cut), and the kernel is
+// built without the chunk path, whose copy of the engine costs it registers (a workgroup per CU
+// for rows of at most 1 KB).
+// PADDED: a row's ids go straight to its row of a.pad_ids, padded (dnatok_bpe_encode_padded).
+template <int NT, int TEAMS, int CAP, bool PLANNED, bool LTAB = false, bool CHARS = false, bool CHUNKS = PLANNED,
+          bool PADDED = false>
 __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     BpeArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
     BpePlan p, int32_t n_rows, int32_t *__restrict__ tok_tmp, int32_t *__restrict__ lengths)
@@ -1031,13 +1075,17 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     __syncthreads();
 
     const int32_t n_items = PLANNED ? p.counts[0] : n_rows;
-    const int32_t n_mc = PLANNED ? p.counts[1] : 0;
+    static_assert(PLANNED || !CHUNKS, "chunks come from the work list");
+    static_assert(!PADDED || (!CHUNKS && !LTAB && TEAMS == 1), "padded rows: whole rows, one team per workgroup");
+    const int32_t n_mc = CHUNKS ? p.counts[1] : 0;
     const int32_t n_single0 = PLANNED ? p.counts[4] : 0, n_single1 = PLANNED ? p.counts[5] : 0;
     // A team's first item is its own number; only the items beyond one per team are handed out
     // through the counter.  (Every team asking the counter at the start of the kernel is a
     // thousand atomics on one address, about 12 ns each, before the last team has its row.)
     const int32_t n_teams = (int32_t)gridDim.x * TEAMS;
     int32_t item = (int32_t)blockIdx.x * TEAMS + team;
+    constexpr bool padded = PADDED;
+    int32_t team_longest = 0;                        // (padded) most tokens in a row of this team
     for (bool first = true;; first = false) {
         if (!first) {
             if (PLANNED) {
@@ -1053,7 +1101,7 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
         if (item >= n_items) break;
         int32_t row = item, k = 0, nc = 1;
         if (PLANNED) {
-            if (item < n_mc) {
+            if (CHUNKS && item < n_mc) {
                 const int4 rc = p.rec[item];
                 row = rc.x; k = rc.y; nc = rc.z;
             } else {
@@ -1066,30 +1114,45 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
                 row = list[j];
             }
         }
+        // (a team is whole waves: its item is the same in every lane, and so is all that follows from it)
+        row = __builtin_amdgcn_readfirstlane(row);
+        k = __builtin_amdgcn_readfirstlane(k);
+        nc = __builtin_amdgcn_readfirstlane(nc);
         const int64_t start = offsets[row];
         const int64_t len = offsets[row + 1] - start;
         // one straight path per iteration (no `continue`): every lane of the team must come
         // back to the fetch above together, or lanes that skipped ahead would re-read the
         // old item while lane 0 has not fetched the next one yet
-        if (nc == 1 && (len > CAP || len <= 0)) {
+        if ((!CHUNKS || nc == 1) && (len > CAP || len <= 0)) {
             // too long: left to the whole-row kernel (row_fail is set); empty: no tokens
             if (tid == 0) lengths[row] = len > CAP ? -1 : 0;
+            if (padded) {
+                for (int64_t i = tid; i < a.pad_stride; i += NT) {
+                    a.pad_ids[(int64_t)row * a.pad_stride + i] = a.pad_id;
+                    if (a.pad_mask) a.pad_mask[(int64_t)row * a.pad_stride + i] = 0;
+                }
+            }
             if (CHARS) {
                 for (int64_t i = tid; i < len; i += NT) {
                     a.char_ids[start + i] = a.char_lut[bytes[start + i]];
                     if (a.char_mask) a.char_mask[start + i] = 1;
                 }
             }
-        } else if (nc == 1) {
+        } else if (!CHUNKS || nc == 1) {
             if (LTAB)
                 bpe_row<NT, uint16_t, (CAP + NT - 1) / NT>(lpt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC,
                                       Q, C, D, red, tid, tok_tmp + start, lengths + row);
-            else
-                bpe_row<NT, uint16_t, (CAP + NT - 1) / NT, CHARS>(
-                    pt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC, Q, C, D, red, tid, tok_tmp + start,
+            else {
+                const int32_t n_tok = bpe_row<NT, uint16_t, (CAP + NT - 1) / NT, CHARS, PADDED>(
+                    pt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC, Q, C, D, red, tid,
+                    padded ? a.pad_ids + (int64_t)row * a.pad_stride : tok_tmp + start,
                     lengths + row, nullptr, 0, 0, nullptr, a.char_lut, CHARS ? a.char_ids + start : nullptr,
-                    CHARS && a.char_mask ? a.char_mask + start : nullptr, 0, (int)len);
-        } else {
+                    CHARS && a.char_mask ? a.char_mask + start : nullptr, 0, (int)len,
+                    padded ? (int)a.pad_stride : 0, a.pad_id,
+                    padded && a.pad_mask ? a.pad_mask + (int64_t)row * a.pad_stride : nullptr, a.pad_remap);
+                team_longest = n_tok > team_longest ? n_tok : team_longest;
+            }
+        } else if (CHUNKS) {
             const int64_t e0 = (int64_t)k * p.core - p.overlap < 0 ? 0 : (int64_t)k * p.core - p.overlap;
             int64_t e1 = (int64_t)(k + 1) * p.core + p.overlap;
             if (e1 > len) e1 = len;
@@ -1109,6 +1172,9 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
         }
         team_sync<NT>();
     }
+    // (padded, one team per workgroup) every workgroup reports once, whether it had a row or not
+    if (padded && a.max_tree && threadIdx.x == 0)
+        publish_max(a.max_tree, (unsigned)team_longest, a.longest);
 }
 
 // One workgroup per chunk of a multi-chunk row: the seam with the chunk to its right.  The two
@@ -1424,8 +1490,9 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
     const size_t o_b2s = up(o_tab + (size_t)slots * sizeof(uint4));
     const size_t o_remap = up(o_b2s + 512);
     const size_t o_ltab = up(o_remap + (out_remap_h ? (size_t)n_symbols * 4 : 0));
-    const size_t total = up(o_ltab + ltab.size() * 4) + 256;
-    std::vector<uint8_t> host(total, 0);
+    const size_t o_trees = up(o_ltab + ltab.size() * 4);
+    const size_t total = up(o_trees + (size_t)kMaxTreeSlots * kTreeWords * 8) + 256;
+    std::vector<uint8_t> host(total, 0);             // (the trees start as zeros)
     memcpy(&host[o_tab], tab.data(), (size_t)slots * sizeof(uint4));
     memcpy(&host[o_b2s], b2s.data(), 512);
     if (out_remap_h) memcpy(&host[o_remap], out_remap_h, (size_t)n_symbols * 4);
@@ -1447,6 +1514,7 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
     t->out_remap = out_remap_h ? (int32_t *)(b + o_remap) : nullptr;
     t->ltab = ltab.empty() ? nullptr : (uint32_t *)(b + o_ltab);
     t->lmul1 = lmul1; t->lmul2 = lmul2;
+    t->max_trees = (unsigned long long *)(b + o_trees);
     *out = t;
     return DNATOK_OK;
 }
@@ -1493,7 +1561,8 @@ constexpr size_t lds_bytes()
     return 512 + 64 + (size_t)TEAMS * (4 * (NT / 64) + 4) * 4 + (size_t)TEAMS * CAP * 15 + (size_t)TEAMS * NT + 64;
 }
 
-// Teams of the LDS kernel that are resident at once (the same for both of its forms).
+// Teams of the LDS kernel that are resident at once: of the form that works through a list with
+// chunks, which holds the most registers (a batch of more rows than that gets a list).
 template <int NT, int TEAMS, int CAP>
 int64_t lds_resident_teams()
 {
@@ -1502,12 +1571,12 @@ int64_t lds_resident_teams()
     return (int64_t)resident * TEAMS;
 }
 
-template <int NT, int TEAMS, int CAP, bool PLANNED, bool CHARS = false>
+template <int NT, int TEAMS, int CAP, bool PLANNED, bool CHARS = false, bool CHUNKS = PLANNED, bool PADDED = false>
 int launch_lds_as(const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets, const BpePlan &p,
                   int64_t n_rows, int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
 {
     const size_t lds = lds_bytes<NT, TEAMS, CAP>();
-    auto kern = bpe_lds_kernel<NT, TEAMS, CAP, PLANNED, false, CHARS>;
+    auto kern = bpe_lds_kernel<NT, TEAMS, CAP, PLANNED, false, CHARS, CHUNKS, PADDED>;
     static bool attr_set = false;
     if (!attr_set) {
         DNATOK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -1516,8 +1585,9 @@ int launch_lds_as(const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets
     }
     const int64_t items = PLANNED ? p.max_items : n_rows;
     int64_t grid = (items + TEAMS - 1) / TEAMS;
-    const int64_t resident = lds_resident_teams<NT, TEAMS, CAP>() / TEAMS;
+    static const int64_t resident = resident_workgroups(kern, NT * TEAMS, lds, 2);    // (of this form)
     if (grid > resident) grid = resident;
+    if (a.max_tree && grid > kTreeRows) grid = kTreeRows;
     if (grid < 1) grid = 1;
     kern<<<(int)grid, NT * TEAMS, lds, s>>>(a, bytes, offsets, p, (int32_t)n_rows, tok_tmp, lengths);
     DNATOK_HIP_TRY(hipGetLastError());
@@ -1570,7 +1640,7 @@ template <int NT, int TEAMS, int CAP>
 int run_lds(bool long_rows, int chunking, const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets,
             const BpePlan &p, int64_t n_rows, int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
 {
-    if (CAP == 1024 && !long_rows && a.ltab && !a.char_ids) {
+    if (CAP == 1024 && !long_rows && a.ltab && !a.char_ids && !a.pad_ids) {
         const int mode = g_table_placement.load(std::memory_order_relaxed);
         if (mode == 2 || (mode == 1 && n_rows <= ltab_resident_teams<NT, TEAMS, 1024>()))
             return launch_lds_ltab<NT, TEAMS, 1024>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
@@ -1584,9 +1654,15 @@ int run_lds(bool long_rows, int chunking, const BpeArgs &a, const uint8_t *bytes
             bpe_expand_kernel<<<(int)((n_rows + 255) / 256), 256, 0, s>>>(offsets, n_rows, p);
             DNATOK_HIP_TRY(hipGetLastError());
         }
-        if (a.char_ids) return launch_lds_as<NT, TEAMS, CAP, true, true>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
-        return launch_lds_as<NT, TEAMS, CAP, true>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+        if (chunking & 1) {
+            if (a.char_ids) return launch_lds_as<NT, TEAMS, CAP, true, true>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+            return launch_lds_as<NT, TEAMS, CAP, true>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+        }
+        if (a.pad_ids) return launch_lds_as<NT, TEAMS, CAP, true, false, false, true>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+        if (a.char_ids) return launch_lds_as<NT, TEAMS, CAP, true, true, false>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+        return launch_lds_as<NT, TEAMS, CAP, true, false, false>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
     }
+    if (a.pad_ids) return launch_lds_as<NT, TEAMS, CAP, false, false, false, true>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
     if (a.char_ids) return launch_lds_as<NT, TEAMS, CAP, false, true>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
     return launch_lds_as<NT, TEAMS, CAP, false>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
 }
@@ -1597,10 +1673,15 @@ int run_lds(bool long_rows, int chunking, const BpeArgs &a, const uint8_t *bytes
 static int bpe_encode_launch(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets, int64_t n_rows,
                              int64_t max_len, const BpePlan &p, int32_t *tok_tmp, int32_t *lengths, hipStream_t s,
                              const int32_t *char_lut = nullptr, int32_t *char_ids = nullptr,
-                             uint8_t *char_mask = nullptr)
+                             uint8_t *char_mask = nullptr, const BpeArgs *padded = nullptr)
 {
     BpeArgs a{t->tab, t->byte_to_sym, t->out_remap, t->shift, t->mul1, t->mul2, t->n_merges, t->ltab, t->lmul1, t->lmul2,
               char_lut, char_ids, char_mask};
+    if (padded) {
+        a.pad_ids = padded->pad_ids; a.pad_mask = padded->pad_mask; a.pad_remap = padded->pad_remap;
+        a.pad_stride = padded->pad_stride; a.pad_id = padded->pad_id;
+        a.max_tree = padded->max_tree; a.longest = padded->longest;
+    }
 
     const bool long_rows = max_len > p.ext;
     int chunking = (long_rows && t->monotone) ? 1 : 0;
@@ -1678,6 +1759,93 @@ extern "C" int dnatok_bpe_encode_with_chars(const dnatok_bpe_t *t, const uint8_t
     const BpePlan p = make_plan((uint8_t *)scratch, n_rows, max_len, total);
     return bpe_encode_launch(t, bytes, offsets, n_rows, max_len, p, tok_tmp, lengths, (hipStream_t)stream, char_lut,
                              char_ids, char_mask);
+}
+
+// Longest row (negative lengths count as 0) by one workgroup: where no tree of atomics carries it.
+__global__ __launch_bounds__(1024) void bpe_longest_kernel(const int32_t *__restrict__ lengths, int64_t n_rows,
+                                                           int32_t *__restrict__ longest)
+{
+    __shared__ uint32_t red[16];
+    uint32_t m = 0;
+    for (int64_t i = threadIdx.x; i < n_rows; i += 1024) {
+        const int32_t v = lengths[i];
+        m = v > 0 && (uint32_t)v > m ? (uint32_t)v : m;
+    }
+    m = wave_max_u32(m);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t all = 0;
+        for (int w = 0; w < 16; ++w) all = all > red[w] ? all : red[w];
+        *longest = (int32_t)all;
+    }
+}
+
+extern "C" int64_t dnatok_bpe_padded_direct_max(void)
+{
+    int core, overlap;
+    chunk_geometry(&core, &overlap, 0, 0);
+    return (int64_t)core + 2 * overlap;
+}
+
+extern "C" int dnatok_bpe_encode_padded(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets,
+                                        int64_t n_rows, int64_t max_len, int64_t total, void *scratch,
+                                        size_t scratch_bytes, int32_t *tok_tmp, const int32_t *remap, int32_t pad_id,
+                                        int64_t stride, int32_t *ids, uint8_t *mask, int32_t *lengths,
+                                        int32_t *longest, void *stream)
+{
+    static const char *who = "dnatok_bpe_encode_padded";
+    DNATOK_REQUIRE(t && offsets && (lengths || n_rows == 0), DNATOK_E_INVALID, "%s: null argument", who);
+    DNATOK_REQUIRE(n_rows >= 0 && max_len >= 0 && total >= 0, DNATOK_E_INVALID, "%s: negative size", who);
+    DNATOK_REQUIRE(max_len < (int64_t)1 << 31 && total / 256 + n_rows < (int64_t)1 << 30, DNATOK_E_TOO_LARGE,
+                   "%s: batch too large", who);
+    DNATOK_REQUIRE(stride >= 1 && stride < (int64_t)1 << 31, DNATOK_E_INVALID, "%s: stride must be in [1, 2^31)", who);
+    DNATOK_REQUIRE(bytes || total == 0, DNATOK_E_INVALID, "%s: null bytes", who);
+    DNATOK_REQUIRE(ids || n_rows == 0, DNATOK_E_INVALID, "%s: null ids", who);
+    hipStream_t s = (hipStream_t)stream;
+    if (n_rows == 0) {
+        if (longest) {
+            bpe_longest_kernel<<<1, 1024, 0, s>>>(lengths, 0, longest);
+            DNATOK_HIP_TRY(hipGetLastError());
+        }
+        return DNATOK_OK;
+    }
+    const BpePlan need = make_plan(nullptr, n_rows, max_len, total);
+    DNATOK_REQUIRE(scratch && scratch_bytes >= need.total_bytes, DNATOK_E_SCRATCH,
+                   "%s: scratch holds %zu bytes, %zu needed", who, scratch_bytes, need.total_bytes);
+    DNATOK_REQUIRE(((uintptr_t)scratch & 255) == 0, DNATOK_E_INVALID, "%s: scratch must be 256-byte aligned", who);
+    const BpePlan p = make_plan((uint8_t *)scratch, n_rows, max_len, total);
+    if (max_len > p.ext) {
+        // rows cut into chunks (or left to the whole-row kernel) are assembled in tok_tmp first
+        DNATOK_REQUIRE(tok_tmp, DNATOK_E_INVALID,
+                       "%s: a batch with a row of more than %d bytes needs tok_tmp (int32[total])", who, p.ext);
+        const int rc = bpe_encode_launch(t, bytes, offsets, n_rows, max_len, p, tok_tmp, lengths, s);
+        if (rc) return rc;
+        if (longest) {
+            bpe_longest_kernel<<<1, 1024, 0, s>>>(lengths, n_rows, longest);
+            DNATOK_HIP_TRY(hipGetLastError());
+        }
+        return dnatok_pad_rows(tok_tmp, offsets, lengths, n_rows, remap, pad_id, stride, stride, ids, mask, nullptr,
+                               stream);
+    }
+    BpeArgs pad{};
+    pad.pad_ids = ids; pad.pad_mask = mask; pad.pad_remap = remap; pad.pad_stride = stride; pad.pad_id = pad_id;
+    pad.longest = longest;
+    if (longest) {
+        std::lock_guard<std::mutex> hold(t->slot_lock);
+        auto it = t->slot_of_stream.find(stream);
+        if (it == t->slot_of_stream.end() && (int)t->slot_of_stream.size() < kMaxTreeSlots)
+            it = t->slot_of_stream.emplace(stream, (int)t->slot_of_stream.size()).first;
+        if (it != t->slot_of_stream.end()) pad.max_tree = t->max_trees + (size_t)it->second * kTreeWords;
+    }
+    const int rc = bpe_encode_launch(t, bytes, offsets, n_rows, max_len, p, nullptr, lengths, s, nullptr, nullptr,
+                                     nullptr, &pad);
+    if (rc) return rc;
+    if (longest && !pad.max_tree) {
+        bpe_longest_kernel<<<1, 1024, 0, s>>>(lengths, n_rows, longest);
+        DNATOK_HIP_TRY(hipGetLastError());
+    }
+    return DNATOK_OK;
 }
 
 // ---- the entry point that allocates nothing -------------------------------------------------

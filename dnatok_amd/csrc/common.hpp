@@ -104,4 +104,63 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v)
     return ~wave_min_u32(~v);
 }
 
+// ---- maximum over the workgroups of a launch, carried by atomics alone ----
+
+constexpr int kTreeRows = 2048;          // workgroups of one launch that can take part
+constexpr int kTreeWords = 1024;         // 512 + 128 + 32 + 8 + 2 + 1 words used, 8 KB per tree
+
+// The longest row of a call without a padding pass (every row padded as far as any row can
+// reach), found without a fence: nothing but atomics carries it.  Every workgroup adds its
+// maximum + 1 into its 16-bit field of a 64-bit word shared by four workgroups; the atomic returns
+// the fields of those that came before, so the workgroup that completes a word knows the maximum
+// of its four, clears the word for the next call and carries the maximum one level up in the same
+// way (a 4-ary tree, `tree` holds its words level by level).  Who completes the root writes
+// max_len.  `mine` is the caller's value + 1 and `before` what its own atomicAdd at the lowest
+// level returned (the caller issues that one itself, as early as it knows its value); one lane
+// calls this.  (One counter and one atomicMax for 256 workgroups cost 3 us, two of them spent
+// queueing at that one address.)
+__device__ __forceinline__ void climb_max_tree(unsigned long long *tree, unsigned idx, unsigned n_here,
+                                               unsigned long long mine, unsigned long long before,
+                                               int32_t *__restrict__ max_len)
+{
+    unsigned long long *level = tree;
+    // words this workgroup completed: cleared when it is done climbing, so that a level costs one
+    // trip to memory (the add, whose answer is waited for) and not two
+    unsigned long long *completed[8];
+    int n_completed = 0;
+    for (;;) {
+        const unsigned long long all = before + (mine << (16 * (idx & 3)));
+        const unsigned members = n_here - (idx & ~3u) < 4u ? n_here - (idx & ~3u) : 4u;
+        unsigned arrived = 0;
+        unsigned long long best = 0;
+#pragma unroll
+        for (int f = 0; f < 4; ++f) {
+            const unsigned long long v = (all >> (16 * f)) & 0xFFFFull;
+            arrived += v != 0;
+            best = v > best ? v : best;
+        }
+        if (arrived < members) break;
+        completed[n_completed++] = level + (idx >> 2);
+        if (n_here <= 4) {
+            *max_len = (int32_t)best - 1;
+            break;
+        }
+        level += (n_here + 3) >> 2;
+        n_here = (n_here + 3) >> 2;
+        idx >>= 2;
+        mine = best;
+        before = atomicAdd(level + (idx >> 2), mine << (16 * (idx & 3)));
+    }
+    for (int i = 0; i < n_completed; ++i) atomicExch(completed[i], 0ull);
+}
+
+// The whole of it for a workgroup that knows its value (< 0xFFFF) only at its end: one lane calls
+// this, every workgroup of the launch exactly once, gridDim.x <= kTreeRows.
+__device__ __forceinline__ void publish_max(unsigned long long *tree, unsigned value, int32_t *__restrict__ max_len)
+{
+    const unsigned long long mine = (unsigned long long)value + 1ull;
+    const unsigned long long before = atomicAdd(tree + (blockIdx.x >> 2), mine << (16 * (blockIdx.x & 3)));
+    climb_max_tree(tree, blockIdx.x, gridDim.x, mine, before, max_len);
+}
+
 }  // namespace dnatok

@@ -66,9 +66,9 @@ constexpr int kMaxSlots = 64;
 static std::atomic<int> g_team_rows{-1};
 constexpr int kMaxSlotStride = 32;       // 64-bit words between two slots (one 256-byte line each)
 // A call whose kernel reports the maximum itself (kmer_team_kernel, publish) gathers it up a tree
-// of 64-bit words with four 16-bit fields each: kTreeRows leaves, four children per word.
-constexpr int kTreeRows = 2048;          // workgroups of one call (a row each, or the persistent grid)
-constexpr int kTreeWords = 1024;         // 512 + 128 + 32 + 8 + 2 + 1 words used, 8 KB per slot
+// of atomics (climb_max_tree): kTreeWords words per slot.
+using dnatok::kTreeRows;
+using dnatok::kTreeWords;
 
 namespace dnatok {
 
@@ -162,51 +162,6 @@ __device__ __forceinline__ void wave_sync()
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
-// The longest row of a call without a padding pass (every row padded as far as any row can
-// reach), found without a fence: nothing but atomics carries it.  Every workgroup adds its
-// maximum + 1 into its 16-bit field of a 64-bit word shared by four workgroups; the atomic returns
-// the fields of those that came before, so the workgroup that completes a word knows the maximum
-// of its four, clears the word for the next call and carries the maximum one level up in the same
-// way (a 4-ary tree, `tree` holds its words level by level).  Who completes the root writes
-// max_len.  `mine` is the caller's value + 1 and `before` what its own atomicAdd at the lowest
-// level returned (the caller issues that one itself, as early as it knows its value); one lane
-// calls this.  (One counter and one atomicMax for 256 workgroups cost 3 us, two of them spent
-// queueing at that one address.)
-__device__ __forceinline__ void climb_max_tree(unsigned long long *tree, unsigned idx, unsigned n_here,
-                                               unsigned long long mine, unsigned long long before,
-                                               int32_t *__restrict__ max_len)
-{
-    unsigned long long *level = tree;
-    // words this workgroup completed: cleared when it is done climbing, so that a level costs one
-    // trip to memory (the add, whose answer is waited for) and not two
-    unsigned long long *completed[8];
-    int n_completed = 0;
-    for (;;) {
-        const unsigned long long all = before + (mine << (16 * (idx & 3)));
-        const unsigned members = n_here - (idx & ~3u) < 4u ? n_here - (idx & ~3u) : 4u;
-        unsigned arrived = 0;
-        unsigned long long best = 0;
-#pragma unroll
-        for (int f = 0; f < 4; ++f) {
-            const unsigned long long v = (all >> (16 * f)) & 0xFFFFull;
-            arrived += v != 0;
-            best = v > best ? v : best;
-        }
-        if (arrived < members) break;
-        completed[n_completed++] = level + (idx >> 2);
-        if (n_here <= 4) {
-            *max_len = (int32_t)best - 1;
-            break;
-        }
-        level += (n_here + 3) >> 2;
-        n_here = (n_here + 3) >> 2;
-        idx >>= 2;
-        mine = best;
-        before = atomicAdd(level + (idx >> 2), mine << (16 * (idx & 3)));
-    }
-    for (int i = 0; i < n_completed; ++i) atomicExch(completed[i], 0ull);
 }
 
 template <int K, bool LUT4_LDS, bool CHARS, bool HAS_MASK>

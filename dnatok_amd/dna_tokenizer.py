@@ -387,6 +387,22 @@ class DNATok:
         left = self.padding_side == "left"
         self._staged_host_ids = None
         if self.bpe_backend is not None:
+            if not left and dtype == torch.int32:
+                # the engine pads the rows itself while it writes them out
+                staged = []
+
+                def stage(ids):
+                    if host_ids:
+                        nbytes = ids.numel() * ids.element_size()
+                        host = self._pinned(nbytes)[:nbytes].view(ids.dtype).view(ids.shape)
+                        host.copy_(ids, non_blocking=True)
+                        staged[:] = [host]
+
+                ids, mask = self.bpe_backend.padded_device(list(seqs), device=device, min_width=min_width,
+                                                           pad_multiple=pad_multiple, stage_ids=stage)
+                if staged and staged[0].shape[1] == ids.stride(0):      # (not those of a first, too narrow, try)
+                    self._staged_host_ids = staged[0][:, :ids.shape[1]]
+                return ids, mask
             tok, offsets, lengths, t_cap = self.bpe_backend.tokens_device(list(seqs), device=device, meta_tail=2)
             return self._pad_bpe_runs(tok, offsets, lengths, t_cap, dtype=dtype, min_width=min_width,
                                       pad_multiple=pad_multiple, host_ids=host_ids, stats_behind_lengths=True)

@@ -463,6 +463,46 @@ class BpeEncoder:
                    "dnatok_bpe_encode")
         return tok_tmp, lengths
 
+    def encode_padded(self, data: torch.Tensor, offsets: torch.Tensor, max_len: int, stride: int, pad_id: int, *,
+                      remap: Optional[torch.Tensor] = None, want_mask: bool = True, want_longest: bool = True,
+                      out=None, tok_tmp: Optional[torch.Tensor] = None):
+        """Engine and padding in one pass: ``ids[B, stride]`` int32 (through ``remap``, ``pad_id``
+        behind a row's tokens), ``mask[B, stride]`` uint8, ``lengths[B]`` (full token counts) and
+        ``longest[1]`` (their maximum; None with ``want_longest=False`` or in ``out``: the caller takes it
+        from the lengths), all on the device.  A row with more tokens than ``stride``
+        keeps its first ``stride``: compare ``longest`` with it.  ``out`` = (ids, mask, lengths,
+        longest) reuses caller buffers.  Rows above ``padded_direct_max()`` bytes go through a token
+        buffer (``tok_tmp``, allocated here when not given)."""
+        _require_cuda(data, torch.uint8, "data")
+        _require_cuda(offsets, torch.int64, "offsets")
+        n_rows = offsets.numel() - 1
+        total = data.numel()
+        dev = data.device
+        stride = int(stride)
+        if out is None:
+            ids = torch.empty((n_rows, stride), dtype=torch.int32, device=dev)
+            mask = torch.empty((n_rows, stride), dtype=torch.uint8, device=dev) if want_mask else None
+            lengths = torch.empty(n_rows, dtype=torch.int32, device=dev)
+            longest = torch.empty(1, dtype=torch.int32, device=dev) if want_longest else None
+        else:
+            ids, mask, lengths, longest = out
+            if ids.shape != (n_rows, stride) or not ids.is_contiguous():
+                raise ValueError("ids must be a contiguous [n_rows, stride] tensor")
+        if int(max_len) > self.padded_direct_max() and tok_tmp is None:
+            tok_tmp = torch.empty(max(total, 1), dtype=torch.int32, device=dev)
+        scratch = self._get_scratch(n_rows, int(max_len), total, dev)
+        _lib.check(_lib.lib().dnatok_bpe_encode_padded(
+            self._h, _ptr(data), _ptr(offsets), n_rows, int(max_len), total, _ptr(scratch), scratch.numel(),
+            _ptr(tok_tmp) if tok_tmp is not None else None, _ptr(remap) if remap is not None else None,
+            int(pad_id), stride, _ptr(ids), _ptr(mask) if mask is not None else None, _ptr(lengths), _ptr(longest),
+            _stream()), "dnatok_bpe_encode_padded")
+        return ids, mask, lengths, longest
+
+    @staticmethod
+    def padded_direct_max() -> int:
+        """Longest row (bytes) that ``encode_padded`` writes without a token buffer."""
+        return int(_lib.lib().dnatok_bpe_padded_direct_max())
+
     def encode_with_chars(self, data: torch.Tensor, offsets: torch.Tensor, max_len: int, char_lut: torch.Tensor, *,
                           tok_tmp: Optional[torch.Tensor] = None, lengths: Optional[torch.Tensor] = None,
                           char_ids: Optional[torch.Tensor] = None, char_mask: Optional[torch.Tensor] = None,

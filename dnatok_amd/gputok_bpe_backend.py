@@ -347,6 +347,7 @@ class GPUTokBPEBackend:
         self._remap_cpu = torch.from_numpy(remap.astype("int64"))          # int64 [V_kernel]
         self._remap_i32 = torch.from_numpy(remap)                          # int32, what the packer reads
         self._remap_cuda: Optional[torch.Tensor] = None
+        self._widths = encoders.WidthGuess()           # how wide the recent batches came out (padded_device)
         size = getattr(hf_tokenizer, "vocab_size", None)
         if callable(size):
             size = None
@@ -389,13 +390,10 @@ class GPUTokBPEBackend:
 
     # ------------------------------------------------------------------- reference API
 
-    def tokens_device(self, seqs: List[str], *, device: object = "cuda", meta_tail: int = 0):
-        """Strings -> the engine's token runs on the device: ``(tok_tmp int32, offsets int64 [B+1],
-        lengths int32 [B], t_cap)`` with row b's kernel-space tokens at
-        ``tok_tmp[offsets[b] : offsets[b] + lengths[b]]`` and t_cap a host-known bound of the row
-        lengths.  What ``encode_batch`` pads; DNATok pads the same runs its own way.  With
-        ``meta_tail`` > 0 the lengths are the head of an int32 allocation with that many more
-        entries behind them (for the padding's statistics: one copy then brings both to the host)."""
+    def bytes_device(self, seqs: List[str], *, device: object = "cuda"):
+        """Strings -> what the engine reads: ``(data uint8, offsets int64 [B+1], t_cap)`` on the
+        device, normalizer applied (on the device where its steps allow), t_cap a host-known bound
+        of the row lengths in bytes."""
         if not seqs:
             raise ValueError("No sequences provided.")
         dev = torch.device(device) if not isinstance(device, torch.device) else device
@@ -420,26 +418,66 @@ class GPUTokBPEBackend:
             norm = [self._normalize(s) for s in seqs]
             data, offsets, lens = encoders.bytes_from_strings(norm, dev, encoding="utf-8")
             t_cap = int(lens.max())
-        t_cap = max(t_cap, 1)
+        return data, offsets, max(t_cap, 1)
+
+    def tokens_device(self, seqs: List[str], *, device: object = "cuda", meta_tail: int = 0):
+        """Strings -> the engine's token runs on the device: ``(tok_tmp int32, offsets int64 [B+1],
+        lengths int32 [B], t_cap)`` with row b's kernel-space tokens at
+        ``tok_tmp[offsets[b] : offsets[b] + lengths[b]]`` and t_cap a host-known bound of the row
+        lengths.  DNATok pads these runs its own way where the engine's own padding does not fit (padding
+        on the left, narrow id types).  With
+        ``meta_tail`` > 0 the lengths are the head of an int32 allocation with that many more
+        entries behind them (for the padding's statistics: one copy then brings both to the host)."""
+        data, offsets, t_cap = self.bytes_device(seqs, device=device)
         n = offsets.numel() - 1
         lengths = torch.empty(n + int(meta_tail), dtype=torch.int32, device=data.device)[:n] if meta_tail else None
         tok, lengths = self._dnatok.tokenize_device(data, offsets, t_cap, lengths=lengths)
         return tok, offsets, lengths, t_cap
 
+    def padded_device(self, seqs: List[str], *, device: object = "cuda", min_width: int = 0,
+                      pad_multiple: int = 1, stage_ids=None) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Strings -> ``(ids int32 [B, T], mask uint8 [B, T])`` on the device, tokenizer ids, padded
+        on the right with ``pad_id`` to the longest row (at least ``min_width``, a multiple of
+        ``pad_multiple``): one engine launch writes the padded rows (``dnatok_bpe_encode_padded``),
+        one copy brings the lengths to the host.  The rows are laid out only as
+        far apart as the recent batches of this backend were wide (``encoders.WidthGuess``); a batch
+        that needs more room is encoded again with room for the worst case (a token per byte).
+        ``stage_ids``: a callable ``(ids) -> None`` run before the wait when the layout was not the
+        worst-case one (DNATok copies the ids to pinned memory there)."""
+        data, offsets, t_cap = self.bytes_device(seqs, device=device)
+        dev = data.device
+        n = offsets.numel() - 1
+
+        def rounded(w: int) -> int:
+            return w + (-w) % pad_multiple if pad_multiple > 1 else w
+
+        worst = rounded(max(int(t_cap), int(min_width), 1))
+        guess = self._widths.next()
+        cap = min(rounded(max(guess + (-guess) % 32, int(min_width))), worst) if guess else worst
+        lengths = torch.empty(n, dtype=torch.int32, device=dev)
+        while True:
+            # (no longest row from the device: the lengths come down anyway, and the launch ends earlier without it)
+            out = (torch.empty((n, cap), dtype=torch.int32, device=dev),
+                   torch.empty((n, cap), dtype=torch.uint8, device=dev), lengths, None)
+            ids, mask, _, _ = self._dnatok.tokenize_padded_device(data, offsets, t_cap, cap, int(self.pad_id),
+                                                                  remap=self._remap_on(dev), out=out)
+            if stage_ids is not None and cap < worst:
+                stage_ids(ids)
+            lengths_h = lengths.cpu().numpy()                            # (the one wait)
+            longest, shortest = int(lengths_h.max()), int(lengths_h.min())
+            if shortest < 0:
+                raise RuntimeError("BPE engine reported a failed row (negative length)")
+            if longest <= cap:
+                break
+            cap = worst                                  # a row was cut: once more, with room for all
+        self._widths.update(longest)
+        width = min(rounded(max(longest, int(min_width))), cap)
+        return ids[:, :width], mask[:, :width]
+
     def encode_batch(self, seqs: List[str], *, device: object = "cuda"
                      ) -> Tuple[torch.Tensor, torch.Tensor]:
-        tok, offsets, lengths, t_cap = self.tokens_device(seqs, device=device)
-        dev, b = tok.device, len(seqs)
-        ids32, mask, longest = encoders.pad_rows(tok, offsets, lengths, self.pad_id, t_cap, fill_to=0,
-                                                 remap=self._remap_on(dev))
-        # the one host sync: the output shape, and with it the smallest length (negative = failed row)
-        width, shortest = torch.stack((longest[0], lengths.min())).tolist()
-        if shortest < 0:
-            raise RuntimeError("BPE engine reported a failed row (negative length)")
-        if width == 0:
-            return (torch.empty((b, 0), dtype=torch.long, device=dev),
-                    torch.empty((b, 0), dtype=torch.uint8, device=dev))
-        return ids32[:, :width].to(torch.long), mask[:, :width].contiguous()
+        ids32, mask = self.padded_device(seqs, device=device)
+        return ids32.to(torch.long), mask.contiguous()
 
     def encode_batch_ids_only(self, seqs: List[str], *, device: object = "cuda") -> torch.Tensor:
         ids, _ = self.encode_batch(seqs, device=device)

@@ -214,6 +214,31 @@ int dnatok_bpe_encode_with_chars(const dnatok_bpe_t *t, const uint8_t *bytes, co
                                  const int32_t *char_lut, int32_t *char_ids, uint8_t *char_mask,
                                  void *stream);
 
+/* dnatok_bpe_encode and dnatok_pad_rows in one pass: row b's ids go straight to ids[b * stride ..]
+ * (int32[n_rows, stride]), through remap (kernel id -> tokenizer id, NULL: none), pad_id behind them
+ * up to the stride, mask (uint8[n_rows, stride], NULL allowed) 1 for a token and 0 for padding.  This
+ * is the tail of GPUTokBPEBackend.encode_batch (the remap LUT and the [B, T_max] padding,
+ * src/gputok_bpe_backend.py:624-638, 660-674) done by the merge engine while it writes a row's
+ * tokens out: no token run in memory in between, no second launch.  lengths[b] receives the row's
+ * full token count and *longest (device int32[1]; NULL: the caller takes it from the lengths, and
+ * the call ends a few microseconds earlier) the largest of them: a row with more tokens than
+ * the stride keeps its first `stride`, so a caller that sized the stride by a guess compares
+ * the longest row with it and, when that is larger, calls again with a stride of at least that (a row
+ * never has more tokens than bytes).  Rows of at most dnatok_bpe_padded_direct_max() bytes are
+ * written this way; a batch with a longer row (max_len above it) is assembled in tok_tmp
+ * (int32[total], NULL allowed otherwise) and padded from there by the kernels of the two calls.
+ * scratch, max_len and errors as for dnatok_bpe_encode. */
+int dnatok_bpe_encode_padded(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets,
+                             int64_t n_rows, int64_t max_len, int64_t total,
+                             void *scratch, size_t scratch_bytes, int32_t *tok_tmp,
+                             const int32_t *remap, int32_t pad_id, int64_t stride,
+                             int32_t *ids, uint8_t *mask, int32_t *lengths, int32_t *longest,
+                             void *stream);
+
+/* Longest row, in bytes, that dnatok_bpe_encode_padded writes without tok_tmp (the size of an
+ * extended chunk: dnatok_bpe_set_chunk_geometry changes it). */
+int64_t dnatok_bpe_padded_direct_max(void);
+
 /* The same encode for callers that cannot allocate device memory or hand over a work buffer: code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
  * counterpart in the reference (whose tokenize_batch grows torch tensors on demand,

@@ -669,6 +669,108 @@ def test_bpe_with_single_character_ids_from_the_same_pass(bpe):
                 np.testing.assert_array_equal(tok[b.offsets[i]:b.offsets[i] + lengths[i]], e, err_msg=f"row {i}")
 
 
+def check_padded(enc, bo, seqs, stride, *, remap_h=None, want_mask=True, want_longest=True, pad_id=-7, out=None,
+                 ref=None):
+    b = util.batch_from_strings(seqs)
+    data, off = to_dev(b)
+    max_len = int(b.lengths().max()) if b.n_seqs else 0
+    remap = None if remap_h is None else torch.from_numpy(remap_h).to(DEV)
+    ids, mask, lengths, longest = enc.encode_padded(data, off, max_len, stride, pad_id, remap=remap,
+                                                    want_mask=want_mask, want_longest=want_longest, out=out)
+    torch.cuda.synchronize()
+    ids_h, len_h = ids.cpu().numpy(), lengths.cpu().numpy()
+    mask_h = mask.cpu().numpy() if mask is not None else None
+    ref = bo.encode_batch(b.data, b.offsets) if ref is None else ref
+    want_longest = max((len(e) for e in ref), default=0)
+    assert longest is None or int(longest.item()) == want_longest
+    for i, e in enumerate(ref):
+        e = np.asarray(e, dtype=np.int64)
+        if remap_h is not None:
+            e = remap_h[e]
+        assert len_h[i] == len(e), f"row {i}"
+        kept = min(len(e), stride)
+        np.testing.assert_array_equal(ids_h[i, :kept], e[:kept], err_msg=f"row {i}")
+        assert (ids_h[i, kept:] == pad_id).all(), f"row {i}: padding"
+        if mask_h is not None:
+            assert (mask_h[i, :kept] == 1).all() and (mask_h[i, kept:] == 0).all(), f"row {i}: mask"
+    return ref
+
+
+def test_bpe_padded_in_one_pass(bpe):
+    """dnatok_bpe_encode_padded: ids, mask, lengths and the longest row as dnatok_bpe_encode followed by
+    dnatok_pad_rows give them, on every route: one row per team, more rows than teams (the work
+    list), every LDS capacity, rows cut by a stride that is too small, empty rows and an empty
+    batch, a second id map or none, a mask or none, and batches with rows long enough to be cut into
+    chunks (assembled in the token buffer first)."""
+    which, enc, bo = bpe
+    say(f"bpe{which} padded in one pass")
+    rng = random.Random(5)
+    rnd = lambda n: "".join(rng.choices("ACGTN", weights=[24, 24, 24, 24, 4], k=n))
+    remap_h = np.random.default_rng(3).permutation(70000).astype(np.int32)
+    short = [rnd(n) for n in (0, 1, 7, 8, 9, 63, 1000, 1024, 0, 333)]
+    ref = check_padded(enc, bo, short, 512)
+    check_padded(enc, bo, short, 512, remap_h=remap_h, want_mask=False, ref=ref)
+    check_padded(enc, bo, short, 100, ref=ref)                     # rows cut by the stride
+    check_padded(enc, bo, short, 100, want_longest=False, ref=ref)  # the caller takes the longest row from the lengths
+    check_padded(enc, bo, short, 1, remap_h=remap_h, ref=ref)
+    check_padded(enc, bo, ["", "", ""], 16)
+    none = enc.encode_padded(torch.empty(0, dtype=torch.uint8, device=DEV), torch.zeros(1, dtype=torch.int64, device=DEV),
+                             0, 8, 0)
+    torch.cuda.synchronize()
+    assert none[0].shape == (0, 8) and int(none[3].item()) == 0
+    for cap_len in (1300, 1536, 2048):                             # the other LDS capacities
+        check_padded(enc, bo, [rnd(cap_len), rnd(5), "", rnd(cap_len - 7)], 640, remap_h=remap_h)
+    many = [rnd(rng.randint(0, 700)) for _ in range(5000)]          # more rows than teams
+    ref = check_padded(enc, bo, many, 256, remap_h=remap_h)
+    check_padded(enc, bo, many, 120, ref=ref)
+    check_padded(enc, bo, many, 256, want_longest=False, ref=ref)
+    # several calls in a row on one stream share the tree that carries the longest row; a smaller batch after a larger one
+    check_padded(enc, bo, many[:1500], 256, ref=ref[:1500])
+    check_padded(enc, bo, many[:3], 256, ref=ref[:3])
+    # rows that are cut into chunks, or redone by the whole-row kernel: through the token buffer
+    long_rows = wl.config5_ragged(40, seed=12).strings() + ["", rnd(5000), "A" * 9000, rnd(20_001)]
+    ref = check_padded(enc, bo, long_rows, 6000, remap_h=remap_h)
+    check_padded(enc, bo, long_rows, 300, ref=ref)
+
+
+def test_bpe_padded_on_two_streams_and_in_a_graph(bpe):
+    """Every stream has its own tree; replays of a captured call give the eager result each time,
+    with eager calls (which use the same tree) in between."""
+    which, enc, bo = bpe
+    say(f"bpe{which} padded: streams and graph")
+    rng = random.Random(9)
+    rnd = lambda n: "".join(rng.choices("ACGT", k=n))
+    seqs_a = [rnd(rng.randint(1, 1000)) for _ in range(700)]
+    seqs_b = [rnd(rng.randint(1, 500)) for _ in range(2500)]
+    s2 = torch.cuda.Stream()
+    ref_a = check_padded(enc, bo, seqs_a, 300)
+    with torch.cuda.stream(s2):
+        ref_b = check_padded(enc, bo, seqs_b, 160)
+    b = util.batch_from_strings(seqs_a)
+    data, off = to_dev(b)
+    max_len = int(b.lengths().max())
+    out = (torch.empty((len(seqs_a), 300), dtype=torch.int32, device=DEV),
+           torch.empty((len(seqs_a), 300), dtype=torch.uint8, device=DEV),
+           torch.empty(len(seqs_a), dtype=torch.int32, device=DEV), torch.empty(1, dtype=torch.int32, device=DEV))
+    eager = [t.clone() for t in enc.encode_padded(data, off, max_len, 300, 0, out=out)]
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        enc.encode_padded(data, off, max_len, 300, 0, out=out)       # the side stream's first call, outside the capture
+        torch.cuda.synchronize()
+        with torch.cuda.graph(g, stream=side):
+            enc.encode_padded(data, off, max_len, 300, 0, out=out)
+    for _ in range(3):
+        for t in out:
+            t.fill_(-1 if t.dtype != torch.uint8 else 7)
+        g.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(out, eager):
+            assert torch.equal(got, want)
+        check_padded(enc, bo, seqs_b[:900], 160, ref=ref_b[:900])
+
+
 def test_bpe_rows_without_a_seam_fall_back_to_the_whole_row_kernel(bpe):
     """Tandem repeats far longer than the chunk overlap: neighbouring chunk runs can stay out
     of phase, no seam is accepted, and the row is redone by the whole-row kernel."""
