@@ -90,6 +90,8 @@ struct BpeArgs {
     int32_t pad_id;
     unsigned long long *max_tree;
     int32_t *longest;
+    // the work list holds no rows: item i is row i (bpe_plan_in_order_kernel)
+    int32_t in_order;
 };
 
 typedef int32_t bpe_int4_a4 __attribute__((ext_vector_type(4), aligned(4)));
@@ -1007,6 +1009,20 @@ __global__ __launch_bounds__(1024) void bpe_plan_kernel(
 }
 
 // The entries of the chunks of the chunked rows: one thread per row, a row of many chunks by its wave.
+// The work list of a batch whose rows are about equally long and all taken whole: nothing but the
+// counters; the rows are dealt in their given order (sorting them by length gains nothing then, and
+// the scan over 16,384 rows by one workgroup takes 19 us).
+__global__ void bpe_plan_in_order_kernel(int32_t n_rows, BpePlan p)
+{
+    if (threadIdx.x == 0) {
+        p.counts[0] = n_rows;
+        p.counts[1] = 0;
+        p.counts[2] = 0;
+        p.counts[3] = 0;
+        for (int q = 0; q < kSingleClasses; ++q) p.counts[4 + q] = 0;
+    }
+}
+
 __global__ __launch_bounds__(256) void bpe_expand_kernel(const int64_t *__restrict__ offsets, int64_t n_rows,
                                                          BpePlan p)
 {
@@ -1104,6 +1120,8 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
             if (CHUNKS && item < n_mc) {
                 const int4 rc = p.rec[item];
                 row = rc.x; k = rc.y; nc = rc.z;
+            } else if (!CHUNKS && a.in_order) {
+                row = item;
             } else {
                 int32_t j = item - n_mc;
                 const int32_t *list = p.single[0];
@@ -1647,12 +1665,17 @@ int run_lds(bool long_rows, int chunking, const BpeArgs &a, const uint8_t *bytes
     }
     const bool planned = long_rows || n_rows > lds_resident_teams<NT, TEAMS, CAP>();
     if (planned) {
-        const int expand_here = chunking >> 1;
-        bpe_plan_kernel<<<1, 1024, 0, s>>>(offsets, n_rows, chunking & 1, expand_here, p);
-        DNATOK_HIP_TRY(hipGetLastError());
-        if ((chunking & 1) && !expand_here) {
-            bpe_expand_kernel<<<(int)((n_rows + 255) / 256), 256, 0, s>>>(offsets, n_rows, p);
+        if (a.in_order) {                            // (no row is cut)
+            bpe_plan_in_order_kernel<<<1, 64, 0, s>>>((int32_t)n_rows, p);
             DNATOK_HIP_TRY(hipGetLastError());
+        } else {
+            const int expand_here = chunking >> 1;
+            bpe_plan_kernel<<<1, 1024, 0, s>>>(offsets, n_rows, chunking & 1, expand_here, p);
+            DNATOK_HIP_TRY(hipGetLastError());
+            if ((chunking & 1) && !expand_here) {
+                bpe_expand_kernel<<<(int)((n_rows + 255) / 256), 256, 0, s>>>(offsets, n_rows, p);
+                DNATOK_HIP_TRY(hipGetLastError());
+            }
         }
         if (chunking & 1) {
             if (a.char_ids) return launch_lds_as<NT, TEAMS, CAP, true, true>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
@@ -1671,7 +1694,7 @@ int run_lds(bool long_rows, int chunking, const BpeArgs &a, const uint8_t *bytes
 
 // The launches of one encode call; p lies inside a scratch buffer that holds p.total_bytes.
 static int bpe_encode_launch(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets, int64_t n_rows,
-                             int64_t max_len, const BpePlan &p, int32_t *tok_tmp, int32_t *lengths, hipStream_t s,
+                             int64_t max_len, int64_t total, const BpePlan &p, int32_t *tok_tmp, int32_t *lengths, hipStream_t s,
                              const int32_t *char_lut = nullptr, int32_t *char_ids = nullptr,
                              uint8_t *char_mask = nullptr, const BpeArgs *padded = nullptr)
 {
@@ -1684,6 +1707,8 @@ static int bpe_encode_launch(const dnatok_bpe_t *t, const uint8_t *bytes, const 
     }
 
     const bool long_rows = max_len > p.ext;
+    // rows of about one length (the mean at least 3/4 of the longest), none cut: dealt in their given order
+    a.in_order = !long_rows && total >= (max_len * n_rows / 4) * 3 ? 1 : 0;
     int chunking = (long_rows && t->monotone) ? 1 : 0;
     // bit 1: the plan kernel writes the chunk entries itself (few rows, few chunks: one launch less)
     if (chunking && n_rows <= kPlanInlineRows && p.max_mc <= kPlanInlineChunks) chunking |= 2;
@@ -1736,7 +1761,7 @@ extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, co
                    "dnatok_bpe_encode: scratch holds %zu bytes, %zu needed", scratch_bytes, need.total_bytes);
     DNATOK_REQUIRE(((uintptr_t)scratch & 255) == 0, DNATOK_E_INVALID, "dnatok_bpe_encode: scratch must be 256-byte aligned");
     const BpePlan p = make_plan((uint8_t *)scratch, n_rows, max_len, total);
-    return bpe_encode_launch(t, bytes, offsets, n_rows, max_len, p, tok_tmp, lengths, (hipStream_t)stream);
+    return bpe_encode_launch(t, bytes, offsets, n_rows, max_len, total, p, tok_tmp, lengths, (hipStream_t)stream);
 }
 
 extern "C" int dnatok_bpe_encode_with_chars(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets,
@@ -1757,7 +1782,7 @@ extern "C" int dnatok_bpe_encode_with_chars(const dnatok_bpe_t *t, const uint8_t
     DNATOK_REQUIRE(((uintptr_t)scratch & 255) == 0, DNATOK_E_INVALID,
                    "dnatok_bpe_encode_with_chars: scratch must be 256-byte aligned");
     const BpePlan p = make_plan((uint8_t *)scratch, n_rows, max_len, total);
-    return bpe_encode_launch(t, bytes, offsets, n_rows, max_len, p, tok_tmp, lengths, (hipStream_t)stream, char_lut,
+    return bpe_encode_launch(t, bytes, offsets, n_rows, max_len, total, p, tok_tmp, lengths, (hipStream_t)stream, char_lut,
                              char_ids, char_mask);
 }
 
@@ -1819,7 +1844,7 @@ extern "C" int dnatok_bpe_encode_padded(const dnatok_bpe_t *t, const uint8_t *by
         // rows cut into chunks (or left to the whole-row kernel) are assembled in tok_tmp first
         DNATOK_REQUIRE(tok_tmp, DNATOK_E_INVALID,
                        "%s: a batch with a row of more than %d bytes needs tok_tmp (int32[total])", who, p.ext);
-        const int rc = bpe_encode_launch(t, bytes, offsets, n_rows, max_len, p, tok_tmp, lengths, s);
+        const int rc = bpe_encode_launch(t, bytes, offsets, n_rows, max_len, total, p, tok_tmp, lengths, s);
         if (rc) return rc;
         if (longest) {
             bpe_longest_kernel<<<1, 1024, 0, s>>>(lengths, n_rows, longest);
@@ -1838,7 +1863,7 @@ extern "C" int dnatok_bpe_encode_padded(const dnatok_bpe_t *t, const uint8_t *by
             it = t->slot_of_stream.emplace(stream, (int)t->slot_of_stream.size()).first;
         if (it != t->slot_of_stream.end()) pad.max_tree = t->max_trees + (size_t)it->second * kTreeWords;
     }
-    const int rc = bpe_encode_launch(t, bytes, offsets, n_rows, max_len, p, nullptr, lengths, s, nullptr, nullptr,
+    const int rc = bpe_encode_launch(t, bytes, offsets, n_rows, max_len, total, p, nullptr, lengths, s, nullptr, nullptr,
                                      nullptr, &pad);
     if (rc) return rc;
     if (longest && !pad.max_tree) {
@@ -1903,5 +1928,5 @@ extern "C" int dnatok_bpe_encode_static(const dnatok_bpe_t *t, const uint8_t *by
     const int rc = static_scratch_ptr(&base);
     if (rc) return rc;
     const BpePlan p = make_plan(base, n_rows, max_len, total, slabs);
-    return bpe_encode_launch(t, bytes, offsets, n_rows, max_len, p, tok_tmp, lengths, (hipStream_t)stream);
+    return bpe_encode_launch(t, bytes, offsets, n_rows, max_len, total, p, tok_tmp, lengths, (hipStream_t)stream);
 }

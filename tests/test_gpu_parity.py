@@ -771,6 +771,21 @@ def test_bpe_padded_on_two_streams_and_in_a_graph(bpe):
         check_padded(enc, bo, seqs_b[:900], 160, ref=ref_b[:900])
 
 
+def test_bpe_more_rows_of_about_one_length_than_teams(bpe):
+    """A batch of more rows than resident teams whose rows are about equally long is dealt in the
+    rows' given order, without the sorted work list: tokens as the oracle's, through the plain call
+    and through the one that pads."""
+    which, enc, bo = bpe
+    say(f"bpe{which} rows of one length, dealt in order")
+    rng = random.Random(23)
+    seqs = ["".join(rng.choices("ACGT", k=rng.randint(290, 300))) for _ in range(4000)]
+    b = util.batch_from_strings(seqs)
+    ref = bo.encode_batch(b.data, b.offsets)
+    for r, e in zip(bpe_rows(enc, b), ref):
+        np.testing.assert_array_equal(r, e)
+    check_padded(enc, bo, seqs, 128, ref=ref)
+
+
 def test_bpe_rows_without_a_seam_fall_back_to_the_whole_row_kernel(bpe):
     """Tandem repeats far longer than the chunk overlap: neighbouring chunk runs can stay out
     of phase, no seam is accepted, and the row is redone by the whole-row kernel."""
