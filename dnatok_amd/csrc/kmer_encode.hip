@@ -43,6 +43,9 @@ struct dnatok_kmer_table {
     int8_t *digit;           // [256]
     int32_t *single;         // [256]
     int32_t *lut4;           // [4^k]  id of an ACGT-only window, or -1
+    int32_t *lut4r;          // the same ids indexed the way kmer_rows_kernel<..., ARITH> forms a window's code
+    int arith;               // the digit table is the plain one (A C G T -> 0 1 2 3, N -> 4, nothing else,
+    uint32_t fold;           // or lower case as well: fold = 0xDFDFDFDF, else 0xFFFFFFFF): digits by arithmetic
     int2 *entry;             // [5^k]  {id, 0} | {-len, offset into flat} | {INT_MIN, 0} = nothing known
     int32_t *flat;           // expansion lists
     // Running maxima of pad-to-longest calls.  Every stream that encodes with this table gets a
@@ -74,7 +77,8 @@ namespace dnatok {
 
 struct KmerArgs {
     const int8_t *digit;
-    const int32_t *single, *lut4;
+    const int32_t *single, *lut4, *lut4r;
+    uint32_t fold;
     const int2 *entry;
     const int32_t *flat;
     int32_t pad_id, missing_id;
@@ -164,7 +168,13 @@ __device__ __forceinline__ void wave_sync()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-template <int K, bool LUT4_LDS, bool CHARS, bool HAS_MASK>
+// ARITH: the digit table is the plain one (see dnatok_kmer_table_create), and the digits of a lane
+// with four whole windows come from the bytes by arithmetic on four bytes at a time instead of a
+// trip to the digit table in LDS per byte: bits 1 and 2 of the ASCII code tell A, C, T and G
+// apart (0, 1, 2, 3); v_perm_b32 with those bits as selectors rebuilds the byte they stand for,
+// and a byte that differs from it is not one of the four.  The window code holds character i in
+// bits 2i, 2i + 1 (a.lut4r is indexed that way).
+template <int K, bool LUT4_LDS, bool CHARS, bool HAS_MASK, bool ARITH>
 __global__ __launch_bounds__(kRowsThreads) void kmer_rows_kernel(
     KmerArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
     int64_t n_rows, int64_t t_cap, int64_t fill_to, int32_t *__restrict__ ids,
@@ -185,8 +195,14 @@ __global__ __launch_bounds__(kRowsThreads) void kmer_rows_kernel(
         // a byte outside the alphabet counts as N inside a window
         s_spell[i] = a.single[(int)"ACGTN"[d < 0 || d > 4 ? 4 : d]];
     }
+    const int32_t *const g_lut4 = ARITH ? a.lut4r : a.lut4;
     if (LUT4_LDS)
-        for (uint32_t i = threadIdx.x; i < POW4; i += kRowsThreads) s_lut4[i] = a.lut4[i];
+        for (uint32_t i = threadIdx.x; i < POW4; i += kRowsThreads) s_lut4[i] = g_lut4[i];
+    // a window's code from the digit table's entries, character i at a time
+    auto with_digit = [](uint32_t c, uint32_t v, int i) -> uint32_t {
+        if (!ARITH) return (c << 2) + v;
+        return c | ((v & (kDigN | kDigBad)) ? (v & (kDigN | kDigBad)) : (((v ^ (v >> 1)) & 3u) << (2 * i)));
+    };
     __syncthreads();          // from here on every wave runs alone (one more barrier at the very end, with `publish`)
 
     const int lane = threadIdx.x & 63;
@@ -278,20 +294,56 @@ __global__ __launch_bounds__(kRowsThreads) void kmer_rows_kernel(
 #pragma unroll
             for (int i = 0; i < K; ++i) w[i] = wn[i];
             fetch(wn, u0 + kWaveUnits);
+            // (ARITH) bytes of the lane that are none of A C G T, as nonzero bytes: only meaningful
+            // for a lane whose bytes all lie inside the row (past its end the loads return zeros)
+            uint32_t odd[ARITH ? K : 1];
+            uint32_t odd_any = 0;
+            if (ARITH) {
+                // the digits of four bytes at a time, packed to one byte per word, then the
+                // windows cut from the string of 2-bit digits
+                uint32_t c8[K];
 #pragma unroll
-            for (int j = 0; j < kUnitsPerLane; ++j) {
-                uint32_t c = 0;
+                for (int i = 0; i < K; ++i) {
+                    const uint32_t d = w[i] & 0x06060606u;                       // digit << 1 in every byte
+                    // pool of the 8-byte permute: byte 0 'A', 2 'C', 4 'T', 6 'G'
+                    odd[i] = (w[i] ^ __builtin_amdgcn_perm(0x00470054u, 0x00430041u, d)) & a.fold;
+                    odd_any |= odd[i];
+                    const uint32_t x1 = (d << 6) | d;                            // bits 7..10, 23..26: two digits each
+                    const uint32_t x2 = (x1 << 12) | x1;                         // bits 19..26: the four digits
+                    c8[i] = (x2 >> 19) & 255u;
+                }
+                uint32_t str[(K + 3) / 4 + 1];
 #pragma unroll
-                for (int i = 0; i < K; ++i) c = (c << 2) + digit_of(j * K + i);
-                code[j] = c;
+                for (int q = 0; q < (K + 3) / 4 + 1; ++q) {
+                    uint32_t v = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (4 * q + e < K) v |= c8[4 * q + e] << (8 * e);
+                    str[q] = v;
+                }
+#pragma unroll
+                for (int j = 0; j < kUnitsPerLane; ++j) {
+                    constexpr uint32_t kCodeMask = POW4 - 1;
+                    const int bit = 2 * K * j;
+                    const uint64_t two = ((uint64_t)str[(bit >> 5) + 1] << 32) | str[bit >> 5];
+                    code[j] = (uint32_t)(two >> (bit & 31)) & kCodeMask;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < kUnitsPerLane; ++j) {
+                    uint32_t c = 0;
+#pragma unroll
+                    for (int i = 0; i < K; ++i) c = (c << 2) + digit_of(j * K + i);
+                    code[j] = c;
+                }
             }
 #pragma unroll
             for (int j = 0; j < kUnitsPerLane; ++j) {
                 const uint32_t idx = code[j] & (POW4 - 1);
-                t[j] = LUT4_LDS ? s_lut4[idx] : a.lut4[idx];
+                t[j] = LUT4_LDS ? s_lut4[idx] : g_lut4[idx];
             }
-            const uint32_t any_flag = code[0] | code[1] | code[2] | code[3];
-            const bool fast = lane_full && any_flag < POW4 && (t[0] | t[1] | t[2] | t[3]) >= 0;
+            const uint32_t any_flag = ARITH ? odd_any : (code[0] | code[1] | code[2] | code[3]);
+            const bool fast = lane_full && (ARITH ? any_flag == 0 : any_flag < POW4) && (t[0] | t[1] | t[2] | t[3]) >= 0;
             const uint64_t rest_mask = __ballot(!fast && !empty);
             const int A = mis + running;           // cell the step's first token goes to
 
@@ -307,6 +359,28 @@ __global__ __launch_bounds__(kRowsThreads) void kmer_rows_kernel(
             if (fast) {
                 lane_cnt = kUnitsPerLane;
             } else if (lane_full) {
+                if (ARITH && odd_any) {
+                    // which windows hold a byte that is none of the four (kDigN on their code), and
+                    // whether such a byte is no N either (kDigBad): the byte that bits 1..3 of a
+                    // byte stand for, with N in the pool
+                    uint32_t foreign = 0;
+#pragma unroll
+                    for (int i = 0; i < K; ++i) {
+                        const uint32_t sel = (w[i] >> 1) & 0x07070707u;           // A 0, C 1, T 2, G 3, N 7
+                        foreign |= w[i] ^ __builtin_amdgcn_perm(0x4E000000u, 0x47544341u, sel);
+                    }
+                    foreign &= a.fold;
+#pragma unroll
+                    for (int j = 0; j < kUnitsPerLane; ++j) {
+                        uint32_t hit = 0;
+#pragma unroll
+                        for (int i = 0; i < K; ++i) {
+                            const int bi = j * K + i;
+                            hit |= odd[bi >> 2] & (0xFFu << (8 * (bi & 3)));
+                        }
+                        if (hit) code[j] |= foreign ? (kDigN | kDigBad) : kDigN;
+                    }
+                }
 #pragma unroll
                 for (int j = 0; j < kUnitsPerLane; ++j) {
                     ex[j] = 0; ey[j] = 0;
@@ -343,12 +417,12 @@ __global__ __launch_bounds__(kRowsThreads) void kmer_rows_kernel(
 #pragma unroll
                         for (int i = 0; i < K; ++i) {
                             const uint32_t v = s_dig[src[u * K + i]];
-                            c = (c << 2) + v;
+                            c = with_digit(c, v, i);
                             if (v & kDigBad) my_status |= DNATOK_ROW_INVALID_BYTE;
                             c5 = c5 * 5 + ((v & (kDigN | kDigBad)) ? 4 : (int)v);
                         }
                         int32_t id = -1;
-                        if (c < POW4) id = LUT4_LDS ? s_lut4[c] : a.lut4[c];
+                        if (c < POW4) id = LUT4_LDS ? s_lut4[c] : g_lut4[c];
                         if (id >= 0) {
                             n = 1;
                         } else {
@@ -407,11 +481,11 @@ __global__ __launch_bounds__(kRowsThreads) void kmer_rows_kernel(
     #pragma unroll
                         for (int i = 0; i < K; ++i) {
                             const uint32_t v = s_dig[src[u * K + i]];
-                            c = (c << 2) + v;
+                            c = with_digit(c, v, i);
                             c5 = c5 * 5 + ((v & (kDigN | kDigBad)) ? 4 : (int)v);
                         }
                         int32_t id = -1;
-                        if (c < POW4) id = LUT4_LDS ? s_lut4[c] : a.lut4[c];
+                        if (c < POW4) id = LUT4_LDS ? s_lut4[c] : g_lut4[c];
                         if (id >= 0) {
                             put(s, id);
                             ++s;
@@ -1060,6 +1134,31 @@ extern "C" int dnatok_kmer_table_create(int k, const int8_t *digit_h, const int3
         for (int i = k - 1; i >= 0; --i) c5 = c5 * 5 + ((c4 >> (2 * i)) & 3);
         lut4[c4] = kmer_lut_h[c5];
     }
+    // The same ids in the order of the code that kmer_rows_kernel<..., ARITH> computes from the bytes
+    // themselves: character i of the window in bits 2i, 2i + 1, as bits 1 and 2 of its ASCII code
+    // (A 0, C 1, T 2, G 3).  That kernel serves the plain digit table: A C G T N -> 0 1 2 3 4, in
+    // upper case alone or in both cases, every other byte outside the alphabet.
+    std::vector<int32_t> lut4r(pow4);
+    for (int64_t c4 = 0; c4 < pow4; ++c4) {
+        int64_t r = 0;
+        for (int i = 0; i < k; ++i) {
+            const int64_t d = (c4 >> (2 * (k - 1 - i))) & 3;       // digit of character i
+            r |= (d ^ (d >> 1)) << (2 * i);
+        }
+        lut4r[r] = lut4[c4];
+    }
+    bool plain_upper = true, plain_lower = true, no_lower = true;
+    for (int b = 0; b < 256; ++b) {
+        const char *u = strchr("ACGTN", b), *l = strchr("acgtn", b);
+        const int want_u = (b && u) ? (int)(u - "ACGTN") : -1, want_l = (b && l) ? (int)(l - "acgtn") : -1;
+        if (want_l >= 0) {
+            plain_lower = plain_lower && digit_h[b] == want_l;
+            no_lower = no_lower && digit_h[b] < 0;
+        } else {
+            plain_upper = plain_upper && (want_u < 0 ? digit_h[b] < 0 : digit_h[b] == want_u);
+        }
+    }
+    const bool arith = plain_upper && (plain_lower || no_lower);
     // entry[c5]: one 8-byte record per window, and whether every window without an id is
     // spelled by its own characters (then the kernel never reads entry / flat)
     std::vector<int2> entry(pow5);
@@ -1088,7 +1187,8 @@ extern "C" int dnatok_kmer_table_create(int k, const int8_t *digit_h, const int3
     const size_t o_digit = 0;
     const size_t o_single = up(o_digit + 256);
     const size_t o_lut4 = up(o_single + 256 * 4);
-    const size_t o_entry = up(o_lut4 + pow4 * 4);
+    const size_t o_lut4r = up(o_lut4 + pow4 * 4);
+    const size_t o_entry = up(o_lut4r + pow4 * 4);
     const size_t o_flat = up(o_entry + pow5 * sizeof(int2));
     const size_t o_slots = up(o_flat + (has_exp ? n_flat * 4 : 0));
     const size_t o_trees = up(o_slots + (size_t)kMaxSlots * kMaxSlotStride * 8);
@@ -1097,6 +1197,7 @@ extern "C" int dnatok_kmer_table_create(int k, const int8_t *digit_h, const int3
     memcpy(&host[o_digit], digit_h, 256);
     memcpy(&host[o_single], single_h, 256 * 4);
     memcpy(&host[o_lut4], lut4.data(), pow4 * 4);
+    memcpy(&host[o_lut4r], lut4r.data(), pow4 * 4);
     memcpy(&host[o_entry], entry.data(), pow5 * sizeof(int2));
     if (has_exp) memcpy(&host[o_flat], exp_flat_h, n_flat * 4);
     void *blob = nullptr;
@@ -1114,6 +1215,9 @@ extern "C" int dnatok_kmer_table_create(int k, const int8_t *digit_h, const int3
     t->digit = (int8_t *)(b + o_digit);
     t->single = (int32_t *)(b + o_single);
     t->lut4 = (int32_t *)(b + o_lut4);
+    t->lut4r = (int32_t *)(b + o_lut4r);
+    t->arith = arith ? 1 : 0;
+    t->fold = arith && plain_lower ? 0xDFDFDFDFu : 0xFFFFFFFFu;
     t->entry = (int2 *)(b + o_entry);
     t->flat = (int32_t *)(b + o_flat);
     t->max_slots = (unsigned long long *)(b + o_slots);
@@ -1158,7 +1262,7 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
     if (to_longest) fill_to = guess;
     if (n_rows == 0) return DNATOK_OK;
     hipStream_t s = (hipStream_t)stream;
-    KmerArgs a{t->digit, t->single, t->lut4, t->entry, t->flat, t->pad_id, t->missing_id};
+    KmerArgs a{t->digit, t->single, t->lut4, t->lut4r, t->fold, t->entry, t->flat, t->pad_id, t->missing_id};
     MaxRef mref{nullptr, nullptr};
     if (to_longest) {
         std::lock_guard<std::mutex> hold(t->slot_lock);
@@ -1184,9 +1288,13 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
     constexpr int64_t kTightStride = 256;
     const bool tight = to_longest && mref.slot && guess > 0 && t_cap - guess <= kTightStride && t_cap < 0xFFFF;
     bool padded_in_kernel = false;
-#define LAUNCH3(KK, L, C, M)                                                                      \
+#define LAUNCH3(KK, L, C, M) \
     do {                                                                                          \
-        static const int resident = resident_workgroups(kmer_rows_kernel<KK, L, C, M>, kRowsThreads, 0, 2); \
+        if (t->arith) LAUNCH4(KK, L, C, M, true); else LAUNCH4(KK, L, C, M, false);               \
+    } while (0)
+#define LAUNCH4(KK, L, C, M, AR)                                                                  \
+    do {                                                                                          \
+        static const int resident = resident_workgroups(kmer_rows_kernel<KK, L, C, M, AR>, kRowsThreads, 0, 2); \
         static const int team_resident = resident_workgroups(kmer_team_kernel<KK, L, C, M>, kKmerThreads, 0, 4); \
         const int team_rows = g_team_rows.load(std::memory_order_relaxed);                       \
         if (n_rows <= (team_rows < 0 ? team_resident : team_rows)) {                              \
@@ -1198,7 +1306,7 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
         }                                                                                         \
         const int64_t grid = want < resident ? want : resident;                                   \
         padded_in_kernel = tight && grid <= kTreeRows;                                            \
-        kmer_rows_kernel<KK, L, C, M><<<(int)grid, kRowsThreads, 0, s>>>(                         \
+        kmer_rows_kernel<KK, L, C, M, AR><<<(int)grid, kRowsThreads, 0, s>>>(                     \
             a, bytes, offsets, n_rows, t_cap, padded_in_kernel ? t_cap : fill_to, ids, mask,      \
             lengths, status, max_len, mref, padded_in_kernel ? 1 : 0);                            \
     } while (0)
@@ -1222,6 +1330,7 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
 #undef LAUNCH
 #undef LAUNCH2
 #undef LAUNCH3
+#undef LAUNCH4
     DNATOK_HIP_TRY(hipGetLastError());
     if (to_longest && !padded_in_kernel)
         return launch_pad(ids, mask, lengths, n_rows, t_cap, max_len, t->pad_id, (int32_t)guess, mref, s);

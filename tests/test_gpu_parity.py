@@ -547,6 +547,49 @@ def test_kmer_general_tables_not_spelled(kmer_kernel_choice):
 
 
 @both_kmer_kernels
+@pytest.mark.parametrize("k", [3, 6, 8])
+@pytest.mark.parametrize("form", ["both_cases", "u_reads_as_t"])
+def test_kmer_digit_tables_of_other_forms(kmer_kernel_choice, k, form):
+    """The kernel that takes a row per wave finds the digits of the plain table (A C G T N in
+    upper case, or in both cases) by arithmetic on the bytes and those of any other table in the
+    table itself: a table that folds the case (lower-case rows, rows of mixed case, bytes that
+    differ from a base in one bit only), and one with a sixth letter, against the oracle's walk
+    through the same tables."""
+    say(f"kmer digit table {form} k={k}")
+    vocab = hf.kmer_vocab(k)
+    t = kmer_tables.tables_from_vocab(vocab, k, 0)
+    digit = kmer_tables.digit_table(fold_case=(form == "both_cases"))
+    if form == "u_reads_as_t":
+        digit[ord("U")] = 3
+    single = t.single.copy()
+    for ch in "acgtnU":
+        single[ord(ch)] = single[ord(ch.upper() if ch != "U" else "T")]
+    enc = encoders.KmerEncoder(k, digit, t.kmer_lut, single, pad_id=1, missing_id=0,
+                               exp_off=t.exp_off, exp_len=t.exp_len, exp_flat=t.exp_flat)
+    ot = O.KmerTables(k, digit, t.kmer_lut, t.exp_off, t.exp_len, t.exp_flat, single, 0)
+    rng = np.random.default_rng(100 + k)
+    letters = list("ACGTNacgtnU")
+    strings = ["".join(rng.choice(letters, p=[.2, .2, .2, .2, .02, .04, .04, .04, .04, .01, .01], size=n))
+               for n in rng.integers(0, 7000, size=40)]
+    strings += ["acgt" * 1500, "ACGTU" * 900, "".join(chr(ord(c) ^ b) for c, b in zip("ACGTN" * 600, [1, 2, 4, 8, 16, 32, 64] * 429)),
+                "ACGT" * 700 + "a!c{g`t@" * 50 + "ACGT" * 700]
+    b = util.batch_from_strings(strings)
+    data, off = to_dev(b)
+    t_cap = max(len(s) for s in strings) + 4
+    t_cap += (-t_cap) % 4
+    ids, mask, lengths, status, max_len = enc.encode_padded(data, off, t_cap)
+    torch.cuda.synchronize()
+    erows, estatus = O.kmer_encode(ot, b.data, b.offsets)
+    np.testing.assert_array_equal(lengths.cpu().numpy(), [r.size for r in erows])
+    np.testing.assert_array_equal(status.cpu().numpy() & 3, estatus)
+    m = int(max_len.item())
+    assert m == max(r.size for r in erows)
+    eids, emask = O.pad_rows(erows, 1, m)
+    np.testing.assert_array_equal(ids[:, :m].cpu().numpy(), eids)
+    np.testing.assert_array_equal(mask[:, :m].cpu().numpy(), emask)
+
+
+@both_kmer_kernels
 def test_kmer_missing_windows_without_expansion(kmer_kernel_choice):
     say("kmer missing windows")
     t = kmer_tables.tables_from_vocab(hf.kmer_vocab(4), 4, 0)
