@@ -553,6 +553,53 @@ def hf_cpu(config: str, threads: int, max_bases: int) -> dict | None:
         return {"error": f"{type(e).__name__}: {e}"}
 
 
+def memory_only_extra(w, dev_ms: float) -> dict:
+    """What this machine gives the 6-mer workload's loads and stores when nothing is computed
+    (dnatok_diag_kmer_shape: the same rows, steps, strides and padding, no arithmetic), and its
+    fastest plain copy (dnatok_diag_copy_tiles), beside the encoder's own step."""
+    import ctypes
+    import torch
+    from dnatok_amd import _lib
+    L = _lib.lib()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+    ids = torch.empty((w.n_rows, w.t_cap), dtype=torch.int32, device="cuda")
+    mask = torch.empty((w.n_rows, w.t_cap), dtype=torch.uint8, device="cuda")
+    fill = sum(w.widths) // 2
+
+    def timed(fn, n):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    shape_ms = timed(lambda: _lib.check(L.dnatok_diag_kmer_shape(ptr(w.sets[0]), ptr(w.off), w.n_rows, w.t_cap, fill,
+                                                                 ptr(ids), ptr(mask), stream), "dnatok_diag_kmer_shape"), 100)
+    del ids, mask
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device="cuda").random_(0, 255)
+    dst = torch.empty_like(src)
+    copy_ms = timed(lambda: _lib.check(L.dnatok_diag_copy_tiles(ptr(src), ptr(dst), n, stream), "dnatok_diag_copy_tiles"), 30)
+    same = bool(torch.equal(src, dst))
+    del src, dst
+    by = w.algorithmic_bytes
+    return {"kmer_shape": {"what": "the workload's loads and stores without the arithmetic: same rows, 1536-byte steps, "
+                                   f"row stride {w.t_cap} cells, padded to {fill} cells",
+                           "device_ms_per_step": shape_ms, "GB/s": by / (shape_ms * 1e-3) / 1e9,
+                           "hbm_frac": by / (shape_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                           "encoder_rate_over_this": shape_ms / dev_ms},
+            "copy_tiles_1GiB": {"what": "device-to-device copy of 1 GiB in contiguous 16 KB tiles per workgroup "
+                                        "(1 GiB read + 1 GiB written)", "device_ms": copy_ms,
+                                "GB/s": 2 * n / (copy_ms * 1e-3) / 1e9, "hbm_frac": 2 * n / (copy_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                                "copied_exactly": same}}
+
+
 def fused_embed_extra():
     """Fused byte -> id -> embedding row kernel on one C1 batch (64 x 8192 bases), bf16 rows of 512:
     1 byte read and 1 KiB written per base; checked against the two-step torch form."""
@@ -873,6 +920,8 @@ def main() -> None:
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if args.config == "C2" and not args.per_call and (args.calibrate_copy or not args.no_extras):
+        result["memory_only"] = memory_only_extra(w, dev_ms)
 
     # HBM bytes per launch come from rocprofv3 counter runs of this same command, which cannot run
     # inside it; the committed summary says when and how they were taken

@@ -21,7 +21,8 @@ EXPORTS = [
     "dnatok_char_unpack_2bit", "dnatok_host_clean_ascii", "dnatok_host_pack_2bit", "dnatok_host_fasta_scan",
     "dnatok_kmer_table_create", "dnatok_kmer_table_destroy", "dnatok_kmer_set_team_rows", "dnatok_kmer_encode_padded",
     "dnatok_bpe_table_create", "dnatok_bpe_table_destroy", "dnatok_bpe_scratch_bytes",
-    "dnatok_bpe_encode", "dnatok_bpe_encode_with_chars", "dnatok_bpe_encode_padded", "dnatok_bpe_padded_direct_max", "dnatok_bpe_static_scratch_bytes", "dnatok_bpe_encode_static",
+    "dnatok_bpe_encode", "dnatok_bpe_encode_with_chars", "dnatok_bpe_encode_padded", "dnatok_bpe_padded_direct_max",
+    "dnatok_diag_copy_tiles", "dnatok_diag_kmer_shape", "dnatok_bpe_static_scratch_bytes", "dnatok_bpe_encode_static",
     "dnatok_bpe_set_chunk_geometry", "dnatok_bpe_set_table_placement", "dnatok_pack_ragged", "dnatok_pad_rows", "dnatok_pad_rows_as",
     "dnatok_normalize_bounds", "dnatok_normalize_rows",
 ]
@@ -108,6 +109,8 @@ def lib() -> ctypes.CDLL:
                                            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
     L.dnatok_bpe_padded_direct_max.argtypes = []
     L.dnatok_bpe_padded_direct_max.restype = c_int64
+    L.dnatok_diag_copy_tiles.argtypes = [c_void_p, c_void_p, c_size_t, c_void_p]
+    L.dnatok_diag_kmer_shape.argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p]
     L.dnatok_bpe_static_scratch_bytes.restype = c_size_t
     L.dnatok_bpe_encode_static.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                            c_void_p, c_void_p, c_void_p]

@@ -8,7 +8,7 @@ import sys
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_HERE, "libdnatok_hip.so")
-SOURCES = ["errors.hip", "char_encode.hip", "kmer_encode.hip", "bpe_encode.hip", "pack.hip", "host_ingest.hip", "normalize.hip"]
+SOURCES = ["errors.hip", "char_encode.hip", "kmer_encode.hip", "bpe_encode.hip", "pack.hip", "host_ingest.hip", "normalize.hip", "diag.hip"]
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # packed-FP32 instruction forms are kept out of all device code
