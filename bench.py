@@ -540,6 +540,25 @@ def time_steps(w: Workload, steps: int, warmup: int):
     return wall_ms, dev_ms
 
 
+def step_spread(w: Workload, steps: int = 100) -> dict:
+    """Device time of single steps (an event between every two of them): median, p5 and p95 in
+    microseconds.  A pass of its own after the timed region, which is bracketed as a whole (the
+    event between two steps costs each of them a microsecond or two)."""
+    import torch
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    for _ in range(10):
+        w.step()
+    torch.cuda.synchronize()
+    marks[0].record()
+    for i in range(steps):
+        w.step()
+        marks[i + 1].record()
+    torch.cuda.synchronize()
+    us = np.array([marks[i].elapsed_time(marks[i + 1]) * 1e3 for i in range(steps)])
+    return {"n": steps, "median_us": float(np.median(us)), "p5_us": float(np.percentile(us, 5)),
+            "p95_us": float(np.percentile(us, 95)), "min_us": float(us.min()), "max_us": float(us.max())}
+
+
 def hf_cpu(config: str, threads: int, max_bases: int) -> dict | None:
     env = dict(os.environ, RAYON_NUM_THREADS=str(threads), TOKENIZERS_PARALLELISM="true")
     cmd = [sys.executable, "-m", "tests.support.hf_baseline", "--config", config, "--budget", "12"]
@@ -912,6 +931,7 @@ def main() -> None:
     }
     if args.config in ("C3", "C4", "C5"):
         result["roofline"]["note"] = BPE_BOUND_NOTE
+    result["step_spread"] = step_spread(w)
 
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").random_(0, 255)
