@@ -35,3 +35,11 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert b"null" in L.dnatok_last_error()
     rc = L.dnatok_kmer_encode_padded(None, None, None, 1, 4, 8, None, None, None, None, None, None)
     assert rc == -1
+    # the entry points that pad BPE rows themselves and the measurement aids check their arguments first as well
+    rc = L.dnatok_bpe_encode_padded(None, None, None, 1, 4, 4, None, 0, None, None, 0, 8, None, None, None, None, None)
+    assert rc == -1 and b"null" in L.dnatok_last_error()
+    rc = L.dnatok_diag_copy_tiles(None, None, 16, None)
+    assert rc == -1 and b"null" in L.dnatok_last_error()
+    rc = L.dnatok_diag_kmer_shape(None, None, 1, 8, 8, None, None, None)
+    assert rc == -1
+    assert L.dnatok_bpe_padded_direct_max() == 2048
