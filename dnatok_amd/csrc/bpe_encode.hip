@@ -92,6 +92,9 @@ struct BpeArgs {
     int32_t *longest;
     // the work list holds no rows: item i is row i (bpe_plan_in_order_kernel)
     int32_t in_order;
+    // items a team takes from its work counter at a time, and the counters in use (a power of two,
+    // at most kDealers and at most the number of teams: every counter needs a team)
+    int32_t grab, dealers;
 };
 
 typedef int32_t bpe_int4_a4 __attribute__((ext_vector_type(4), aligned(4)));
@@ -800,8 +803,17 @@ constexpr int kLongGrid = 64;            // slabs of scratch for the whole-row f
 // teams idle for its whole duration (ragged benchmark batch: 0.299 -> 0.289 ms).
 constexpr int kSingleClasses = 3;
 
+// The items beyond one per team are handed out through kDealers counters instead of one: an
+// atomic on one address takes its turn behind all others (about 12 ns each), which for 100,000
+// short rows is longer than their merging.  Counter c hands out the items whose number is c modulo
+// kDealers, to the teams whose number is c modulo kDealers: every counter's share of the list,
+// which runs from large items to small ones, looks like the whole.
+constexpr int kDealers = 16;
+constexpr int kDealerStride = 64;         // int32 words between two counters (256 bytes)
+
 struct BpePlan {                          // device arrays inside the scratch buffer
-    int32_t *counts;      // [0] items, [1] chunk items, [2] work counter, [3] failed rows, [4 + c] single rows of class c
+    int32_t *counts;      // [0] items, [1] chunk items, [3] failed rows, [4 + c] single rows of class c
+    int32_t *deal;        // [kDealers * kDealerStride] the work counters
     int32_t *mc_off;      // [n_rows + 1] first chunk slot of a row (multi-chunk rows only)
     int4 *rec;           // [max_mc] a chunk item: {row, chunk of the row, chunks of the row, row length}
     int32_t *single[kSingleClasses];   // [n_rows] each: the rows that are one item, longest class first
@@ -861,6 +873,7 @@ static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t
     size_t o = 0;
     auto take = [&](size_t bytes) { size_t at = o; o = up(o + bytes); return at; };
     const size_t o_counts = take(64);
+    const size_t o_deal = take(4 * (size_t)kDealers * kDealerStride);
     const size_t o_mc_off = take(4 * (size_t)(n_rows + 1));
     const size_t o_rec = take(16 * (size_t)p.max_mc);
     size_t o_single[kSingleClasses];
@@ -876,6 +889,7 @@ static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t
     p.total_bytes = o + 256;
     if (base) {
         p.counts = (int32_t *)(base + o_counts);
+        p.deal = (int32_t *)(base + o_deal);
         p.mc_off = (int32_t *)(base + o_mc_off);
         p.rec = (int4 *)(base + o_rec);
         for (int c = 0; c < kSingleClasses; ++c) p.single[c] = (int32_t *)(base + o_single[c]);
@@ -997,6 +1011,7 @@ __global__ __launch_bounds__(1024) void bpe_plan_kernel(
             p.rec[c] = make_int4(row, c - first, next - first, s_len[row]);
         }
     }
+    if (threadIdx.x < kDealers) p.deal[threadIdx.x * kDealerStride] = 0;
     if (threadIdx.x == 0) {
         int32_t items = carry[0];
         for (int q = 0; q < kSingleClasses; ++q) { p.counts[4 + q] = carry[1 + q]; items += carry[1 + q]; }
@@ -1021,6 +1036,7 @@ __global__ void bpe_plan_in_order_kernel(int32_t n_rows, BpePlan p)
         p.counts[3] = 0;
         for (int q = 0; q < kSingleClasses; ++q) p.counts[4 + q] = 0;
     }
+    if (threadIdx.x < kDealers) p.deal[threadIdx.x * kDealerStride] = 0;
 }
 
 __global__ __launch_bounds__(256) void bpe_expand_kernel(const int64_t *__restrict__ offsets, int64_t n_rows,
@@ -1092,7 +1108,7 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
 
     const int32_t n_items = PLANNED ? p.counts[0] : n_rows;
     static_assert(PLANNED || !CHUNKS, "chunks come from the work list");
-    static_assert(!PADDED || (!CHUNKS && !LTAB && TEAMS == 1), "padded rows: whole rows, one team per workgroup");
+    static_assert(!PADDED || (!CHUNKS && !LTAB), "padded rows: whole rows");
     const int32_t n_mc = CHUNKS ? p.counts[1] : 0;
     const int32_t n_single0 = PLANNED ? p.counts[4] : 0, n_single1 = PLANNED ? p.counts[5] : 0;
     // A team's first item is its own number; only the items beyond one per team are handed out
@@ -1100,16 +1116,25 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     // thousand atomics on one address, about 12 ns each, before the last team has its row.)
     const int32_t n_teams = (int32_t)gridDim.x * TEAMS;
     int32_t item = (int32_t)blockIdx.x * TEAMS + team;
+    int32_t left = 0;                                // items of the team's current share still to come
+    const int32_t dealer = item & (a.dealers - 1);
+    // the first item beyond the teams' own that this team's counter hands out
+    const int32_t dealt_from = n_teams + ((dealer - n_teams) & (a.dealers - 1));
     constexpr bool padded = PADDED;
     int32_t team_longest = 0;                        // (padded) most tokens in a row of this team
     for (bool first = true;; first = false) {
         if (!first) {
-            if (PLANNED) {
-                if (n_teams >= n_items) break;       // nothing was left for the counter
-                if (tid == 0) *next_item = n_teams + atomicAdd(&p.counts[2], 1);
+            if (PLANNED && left > 0) {               // (the same in every lane)
+                item += a.dealers;
+                --left;
+            } else if (PLANNED) {
+                if (n_teams >= n_items) break;       // nothing was left for the counters
+                if (tid == 0)
+                    *next_item = dealt_from + a.dealers * atomicAdd(&p.deal[dealer * kDealerStride], a.grab);
                 team_sync<NT>();
                 item = *next_item;
                 team_sync<NT>();
+                left = a.grab - 1;
             } else {
                 item += n_teams;
             }
@@ -1190,9 +1215,22 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
         }
         team_sync<NT>();
     }
-    // (padded, one team per workgroup) every workgroup reports once, whether it had a row or not
-    if (padded && a.max_tree && threadIdx.x == 0)
-        publish_max(a.max_tree, (unsigned)team_longest, a.longest);
+    // (padded) every workgroup reports once, whether it had a row or not
+    if (padded && a.max_tree) {
+        if (TEAMS == 1) {
+            if (threadIdx.x == 0) publish_max(a.max_tree, (unsigned)team_longest, a.longest);
+        } else {
+            __shared__ int32_t s_longest[TEAMS];
+            if (tid == 0) s_longest[team] = team_longest;
+            __syncthreads();                         // (every team has left its loop)
+            if (threadIdx.x == 0) {
+                int32_t m = 0;
+#pragma unroll
+                for (int q = 0; q < TEAMS; ++q) m = s_longest[q] > m ? s_longest[q] : m;
+                publish_max(a.max_tree, (unsigned)m, a.longest);
+            }
+        }
+    }
 }
 
 // One workgroup per chunk of a multi-chunk row: the seam with the chunk to its right.  The two
@@ -1607,7 +1645,17 @@ int launch_lds_as(const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets
     if (grid > resident) grid = resident;
     if (a.max_tree && grid > kTreeRows) grid = kTreeRows;
     if (grid < 1) grid = 1;
-    kern<<<(int)grid, NT * TEAMS, lds, s>>>(a, bytes, offsets, p, (int32_t)n_rows, tok_tmp, lengths);
+    // a team's share per trip to its work counter: one item, and with very many items 1/32 of
+    // what a team takes in all, at most 8 (the last shares decide how evenly the teams end)
+    BpeArgs a2 = a;
+    const int64_t per_team = PLANNED ? (items - grid * TEAMS) / (grid * TEAMS * 32) : 1;
+    a2.grab = (int32_t)(per_team < 1 ? 1 : (per_team > 8 ? 8 : per_team));
+    // several counters for the wave-sized teams of short rows (thousands of teams, items of a few
+    // microseconds); one for the 256-thread teams, whose items last far longer than a turn at the
+    // counter and end most evenly when any team may take the last of them
+    a2.dealers = TEAMS > 1 ? kDealers : 1;
+    while (a2.dealers > grid * TEAMS) a2.dealers >>= 1;
+    kern<<<(int)grid, NT * TEAMS, lds, s>>>(a2, bytes, offsets, p, (int32_t)n_rows, tok_tmp, lengths);
     DNATOK_HIP_TRY(hipGetLastError());
     return DNATOK_OK;
 }
@@ -1658,10 +1706,12 @@ template <int NT, int TEAMS, int CAP>
 int run_lds(bool long_rows, int chunking, const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets,
             const BpePlan &p, int64_t n_rows, int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
 {
-    if (CAP == 1024 && !long_rows && a.ltab && !a.char_ids && !a.pad_ids) {
-        const int mode = g_table_placement.load(std::memory_order_relaxed);
-        if (mode == 2 || (mode == 1 && n_rows <= ltab_resident_teams<NT, TEAMS, 1024>()))
-            return launch_lds_ltab<NT, TEAMS, 1024>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    if constexpr (CAP == 1024) {
+        if (!long_rows && a.ltab && !a.char_ids && !a.pad_ids) {
+            const int mode = g_table_placement.load(std::memory_order_relaxed);
+            if (mode == 2 || (mode == 1 && n_rows <= ltab_resident_teams<NT, TEAMS, 1024>()))
+                return launch_lds_ltab<NT, TEAMS, 1024>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+        }
     }
     const bool planned = long_rows || n_rows > lds_resident_teams<NT, TEAMS, CAP>();
     if (planned) {
@@ -1716,7 +1766,12 @@ static int bpe_encode_launch(const dnatok_bpe_t *t, const uint8_t *bytes, const 
     // less LDS per workgroup means more workgroups per CU
     int rc;
     const int64_t work_len = max_len < p.ext ? max_len : p.ext;    // longest piece the LDS kernel sees
-    if (work_len <= 1024)        rc = run_lds<256, 1, 1024>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    // short rows: a wave per row, four rows to a workgroup (a 256-thread team would leave most of
+    // its lanes without a position, and a row's time is its rounds, not its length)
+    if (work_len <= 256)         rc = run_lds<64, 4, 256>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    else if (work_len <= 384)    rc = run_lds<64, 4, 384>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    else if (work_len <= 512)    rc = run_lds<64, 4, 512>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    else if (work_len <= 1024)   rc = run_lds<256, 1, 1024>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
     else if (work_len <= 1408)   rc = run_lds<256, 1, 1408>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
     else if (work_len <= 1536)   rc = run_lds<256, 1, 1536>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
     else if (work_len <= 2048)   rc = run_lds<256, 1, 2048>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);

@@ -829,6 +829,37 @@ def test_bpe_more_rows_of_about_one_length_than_teams(bpe):
     check_padded(enc, bo, seqs, 128, ref=ref)
 
 
+@pytest.mark.parametrize("longest", [250, 380, 500])
+def test_bpe_many_short_rows_a_wave_each(bpe, longest):
+    """Batches whose rows are at most 256 / 384 / 512 bytes long go to teams of one wave (four rows to a
+    workgroup), more rows than teams through several work counters: every row as the oracle has it,
+    through the plain call, the one that pads, and the one that also writes the single-character ids;
+    a few rows only, empty rows, rows of one length (dealt in order) and ragged ones."""
+    which, enc, bo = bpe
+    say(f"bpe{which} short rows, longest {longest}")
+    rng = random.Random(1000 + longest)
+    rnd = lambda n: "".join(rng.choices("ACGTN", weights=[24, 24, 24, 24, 4], k=n))
+    lut = np.arange(256, dtype=np.int32) + 3
+    lut_dev = torch.from_numpy(lut).to(DEV)
+    batches = [[rnd(rng.randint(0, longest)) for _ in range(9000)],
+               [rnd(rng.randint(longest - 8, longest)) for _ in range(7000)],
+               [rnd(longest), "", rnd(1), rnd(longest - 1), ""],
+               [rnd(rng.randint(1, longest)) for _ in range(300)]]
+    for seqs in batches:
+        b = util.batch_from_strings(seqs)
+        ref = bo.encode_batch(b.data, b.offsets)
+        for r, e in zip(bpe_rows(enc, b), ref):
+            np.testing.assert_array_equal(r, e)
+        check_padded(enc, bo, seqs, 160, ref=ref)
+        data, off = to_dev(b)
+        tok, lengths, cids, _ = enc.encode_with_chars(data, off, int(b.lengths().max()), lut_dev, want_char_mask=False)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(cids[:b.data.size].cpu().numpy(), lut[b.data])
+        tok, lengths = tok.cpu().numpy(), lengths.cpu().numpy()
+        for i, e in enumerate(ref):
+            np.testing.assert_array_equal(tok[b.offsets[i]:b.offsets[i] + lengths[i]], e, err_msg=f"row {i}")
+
+
 def test_bpe_rows_without_a_seam_fall_back_to_the_whole_row_kernel(bpe):
     """Tandem repeats far longer than the chunk overlap: neighbouring chunk runs can stay out
     of phase, no seam is accepted, and the row is redone by the whole-row kernel."""
