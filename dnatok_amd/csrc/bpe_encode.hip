@@ -1757,8 +1757,10 @@ static int bpe_encode_launch(const dnatok_bpe_t *t, const uint8_t *bytes, const 
     }
 
     const bool long_rows = max_len > p.ext;
-    // rows of about one length (the mean at least 3/4 of the longest), none cut: dealt in their given order
-    a.in_order = !long_rows && total >= (max_len * n_rows / 4) * 3 ? 1 : 0;
+    // rows of about one length (the mean at least 3/4 of the longest), none cut: dealt in their given
+    // order; and so are very many short rows of any lengths (sorting 100,000 of them costs the one
+    // workgroup that does it 115 us, their unsorted end at most the time of one row, about 25 us)
+    a.in_order = !long_rows && (total >= (max_len * n_rows / 4) * 3 || (max_len <= 512 && n_rows >= 8192)) ? 1 : 0;
     int chunking = (long_rows && t->monotone) ? 1 : 0;
     // bit 1: the plan kernel writes the chunk entries itself (few rows, few chunks: one launch less)
     if (chunking && n_rows <= kPlanInlineRows && p.max_mc <= kPlanInlineChunks) chunking |= 2;

@@ -841,7 +841,8 @@ def test_bpe_many_short_rows_a_wave_each(bpe, longest):
     rnd = lambda n: "".join(rng.choices("ACGTN", weights=[24, 24, 24, 24, 4], k=n))
     lut = np.arange(256, dtype=np.int32) + 3
     lut_dev = torch.from_numpy(lut).to(DEV)
-    batches = [[rnd(rng.randint(0, longest)) for _ in range(9000)],
+    batches = [[rnd(rng.randint(0, longest)) for _ in range(9000)],       # so many that they are dealt unsorted
+               [rnd(rng.randint(0, longest)) for _ in range(7500)],       # more than teams: the sorted work list
                [rnd(rng.randint(longest - 8, longest)) for _ in range(7000)],
                [rnd(longest), "", rnd(1), rnd(longest - 1), ""],
                [rnd(rng.randint(1, longest)) for _ in range(300)]]
