@@ -766,6 +766,49 @@ def pathological_extra():
     return out
 
 
+def short_reads_extra():
+    """BPE (vocabulary 4096) on batches of short reads, 100 to 300 bp each, padded by the engine: the
+    shape of a sequencing run rather than of the five configurations.  Rows this short go to teams
+    of one wave and are handed out through several work counters; the last 512 rows of every batch
+    are checked against the Hugging Face tokenizer run here."""
+    import torch
+    from dnatok_amd import bpe_vocab, encoders
+    from tests.support import hf_tokenizers as hf
+    with open(hf.bpe_tokenizer_path("4096")) as fh:
+        cfg = json.load(fh)
+    kv = bpe_vocab.KernelVocab(bpe_vocab.split_merges(cfg["model"]["merges"]))
+    vocab = cfg["model"]["vocab"]
+    enc = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv), out_remap=kv.remap_to(vocab, vocab["[UNK]"]))
+    tk = hf.load_bpe_tokenizer("4096")
+    rng = np.random.Generator(np.random.PCG64(1006))
+    out = {}
+    for n_rows in (4096, 20_000, 100_000):
+        lens = rng.integers(100, 301, n_rows)
+        off_h = np.zeros(n_rows + 1, dtype=np.int64)
+        off_h[1:] = np.cumsum(lens)
+        host = rng.choice(np.frombuffer(b"ACGT", dtype=np.uint8), int(off_h[-1]), p=[.295, .205, .205, .295])
+        data, off = _dev(host), _dev(off_h)
+        stride = 128
+        buf = (torch.empty((n_rows, stride), dtype=torch.int32, device="cuda"),
+               torch.empty((n_rows, stride), dtype=torch.uint8, device="cuda"),
+               torch.empty(n_rows, dtype=torch.int32, device="cuda"), torch.empty(1, dtype=torch.int32, device="cuda"))
+
+        class W:
+            def step(self):
+                enc.encode_padded(data, off, 300, stride, vocab["[PAD]"], out=buf)
+        W().step()
+        torch.cuda.synchronize()
+        ln = buf[2].cpu().numpy()
+        assert int(buf[3].item()) == int(ln.max()) <= stride
+        first = n_rows - 512
+        want = hf_live_rows(tk, host[off_h[first]:], off_h[first:] - off_h[first])
+        same_rows([buf[0][first + r, :ln[first + r]].cpu().numpy() for r in range(512)], want, f"short reads, {n_rows} rows")
+        _, dm = time_steps(W(), 50, 10)
+        out[f"{n_rows}_rows"] = {"bases": int(off_h[-1]), "device_us_per_call": dm * 1e3,
+                                 "mbp_per_s": float(off_h[-1]) / (dm * 1e-3) / 1e6}
+    return out
+
+
 def kmer_rows_with_n_extra():
     """The 6-mer encoder on 65,536 rows of 6000 bp that differ only in where they hold N: none, one
     per row (anywhere / at the start: every later step of the row is then written shifted), 32
@@ -890,7 +933,8 @@ def main() -> None:
     ap.add_argument("--config", default="C2", choices=["C1", "C2", "C3", "C4", "C5"])
     ap.add_argument("--per-call", action="store_true", help="time one exact batch instead of the sustained form")
     ap.add_argument("--no-extras", action="store_true")
-    ap.add_argument("--only-extra", default="", choices=["", "merge_table_placement", "pathological", "kmer_rows_with_n"],
+    ap.add_argument("--only-extra", default="", choices=["", "merge_table_placement", "pathological", "kmer_rows_with_n",
+                                                         "short_reads"],
                     help="run only this extra after the headline (for profiling it)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -974,7 +1018,8 @@ def main() -> None:
     if args.only_extra:
         result[args.only_extra] = {"merge_table_placement": merge_table_placement_extra,
                                    "pathological": pathological_extra,
-                                   "kmer_rows_with_n": kmer_rows_with_n_extra}[args.only_extra]()
+                                   "kmer_rows_with_n": kmer_rows_with_n_extra,
+                                   "short_reads": short_reads_extra}[args.only_extra]()
     elif not args.no_extras:
         per_call = {}
         for cfg in ["C1", "C2", "C3", "C4", "C5"]:
@@ -1026,6 +1071,7 @@ def main() -> None:
         result["unpack_2bit"] = unpack_2bit_extra()
         result["device_normalizer"] = device_normalizer_extra()
         result["pathological"] = pathological_extra()
+        result["short_reads"] = short_reads_extra()
         result["merge_table_placement"] = merge_table_placement_extra()
 
     print(json.dumps(result), flush=True)
