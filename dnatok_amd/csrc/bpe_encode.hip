@@ -95,6 +95,10 @@ struct BpeArgs {
     // items a team takes from its work counter at a time, and the counters in use (a power of two,
     // at most kDealers and at most the number of teams: every counter needs a team)
     int32_t grab, dealers;
+    // which part of the work list a launch works through: 0 all of it, 1 all but the class of the
+    // shortest rows, 2 that class alone (a batch of mostly short rows with a few long ones is split
+    // between a launch with 256-thread teams and one with teams of one wave)
+    int32_t part;
 };
 
 typedef int32_t bpe_int4_a4 __attribute__((ext_vector_type(4), aligned(4)));
@@ -813,7 +817,7 @@ constexpr int kDealerStride = 64;         // int32 words between two counters (2
 
 struct BpePlan {                          // device arrays inside the scratch buffer
     int32_t *counts;      // [0] items, [1] chunk items, [3] failed rows, [4 + c] single rows of class c
-    int32_t *deal;        // [kDealers * kDealerStride] the work counters
+    int32_t *deal;        // [2][kDealers * kDealerStride] the work counters (second bank: a launch for the shortest rows alone)
     int32_t *mc_off;      // [n_rows + 1] first chunk slot of a row (multi-chunk rows only)
     int4 *rec;           // [max_mc] a chunk item: {row, chunk of the row, chunks of the row, row length}
     int32_t *single[kSingleClasses];   // [n_rows] each: the rows that are one item, longest class first
@@ -873,7 +877,7 @@ static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t
     size_t o = 0;
     auto take = [&](size_t bytes) { size_t at = o; o = up(o + bytes); return at; };
     const size_t o_counts = take(64);
-    const size_t o_deal = take(4 * (size_t)kDealers * kDealerStride);
+    const size_t o_deal = take(2 * 4 * (size_t)kDealers * kDealerStride);
     const size_t o_mc_off = take(4 * (size_t)(n_rows + 1));
     const size_t o_rec = take(16 * (size_t)p.max_mc);
     size_t o_single[kSingleClasses];
@@ -1011,7 +1015,7 @@ __global__ __launch_bounds__(1024) void bpe_plan_kernel(
             p.rec[c] = make_int4(row, c - first, next - first, s_len[row]);
         }
     }
-    if (threadIdx.x < kDealers) p.deal[threadIdx.x * kDealerStride] = 0;
+    if (threadIdx.x < 2 * kDealers) p.deal[threadIdx.x * kDealerStride] = 0;
     if (threadIdx.x == 0) {
         int32_t items = carry[0];
         for (int q = 0; q < kSingleClasses; ++q) { p.counts[4 + q] = carry[1 + q]; items += carry[1 + q]; }
@@ -1036,7 +1040,7 @@ __global__ void bpe_plan_in_order_kernel(int32_t n_rows, BpePlan p)
         p.counts[3] = 0;
         for (int q = 0; q < kSingleClasses; ++q) p.counts[4 + q] = 0;
     }
-    if (threadIdx.x < kDealers) p.deal[threadIdx.x * kDealerStride] = 0;
+    if (threadIdx.x < 2 * kDealers) p.deal[threadIdx.x * kDealerStride] = 0;
 }
 
 __global__ __launch_bounds__(256) void bpe_expand_kernel(const int64_t *__restrict__ offsets, int64_t n_rows,
@@ -1106,7 +1110,10 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     const LdsPairTable lpt{ltab, ltab + kLdsTabSlots, a.lmul1, a.lmul2};
     __syncthreads();
 
-    const int32_t n_items = PLANNED ? p.counts[0] : n_rows;
+    const int32_t n_shortest = PLANNED ? p.counts[4 + kSingleClasses - 1] : 0;
+    const int32_t n_items = !PLANNED ? n_rows
+                            : (a.part == 2 ? n_shortest : p.counts[0] - (a.part == 1 ? n_shortest : 0));
+    int32_t *const deal = PLANNED ? p.deal + (a.part == 2 ? kDealers * kDealerStride : 0) : nullptr;
     static_assert(PLANNED || !CHUNKS, "chunks come from the work list");
     static_assert(!PADDED || (!CHUNKS && !LTAB), "padded rows: whole rows");
     const int32_t n_mc = CHUNKS ? p.counts[1] : 0;
@@ -1130,7 +1137,7 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
             } else if (PLANNED) {
                 if (n_teams >= n_items) break;       // nothing was left for the counters
                 if (tid == 0)
-                    *next_item = dealt_from + a.dealers * atomicAdd(&p.deal[dealer * kDealerStride], a.grab);
+                    *next_item = dealt_from + a.dealers * atomicAdd(&deal[dealer * kDealerStride], a.grab);
                 team_sync<NT>();
                 item = *next_item;
                 team_sync<NT>();
@@ -1147,6 +1154,8 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
                 row = rc.x; k = rc.y; nc = rc.z;
             } else if (!CHUNKS && a.in_order) {
                 row = item;
+            } else if (!CHUNKS && a.part == 2) {
+                row = p.single[kSingleClasses - 1][item];
             } else {
                 int32_t j = item - n_mc;
                 const int32_t *list = p.single[0];
@@ -1611,6 +1620,26 @@ extern "C" size_t dnatok_bpe_scratch_bytes(const dnatok_bpe_t *t, int64_t n_rows
 
 namespace {
 
+// Longest row (negative lengths count as 0) by one workgroup: where no tree of atomics carries it.
+__global__ __launch_bounds__(1024) void bpe_longest_kernel(const int32_t *__restrict__ lengths, int64_t n_rows,
+                                                           int32_t *__restrict__ longest)
+{
+    __shared__ uint32_t red[16];
+    uint32_t m = 0;
+    for (int64_t i = threadIdx.x; i < n_rows; i += 1024) {
+        const int32_t v = lengths[i];
+        m = v > 0 && (uint32_t)v > m ? (uint32_t)v : m;
+    }
+    m = wave_max_u32(m);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t all = 0;
+        for (int w = 0; w < 16; ++w) all = all > red[w] ? all : red[w];
+        *longest = (int32_t)all;
+    }
+}
+
 template <int NT, int TEAMS, int CAP>
 constexpr size_t lds_bytes()
 {
@@ -1703,8 +1732,9 @@ int launch_lds_ltab(const BpeArgs &a, const uint8_t *bytes, const int64_t *offse
 // (16 x 1024 rows of 1 KB: 0.60 ms with fixed shares, 0.46 ms dealt).  A batch of at most one row
 // per team needs neither list nor counter.
 template <int NT, int TEAMS, int CAP>
-int run_lds(bool long_rows, int chunking, const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets,
-            const BpePlan &p, int64_t n_rows, int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
+int run_lds_part(bool long_rows, int chunking, bool force_plan, const BpeArgs &a, const uint8_t *bytes,
+                 const int64_t *offsets, const BpePlan &p, int64_t n_rows, int32_t *tok_tmp, int32_t *lengths,
+                 hipStream_t s)
 {
     if constexpr (CAP == 1024) {
         if (!long_rows && a.ltab && !a.char_ids && !a.pad_ids) {
@@ -1713,7 +1743,7 @@ int run_lds(bool long_rows, int chunking, const BpeArgs &a, const uint8_t *bytes
                 return launch_lds_ltab<NT, TEAMS, 1024>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
         }
     }
-    const bool planned = long_rows || n_rows > lds_resident_teams<NT, TEAMS, CAP>();
+    const bool planned = long_rows || force_plan || n_rows > lds_resident_teams<NT, TEAMS, CAP>();
     if (planned) {
         if (a.in_order) {                            // (no row is cut)
             bpe_plan_in_order_kernel<<<1, 64, 0, s>>>((int32_t)n_rows, p);
@@ -1738,6 +1768,26 @@ int run_lds(bool long_rows, int chunking, const BpeArgs &a, const uint8_t *bytes
     if (a.pad_ids) return launch_lds_as<NT, TEAMS, CAP, false, false, false, true>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
     if (a.char_ids) return launch_lds_as<NT, TEAMS, CAP, false, true>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
     return launch_lds_as<NT, TEAMS, CAP, false>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+}
+
+template <int NT, int TEAMS, int CAP>
+int run_lds(bool long_rows, int chunking, bool split, const BpeArgs &a_in, const uint8_t *bytes, const int64_t *offsets,
+            const BpePlan &p, int64_t n_rows, int32_t *tok_tmp, int32_t *lengths, hipStream_t s)
+{
+    // split: the rows of the shortest class (at most a quarter of an extended chunk: 512 bytes) get
+    // a launch of their own with teams of one wave, after the launch for everything else
+    BpeArgs a = a_in;
+    a.part = split ? 1 : 0;
+    if (split) {
+        BpeArgs b = a_in;
+        b.part = 2;
+        const int rc = run_lds_part<NT, TEAMS, CAP>(long_rows, chunking, true, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+        if (rc) return rc;
+        if (b.pad_ids) return launch_lds_as<64, 4, 512, true, false, false, true>(b, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+        if (b.char_ids) return launch_lds_as<64, 4, 512, true, true, false>(b, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+        return launch_lds_as<64, 4, 512, true, false, false>(b, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    }
+    return run_lds_part<NT, TEAMS, CAP>(long_rows, chunking, false, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
 }
 
 }  // namespace
@@ -1768,16 +1818,26 @@ static int bpe_encode_launch(const dnatok_bpe_t *t, const uint8_t *bytes, const 
     // less LDS per workgroup means more workgroups per CU
     int rc;
     const int64_t work_len = max_len < p.ext ? max_len : p.ext;    // longest piece the LDS kernel sees
+    // Mostly short rows with some long ones among them (the mean at most 384 bytes, the longest above
+    // 512): the short ones, which a 256-thread team would take as long over as over a row of 1 KB,
+    // get a launch of their own.  The two launches cannot both carry the longest row up the one
+    // tree: it is taken from the lengths afterwards.
+    const bool split = work_len > 512 && n_rows >= 1024 && total / n_rows <= 384 && p.ext / 4 <= 512;
+    int32_t *const longest_after = split && a.max_tree ? a.longest : nullptr;
+    if (split) {
+        a.in_order = 0;
+        a.max_tree = nullptr;
+    }
     // short rows: a wave per row, four rows to a workgroup (a 256-thread team would leave most of
     // its lanes without a position, and a row's time is its rounds, not its length)
-    if (work_len <= 256)         rc = run_lds<64, 4, 256>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
-    else if (work_len <= 384)    rc = run_lds<64, 4, 384>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
-    else if (work_len <= 512)    rc = run_lds<64, 4, 512>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
-    else if (work_len <= 1024)   rc = run_lds<256, 1, 1024>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
-    else if (work_len <= 1408)   rc = run_lds<256, 1, 1408>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
-    else if (work_len <= 1536)   rc = run_lds<256, 1, 1536>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
-    else if (work_len <= 2048)   rc = run_lds<256, 1, 2048>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
-    else                         rc = run_lds<256, 1, kLdsCap>(long_rows, chunking, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    if (work_len <= 256)         rc = run_lds<64, 4, 256>(long_rows, chunking, split, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    else if (work_len <= 384)    rc = run_lds<64, 4, 384>(long_rows, chunking, split, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    else if (work_len <= 512)    rc = run_lds<64, 4, 512>(long_rows, chunking, split, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    else if (work_len <= 1024)   rc = run_lds<256, 1, 1024>(long_rows, chunking, split, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    else if (work_len <= 1408)   rc = run_lds<256, 1, 1408>(long_rows, chunking, split, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    else if (work_len <= 1536)   rc = run_lds<256, 1, 1536>(long_rows, chunking, split, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    else if (work_len <= 2048)   rc = run_lds<256, 1, 2048>(long_rows, chunking, split, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
+    else                         rc = run_lds<256, 1, kLdsCap>(long_rows, chunking, split, a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
     if (rc) return rc;
     if (long_rows) {
         if (chunking) {
@@ -1789,6 +1849,10 @@ static int bpe_encode_launch(const dnatok_bpe_t *t, const uint8_t *bytes, const 
         }
         bpe_long_kernel<kLongThreads><<<p.n_slabs, kLongThreads, 0, s>>>(a, bytes, offsets, n_rows, max_len, p,
                                                                         tok_tmp, lengths);
+        DNATOK_HIP_TRY(hipGetLastError());
+    }
+    if (longest_after) {
+        bpe_longest_kernel<<<1, 1024, 0, s>>>(lengths, n_rows, longest_after);
         DNATOK_HIP_TRY(hipGetLastError());
     }
     return DNATOK_OK;
@@ -1841,26 +1905,6 @@ extern "C" int dnatok_bpe_encode_with_chars(const dnatok_bpe_t *t, const uint8_t
     const BpePlan p = make_plan((uint8_t *)scratch, n_rows, max_len, total);
     return bpe_encode_launch(t, bytes, offsets, n_rows, max_len, total, p, tok_tmp, lengths, (hipStream_t)stream, char_lut,
                              char_ids, char_mask);
-}
-
-// Longest row (negative lengths count as 0) by one workgroup: where no tree of atomics carries it.
-__global__ __launch_bounds__(1024) void bpe_longest_kernel(const int32_t *__restrict__ lengths, int64_t n_rows,
-                                                           int32_t *__restrict__ longest)
-{
-    __shared__ uint32_t red[16];
-    uint32_t m = 0;
-    for (int64_t i = threadIdx.x; i < n_rows; i += 1024) {
-        const int32_t v = lengths[i];
-        m = v > 0 && (uint32_t)v > m ? (uint32_t)v : m;
-    }
-    m = wave_max_u32(m);
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        uint32_t all = 0;
-        for (int w = 0; w < 16; ++w) all = all > red[w] ? all : red[w];
-        *longest = (int32_t)all;
-    }
 }
 
 extern "C" int64_t dnatok_bpe_padded_direct_max(void)

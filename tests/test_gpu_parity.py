@@ -861,6 +861,39 @@ def test_bpe_many_short_rows_a_wave_each(bpe, longest):
             np.testing.assert_array_equal(tok[b.offsets[i]:b.offsets[i] + lengths[i]], e, err_msg=f"row {i}")
 
 
+@pytest.mark.parametrize("long_ones", ["up to 1 KB", "up to 2 KB", "cut into chunks"])
+def test_bpe_mostly_short_rows_with_some_long_ones(bpe, long_ones):
+    """A batch of mostly short rows with a few long ones among them is split between two launches (the
+    shortest class of the work list to teams of one wave, the rest to 256-thread teams): every row as
+    the oracle has it, through the plain call, the one that pads (whose longest row then comes from
+    the lengths) and the one that also writes the single-character ids."""
+    which, enc, bo = bpe
+    say(f"bpe{which} mostly short rows, long ones {long_ones}")
+    rng = random.Random(77)
+    rnd = lambda n: "".join(rng.choices("ACGTN", weights=[24, 24, 24, 24, 4], k=n))
+    seqs = [rnd(rng.randint(0, 320)) for _ in range(6000)]
+    extra = {"up to 1 KB": [rnd(rng.randint(513, 1000)) for _ in range(40)],
+             "up to 2 KB": [rnd(rng.randint(400, 2048)) for _ in range(60)],
+             "cut into chunks": [rnd(rng.randint(400, 2048)) for _ in range(30)] + [rnd(5000), rnd(20_001), "A" * 7000]}[long_ones]
+    for e in extra:
+        seqs.insert(rng.randint(0, len(seqs)), e)
+    b = util.batch_from_strings(seqs)
+    ref = bo.encode_batch(b.data, b.offsets)
+    for r, e in zip(bpe_rows(enc, b), ref):
+        np.testing.assert_array_equal(r, e)
+    check_padded(enc, bo, seqs, 520 if long_ones != "cut into chunks" else 6000, ref=ref)
+    check_padded(enc, bo, seqs, 96, want_longest=False, ref=ref)
+    lut = np.arange(256, dtype=np.int32) + 3
+    data, off = to_dev(b)
+    tok, lengths, cids, _ = enc.encode_with_chars(data, off, int(b.lengths().max()), torch.from_numpy(lut).to(DEV),
+                                                  want_char_mask=False)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(cids[:b.data.size].cpu().numpy(), lut[b.data])
+    tok, lengths = tok.cpu().numpy(), lengths.cpu().numpy()
+    for i, e in enumerate(ref):
+        np.testing.assert_array_equal(tok[b.offsets[i]:b.offsets[i] + lengths[i]], e, err_msg=f"row {i}")
+
+
 def test_bpe_rows_without_a_seam_fall_back_to_the_whole_row_kernel(bpe):
     """Tandem repeats far longer than the chunk overlap: neighbouring chunk runs can stay out
     of phase, no seam is accepted, and the row is redone by the whole-row kernel."""
