@@ -806,7 +806,41 @@ def short_reads_extra():
         _, dm = time_steps(W(), 50, 10)
         out[f"{n_rows}_rows"] = {"bases": int(off_h[-1]), "device_us_per_call": dm * 1e3,
                                  "mbp_per_s": float(off_h[-1]) / (dm * 1e-3) / 1e6}
+        if n_rows == 100_000:
+            out["6mer_100000_rows"] = short_reads_kmer(host, off_h, data, off)
     return out
+
+
+def short_reads_kmer(host, off_h, data, off) -> dict:
+    """The same reads through the 6-mer encoder (rows 128 cells apart, padded to the longest),
+    the last 512 rows checked against the Hugging Face tokenizer run here."""
+    import torch
+    from dnatok_amd import encoders, kmer_tables
+    from tests.support import hf_tokenizers as hf
+    vocab = hf.kmer_vocab(6)
+    t = kmer_tables.tables_from_vocab(vocab, 6, vocab["<unk>"])
+    enc = encoders.KmerEncoder(6, t.digit, t.kmer_lut, t.single, vocab["<pad>"], vocab["<unk>"],
+                               t.exp_off, t.exp_len, t.exp_flat)
+    n_rows = off_h.size - 1
+    buf = (torch.empty((n_rows, 128), dtype=torch.int32, device="cuda"), torch.empty((n_rows, 128), dtype=torch.uint8, device="cuda"),
+           torch.empty(n_rows, dtype=torch.int32, device="cuda"), torch.empty(n_rows, dtype=torch.int32, device="cuda"),
+           torch.empty(1, dtype=torch.int32, device="cuda"))
+
+    class W:
+        def step(self):
+            enc.encode_padded(data, off, 128, fill_to=0, width_guess=64, out=buf)
+    W().step()
+    torch.cuda.synchronize()
+    ln = buf[2].cpu().numpy()
+    width = int(buf[4].item())
+    assert width == int(ln.max()) and int(buf[3].abs().sum().item()) == 0
+    first = n_rows - 512
+    want = hf_live_rows(hf.build_kmer_tokenizer(6), host[off_h[first]:], off_h[first:] - off_h[first])
+    same_rows([buf[0][first + r, :ln[first + r]].cpu().numpy() for r in range(512)], want, "short reads, 6-mer")
+    _, dm = time_steps(W(), 50, 10)
+    by = int(off_h[-1]) + 5 * n_rows * width + 4 * n_rows
+    return {"bases": int(off_h[-1]), "device_us_per_call": dm * 1e3, "mbp_per_s": float(off_h[-1]) / (dm * 1e-3) / 1e6,
+            "hbm_frac": by / (dm * 1e-3) / 1e9 / HBM_PEAK_GBS}
 
 
 def kmer_rows_with_n_extra():
