@@ -686,6 +686,257 @@ __global__ __launch_bounds__(kRowsThreads) void kmer_rows_kernel(
     }
 }
 
+// ---- short rows: sixteen lanes per row -----------------------------------------------------------
+//
+// A read of a few hundred bases is one step of kmer_rows_kernel in which a sixth of the lanes
+// take part, and the row's fixed work is then all there is.  Here a row belongs to 16 lanes (four
+// rows to a wave, sixteen to a workgroup) that walk it in steps of 64 windows: the digits by
+// arithmetic on the bytes (the plain digit table only, see ARITH above), the positions by a scan
+// over the 16 lanes (DPP row operations stay inside them), the tokens stored by the lanes
+// themselves, a 16-byte store for a lane of four plain windows on a 16-byte boundary and single
+// cells otherwise: no staging, no LDS beyond the tables.  For tables that spell every window
+// without an id by its characters (CHARS above) and row strides of at most kGroupsMaxStride cells.
+constexpr int kGroupThreads = 256;
+constexpr int kGroupsMaxStride = 256;
+
+// inclusive sum over the 16 lanes of a DPP row
+__device__ __forceinline__ uint32_t row16_inclusive_sum(uint32_t v)
+{
+    v += dpp_row_shr_zero<1>(v);
+    v += dpp_row_shr_zero<2>(v);
+    v += dpp_row_shr_zero<4>(v);
+    v += dpp_row_shr_zero<8>(v);
+    return v;
+}
+
+// the value of the last of a lane's 16
+__device__ __forceinline__ uint32_t row16_last(uint32_t v)
+{
+    const int src = (int)((threadIdx.x & 63) | 15);
+    return (uint32_t)__builtin_amdgcn_ds_bpermute(src << 2, (int)v);
+}
+
+template <int K, bool LUT4_LDS, bool HAS_MASK>
+__global__ __launch_bounds__(kGroupThreads) void kmer_groups_kernel(
+    KmerArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
+    int64_t n_rows, int64_t t_cap, int64_t fill_to, int32_t *__restrict__ ids,
+    uint8_t *__restrict__ mask, int32_t *__restrict__ lengths, int32_t *__restrict__ status,
+    int32_t *__restrict__ max_len, MaxRef mref, int publish)
+{
+    constexpr uint32_t POW4 = 1u << (2 * K);
+    constexpr int kLaneBytes = kUnitsPerLane * K;                 // bytes of a lane's four windows
+    __shared__ int32_t s_single[256];
+    __shared__ int32_t s_spell[256];
+    __shared__ int32_t s_lut4[LUT4_LDS ? POW4 : 1];
+    __shared__ uint32_t s_wave_max[kGroupThreads / 64];
+    for (int i = threadIdx.x; i < 256; i += kGroupThreads) {
+        const int d = a.digit[i];
+        s_single[i] = a.single[i];
+        s_spell[i] = a.single[(int)"ACGTN"[d < 0 || d > 4 ? 4 : d]];
+    }
+    if (LUT4_LDS)
+        for (uint32_t i = threadIdx.x; i < POW4; i += kGroupThreads) s_lut4[i] = a.lut4r[i];
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63, gl = lane & 15;
+    const int cap = (int)t_cap;                                   // (at most kGroupsMaxStride)
+    const int fill = fill_to > cap ? cap : (int)fill_to;
+    const int64_t group = ((int64_t)blockIdx.x * kGroupThreads + threadIdx.x) >> 4;
+    const int64_t n_groups = (int64_t)gridDim.x * (kGroupThreads / 16);
+    const unsigned long long slot_gen = mref.slot ? mref.slot[1] : 0ull;
+    const int64_t total = offsets[n_rows];
+    uint32_t group_max = 0;
+
+    // every group of the wave makes the same number of trips (a group without a row idles), so
+    // that the wave's loads can share one descriptor per trip
+    const int64_t wave_first = group - (lane >> 4);
+    for (int64_t row0 = wave_first; row0 < n_rows; row0 += n_groups) {
+        const int64_t row = row0 + (lane >> 4);
+        const bool have = row < n_rows;
+        const int64_t start = have ? offsets[row] : 0;
+        const int len = have ? (int)(offsets[row + 1] - start) : 0;
+        const int full = len / K, tail = len - full * K;
+        const int n_slots = full + (tail ? 1 : 0);                // windows, and one slot for the trailing characters
+        int32_t *out = ids + row * t_cap;
+        uint8_t *mout = HAS_MASK ? mask + row * t_cap : nullptr;
+        int running = 0;
+        bool foreign_seen = false;
+
+        const int steps = (n_slots + 63) >> 6;
+        const int wave_steps = (int)wave_max_u32((uint32_t)steps);        // (wave-uniform loop: the loads are wave-wide)
+        for (int st = 0; st < wave_steps; ++st) {
+            const int wb = st * 64 + gl * kUnitsPerLane;          // the lane's first window
+            // the lane's 4K bytes, a word at a time; what lies past the row's end (the next rows'
+            // bytes) is read and ignored, what lies past the end of the batch is not read
+            const int64_t pos = start + (int64_t)wb * K;
+            uint32_t w[K];
+#pragma unroll
+            for (int i = 0; i < K; ++i) {
+                const int64_t at = pos + 4 * i;
+                uint32_t v = 0;
+                if (wb < n_slots) {
+                    if (at + 4 <= total) {
+                        v = *reinterpret_cast<const u32_a1 *>(bytes + at);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (at + e < total) v |= (uint32_t)bytes[at + e] << (8 * e);
+                    }
+                }
+                w[i] = v;
+            }
+            // digits, codes and the bytes that are no base, as in kmer_rows_kernel<..., ARITH>
+            uint32_t odd[K], c8[K];
+#pragma unroll
+            for (int i = 0; i < K; ++i) {
+                const uint32_t d = w[i] & 0x06060606u;
+                odd[i] = (w[i] ^ __builtin_amdgcn_perm(0x00470054u, 0x00430041u, d)) & a.fold;
+                const uint32_t x1 = (d << 6) | d, x2 = (x1 << 12) | x1;
+                c8[i] = (x2 >> 19) & 255u;
+            }
+            uint32_t str[(K + 3) / 4 + 1];
+#pragma unroll
+            for (int q = 0; q < (K + 3) / 4 + 1; ++q) {
+                uint32_t v = 0;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (4 * q + e < K) v |= c8[4 * q + e] << (8 * e);
+                str[q] = v;
+            }
+            // per slot: its token count, and for a plain window its id
+            int32_t t[kUnitsPerLane];
+            uint32_t cnt[kUnitsPerLane], lane_cnt = 0;
+            bool spelled_any = false;
+#pragma unroll
+            for (int j = 0; j < kUnitsPerLane; ++j) {
+                const int bit = 2 * K * j;
+                const uint64_t two = ((uint64_t)str[(bit >> 5) + 1] << 32) | str[bit >> 5];
+                const uint32_t code = (uint32_t)(two >> (bit & 31)) & (POW4 - 1);
+                t[j] = LUT4_LDS ? s_lut4[code] : a.lut4r[code];
+                uint32_t hit = 0;
+#pragma unroll
+                for (int i = 0; i < K; ++i) {
+                    const int bi = j * K + i;
+                    hit |= odd[bi >> 2] & (0xFFu << (8 * (bi & 3)));
+                }
+                const int slot = wb + j;
+                uint32_t c = 0;
+                if (slot < full) {
+                    c = (hit == 0 && t[j] >= 0) ? 1u : (uint32_t)K;
+                    if (c != 1u) { t[j] = -1; spelled_any = true; }
+                } else if (slot == full && tail) {
+                    c = (uint32_t)tail;
+                    t[j] = -2;                                     // the trailing characters
+                }
+                cnt[j] = c;
+                lane_cnt += c;
+            }
+            // a byte of a window (not of the trailing characters) that is neither a base nor N: the
+            // row is flagged
+            if (spelled_any) {
+                const int in_windows = full - wb < kUnitsPerLane ? (full - wb) * K : kLaneBytes;     // bytes of whole windows
+                uint32_t f = 0;
+#pragma unroll
+                for (int i = 0; i < K; ++i) {
+                    const uint32_t sel = (w[i] >> 1) & 0x07070707u;               // A 0, C 1, T 2, G 3, N 7
+                    const int nb = in_windows - 4 * i;
+                    const uint32_t m = nb >= 4 ? 0xFFFFFFFFu : (nb <= 0 ? 0u : ((1u << (8 * nb)) - 1u));
+                    f |= (w[i] ^ __builtin_amdgcn_perm(0x4E000000u, 0x47544341u, sel)) & m;
+                }
+                if (f & a.fold) foreign_seen = true;
+            }
+            const uint32_t inc = row16_inclusive_sum(lane_cnt);
+            const uint32_t step_total = row16_last(inc);
+            uint32_t s = (uint32_t)running + inc - lane_cnt;      // cell of the lane's first token
+
+            auto byte_of = [&](int bi) -> uint32_t { return (w[bi >> 2] >> (8 * (bi & 3))) & 255u; };
+            if (lane_cnt == kUnitsPerLane && cnt[0] == 1 && cnt[1] == 1 && cnt[2] == 1 && cnt[3] == 1 &&
+                (t[0] | t[1] | t[2] | t[3]) >= 0 && (s & 3u) == 0 && (int)s + 4 <= cap && ((reinterpret_cast<uintptr_t>(out) & 15) == 0)) {
+                const int4v x = {t[0], t[1], t[2], t[3]};
+                __builtin_nontemporal_store(x, reinterpret_cast<int4v *>(out + s));
+            } else if (lane_cnt) {
+#pragma unroll
+                for (int j = 0; j < kUnitsPerLane; ++j) {
+                    if (cnt[j] == 0) continue;
+                    if (t[j] >= 0) {
+                        if ((int)s < cap) out[s] = t[j];
+                        s += 1;
+                    } else if (t[j] == -1) {
+#pragma unroll
+                        for (int i = 0; i < K; ++i)
+                            if ((int)s + i < cap) out[s + i] = s_spell[byte_of(j * K + i)];
+                        s += K;
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < K - 1; ++i)
+                            if (i < tail && (int)s + i < cap) out[s + i] = s_single[byte_of(j * K + i)];
+                        s += (uint32_t)tail;
+                    }
+                }
+            }
+            running += (int)step_total;
+        }
+
+        // the row's end: mask, padding, length and status, by the row's 16 lanes
+        const int stored = running < cap ? running : cap;
+        const int upto = fill > stored ? fill : stored;
+        if (HAS_MASK && have) {
+            for (int c = 4 * gl; c < upto; c += 64) {
+                const int ones = stored - c;                       // cells of this word that hold a token
+                const uint32_t v = ones >= 4 ? 0x01010101u : (ones <= 0 ? 0u : (0x01010101u >> (8 * (4 - ones))));
+                if (c + 4 <= upto && ((reinterpret_cast<uintptr_t>(mout) & 3) == 0)) {
+                    *reinterpret_cast<uint32_t *>(mout + c) = v;
+                } else {
+                    for (int e = 0; e < 4; ++e)
+                        if (c + e < upto) mout[c + e] = (uint8_t)((v >> (8 * e)) & 1u);
+                }
+            }
+        }
+        if (have) {
+            for (int c = (stored & ~3) + 4 * gl; c < fill; c += 64) {
+                if (c >= stored && c + 4 <= fill && ((reinterpret_cast<uintptr_t>(out) & 15) == 0)) {
+                    const int4v x = {a.pad_id, a.pad_id, a.pad_id, a.pad_id};
+                    __builtin_nontemporal_store(x, reinterpret_cast<int4v *>(out + c));
+                } else {
+                    for (int e = 0; e < 4; ++e)
+                        if (c + e >= stored && c + e < fill) out[c + e] = a.pad_id;
+                }
+            }
+        }
+        const uint64_t bad = __ballot(foreign_seen);
+        if (have && gl == 0) {
+            lengths[row] = running;
+            if (status) {
+                int32_t v = ((bad >> (lane & 48)) & 0xFFFFull) ? DNATOK_ROW_INVALID_BYTE : 0;
+                if (running > cap) v |= DNATOK_ROW_TRUNCATED;
+                status[row] = v;
+            }
+        }
+        if (have && (uint32_t)stored > group_max) group_max = (uint32_t)stored;
+    }
+
+    // the longest row: as kmer_rows_kernel reports it
+    const uint32_t wmax = wave_max_u32(group_max);
+    if (publish) {
+        if (lane == 0) s_wave_max[threadIdx.x >> 6] = wmax;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            uint32_t m = 0;
+#pragma unroll
+            for (int q = 0; q < kGroupThreads / 64; ++q) m = s_wave_max[q] > m ? s_wave_max[q] : m;
+            publish_max(mref.tree, m, max_len);
+        }
+        return;
+    }
+    if (mref.slot) {
+        const unsigned long long v = (slot_gen << 32) | (unsigned long long)wmax;
+        const bool first_wave = blockIdx.x == 0 && threadIdx.x < 64;
+        if (lane == 0 && (wmax > 0 || first_wave) && __builtin_nontemporal_load(mref.slot) < v) atomicMax(mref.slot, v);
+    } else if (max_len && lane == 0 && wmax > 0 && (uint32_t)__builtin_nontemporal_load(max_len) < wmax) {
+        atomicMax(max_len, (int32_t)wmax);
+    }
+}
+
 // ---- few rows: a workgroup per row ---------------------------------------------------------------
 //
 // With fewer rows than workgroups fit the chip (one 256-row batch), a wave per row leaves most of
@@ -1288,6 +1539,37 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
     constexpr int64_t kTightStride = 256;
     const bool tight = to_longest && mref.slot && guess > 0 && t_cap - guess <= kTightStride && t_cap < 0xFFFF;
     bool padded_in_kernel = false;
+    // short rows (a row stride of at most kGroupsMaxStride cells says so), the plain digit table,
+    // every window without an id spelled by its characters: sixteen lanes per row
+    if (t->arith && t->chars_mode && t_cap > 0 && t_cap <= kGroupsMaxStride && (t_cap & 3) == 0 && (!to_longest || tight)) {
+#define GROUPS2(KK, L, M)                                                                         \
+    do {                                                                                          \
+        static const int resident = resident_workgroups(kmer_groups_kernel<KK, L, M>, kGroupThreads, 0, 8); \
+        int64_t grid = (n_rows + kGroupThreads / 16 - 1) / (kGroupThreads / 16);                  \
+        if (grid > resident) grid = resident;                                                     \
+        if (grid > kTreeRows) grid = kTreeRows;                                                   \
+        kmer_groups_kernel<KK, L, M><<<(int)grid, kGroupThreads, 0, s>>>(                         \
+            a, bytes, offsets, n_rows, t_cap, tight ? t_cap : fill_to, ids, mask, lengths, status, max_len, mref, \
+            tight ? 1 : 0);                                                                       \
+    } while (0)
+#define GROUPS(KK, L)                                                                             \
+    do {                                                                                          \
+        if (mask) GROUPS2(KK, L, true); else GROUPS2(KK, L, false);                               \
+    } while (0)
+        switch (t->k) {
+            case 2: GROUPS(2, true); break;
+            case 3: GROUPS(3, true); break;
+            case 4: GROUPS(4, true); break;
+            case 5: GROUPS(5, true); break;
+            case 6: GROUPS(6, true); break;
+            case 7: GROUPS(7, false); break;
+            default: GROUPS(8, false); break;
+        }
+#undef GROUPS
+#undef GROUPS2
+        DNATOK_HIP_TRY(hipGetLastError());
+        return DNATOK_OK;
+    }
 #define LAUNCH3(KK, L, C, M) \
     do {                                                                                          \
         if (t->arith) LAUNCH4(KK, L, C, M, true); else LAUNCH4(KK, L, C, M, false);               \

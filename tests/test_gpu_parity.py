@@ -589,6 +589,53 @@ def test_kmer_digit_tables_of_other_forms(kmer_kernel_choice, k, form):
     np.testing.assert_array_equal(mask[:, :m].cpu().numpy(), emask)
 
 
+@pytest.mark.parametrize("k", [2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("fold", [False, True])
+def test_kmer_short_rows_sixteen_lanes_each(k, fold):
+    """Row strides of at most 256 cells send a batch to the kernel that gives a row sixteen lanes:
+    reads of a few hundred bases with N, lower case (a table that folds the case, and one that does
+    not), foreign bytes, every tail length, empty rows, rows of more than one step of 64 windows and
+    rows cut by the stride; padded to a fixed width, to the longest row with a guess (one launch), and
+    to the longest row without one (the wave-per-row kernel), all against the oracle."""
+    say(f"kmer short rows k={k} fold={fold}")
+    vocab = hf.kmer_vocab(k)
+    t = kmer_tables.tables_from_vocab(vocab, k, 0)
+    digit = kmer_tables.digit_table(fold_case=fold)
+    single = t.single.copy()
+    for ch in "acgtn":
+        single[ord(ch)] = single[ord(ch.upper())] if fold else 0
+    enc = encoders.KmerEncoder(k, digit, t.kmer_lut, single, pad_id=1, missing_id=0,
+                               exp_off=t.exp_off, exp_len=t.exp_len, exp_flat=t.exp_flat)
+    ot = O.KmerTables(k, digit, t.kmer_lut, t.exp_off, t.exp_len, t.exp_flat, single, 0)
+    rng = np.random.default_rng(40 + k)
+    letters = list("ACGTNacgtx")
+    p = [.22, .22, .22, .22, .03, .02, .02, .02, .02, .01]
+    strings = ["".join(rng.choice(letters, p=p, size=n)) for n in rng.integers(0, 64 * k + 40, size=3000)]
+    strings[:8] = ["", "A", "ACGT"[:k - 1], "ACGTACGT"[:k], "N" * (3 * k + 1), "ACGT" * 400, "x" * 50, "ACGTN" * 90]
+    strings += ["".join(rng.choice(list("ACGT"), size=n)) for n in rng.integers(100, 301, size=2000)]
+    b = util.batch_from_strings(strings)
+    data, off = to_dev(b)
+    erows, estatus = O.kmer_encode(ot, b.data, b.offsets)
+    elen = np.array([r.size for r in erows])
+    for cap in (64, 128, 256):
+        for fill_to, guess in ((cap, 0), (0, cap - 7), (0, 0)):
+            ids, mask, lengths, status, max_len = enc.encode_padded(data, off, cap, fill_to=fill_to, width_guess=guess)
+            torch.cuda.synchronize()
+            np.testing.assert_array_equal(lengths.cpu().numpy(), elen)
+            st = status.cpu().numpy()
+            np.testing.assert_array_equal(st & 3, estatus)
+            np.testing.assert_array_equal((st & 4) != 0, elen > cap)
+            width = fill_to if fill_to else min(cap, int(elen.max()))
+            assert int(max_len.item()) == min(cap, int(elen.max()))
+            eids, emask = O.pad_rows(erows, 1, width)
+            np.testing.assert_array_equal(ids[:, :width].cpu().numpy(), eids)
+            np.testing.assert_array_equal(mask[:, :width].cpu().numpy(), emask)
+    ids, mask, lengths, status, max_len = enc.encode_padded(data, off, 128, fill_to=128, want_mask=False)
+    torch.cuda.synchronize()
+    assert mask is None
+    np.testing.assert_array_equal(ids.cpu().numpy(), O.pad_rows(erows, 1, 128)[0])
+
+
 @both_kmer_kernels
 def test_kmer_missing_windows_without_expansion(kmer_kernel_choice):
     say("kmer missing windows")
