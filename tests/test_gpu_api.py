@@ -291,6 +291,23 @@ def test_kmer_stream_of_batches_with_a_much_wider_one_in_between():
         assert torch.equal(h.encode_batch_to_ids(seqs), want)
 
 
+def test_kmer_stream_of_batches_of_short_reads():
+    """Batches of reads of 100-300 bases: from the second batch on the rows lie a guess apart (at most
+    256 cells), which sends them to the k-mer kernel for short rows; every batch as the tokenizer
+    has it, a row with a foreign byte (which goes back to the tokenizer) included."""
+    tok = MockKmerTokenizer(4)
+    h = DNATok(RecordingEmbedder(tok))
+    h.discover()
+    assert h.kmer_k == 4
+    rng = random.Random(12)
+    for batch in range(5):
+        seqs = ["".join(rng.choices("ACGTN", weights=[24, 24, 24, 24, 4], k=rng.randint(100, 300))) for _ in range(3000)]
+        if batch == 3:
+            seqs[7] = seqs[7][:50] + "x" + seqs[7][51:]
+        want = tok(seqs, padding=True, return_tensors="pt")["input_ids"]
+        assert torch.equal(h.encode_batch_to_ids(seqs), want), batch
+
+
 def test_kmer_multi_token_windows_follow_the_tokenizer():
     tok = FakeKmerTokenizer(3)
     emb = RecordingEmbedder(tok, 256)
