@@ -697,7 +697,7 @@ __global__ __launch_bounds__(kRowsThreads) void kmer_rows_kernel(
 // cells otherwise: no staging, no LDS beyond the tables.  For tables that spell every window
 // without an id by its characters (CHARS above) and row strides of at most kGroupsMaxStride cells.
 constexpr int kGroupThreads = 256;
-constexpr int kGroupsMaxStride = 256;
+constexpr int kGroupsMaxStride = 384;
 
 // inclusive sum over the 16 lanes of a DPP row
 __device__ __forceinline__ uint32_t row16_inclusive_sum(uint32_t v)

@@ -293,7 +293,7 @@ def test_kmer_stream_of_batches_with_a_much_wider_one_in_between():
 
 def test_kmer_stream_of_batches_of_short_reads():
     """Batches of reads of 100-300 bases: from the second batch on the rows lie a guess apart (at most
-    256 cells), which sends them to the k-mer kernel for short rows; every batch as the tokenizer
+    384 cells), which sends them to the k-mer kernel for short rows; every batch as the tokenizer
     has it, a row with a foreign byte (which goes back to the tokenizer) included."""
     tok = MockKmerTokenizer(4)
     h = DNATok(RecordingEmbedder(tok))

@@ -592,7 +592,7 @@ def test_kmer_digit_tables_of_other_forms(kmer_kernel_choice, k, form):
 @pytest.mark.parametrize("k", [2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("fold", [False, True])
 def test_kmer_short_rows_sixteen_lanes_each(k, fold):
-    """Row strides of at most 256 cells send a batch to the kernel that gives a row sixteen lanes:
+    """Row strides of at most 384 cells send a batch to the kernel that gives a row sixteen lanes:
     reads of a few hundred bases with N, lower case (a table that folds the case, and one that does
     not), foreign bytes, every tail length, empty rows, rows of more than one step of 64 windows and
     rows cut by the stride; padded to a fixed width, to the longest row with a guess (one launch), and
@@ -617,7 +617,7 @@ def test_kmer_short_rows_sixteen_lanes_each(k, fold):
     data, off = to_dev(b)
     erows, estatus = O.kmer_encode(ot, b.data, b.offsets)
     elen = np.array([r.size for r in erows])
-    for cap in (64, 128, 256):
+    for cap in (64, 128, 384):
         for fill_to, guess in ((cap, 0), (0, cap - 7), (0, 0)):
             ids, mask, lengths, status, max_len = enc.encode_padded(data, off, cap, fill_to=fill_to, width_guess=guess)
             torch.cuda.synchronize()
