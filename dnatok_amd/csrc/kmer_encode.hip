@@ -1541,7 +1541,9 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
     bool padded_in_kernel = false;
     // short rows (a row stride of at most kGroupsMaxStride cells says so), the plain digit table,
     // every window without an id spelled by its characters: sixteen lanes per row
-    if (t->arith && t->chars_mode && t_cap > 0 && t_cap <= kGroupsMaxStride && (t_cap & 3) == 0 && (!to_longest || tight)) {
+    const bool by_groups = t->arith && t->chars_mode && t_cap > 0 && t_cap <= kGroupsMaxStride && (t_cap & 3) == 0;
+    if (by_groups) {
+        padded_in_kernel = tight;
 #define GROUPS2(KK, L, M)                                                                         \
     do {                                                                                          \
         static const int resident = resident_workgroups(kmer_groups_kernel<KK, L, M>, kGroupThreads, 0, 8); \
@@ -1567,8 +1569,6 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
         }
 #undef GROUPS
 #undef GROUPS2
-        DNATOK_HIP_TRY(hipGetLastError());
-        return DNATOK_OK;
     }
 #define LAUNCH3(KK, L, C, M) \
     do {                                                                                          \
@@ -1600,7 +1600,7 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
     do {                                                                                          \
         if (t->chars_mode) LAUNCH2(KK, L, true); else LAUNCH2(KK, L, false);                      \
     } while (0)
-    switch (t->k) {
+    if (!by_groups) switch (t->k) {
         case 2: LAUNCH(2, true); break;
         case 3: LAUNCH(3, true); break;
         case 4: LAUNCH(4, true); break;

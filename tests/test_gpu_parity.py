@@ -596,7 +596,7 @@ def test_kmer_short_rows_sixteen_lanes_each(k, fold):
     reads of a few hundred bases with N, lower case (a table that folds the case, and one that does
     not), foreign bytes, every tail length, empty rows, rows of more than one step of 64 windows and
     rows cut by the stride; padded to a fixed width, to the longest row with a guess (one launch), and
-    to the longest row without one (the wave-per-row kernel), all against the oracle."""
+    to the longest row without one (a padding launch follows), all against the oracle."""
     say(f"kmer short rows k={k} fold={fold}")
     vocab = hf.kmer_vocab(k)
     t = kmer_tables.tables_from_vocab(vocab, k, 0)
