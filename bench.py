@@ -578,8 +578,18 @@ def memory_only_extra(w, dev_ms: float) -> dict:
     fastest plain copy (dnatok_diag_copy_tiles), beside the encoder's own step."""
     import ctypes
     import torch
-    from dnatok_amd import _lib
-    L = _lib.lib()
+    from dnatok_amd import build as _build
+    # the measurement kernels are a library of their own (include/dnatok_diag.h), not part of the product
+    L = ctypes.CDLL(_build.DIAG_LIB_PATH)
+    L.dnatok_last_error.restype = ctypes.c_char_p
+    L.dnatok_diag_copy_tiles.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    L.dnatok_diag_kmer_shape.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+
+    def ok(rc, what):
+        if rc != 0:
+            raise RuntimeError(f"{what} failed ({rc}): {L.dnatok_last_error().decode(errors='replace')}")
+
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     ptr = lambda t: ctypes.c_void_p(t.data_ptr())
     ids = torch.empty((w.n_rows, w.t_cap), dtype=torch.int32, device="cuda")
@@ -598,13 +608,13 @@ def memory_only_extra(w, dev_ms: float) -> dict:
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / n
 
-    shape_ms = timed(lambda: _lib.check(L.dnatok_diag_kmer_shape(ptr(w.sets[0]), ptr(w.off), w.n_rows, w.t_cap, fill,
+    shape_ms = timed(lambda: ok(L.dnatok_diag_kmer_shape(ptr(w.sets[0]), ptr(w.off), w.n_rows, w.t_cap, fill,
                                                                  ptr(ids), ptr(mask), stream), "dnatok_diag_kmer_shape"), 100)
     del ids, mask
     n = 1 << 30
     src = torch.empty(n, dtype=torch.uint8, device="cuda").random_(0, 255)
     dst = torch.empty_like(src)
-    copy_ms = timed(lambda: _lib.check(L.dnatok_diag_copy_tiles(ptr(src), ptr(dst), n, stream), "dnatok_diag_copy_tiles"), 30)
+    copy_ms = timed(lambda: ok(L.dnatok_diag_copy_tiles(ptr(src), ptr(dst), n, stream), "dnatok_diag_copy_tiles"), 30)
     same = bool(torch.equal(src, dst))
     del src, dst
     by = w.algorithmic_bytes
@@ -914,7 +924,7 @@ def kmer_rows_with_n_extra():
 
 def merge_table_placement_extra():
     """The BPE merge table of the 4096 vocabulary in global memory (L2; the default) against its compact
-    48 KB form kept in LDS by every workgroup (`dnatok_bpe_set_table_placement`), on batches of 1 KB rows:
+    48 KB form kept in LDS by every workgroup (`dnatok_bpe_table_set_placement`), on batches of 1 KB rows:
     512 rows (one per workgroup resident with the table in LDS) and the C3 batch of 1024 rows (two rounds
     of workgroups with the table in LDS).  Tokens compared between the placements and, for C3, with the
     golden vectors."""
@@ -927,7 +937,7 @@ def merge_table_placement_extra():
     kv = bpe_vocab.KernelVocab(bpe_vocab.split_merges(cfg["model"]["merges"]))
     vocab = cfg["model"]["vocab"]
     enc = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv), out_remap=kv.remap_to(vocab, vocab["[UNK]"]))
-    place = _lib.lib().dnatok_bpe_set_table_placement
+    place = enc.set_table_placement
     out = {}
     try:
         for rows in (512, 1024):
@@ -937,7 +947,7 @@ def merge_table_placement_extra():
             lengths = torch.empty(rows, dtype=torch.int32, device="cuda")
             seen = {}
             for name, mode in (("global_memory", 0), ("lds", 2)):
-                assert place(mode) == 0
+                place(mode)
                 enc.encode(data, off, 1024, tok_tmp=tok, lengths=lengths)
                 torch.cuda.synchronize()
                 ln = lengths.cpu().numpy()

@@ -19,11 +19,11 @@ EXPORTS = [
     "dnatok_char_encode_padded", "dnatok_char_encode_padded_as", "dnatok_char_encode_packed",
     "dnatok_char_embed_packed",
     "dnatok_char_unpack_2bit", "dnatok_host_clean_ascii", "dnatok_host_pack_2bit", "dnatok_host_fasta_scan",
-    "dnatok_kmer_table_create", "dnatok_kmer_table_destroy", "dnatok_kmer_set_team_rows", "dnatok_kmer_encode_padded",
+    "dnatok_kmer_table_create", "dnatok_kmer_table_destroy", "dnatok_kmer_table_set_team_rows", "dnatok_kmer_encode_padded",
     "dnatok_bpe_table_create", "dnatok_bpe_table_destroy", "dnatok_bpe_scratch_bytes",
     "dnatok_bpe_encode", "dnatok_bpe_encode_with_chars", "dnatok_bpe_encode_padded", "dnatok_bpe_padded_direct_max",
-    "dnatok_diag_copy_tiles", "dnatok_diag_kmer_shape", "dnatok_bpe_static_scratch_bytes", "dnatok_bpe_encode_static",
-    "dnatok_bpe_set_chunk_geometry", "dnatok_bpe_set_table_placement", "dnatok_pack_ragged", "dnatok_pad_rows", "dnatok_pad_rows_as",
+    "dnatok_bpe_static_scratch_bytes", "dnatok_bpe_encode_static",
+    "dnatok_bpe_table_set_chunk_geometry", "dnatok_bpe_table_set_placement", "dnatok_pack_ragged", "dnatok_pad_rows", "dnatok_pad_rows_as",
     "dnatok_normalize_bounds", "dnatok_normalize_rows",
 ]
 
@@ -90,7 +90,7 @@ def lib() -> ctypes.CDLL:
                                            c_int64, c_void_p, c_int32, c_int32, POINTER(c_void_p)]
     L.dnatok_kmer_table_destroy.argtypes = [c_void_p]
     L.dnatok_kmer_table_destroy.restype = None
-    L.dnatok_kmer_set_team_rows.argtypes = [c_int32]
+    L.dnatok_kmer_table_set_team_rows.argtypes = [c_void_p, c_int32]
     L.dnatok_kmer_encode_padded.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
     L.dnatok_bpe_table_create.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32,
@@ -107,15 +107,13 @@ def lib() -> ctypes.CDLL:
     L.dnatok_bpe_encode_padded.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                            c_void_p, c_size_t, c_void_p, c_void_p, c_int32, c_int64,
                                            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
-    L.dnatok_bpe_padded_direct_max.argtypes = []
+    L.dnatok_bpe_padded_direct_max.argtypes = [c_void_p]
     L.dnatok_bpe_padded_direct_max.restype = c_int64
-    L.dnatok_diag_copy_tiles.argtypes = [c_void_p, c_void_p, c_size_t, c_void_p]
-    L.dnatok_diag_kmer_shape.argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p]
     L.dnatok_bpe_static_scratch_bytes.restype = c_size_t
     L.dnatok_bpe_encode_static.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                            c_void_p, c_void_p, c_void_p]
-    L.dnatok_bpe_set_chunk_geometry.argtypes = [c_int32, c_int32]
-    L.dnatok_bpe_set_table_placement.argtypes = [c_int32]
+    L.dnatok_bpe_table_set_chunk_geometry.argtypes = [c_void_p, c_int32, c_int32]
+    L.dnatok_bpe_table_set_placement.argtypes = [c_void_p, c_int32]
     L.dnatok_pack_ragged.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_void_p]
     L.dnatok_pad_rows.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int32, c_int64,

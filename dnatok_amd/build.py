@@ -8,7 +8,10 @@ import sys
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_HERE, "libdnatok_hip.so")
-SOURCES = ["errors.hip", "char_encode.hip", "kmer_encode.hip", "bpe_encode.hip", "pack.hip", "host_ingest.hip", "normalize.hip", "diag.hip"]
+SOURCES = ["errors.hip", "char_encode.hip", "kmer_encode.hip", "bpe_encode.hip", "pack.hip", "host_ingest.hip", "normalize.hip"]
+# bench.py's memory-only kernels: a library of their own (include/dnatok_diag.h), not part of the product
+DIAG_LIB_PATH = os.path.join(_HERE, "libdnatok_diag.so")
+DIAG_SOURCES = ["diag.hip", "errors.hip"]
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # packed-FP32 instruction forms are kept out of all device code
@@ -45,13 +48,14 @@ def build_extension(verbose: bool = False) -> str:
     """Compile every HIP source for gfx950 and link the shared library. Always rebuilds."""
     objs = []
     procs = []
-    for src in SOURCES:
+    for src in SOURCES + [x for x in DIAG_SOURCES if x not in SOURCES]:
         obj = os.path.join(CSRC, src.replace(".hip", ".o"))
         cmd = [hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
-        objs.append(obj)
+        if src in SOURCES:
+            objs.append(obj)
     failed = False
     for src, p in procs:
         out, _ = p.communicate()
@@ -67,6 +71,8 @@ def build_extension(verbose: bool = False) -> str:
         raise RuntimeError("hipcc failed")
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]
     subprocess.check_call(cmd)
+    diag_objs = [os.path.join(CSRC, x.replace(".hip", ".o")) for x in DIAG_SOURCES]
+    subprocess.check_call([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", DIAG_LIB_PATH, *diag_objs])
     build_hostpack(verbose)
     return LIB_PATH
 

@@ -57,6 +57,10 @@ struct dnatok_bpe_table {
     unsigned long long *max_trees;
     mutable std::mutex slot_lock;
     mutable std::unordered_map<void *, int> slot_of_stream;
+    // Test and measurement switches of this table (dnatok_bpe_table_set_chunk_geometry,
+    // dnatok_bpe_table_set_placement); 0 / 0 / 0 are the shipped choices.  A call reads them once,
+    // when it starts.
+    std::atomic<int> chunk_core{0}, chunk_overlap{0}, placement{0};
 };
 
 constexpr int kMaxTreeSlots = 64;
@@ -99,6 +103,8 @@ struct BpeArgs {
     // shortest rows, 2 that class alone (a batch of mostly short rows with a few long ones is split
     // between a launch with 256-thread teams and one with teams of one wave)
     int32_t part;
+    // host side only: where the merge table is kept (dnatok_bpe_table_set_placement)
+    int32_t placement;
 };
 
 typedef int32_t bpe_int4_a4 __attribute__((ext_vector_type(4), aligned(4)));
@@ -839,20 +845,19 @@ static size_t long_slab_bytes(int64_t max_len)
     return ((n * 26) + 255) & ~(size_t)255;     // 16 (records) + 2 + 2 (product, gate) + 2 + 4 (queues)
 }
 
-// Chunk geometry of the calls that follow (process-wide).  The shipped values are the constants
-// above; dnatok_bpe_set_chunk_geometry lets a test run the chunk / seam / fallback machinery with
+// Chunk geometry of a table's calls.  The shipped values are the constants above;
+// dnatok_bpe_table_set_chunk_geometry lets a test run the chunk / seam / fallback machinery with
 // chunks so small that every few hundred bytes of a row hold a seam.
-static std::atomic<int> g_chunk_core{kChunkCore}, g_chunk_overlap{kChunkOverlap};
-static std::atomic<int> g_table_placement{0};      // dnatok_bpe_set_table_placement
 
 // A batch whose long rows make far fewer chunks than teams fit the chip (a few rows of a few
 // thousand bytes each) is cut finer, down to a core of 512 bytes: more, shorter items run side by
 // side, and the batch is latency-bound either way (one row of 100 kbp: 48 -> 38 us per call).
 // Only with the shipped geometry, and only when the batch has long rows at all.
-static void chunk_geometry(int *core, int *overlap, int64_t max_len, int64_t total)
+static void chunk_geometry(const dnatok_bpe_t *t, int *core, int *overlap, int64_t max_len, int64_t total)
 {
-    *core = g_chunk_core.load(std::memory_order_relaxed);
-    *overlap = g_chunk_overlap.load(std::memory_order_relaxed);
+    *core = t ? t->chunk_core.load(std::memory_order_relaxed) : 0;
+    *overlap = t ? t->chunk_overlap.load(std::memory_order_relaxed) : 0;
+    if (*core == 0 || *overlap == 0) { *core = kChunkCore; *overlap = kChunkOverlap; }
     if (*core == kChunkCore && *overlap == kChunkOverlap && max_len > kChunkCore + 2 * kChunkOverlap) {
         constexpr int64_t kTeams = 1024;                 // about what is resident at once
         int64_t c = (total / kTeams + 127) & ~(int64_t)127;
@@ -861,11 +866,11 @@ static void chunk_geometry(int *core, int *overlap, int64_t max_len, int64_t tot
     }
 }
 
-static BpePlan make_plan(uint8_t *base, int64_t n_rows, int64_t max_len, int64_t total,
+static BpePlan make_plan(const dnatok_bpe_t *t, uint8_t *base, int64_t n_rows, int64_t max_len, int64_t total,
                          int64_t max_slabs = kLongGrid)
 {
     BpePlan p{};
-    chunk_geometry(&p.core, &p.overlap, max_len, total);
+    chunk_geometry(t, &p.core, &p.overlap, max_len, total);
     p.ext = p.core + 2 * p.overlap;
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
     const bool chunks = max_len > p.ext;
@@ -1584,22 +1589,24 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
     return DNATOK_OK;
 }
 
-extern "C" int dnatok_bpe_set_chunk_geometry(int32_t core, int32_t overlap)
+extern "C" int dnatok_bpe_table_set_chunk_geometry(dnatok_bpe_t *t, int32_t core, int32_t overlap)
 {
-    if (core == 0 && overlap == 0) { core = kChunkCore; overlap = kChunkOverlap; }
-    DNATOK_REQUIRE(core >= 256 && overlap >= 32 && core > 2 * overlap && core + 2 * overlap <= kLdsCap,
+    DNATOK_REQUIRE(t, DNATOK_E_INVALID, "dnatok_bpe_table_set_chunk_geometry: null table");
+    DNATOK_REQUIRE((core == 0 && overlap == 0) ||
+                       (core >= 256 && overlap >= 32 && core > 2 * overlap && core + 2 * overlap <= kLdsCap),
                    DNATOK_E_INVALID,
-                   "dnatok_bpe_set_chunk_geometry: need core >= 256, overlap >= 32, core > 2 * overlap, "
-                   "core + 2 * overlap <= %d", kLdsCap);
-    g_chunk_core.store(core, std::memory_order_relaxed);
-    g_chunk_overlap.store(overlap, std::memory_order_relaxed);
+                   "dnatok_bpe_table_set_chunk_geometry: need core >= 256, overlap >= 32, core > 2 * overlap, "
+                   "core + 2 * overlap <= %d (or 0, 0 for the shipped geometry)", kLdsCap);
+    t->chunk_core.store(core, std::memory_order_relaxed);
+    t->chunk_overlap.store(overlap, std::memory_order_relaxed);
     return DNATOK_OK;
 }
 
-extern "C" int dnatok_bpe_set_table_placement(int32_t mode)
+extern "C" int dnatok_bpe_table_set_placement(dnatok_bpe_t *t, int32_t mode)
 {
-    DNATOK_REQUIRE(mode >= 0 && mode <= 2, DNATOK_E_INVALID, "dnatok_bpe_set_table_placement: mode is 0, 1 or 2");
-    g_table_placement.store(mode, std::memory_order_relaxed);
+    DNATOK_REQUIRE(t, DNATOK_E_INVALID, "dnatok_bpe_table_set_placement: null table");
+    DNATOK_REQUIRE(mode >= 0 && mode <= 2, DNATOK_E_INVALID, "dnatok_bpe_table_set_placement: mode is 0, 1 or 2");
+    t->placement.store(mode, std::memory_order_relaxed);
     return DNATOK_OK;
 }
 
@@ -1613,9 +1620,8 @@ extern "C" void dnatok_bpe_table_destroy(dnatok_bpe_t *t)
 extern "C" size_t dnatok_bpe_scratch_bytes(const dnatok_bpe_t *t, int64_t n_rows, int64_t max_len,
                                            int64_t total)
 {
-    (void)t;
     if (n_rows <= 0) return 256;
-    return make_plan(nullptr, n_rows, max_len, total).total_bytes;
+    return make_plan(t, nullptr, n_rows, max_len, total).total_bytes;
 }
 
 namespace {
@@ -1662,11 +1668,12 @@ int launch_lds_as(const BpeArgs &a, const uint8_t *bytes, const int64_t *offsets
 {
     const size_t lds = lds_bytes<NT, TEAMS, CAP>();
     auto kern = bpe_lds_kernel<NT, TEAMS, CAP, PLANNED, false, CHARS, CHUNKS, PADDED>;
-    static bool attr_set = false;
-    if (!attr_set) {
+    // (once per kernel form; two threads that both find it unset both set it, to the same value)
+    static std::atomic<bool> attr_set{false};
+    if (!attr_set.load(std::memory_order_acquire)) {
         DNATOK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_set = true;
+        attr_set.store(true, std::memory_order_release);
     }
     const int64_t items = PLANNED ? p.max_items : n_rows;
     int64_t grid = (items + TEAMS - 1) / TEAMS;
@@ -1711,11 +1718,12 @@ int launch_lds_ltab(const BpeArgs &a, const uint8_t *bytes, const int64_t *offse
 {
     const size_t lds = lds_bytes<NT, TEAMS, CAP>() + kLdsTabWords * 4 + 16;
     auto kern = bpe_lds_kernel<NT, TEAMS, CAP, false, true>;
-    static bool attr_set = false;
-    if (!attr_set) {
+    // (once per kernel form; two threads that both find it unset both set it, to the same value)
+    static std::atomic<bool> attr_set{false};
+    if (!attr_set.load(std::memory_order_acquire)) {
         DNATOK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_set = true;
+        attr_set.store(true, std::memory_order_release);
     }
     int64_t grid = (n_rows + TEAMS - 1) / TEAMS;
     const int64_t resident = ltab_resident_teams<NT, TEAMS, CAP>() / TEAMS;
@@ -1737,8 +1745,10 @@ int run_lds_part(bool long_rows, int chunking, bool force_plan, const BpeArgs &a
                  hipStream_t s)
 {
     if constexpr (CAP == 1024) {
-        if (!long_rows && a.ltab && !a.char_ids && !a.pad_ids) {
-            const int mode = g_table_placement.load(std::memory_order_relaxed);
+        // (only for a batch that one launch encodes whole: with force_plan or a part of a split
+        // batch the work list decides which rows a launch takes, and this form has none)
+        if (!long_rows && !force_plan && a.part == 0 && a.ltab && !a.char_ids && !a.pad_ids) {
+            const int mode = a.placement;
             if (mode == 2 || (mode == 1 && n_rows <= ltab_resident_teams<NT, TEAMS, 1024>()))
                 return launch_lds_ltab<NT, TEAMS, 1024>(a, bytes, offsets, p, n_rows, tok_tmp, lengths, s);
         }
@@ -1800,6 +1810,7 @@ static int bpe_encode_launch(const dnatok_bpe_t *t, const uint8_t *bytes, const 
 {
     BpeArgs a{t->tab, t->byte_to_sym, t->out_remap, t->shift, t->mul1, t->mul2, t->n_merges, t->ltab, t->lmul1, t->lmul2,
               char_lut, char_ids, char_mask};
+    a.placement = t->placement.load(std::memory_order_relaxed);
     if (padded) {
         a.pad_ids = padded->pad_ids; a.pad_mask = padded->pad_mask; a.pad_remap = padded->pad_remap;
         a.pad_stride = padded->pad_stride; a.pad_id = padded->pad_id;
@@ -1877,11 +1888,11 @@ extern "C" int dnatok_bpe_encode(const dnatok_bpe_t *t, const uint8_t *bytes, co
     const int bad = bpe_encode_check("dnatok_bpe_encode", t, bytes, offsets, n_rows, max_len, total, tok_tmp, lengths);
     if (bad) return bad;
     if (n_rows == 0) return DNATOK_OK;
-    const BpePlan need = make_plan(nullptr, n_rows, max_len, total);
+    const BpePlan need = make_plan(t, nullptr, n_rows, max_len, total);
     DNATOK_REQUIRE(scratch && scratch_bytes >= need.total_bytes, DNATOK_E_SCRATCH,
                    "dnatok_bpe_encode: scratch holds %zu bytes, %zu needed", scratch_bytes, need.total_bytes);
     DNATOK_REQUIRE(((uintptr_t)scratch & 255) == 0, DNATOK_E_INVALID, "dnatok_bpe_encode: scratch must be 256-byte aligned");
-    const BpePlan p = make_plan((uint8_t *)scratch, n_rows, max_len, total);
+    const BpePlan p = make_plan(t, (uint8_t *)scratch, n_rows, max_len, total);
     return bpe_encode_launch(t, bytes, offsets, n_rows, max_len, total, p, tok_tmp, lengths, (hipStream_t)stream);
 }
 
@@ -1897,20 +1908,20 @@ extern "C" int dnatok_bpe_encode_with_chars(const dnatok_bpe_t *t, const uint8_t
     DNATOK_REQUIRE(char_lut && (char_ids || total == 0), DNATOK_E_INVALID,
                    "dnatok_bpe_encode_with_chars: char_lut and char_ids are required");
     if (n_rows == 0) return DNATOK_OK;
-    const BpePlan need = make_plan(nullptr, n_rows, max_len, total);
+    const BpePlan need = make_plan(t, nullptr, n_rows, max_len, total);
     DNATOK_REQUIRE(scratch && scratch_bytes >= need.total_bytes, DNATOK_E_SCRATCH,
                    "dnatok_bpe_encode_with_chars: scratch holds %zu bytes, %zu needed", scratch_bytes, need.total_bytes);
     DNATOK_REQUIRE(((uintptr_t)scratch & 255) == 0, DNATOK_E_INVALID,
                    "dnatok_bpe_encode_with_chars: scratch must be 256-byte aligned");
-    const BpePlan p = make_plan((uint8_t *)scratch, n_rows, max_len, total);
+    const BpePlan p = make_plan(t, (uint8_t *)scratch, n_rows, max_len, total);
     return bpe_encode_launch(t, bytes, offsets, n_rows, max_len, total, p, tok_tmp, lengths, (hipStream_t)stream, char_lut,
                              char_ids, char_mask);
 }
 
-extern "C" int64_t dnatok_bpe_padded_direct_max(void)
+extern "C" int64_t dnatok_bpe_padded_direct_max(const dnatok_bpe_t *t)
 {
     int core, overlap;
-    chunk_geometry(&core, &overlap, 0, 0);
+    chunk_geometry(t, &core, &overlap, 0, 0);
     return (int64_t)core + 2 * overlap;
 }
 
@@ -1936,11 +1947,11 @@ extern "C" int dnatok_bpe_encode_padded(const dnatok_bpe_t *t, const uint8_t *by
         }
         return DNATOK_OK;
     }
-    const BpePlan need = make_plan(nullptr, n_rows, max_len, total);
+    const BpePlan need = make_plan(t, nullptr, n_rows, max_len, total);
     DNATOK_REQUIRE(scratch && scratch_bytes >= need.total_bytes, DNATOK_E_SCRATCH,
                    "%s: scratch holds %zu bytes, %zu needed", who, scratch_bytes, need.total_bytes);
     DNATOK_REQUIRE(((uintptr_t)scratch & 255) == 0, DNATOK_E_INVALID, "%s: scratch must be 256-byte aligned", who);
-    const BpePlan p = make_plan((uint8_t *)scratch, n_rows, max_len, total);
+    const BpePlan p = make_plan(t, (uint8_t *)scratch, n_rows, max_len, total);
     if (max_len > p.ext) {
         // rows cut into chunks (or left to the whole-row kernel) are assembled in tok_tmp first
         DNATOK_REQUIRE(tok_tmp, DNATOK_E_INVALID,
@@ -2017,10 +2028,10 @@ extern "C" int dnatok_bpe_encode_static(const dnatok_bpe_t *t, const uint8_t *by
     // Fewer slabs for the whole-row fallback kernel (fewer rows redone at once) before giving up:
     // the slabs are what grows with the longest row.
     int64_t slabs = kLongGrid;
-    BpePlan need = make_plan(nullptr, n_rows, max_len, total, slabs);
+    BpePlan need = make_plan(t, nullptr, n_rows, max_len, total, slabs);
     while (need.total_bytes > kStaticScratchBytes && slabs > 1) {
         slabs /= 2;
-        need = make_plan(nullptr, n_rows, max_len, total, slabs);
+        need = make_plan(t, nullptr, n_rows, max_len, total, slabs);
     }
     DNATOK_REQUIRE(need.total_bytes <= kStaticScratchBytes, DNATOK_E_TOO_LARGE,
                    "dnatok_bpe_encode_static: this batch needs %zu bytes of work space, the built-in buffer holds "
@@ -2028,6 +2039,6 @@ extern "C" int dnatok_bpe_encode_static(const dnatok_bpe_t *t, const uint8_t *by
     uint8_t *base = nullptr;
     const int rc = static_scratch_ptr(&base);
     if (rc) return rc;
-    const BpePlan p = make_plan(base, n_rows, max_len, total, slabs);
+    const BpePlan p = make_plan(t, base, n_rows, max_len, total, slabs);
     return bpe_encode_launch(t, bytes, offsets, n_rows, max_len, total, p, tok_tmp, lengths, (hipStream_t)stream);
 }

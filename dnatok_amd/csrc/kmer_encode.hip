@@ -60,13 +60,12 @@ struct dnatok_kmer_table {
     unsigned long long *max_trees;       // kTreeWords words per slot (see kmer_team_kernel)
     mutable std::mutex slot_lock;
     mutable std::unordered_map<void *, int> slot_of_stream;
+    // Batches of up to this many rows are encoded by kmer_team_kernel (a workgroup per row); -1: as
+    // many rows as workgroups of that kernel fit the chip at once.  (dnatok_kmer_table_set_team_rows)
+    std::atomic<int> team_rows{-1};
 };
 
 constexpr int kMaxSlots = 64;
-
-// Batches of up to this many rows are encoded by kmer_team_kernel (a workgroup per row); -1: as
-// many rows as workgroups of that kernel fit the chip at once.  (dnatok_kmer_set_team_rows)
-static std::atomic<int> g_team_rows{-1};
 constexpr int kMaxSlotStride = 32;       // 64-bit words between two slots (one 256-byte line each)
 // A call whose kernel reports the maximum itself (kmer_team_kernel, publish) gathers it up a tree
 // of atomics (climb_max_tree): kTreeWords words per slot.
@@ -1477,10 +1476,11 @@ extern "C" int dnatok_kmer_table_create(int k, const int8_t *digit_h, const int3
     return DNATOK_OK;
 }
 
-extern "C" int dnatok_kmer_set_team_rows(int32_t max_rows)
+extern "C" int dnatok_kmer_table_set_team_rows(dnatok_kmer_t *t, int32_t max_rows)
 {
-    DNATOK_REQUIRE(max_rows >= -1, DNATOK_E_INVALID, "dnatok_kmer_set_team_rows: -1 (automatic), 0 (never) or a row count");
-    g_team_rows.store(max_rows, std::memory_order_relaxed);
+    DNATOK_REQUIRE(t, DNATOK_E_INVALID, "dnatok_kmer_table_set_team_rows: null table");
+    DNATOK_REQUIRE(max_rows >= -1, DNATOK_E_INVALID, "dnatok_kmer_table_set_team_rows: -1 (automatic), 0 (never) or a row count");
+    t->team_rows.store(max_rows, std::memory_order_relaxed);
     return DNATOK_OK;
 }
 
@@ -1578,7 +1578,7 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
     do {                                                                                          \
         static const int resident = resident_workgroups(kmer_rows_kernel<KK, L, C, M, AR>, kRowsThreads, 0, 2); \
         static const int team_resident = resident_workgroups(kmer_team_kernel<KK, L, C, M>, kKmerThreads, 0, 4); \
-        const int team_rows = g_team_rows.load(std::memory_order_relaxed);                       \
+        const int team_rows = t->team_rows.load(std::memory_order_relaxed);                         \
         if (n_rows <= (team_rows < 0 ? team_resident : team_rows)) {                              \
             padded_in_kernel = tight && n_rows <= kTreeRows;                                      \
             kmer_team_kernel<KK, L, C, M><<<(int)n_rows, kKmerThreads, 0, s>>>(                   \

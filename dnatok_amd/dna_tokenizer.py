@@ -387,25 +387,8 @@ class DNATok:
         left = self.padding_side == "left"
         self._staged_host_ids = None
         if self.bpe_backend is not None:
-            if not left and dtype == torch.int32:
-                # the engine pads the rows itself while it writes them out
-                staged = []
-
-                def stage(ids):
-                    if host_ids:
-                        nbytes = ids.numel() * ids.element_size()
-                        host = self._pinned(nbytes)[:nbytes].view(ids.dtype).view(ids.shape)
-                        host.copy_(ids, non_blocking=True)
-                        staged[:] = [host]
-
-                ids, mask = self.bpe_backend.padded_device(list(seqs), device=device, min_width=min_width,
-                                                           pad_multiple=pad_multiple, stage_ids=stage)
-                if staged and staged[0].shape[1] == ids.stride(0):      # (not those of a first, too narrow, try)
-                    self._staged_host_ids = staged[0][:, :ids.shape[1]]
-                return ids, mask
-            tok, offsets, lengths, t_cap = self.bpe_backend.tokens_device(list(seqs), device=device, meta_tail=2)
-            return self._pad_bpe_runs(tok, offsets, lengths, t_cap, dtype=dtype, min_width=min_width,
-                                      pad_multiple=pad_multiple, host_ids=host_ids, stats_behind_lengths=True)
+            return self._encode_bpe_rows(list(seqs), device, dtype=dtype, min_width=min_width,
+                                         pad_multiple=pad_multiple, host_ids=host_ids)
         data, offsets, lens = encoders.bytes_from_strings(seqs, device)
         if self._kmer_enc is not None:
             return self._encode_kmer_device(seqs, data, offsets, lens, dtype=dtype, min_width=min_width,
@@ -414,6 +397,73 @@ class DNATok:
         if pad_multiple > 1 and width % pad_multiple:
             width += pad_multiple - width % pad_multiple
         return self._char_enc.encode_padded(data, offsets, width, pad_left=left, dtype=dtype)
+
+    def _encode_bpe_rows(self, seqs: List[str], device, *, dtype: torch.dtype, min_width: int,
+                         pad_multiple: int, host_ids: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+        """BPE rows with the reference's fallback chain (src/dna_tokenizer.py:2066-2100: any failure
+        of the backend ends at the tokenizer itself, with a warning).  Finer than the reference
+        where the backend says which rows it cannot reproduce (``UnsupportedRows``: white space
+        under a pre-tokenizer, a character outside the vocabulary without unk_token): those rows
+        alone get the tokenizer's ids, the others stay on the GPU, as the k-mer path splices its
+        rows.  The reference's middle link (CachedLMM, approximate) is not part of this build."""
+        from .gputok_bpe_backend import UnsupportedRows
+        try:
+            return self._bpe_rows_on_gpu(seqs, device, dtype=dtype, min_width=min_width,
+                                         pad_multiple=pad_multiple, host_ids=host_ids)
+        except UnsupportedRows as e:
+            self._staged_host_ids = None
+            bad = e.rows
+            self.log.warning("BPE backend: %d of %d rows go to the tokenizer (%s)", len(bad), len(seqs), e)
+            fixed = self._tok_ids([seqs[i] for i in bad])
+            is_bad = set(bad)
+            keep = [i for i in range(len(seqs)) if i not in is_bad]
+            if not keep:
+                return self._tokenizer_rows_device(seqs, device, dtype=dtype, min_width=min_width,
+                                                   pad_multiple=pad_multiple)
+            try:
+                good_ids, good_mask = self._bpe_rows_on_gpu([seqs[i] for i in keep], device, dtype=dtype,
+                                                            min_width=min_width, pad_multiple=pad_multiple,
+                                                            host_ids=False)
+            except Exception as e2:
+                self.log.warning("BPE backend failed (%s); falling back to the tokenizer.", e2)
+                return self._tokenizer_rows_device(seqs, device, dtype=dtype, min_width=min_width,
+                                                   pad_multiple=pad_multiple)
+            # the clean rows at their places in a batch of the full height, then the others spliced in
+            n, w = len(seqs), good_ids.shape[1]
+            ids = torch.full((n, w), int(self.id_pad), dtype=good_ids.dtype, device=good_ids.device)
+            mask = torch.zeros((n, w), dtype=torch.uint8, device=good_ids.device)
+            at = torch.as_tensor(keep, dtype=torch.int64, device=good_ids.device)
+            ids[at] = good_ids
+            mask[at] = good_mask
+            return self._splice_tokenizer_rows(ids, mask, bad, fixed, pad_multiple=pad_multiple)
+        except Exception as e:
+            self._staged_host_ids = None
+            self.log.warning("BPE backend failed (%s); falling back to the tokenizer.", e)
+            return self._tokenizer_rows_device(seqs, device, dtype=dtype, min_width=min_width,
+                                               pad_multiple=pad_multiple)
+
+    def _bpe_rows_on_gpu(self, seqs: List[str], device, *, dtype: torch.dtype, min_width: int,
+                         pad_multiple: int, host_ids: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+        left = self.padding_side == "left"
+        if not left and dtype == torch.int32:
+            # the engine pads the rows itself while it writes them out
+            staged = []
+
+            def stage(ids):
+                if host_ids:
+                    nbytes = ids.numel() * ids.element_size()
+                    host = self._pinned(nbytes)[:nbytes].view(ids.dtype).view(ids.shape)
+                    host.copy_(ids, non_blocking=True)
+                    staged[:] = [host]
+
+            ids, mask = self.bpe_backend.padded_device(seqs, device=device, min_width=min_width,
+                                                       pad_multiple=pad_multiple, stage_ids=stage)
+            if staged and staged[0].shape[1] == ids.stride(0):      # (not those of a first, too narrow, try)
+                self._staged_host_ids = staged[0][:, :ids.shape[1]]
+            return ids, mask
+        tok, offsets, lengths, t_cap = self.bpe_backend.tokens_device(seqs, device=device, meta_tail=2)
+        return self._pad_bpe_runs(tok, offsets, lengths, t_cap, dtype=dtype, min_width=min_width,
+                                  pad_multiple=pad_multiple, host_ids=host_ids, stats_behind_lengths=True)
 
     def _pad_bpe_runs(self, tok, offsets, lengths, t_cap: int, *, dtype, min_width: int, pad_multiple: int,
                       host_ids: bool = False, stats_behind_lengths: bool = False):
@@ -492,9 +542,14 @@ class DNATok:
                 ids, mask = self.encode_batch_device([rows[i] for i in range(len(names))], device=device)
                 return ids, mask, names
             t_cap = max(int(lens.max()), 1)
-            tok, lengths = be._dnatok.tokenize_device(data, offsets, t_cap)
-            ids, mask = self._pad_bpe_runs(tok, offsets, lengths, t_cap, dtype=torch.int32, min_width=min_width,
-                                           pad_multiple=1)
+            try:
+                tok, lengths = be._dnatok.tokenize_device(data, offsets, t_cap)
+                ids, mask = self._pad_bpe_runs(tok, offsets, lengths, t_cap, dtype=torch.int32,
+                                               min_width=min_width, pad_multiple=1)
+            except Exception as e:
+                self.log.warning("BPE backend failed (%s); falling back to the tokenizer.", e)
+                ids, mask = self._tokenizer_rows_device([rows[i] for i in range(len(names))], device,
+                                                        dtype=torch.int32, min_width=min_width, pad_multiple=1)
             return ids, mask, names
         if self._kmer_enc is not None:
             ids, mask = self._encode_kmer_device(rows, data, offsets, lens, dtype=torch.int32, min_width=min_width,
@@ -591,30 +646,62 @@ class DNATok:
         if need.any() and not self.allow_incomplete_kmer_lut:
             self._staged_host_ids = None
             rows = np.nonzero(need)[0].tolist()
-            fixed = self._tok_ids([seqs[i] for i in rows])
-            new_w = max(width, max(len(r) for r in fixed))
-            if pad_multiple > 1 and new_w % pad_multiple:
-                new_w += pad_multiple - new_w % pad_multiple
-            if new_w > width:
-                extra = new_w - width
-                pad_i = torch.full((n, extra), int(self.id_pad), dtype=ids.dtype, device=ids.device)
-                pad_m = torch.zeros((n, extra), dtype=torch.uint8, device=ids.device)
-                ids = torch.cat([pad_i, ids], dim=1) if left else torch.cat([ids, pad_i], dim=1)
-                mask = torch.cat([pad_m, mask], dim=1) if left else torch.cat([mask, pad_m], dim=1)
-            else:
-                ids, mask = ids.clone(), mask.clone()
-            for i, r in zip(rows, fixed):
-                ids[i] = int(self.id_pad)
-                mask[i] = 0
-                if r:
-                    cur = torch.as_tensor(r, dtype=ids.dtype, device=ids.device)
-                    if left:
-                        ids[i, new_w - len(r):] = cur
-                        mask[i, new_w - len(r):] = 1
-                    else:
-                        ids[i, :len(r)] = cur
-                        mask[i, :len(r)] = 1
+            ids, mask = self._splice_tokenizer_rows(ids, mask, rows, self._tok_ids([seqs[i] for i in rows]),
+                                                    pad_multiple=pad_multiple)
         return ids, mask
+
+    def _splice_tokenizer_rows(self, ids: torch.Tensor, mask: torch.Tensor, rows: List[int],
+                               fixed: List[List[int]], *, pad_multiple: int = 1):
+        """Rows ``rows`` of a padded batch on the device get the tokenizer's own ids ``fixed``; the
+        batch grows (on ``padding_side``) when one of them is longer than it is wide."""
+        left = self.padding_side == "left"
+        n, width = ids.shape
+        new_w = max(width, max((len(r) for r in fixed), default=0))
+        if pad_multiple > 1 and new_w % pad_multiple:
+            new_w += pad_multiple - new_w % pad_multiple
+        if new_w > width:
+            extra = new_w - width
+            pad_i = torch.full((n, extra), int(self.id_pad), dtype=ids.dtype, device=ids.device)
+            pad_m = torch.zeros((n, extra), dtype=torch.uint8, device=ids.device)
+            ids = torch.cat([pad_i, ids], dim=1) if left else torch.cat([ids, pad_i], dim=1)
+            mask = torch.cat([pad_m, mask], dim=1) if left else torch.cat([mask, pad_m], dim=1)
+        else:
+            ids, mask = ids.clone(), mask.clone()
+        for i, r in zip(rows, fixed):
+            ids[i] = int(self.id_pad)
+            mask[i] = 0
+            if r:
+                cur = torch.as_tensor(r, dtype=ids.dtype, device=ids.device)
+                if left:
+                    ids[i, new_w - len(r):] = cur
+                    mask[i, new_w - len(r):] = 1
+                else:
+                    ids[i, :len(r)] = cur
+                    mask[i, :len(r)] = 1
+        return ids, mask
+
+    def _tokenizer_rows_device(self, seqs: Sequence[str], device, *, dtype: torch.dtype, min_width: int,
+                               pad_multiple: int) -> Tuple[torch.Tensor, torch.Tensor]:
+        """The whole batch through the tokenizer itself, laid out as the device paths lay it out
+        (padding side, least width, multiple, id type): where a fast path ends when it cannot serve
+        a batch (reference: _tokenize_batch_cpu, src/dna_tokenizer.py:1591-1777, 2100)."""
+        fixed = self._tok_ids(seqs)
+        width = max(max((len(r) for r in fixed), default=0), int(min_width))
+        if pad_multiple > 1 and width % pad_multiple:
+            width += pad_multiple - width % pad_multiple
+        ids = torch.full((len(fixed), width), int(self.id_pad), dtype=dtype)
+        mask = torch.zeros((len(fixed), width), dtype=torch.uint8)
+        left = self.padding_side == "left"
+        for i, r in enumerate(fixed):
+            if r:
+                cur = torch.as_tensor(r, dtype=dtype)
+                if left:
+                    ids[i, width - len(r):] = cur
+                    mask[i, width - len(r):] = 1
+                else:
+                    ids[i, :len(r)] = cur
+                    mask[i, :len(r)] = 1
+        return ids.to(device), mask.to(device)
 
     def encode_batch_to_ids(self, seqs: List[str]) -> torch.Tensor:
         """CPU pinned int64 [B, T] (reference: 2049-2148)."""

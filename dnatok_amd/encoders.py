@@ -386,6 +386,11 @@ class KmerEncoder:
             except Exception:
                 pass
 
+    def set_team_rows(self, max_rows: int) -> None:
+        """Test and measurement hook (``dnatok_kmer_table_set_team_rows``): batches of up to
+        ``max_rows`` rows get a workgroup per row, larger ones a wave per row; -1 = automatic."""
+        _lib.check(_lib.lib().dnatok_kmer_table_set_team_rows(self._h, int(max_rows)), "dnatok_kmer_table_set_team_rows")
+
     def encode_padded(self, data: torch.Tensor, offsets: torch.Tensor, t_cap: int, *,
                       fill_to: int = 0, width_guess: int = 0, want_mask: bool = True, out=None):
         """Returns (ids[B, t_cap], mask, lengths[B], status[B], max_len[1]); with fill_to = 0 the
@@ -498,10 +503,20 @@ class BpeEncoder:
             _stream()), "dnatok_bpe_encode_padded")
         return ids, mask, lengths, longest
 
-    @staticmethod
-    def padded_direct_max() -> int:
+    def padded_direct_max(self) -> int:
         """Longest row (bytes) that ``encode_padded`` writes without a token buffer."""
-        return int(_lib.lib().dnatok_bpe_padded_direct_max())
+        return int(_lib.lib().dnatok_bpe_padded_direct_max(self._h))
+
+    def set_chunk_geometry(self, core: int, overlap: int) -> None:
+        """Test hook (``dnatok_bpe_table_set_chunk_geometry``): this encoder's calls cut long rows
+        into chunks of ``core`` bytes extended by ``overlap`` on both sides; (0, 0) = shipped."""
+        _lib.check(_lib.lib().dnatok_bpe_table_set_chunk_geometry(self._h, int(core), int(overlap)),
+                   "dnatok_bpe_table_set_chunk_geometry")
+
+    def set_table_placement(self, mode: int) -> None:
+        """Measurement hook (``dnatok_bpe_table_set_placement``): 0 = merge table in global memory
+        (default), 1 / 2 = its compact form in LDS where the batch allows."""
+        _lib.check(_lib.lib().dnatok_bpe_table_set_placement(self._h, int(mode)), "dnatok_bpe_table_set_placement")
 
     def encode_with_chars(self, data: torch.Tensor, offsets: torch.Tensor, max_len: int, char_lut: torch.Tensor, *,
                           tok_tmp: Optional[torch.Tensor] = None, lengths: Optional[torch.Tensor] = None,

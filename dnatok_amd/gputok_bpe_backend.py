@@ -282,6 +282,17 @@ def _reconstruct_gputok_vocab(merges: Sequence[str]) -> List[str]:
 
 # ------------------------------------------------------------------------- backend
 
+class UnsupportedRows(ValueError):
+    """Rows of a batch that the tokenizer cuts or drops characters from (white space with a
+    pre-tokenizer, a character outside the vocabulary without unk_token), which the engine does
+    not reproduce.  ``rows`` holds their indices in the batch, in rising order: a caller that
+    owns the tokenizer (DNATok) encodes those rows with it and the others on the GPU."""
+
+    def __init__(self, rows: List[int], message: str) -> None:
+        super().__init__(message)
+        self.rows = list(rows)
+
+
 class GPUTokBPEBackend:
     """HF-compatible GPU BPE encoder (reference: src/gputok_bpe_backend.py:396-679)."""
 
@@ -303,8 +314,9 @@ class GPUTokBPEBackend:
         self._normalize_device = _compile_device_normalizer(cfg) if self._normalize is not None else None
         # What the engine cannot reproduce depends on the input for two kinds of tokenizer: with a
         # pre-tokenizer, white space inside a row cuts it into words (and is dropped); without an
-        # unk_token, characters outside the vocabulary are dropped.  Such input raises ValueError
-        # (DNATok then takes the row to the tokenizer itself).
+        # unk_token, characters outside the vocabulary are dropped.  Such input raises UnsupportedRows
+        # (a ValueError naming the rows; DNATok catches it and gives those rows to the tokenizer
+        # itself, the reference's fallback of src/dna_tokenizer.py:2066-2100 row by row).
         self._input_guard: Optional[_re.Pattern] = None
         guard = []
         if cfg.get("pre_tokenizer") is not None:
@@ -404,8 +416,10 @@ class GPUTokBPEBackend:
                 seqs = [self._normalize(s) for s in seqs]
             hit = self._input_guard.search("".join(seqs))
             if hit is not None:
-                raise ValueError(f"character {hit.group(0)!r} is cut or dropped by this tokenizer "
-                                 "(pre-tokenizer / no unk_token); not reproduced by the GPU engine")
+                rows = [i for i, s in enumerate(seqs) if self._input_guard.search(s) is not None]
+                raise UnsupportedRows(rows, f"character {hit.group(0)!r} (row {rows[0]}; {len(rows)} of "
+                                      f"{len(seqs)} rows) is cut or dropped by this tokenizer (pre-tokenizer / "
+                                      "no unk_token); not reproduced by the GPU engine")
         if self._normalize is None or self._input_guard is not None:
             data, offsets, lens = encoders.bytes_from_strings(seqs, dev, encoding="utf-8")
             t_cap = int(lens.max())

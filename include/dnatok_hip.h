@@ -143,12 +143,13 @@ int  dnatok_kmer_table_create(int k, const int8_t *digit_h, const int32_t *kmer_
                               dnatok_kmer_t **out);
 void dnatok_kmer_table_destroy(dnatok_kmer_t *t);
 
-/* Which of the two k-mer kernels the calls that follow use (process-wide; no counterpart in the
- * reference; a switch for tests and measurements, results are identical).  A batch of up to
- * max_rows rows is encoded with a workgroup per row (four waves share a row: the latency of a small
- * batch), a larger one with a wave per row (the bandwidth of a large one).  -1 (default): as many
- * rows as workgroups fit the chip at once; 0: always a wave per row. */
-int dnatok_kmer_set_team_rows(int32_t max_rows);
+/* TEST AND MEASUREMENT ONLY (no counterpart in the reference; results are identical either way).
+ * Which of the two k-mer kernels the calls with this table use.  A batch of up to max_rows rows is
+ * encoded with a workgroup per row (four waves share a row: the latency of a small batch), a
+ * larger one with a wave per row (the bandwidth of a large one).  -1 (default): as many rows as
+ * workgroups fit the chip at once; 0: always a wave per row.  The setting belongs to the table
+ * object; a call reads it once when it starts. */
+int dnatok_kmer_table_set_team_rows(dnatok_kmer_t *t, int32_t max_rows);
 
 /* ids int32[n_rows, t_cap], mask uint8[n_rows, t_cap] (NULL allowed): t_cap is the row stride.
  * lengths int32[n_rows] receives each row's token count (also when it exceeds t_cap),
@@ -235,9 +236,10 @@ int dnatok_bpe_encode_padded(const dnatok_bpe_t *t, const uint8_t *bytes, const 
                              int32_t *ids, uint8_t *mask, int32_t *lengths, int32_t *longest,
                              void *stream);
 
-/* Longest row, in bytes, that dnatok_bpe_encode_padded writes without tok_tmp (the size of an
- * extended chunk: dnatok_bpe_set_chunk_geometry changes it). */
-int64_t dnatok_bpe_padded_direct_max(void);
+/* Longest row, in bytes, that dnatok_bpe_encode_padded writes without tok_tmp with this table
+ * (the size of an extended chunk, 2048 unless dnatok_bpe_table_set_chunk_geometry changed it;
+ * t = NULL: the shipped value). */
+int64_t dnatok_bpe_padded_direct_max(const dnatok_bpe_t *t);
 
 /* The same encode for callers that cannot allocate device memory or hand over a work buffer: code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
@@ -257,22 +259,23 @@ int dnatok_bpe_encode_static(const dnatok_bpe_t *t, const uint8_t *bytes, const 
                              int64_t n_rows, int64_t max_len, int64_t total,
                              int32_t *tok_tmp, int32_t *lengths, void *stream);
 
-/* Test hook, no counterpart in the reference: sets the geometry the calls that follow (in this
- * process) cut rows longer than core + 2 * overlap bytes with: chunks of `core` bytes, extended by
- * `overlap` bytes on both sides, joined at seams inside the overlaps.  The shipped geometry is
- * (1792, 128); (0, 0) restores it.  Tests pass small chunks so that rows of a few kilobytes go
- * through thousands of seams and whole-row fallbacks.  Results never depend on the geometry.
- * Not synchronised with encode calls in flight on other threads. */
-int dnatok_bpe_set_chunk_geometry(int32_t core, int32_t overlap);
+/* TEST ONLY, no counterpart in the reference: the geometry the calls with this table cut rows
+ * longer than core + 2 * overlap bytes with: chunks of `core` bytes, extended by `overlap` bytes on
+ * both sides, joined at seams inside the overlaps.  The shipped geometry is (1792, 128); (0, 0)
+ * restores it.  Tests pass small chunks so that rows of a few kilobytes go through thousands of
+ * seams and whole-row fallbacks.  Results never depend on the geometry.  The setting belongs to the
+ * table object; a call reads it once when it starts (size the scratch buffer after setting it). */
+int dnatok_bpe_table_set_chunk_geometry(dnatok_bpe_t *t, int32_t core, int32_t overlap);
 
-/* Where the merge table of the calls that follow is kept (process-wide; no counterpart in the
- * reference, whose kernel reads its hash table from global memory, dnatok_bpe.cu:822-837).  A table
- * of at most 8192 symbols and 4095 rules also has a compact form of 48 KB.  mode 0 (default): every
- * batch reads the table from global memory (L2), which measured faster.  mode 1: a batch of rows of
- * at most 1024 bytes, few enough for one row per resident workgroup with those 48 KB added to each,
- * is encoded by workgroups that keep the compact form in LDS.  mode 2: the compact form for every
- * batch of rows of at most 1024 bytes (for measurements).  Results are identical in all modes. */
-int dnatok_bpe_set_table_placement(int32_t mode);
+/* MEASUREMENT ONLY: where the merge table of the calls with this table object is kept (no
+ * counterpart in the reference, whose kernel reads its hash table from global memory,
+ * dnatok_bpe.cu:822-837).  A table of at most 8192 symbols and 4095 rules also has a compact form
+ * of 48 KB.  mode 0 (default): every batch reads the table from global memory (L2), which measured
+ * faster.  mode 1: a batch of rows of at most 1024 bytes, few enough for one row per resident
+ * workgroup with those 48 KB added to each, is encoded by workgroups that keep the compact form in
+ * LDS.  mode 2: the compact form for every batch of rows of at most 1024 bytes that one launch
+ * encodes whole.  Results are identical in all modes. */
+int dnatok_bpe_table_set_placement(dnatok_bpe_t *t, int32_t mode);
 
 /* ---------------------------------------------------------------------------------------
  * Ragged-batch packer: turns per-row token runs (tok_tmp + in_offsets + lengths, as the BPE
@@ -351,23 +354,6 @@ int dnatok_normalize_rows(const dnatok_norm_step *steps_h, int32_t n_steps, cons
                           const int64_t *offsets, int64_t n_rows, int64_t total, int64_t max_len,
                           uint8_t *out_bytes, int64_t out_capacity, int64_t *out_offsets,
                           void *scratch, size_t scratch_bytes, void *stream);
-
-/* ---------------------------------------------------------------------------------------
- * Measurement aids.  No counterpart in the reference: kernels that move memory in a given shape
- * and do nothing else, so that an encoder's rate can be set against what the machine gives that
- * shape (bench.py reports both).
- * ------------------------------------------------------------------------------------- */
-
-/* dst[0 .. bytes) = src[0 .. bytes): a workgroup copies contiguous 16 KB tiles (the fastest plain
- * copy measured on an MI355X).  Both buffers and the size are multiples of 16 bytes. */
-int dnatok_diag_copy_tiles(const void *src, void *dst, size_t bytes, void *stream);
-
-/* The loads and stores of dnatok_kmer_encode_padded's kernel for k = 6 on rows of plain bases,
- * without its arithmetic: rows read in steps of 1536 bytes (24 per lane), len / 6 ids and mask
- * bytes written per row (ids int32[n_rows, t_cap], mask uint8[n_rows, t_cap]; what is written
- * is not a tokenization), the cells up to fill_to as padding.  t_cap is a multiple of 4. */
-int dnatok_diag_kmer_shape(const uint8_t *bytes, const int64_t *offsets, int64_t n_rows,
-                           int64_t t_cap, int64_t fill_to, int32_t *ids, uint8_t *mask, void *stream);
 
 #ifdef __cplusplus
 }

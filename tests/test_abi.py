@@ -35,11 +35,25 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert b"null" in L.dnatok_last_error()
     rc = L.dnatok_kmer_encode_padded(None, None, None, 1, 4, 8, None, None, None, None, None, None)
     assert rc == -1
-    # the entry points that pad BPE rows themselves and the measurement aids check their arguments first as well
+    # the entry point that pads BPE rows itself checks its arguments first as well
     rc = L.dnatok_bpe_encode_padded(None, None, None, 1, 4, 4, None, 0, None, None, 0, 8, None, None, None, None, None)
     assert rc == -1 and b"null" in L.dnatok_last_error()
-    rc = L.dnatok_diag_copy_tiles(None, None, 16, None)
-    assert rc == -1 and b"null" in L.dnatok_last_error()
-    rc = L.dnatok_diag_kmer_shape(None, None, 1, 8, 8, None, None, None)
-    assert rc == -1
-    assert L.dnatok_bpe_padded_direct_max() == 2048
+    assert L.dnatok_bpe_padded_direct_max(None) == 2048
+    # the per-table test switches refuse a null table
+    assert L.dnatok_kmer_table_set_team_rows(None, 0) == -1 and b"null" in L.dnatok_last_error()
+    assert L.dnatok_bpe_table_set_chunk_geometry(None, 256, 32) == -1
+    assert L.dnatok_bpe_table_set_placement(None, 0) == -1
+
+
+def test_measurement_library_is_separate():
+    """bench.py's memory-only kernels live in libdnatok_diag.so (include/dnatok_diag.h), not in the
+    product library."""
+    from dnatok_amd import build
+    assert os.path.exists(build.DIAG_LIB_PATH), "build with: python -m dnatok_amd.build"
+    D = ctypes.CDLL(build.DIAG_LIB_PATH)
+    D.dnatok_last_error.restype = ctypes.c_char_p
+    D.dnatok_diag_copy_tiles.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    assert D.dnatok_diag_copy_tiles(None, None, 16, None) == -1 and b"null" in D.dnatok_last_error()
+    assert D.dnatok_diag_kmer_shape(None, None, 1, 8, 8, None, None, None) == -1
+    P = ctypes.CDLL(_lib.LIB_PATH)
+    assert not hasattr(P, "dnatok_diag_copy_tiles") and not hasattr(P, "dnatok_diag_kmer_shape")

@@ -368,7 +368,8 @@ def test_bpe_backend_with_normalizer():
 def test_bpe_backend_guards_input_it_cannot_reproduce():
     """Without an unk_token the library drops characters outside the vocabulary; with a
     pre-tokenizer it cuts rows at white space.  Rows without such characters are identical, rows
-    with them raise ValueError (DNATok then takes the batch to the tokenizer itself)."""
+    with them raise UnsupportedRows, a ValueError that names them (DNATok catches it and takes those rows
+    to the tokenizer itself: test_dnatok_bpe_rows_the_engine_cannot_reproduce_go_to_the_tokenizer)."""
     import json
     from tokenizers import Tokenizer
     cfg = json.loads(json.dumps(util.tokenizer_json("4096")))
@@ -380,8 +381,9 @@ def test_bpe_backend_guards_input_it_cannot_reproduce():
     ids, mask = be.encode_batch(seqs)
     for i, e in enumerate(tk.encode_batch(seqs, add_special_tokens=False)):
         assert ids[i, :len(e.ids)].tolist() == e.ids and int(mask[i].sum()) == len(e.ids)
-    with pytest.raises(ValueError):
-        be.encode_batch(seqs + ["ACXGT"])
+    with pytest.raises(ValueError) as caught:
+        be.encode_batch(seqs[:3] + ["ACXGT"] + seqs[3:] + ["xx"])
+    assert caught.value.rows == [3, len(seqs) + 1]
     cfg = json.loads(json.dumps(util.tokenizer_json("4096")))
     cfg["pre_tokenizer"] = {"type": "Whitespace"}
     tk = Tokenizer.from_str(json.dumps(cfg))
@@ -571,6 +573,104 @@ def _bpe_wrapped(side):
             return tk.get_vocab()
 
     return Wrapped()
+
+
+def _bpe_wrapped_from(cfg, side):
+    import json
+    from tokenizers import Tokenizer
+    tk = Tokenizer.from_str(json.dumps(cfg))
+
+    class Wrapped:
+        pad_token_id, padding_side = 3, side
+        unk_token_id = 0 if cfg["model"].get("unk_token") is not None else None
+        backend_tokenizer = tk
+
+        def __call__(self, texts, add_special_tokens=False, **kw):
+            return {"input_ids": [e.ids for e in tk.encode_batch(list(texts), add_special_tokens=False)]}
+
+        def get_vocab(self):
+            return tk.get_vocab()
+
+    return Wrapped()
+
+
+@pytest.mark.parametrize("side", ["left", "right"])
+@pytest.mark.parametrize("kind", ["whitespace", "no_unk"])
+def test_dnatok_bpe_rows_the_engine_cannot_reproduce_go_to_the_tokenizer(kind, side, caplog):
+    """The reference's DNATok never raises on a BPE batch: whatever its backend cannot do ends at
+    the tokenizer itself (src/dna_tokenizer.py:2066-2100).  Here the backend names the rows it cannot
+    reproduce (white space under a pre-tokenizer, which cuts the row into words; a character outside
+    the vocabulary without unk_token, which is dropped); those rows get the tokenizer's ids, the
+    others stay on the GPU.  Expected in every case: the tokenizer's own rows, padded in plain
+    Python on the tokenizer's side."""
+    import json
+    import logging
+    cfg = json.loads(json.dumps(util.tokenizer_json("4096")))
+    if kind == "whitespace":
+        cfg["pre_tokenizer"] = {"type": "Whitespace"}
+        odd = ["ACGT ACGTTTGA", "A C G T", " ACGTAC", "ACGTACGTAGCTAGCTAGCATCGATCGATCGACTAGCTAGCTAC\nACGT" * 30]
+    else:
+        cfg["model"]["unk_token"] = None
+        odd = ["ACXGT", "xxxx", "ACGTACGTAGCTAGCTAGCATCGATCGATCGACTAGCTAGCTAC" * 30 + "acgt", "ACGTNNNNRY"]
+    tok = _bpe_wrapped_from(cfg, side)
+    h = DNATok(RecordingEmbedder(tok, vocab=8192), padding_side=side)
+    h.discover()
+    assert h.bpe_backend is not None and h.bpe_backend._input_guard is not None
+    clean = random_seqs(9, 300, alphabet="ACGT", seed=31) + ["ACGTACGTACGT", "A"]
+    mixed = clean[:4] + odd[:2] + clean[4:] + odd[2:]
+    for seqs, n_odd in ((clean, 0), (mixed, len(odd)), (odd, len(odd)), ([odd[0]], 1), (clean, 0)):
+        caplog.clear()
+        with caplog.at_level(logging.WARNING, logger=h.log.name):
+            want = h._tokenize_batch_cpu(seqs)
+            got = h.encode_batch_to_ids(seqs)
+            assert got.dtype == torch.int64 and got.shape == want.shape and torch.equal(got, want), (kind, side)
+            ids, mask = h.encode_batch_device(seqs)
+            assert ids.is_cuda and ids.dtype == torch.int32 and torch.equal(ids.cpu().long(), want)
+            lens = torch.tensor([len(r) for r in h._tok_ids(seqs)])
+            col = torch.arange(want.shape[1])[None, :]
+            inside = (col >= want.shape[1] - lens[:, None]) if side == "left" else (col < lens[:, None])
+            assert torch.equal(mask.cpu().bool(), inside)
+            ids8, mask8 = h.encode_batch_with_padding(seqs, 10_000, pad_to_max=False, pad_multiple=8)
+            assert ids8.shape[1] % 8 == 0 and ids8.shape[1] - want.shape[1] in range(8)
+            for i, n in enumerate(lens.tolist()):
+                sl = slice(ids8.shape[1] - n, ids8.shape[1]) if side == "left" else slice(0, n)
+                assert ids8[i, sl].cpu().long().tolist() == h._tok_ids([seqs[i]])[0] and int(mask8[i].sum()) == n
+        warned = [r for r in caplog.records if "tokenizer" in r.getMessage()]
+        assert bool(warned) == bool(n_odd), (kind, side, n_odd, [r.getMessage() for r in caplog.records])
+
+
+@pytest.mark.parametrize("side", ["left", "right"])
+def test_dnatok_bpe_backend_failure_falls_back_to_the_tokenizer(side, monkeypatch, caplog):
+    """Fault injection as in the reference's tests/test_bytes_path_fallback.py:56-75: the backend's
+    entry points raise, and DNATok answers with the tokenizer's own rows and a warning."""
+    import logging
+    tok = _bpe_wrapped(side)
+    h = DNATok(RecordingEmbedder(tok, vocab=8192), padding_side=side)
+    h.discover()
+    seqs = random_seqs(7, 200, alphabet="ACGT", seed=41) + ["ACGT"]
+    want = h._tokenize_batch_cpu(seqs)
+    assert torch.equal(h.encode_batch_to_ids(seqs), want)
+
+    def boom(*args, **kwargs):
+        raise RuntimeError("forced failure")
+
+    monkeypatch.setattr(h.bpe_backend, "padded_device", boom)
+    monkeypatch.setattr(h.bpe_backend, "tokens_device", boom)
+    with caplog.at_level(logging.WARNING, logger=h.log.name):
+        got = h.encode_batch_to_ids(seqs)
+        ids, mask = h.encode_batch_device(seqs)
+    assert torch.equal(got, want) and torch.equal(ids.cpu().long(), want)
+    assert torch.equal(mask.cpu().bool(), want != 3)
+    assert any("forced failure" in r.getMessage() for r in caplog.records)
+    # a failed row (negative length from the engine) ends the same way
+    monkeypatch.undo()
+
+    def failed_row(*args, **kwargs):
+        raise RuntimeError("BPE engine reported a failed row (negative length)")
+
+    monkeypatch.setattr(h, "_pad_bpe_runs", failed_row)
+    monkeypatch.setattr(h.bpe_backend, "padded_device", failed_row)
+    assert torch.equal(h.encode_batch_to_ids(seqs), want)
 
 
 @pytest.mark.parametrize("side", ["left", "right"])

@@ -176,13 +176,22 @@ def test_char_c5_packed(char_enc):
 # ----------------------------------------------------------------- k-mer
 
 @pytest.fixture
-def kmer_kernel_choice(request):
+def kmer_kernel_choice(request, monkeypatch):
     """Which k-mer kernel the test's batches get: a wave per row (forced for all batches) or the
-    automatic choice, which gives the batches of these tests a workgroup per row."""
-    from dnatok_amd import _lib
-    _lib.lib().dnatok_kmer_set_team_rows(0 if request.param == "rows_by_wave" else -1)
+    automatic choice, which gives the batches of these tests a workgroup per row.  The switch
+    belongs to the table object, so every encoder is set before each of its calls."""
+    rows = 0 if request.param == "rows_by_wave" else -1
+    plain = encoders.KmerEncoder.encode_padded
+
+    def encode_padded(self, *args, **kwargs):
+        self.set_team_rows(rows)
+        try:
+            return plain(self, *args, **kwargs)
+        finally:
+            self.set_team_rows(-1)
+
+    monkeypatch.setattr(encoders.KmerEncoder, "encode_padded", encode_padded)
     yield request.param
-    _lib.lib().dnatok_kmer_set_team_rows(-1)
 
 
 both_kmer_kernels = pytest.mark.parametrize("kmer_kernel_choice", ["rows_by_wave", "rows_by_workgroup"], indirect=True)
@@ -979,10 +988,8 @@ def test_bpe_small_chunks_many_seams_and_fallbacks(bpe, core, overlap):
     kernel.  Every row is compared with the oracle."""
     which, enc, bo = bpe
     say(f"bpe{which} chunks of {core} + 2 x {overlap}")
-    from dnatok_amd import _lib
-    L = _lib.lib()
     ext = core + 2 * overlap
-    _lib.check(L.dnatok_bpe_set_chunk_geometry(core, overlap), "dnatok_bpe_set_chunk_geometry")
+    enc.set_chunk_geometry(core, overlap)
     try:
         rng = random.Random(int(which) + core)
         n_rows = n_chunked = n_failed = 0
@@ -1005,7 +1012,7 @@ def test_bpe_small_chunks_many_seams_and_fallbacks(bpe, core, overlap):
         say(f"  {n_rows} rows, {n_chunked} chunked, {n_failed} redone by the whole-row kernel")
         assert n_rows >= 2000 and 0 < n_failed < n_chunked       # seams accepted and seams refused
     finally:
-        _lib.check(L.dnatok_bpe_set_chunk_geometry(0, 0), "dnatok_bpe_set_chunk_geometry")
+        enc.set_chunk_geometry(0, 0)
 
 
 def test_bpe_compact_table_in_lds_gives_the_same_tokens():
@@ -1024,16 +1031,26 @@ def test_bpe_compact_table_in_lds_gives_the_same_tokens():
             for _ in range(300)] + ["A" * 1024, "AC" * 512, ""]
     small = util.batch_from_strings(seqs)
     want = [np.asarray(r) for r in bo.encode_batch(small.data, small.offsets)]
-    place = _lib.lib().dnatok_bpe_set_table_placement
+    # many mostly short rows with some of 600-1000 bytes among them: the batch is split between two
+    # launches that share a work list, which the compact form (one launch, no list) must stay out of
+    rng2 = random.Random(6)
+    split_seqs = ["".join(rng2.choice("ACGT") for _ in range(rng2.randint(20, 300))) for _ in range(1500)]
+    for at in range(0, 1500, 60):
+        split_seqs[at] = "".join(rng2.choice("ACGT") for _ in range(rng2.randint(600, 1000)))
+    split = util.batch_from_strings(split_seqs)
+    want_split = [np.asarray(r) for r in bo.encode_batch(split.data, split.offsets)]
     try:
         for mode in (0, 1, 2):
-            assert place(mode) == 0
+            enc.set_table_placement(mode)
             for s, r, e in zip(seqs, bpe_rows(enc, small), want):
                 np.testing.assert_array_equal(r, e, err_msg=f"mode {mode}: {s[:20]}")
             util.check_against_golden("C3_bpe4096", bpe_rows(enc, wl.config3_bpe4096()))
-        assert place(3) != 0
+            for i, (r, e) in enumerate(zip(bpe_rows(enc, split), want_split)):
+                np.testing.assert_array_equal(r, e, err_msg=f"mode {mode}: split batch row {i}")
+        with pytest.raises(_lib.DnatokError):
+            enc.set_table_placement(3)
     finally:
-        place(0)
+        enc.set_table_placement(0)
 
 
 def test_bpe_c4_golden():
