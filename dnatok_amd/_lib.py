@@ -21,7 +21,7 @@ EXPORTS = [
     "dnatok_char_unpack_2bit", "dnatok_host_clean_ascii", "dnatok_host_pack_2bit", "dnatok_host_fasta_scan",
     "dnatok_kmer_table_create", "dnatok_kmer_table_destroy", "dnatok_kmer_table_set_team_rows", "dnatok_kmer_encode_padded",
     "dnatok_bpe_table_create", "dnatok_bpe_table_destroy", "dnatok_bpe_scratch_bytes",
-    "dnatok_bpe_encode", "dnatok_bpe_encode_with_chars", "dnatok_bpe_encode_padded", "dnatok_bpe_padded_direct_max",
+    "dnatok_bpe_encode", "dnatok_bpe_encode_with_chars", "dnatok_bpe_encode_padded", "dnatok_bpe_encode_padded_as", "dnatok_bpe_padded_direct_max",
     "dnatok_bpe_static_scratch_bytes", "dnatok_bpe_encode_static",
     "dnatok_bpe_table_set_chunk_geometry", "dnatok_bpe_table_set_placement", "dnatok_pack_ragged", "dnatok_pad_rows", "dnatok_pad_rows_as",
     "dnatok_normalize_bounds", "dnatok_normalize_rows",
@@ -107,6 +107,9 @@ def lib() -> ctypes.CDLL:
     L.dnatok_bpe_encode_padded.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                            c_void_p, c_size_t, c_void_p, c_void_p, c_int32, c_int64,
                                            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    L.dnatok_bpe_encode_padded_as.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                                              c_void_p, c_size_t, c_void_p, c_void_p, c_int32, c_int64, c_int,
+                                              c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]
     L.dnatok_bpe_padded_direct_max.argtypes = [c_void_p]
     L.dnatok_bpe_padded_direct_max.restype = c_int64
     L.dnatok_bpe_static_scratch_bytes.restype = c_size_t

@@ -87,7 +87,8 @@ struct BpeArgs {
     // ids go to pad_ids[b * pad_stride ..], through pad_remap when given, pad_id behind them up to
     // the stride, 1 / 0 to pad_mask (null: no mask); the longest row's token count goes up max_tree
     // (null: the caller finds it from the lengths) into *longest
-    int32_t *pad_ids;
+    void *pad_ids;               // [n_rows, pad_stride] of pad_elem-byte integers (1, 2, 4 or 8)
+    int32_t pad_elem, pad_left;  // pad_left: a row's tokens end at its last cell instead of starting at its first
     uint8_t *pad_mask;
     const int32_t *pad_remap;
     int64_t pad_stride;
@@ -291,7 +292,7 @@ __device__ __forceinline__ int32_t bpe_row(
     const int32_t *__restrict__ char_lut = nullptr, int32_t *__restrict__ char_ids = nullptr,
     uint8_t *__restrict__ char_mask = nullptr, const int char_lo = 0, const int char_hi = 0,
     const int pad_stride = 0, const int32_t pad_id = 0, uint8_t *__restrict__ pad_mask = nullptr,
-    const int32_t *__restrict__ remap2 = nullptr)
+    const int32_t *__restrict__ remap2 = nullptr, const int pad_elem = 4, const int pad_left = 0)
 {
     static_assert(!CHARS || PER > 0, "the single-character ids are written from the staged bytes");
     constexpr IT NIL = (IT)~(IT)0;
@@ -742,6 +743,21 @@ __device__ __forceinline__ int32_t bpe_row(
     uint32_t *wave_cnt = reinterpret_cast<uint32_t *>(NS);           // [kBlockPasses][NW]
     const int lane = tid & 63;
     uint32_t done = 0;                                               // tokens of earlier blocks of passes
+    // cell c of a padded row, in the row's own integer width
+    auto put_cell = [&](int c, int32_t v) {
+        if (!PAD || pad_elem == 4) out[c] = v;
+        else if (pad_elem == 8) reinterpret_cast<int64_t *>(out)[c] = (int64_t)v;
+        else if (pad_elem == 2) reinterpret_cast<int16_t *>(out)[c] = (int16_t)v;
+        else reinterpret_cast<uint8_t *>(out)[c] = (uint8_t)v;
+    };
+    // padding on the left: the row's tokens end at its last cell, so their number comes first
+    int shift = 0;
+    if (PAD && pad_left) {
+        uint32_t mine = 0, total;
+        for (int i = tid; i < n0; i += NT) mine += (uint32_t)(P[i].s != DEAD);
+        (void)team_exclusive_sum<NT>(mine, red, wv, total);
+        shift = pad_stride - (int)(total < (uint32_t)pad_stride ? total : (uint32_t)pad_stride);
+    }
     for (int i0 = 0; i0 < n0; i0 += kBlockPasses * NT) {
         uint32_t sy[kBlockPasses], before[kBlockPasses];
 #pragma unroll
@@ -767,7 +783,7 @@ __device__ __forceinline__ int32_t bpe_row(
             if (sy[k] != kNone && (!PAD || cell < (uint32_t)pad_stride)) {
                 int32_t id = out_remap ? out_remap[sy[k]] : (int32_t)sy[k];
                 if (PAD && remap2) id = remap2[id];
-                out[cell] = id;
+                put_cell(shift + (int)cell, id);
             }
         }
         done = at;
@@ -776,9 +792,10 @@ __device__ __forceinline__ int32_t bpe_row(
     if (tid == 0) *out_len = stuck ? -2 : (int32_t)done;
     if (PAD) {
         const int kept = (int)done < pad_stride ? (int)done : pad_stride;
-        for (int i = kept + tid; i < pad_stride; i += NT) out[i] = pad_id;
+        const int pad_from = pad_left ? 0 : kept, pad_to = pad_left ? pad_stride - kept : pad_stride;
+        for (int i = pad_from + tid; i < pad_to; i += NT) put_cell(i, pad_id);
         if (pad_mask)
-            for (int i = tid; i < pad_stride; i += NT) pad_mask[i] = i < kept ? 1 : 0;
+            for (int i = tid; i < pad_stride; i += NT) pad_mask[i] = (i >= pad_from && i < pad_to) ? 0 : 1;
     }
     return (int32_t)done;
 }
@@ -1185,8 +1202,12 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
             if (tid == 0) lengths[row] = len > CAP ? -1 : 0;
             if (padded) {
                 for (int64_t i = tid; i < a.pad_stride; i += NT) {
-                    a.pad_ids[(int64_t)row * a.pad_stride + i] = a.pad_id;
-                    if (a.pad_mask) a.pad_mask[(int64_t)row * a.pad_stride + i] = 0;
+                    const int64_t at = (int64_t)row * a.pad_stride + i;
+                    if (a.pad_elem == 4) reinterpret_cast<int32_t *>(a.pad_ids)[at] = a.pad_id;
+                    else if (a.pad_elem == 8) reinterpret_cast<int64_t *>(a.pad_ids)[at] = (int64_t)a.pad_id;
+                    else if (a.pad_elem == 2) reinterpret_cast<int16_t *>(a.pad_ids)[at] = (int16_t)a.pad_id;
+                    else reinterpret_cast<uint8_t *>(a.pad_ids)[at] = (uint8_t)a.pad_id;
+                    if (a.pad_mask) a.pad_mask[at] = 0;
                 }
             }
             if (CHARS) {
@@ -1202,11 +1223,14 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
             else {
                 const int32_t n_tok = bpe_row<NT, uint16_t, (CAP + NT - 1) / NT, CHARS, PADDED>(
                     pt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC, Q, C, D, red, tid,
-                    padded ? a.pad_ids + (int64_t)row * a.pad_stride : tok_tmp + start,
+                    padded ? reinterpret_cast<int32_t *>(reinterpret_cast<char *>(a.pad_ids) +
+                                                         (int64_t)row * a.pad_stride * a.pad_elem)
+                           : tok_tmp + start,
                     lengths + row, nullptr, 0, 0, nullptr, a.char_lut, CHARS ? a.char_ids + start : nullptr,
                     CHARS && a.char_mask ? a.char_mask + start : nullptr, 0, (int)len,
                     padded ? (int)a.pad_stride : 0, a.pad_id,
-                    padded && a.pad_mask ? a.pad_mask + (int64_t)row * a.pad_stride : nullptr, a.pad_remap);
+                    padded && a.pad_mask ? a.pad_mask + (int64_t)row * a.pad_stride : nullptr, a.pad_remap,
+                    padded ? a.pad_elem : 4, padded ? a.pad_left : 0);
                 team_longest = n_tok > team_longest ? n_tok : team_longest;
             }
         } else if (CHUNKS) {
@@ -1813,6 +1837,7 @@ static int bpe_encode_launch(const dnatok_bpe_t *t, const uint8_t *bytes, const 
     a.placement = t->placement.load(std::memory_order_relaxed);
     if (padded) {
         a.pad_ids = padded->pad_ids; a.pad_mask = padded->pad_mask; a.pad_remap = padded->pad_remap;
+        a.pad_elem = padded->pad_elem; a.pad_left = padded->pad_left;
         a.pad_stride = padded->pad_stride; a.pad_id = padded->pad_id;
         a.max_tree = padded->max_tree; a.longest = padded->longest;
     }
@@ -1925,13 +1950,15 @@ extern "C" int64_t dnatok_bpe_padded_direct_max(const dnatok_bpe_t *t)
     return (int64_t)core + 2 * overlap;
 }
 
-extern "C" int dnatok_bpe_encode_padded(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets,
-                                        int64_t n_rows, int64_t max_len, int64_t total, void *scratch,
-                                        size_t scratch_bytes, int32_t *tok_tmp, const int32_t *remap, int32_t pad_id,
-                                        int64_t stride, int32_t *ids, uint8_t *mask, int32_t *lengths,
-                                        int32_t *longest, void *stream)
+extern "C" int dnatok_bpe_encode_padded_as(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets,
+                                           int64_t n_rows, int64_t max_len, int64_t total, void *scratch,
+                                           size_t scratch_bytes, int32_t *tok_tmp, const int32_t *remap, int32_t pad_id,
+                                           int64_t stride, int pad_left, void *ids, int32_t id_bytes, uint8_t *mask,
+                                           int32_t *lengths, int32_t *longest, void *stream)
 {
-    static const char *who = "dnatok_bpe_encode_padded";
+    static const char *who = "dnatok_bpe_encode_padded_as";
+    DNATOK_REQUIRE(id_bytes == 1 || id_bytes == 2 || id_bytes == 4 || id_bytes == 8, DNATOK_E_INVALID,
+                   "%s: id_bytes must be 1, 2, 4 or 8", who);
     DNATOK_REQUIRE(t && offsets && (lengths || n_rows == 0), DNATOK_E_INVALID, "%s: null argument", who);
     DNATOK_REQUIRE(n_rows >= 0 && max_len >= 0 && total >= 0, DNATOK_E_INVALID, "%s: negative size", who);
     DNATOK_REQUIRE(max_len < (int64_t)1 << 31 && total / 256 + n_rows < (int64_t)1 << 30, DNATOK_E_TOO_LARGE,
@@ -1962,11 +1989,12 @@ extern "C" int dnatok_bpe_encode_padded(const dnatok_bpe_t *t, const uint8_t *by
             bpe_longest_kernel<<<1, 1024, 0, s>>>(lengths, n_rows, longest);
             DNATOK_HIP_TRY(hipGetLastError());
         }
-        return dnatok_pad_rows(tok_tmp, offsets, lengths, n_rows, remap, pad_id, stride, stride, ids, mask, nullptr,
-                               stream);
+        return dnatok_pad_rows_as(tok_tmp, offsets, lengths, n_rows, remap, pad_id, stride, stride, 0, 0,
+                                  pad_left ? 1 : 0, ids, id_bytes, mask, nullptr, nullptr, stream);
     }
     BpeArgs pad{};
     pad.pad_ids = ids; pad.pad_mask = mask; pad.pad_remap = remap; pad.pad_stride = stride; pad.pad_id = pad_id;
+    pad.pad_elem = id_bytes; pad.pad_left = pad_left ? 1 : 0;
     pad.longest = longest;
     if (longest) {
         std::lock_guard<std::mutex> hold(t->slot_lock);
@@ -1983,6 +2011,16 @@ extern "C" int dnatok_bpe_encode_padded(const dnatok_bpe_t *t, const uint8_t *by
         DNATOK_HIP_TRY(hipGetLastError());
     }
     return DNATOK_OK;
+}
+
+extern "C" int dnatok_bpe_encode_padded(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets,
+                                        int64_t n_rows, int64_t max_len, int64_t total, void *scratch,
+                                        size_t scratch_bytes, int32_t *tok_tmp, const int32_t *remap, int32_t pad_id,
+                                        int64_t stride, int32_t *ids, uint8_t *mask, int32_t *lengths,
+                                        int32_t *longest, void *stream)
+{
+    return dnatok_bpe_encode_padded_as(t, bytes, offsets, n_rows, max_len, total, scratch, scratch_bytes, tok_tmp, remap,
+                                       pad_id, stride, 0, ids, 4, mask, lengths, longest, stream);
 }
 
 // ---- the entry point that allocates nothing -------------------------------------------------

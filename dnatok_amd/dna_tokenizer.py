@@ -444,26 +444,24 @@ class DNATok:
 
     def _bpe_rows_on_gpu(self, seqs: List[str], device, *, dtype: torch.dtype, min_width: int,
                          pad_multiple: int, host_ids: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+        # the engine pads the rows itself while it writes them out: side, width and id type are final
         left = self.padding_side == "left"
-        if not left and dtype == torch.int32:
-            # the engine pads the rows itself while it writes them out
-            staged = []
+        staged = []
 
-            def stage(ids):
-                if host_ids:
-                    nbytes = ids.numel() * ids.element_size()
-                    host = self._pinned(nbytes)[:nbytes].view(ids.dtype).view(ids.shape)
-                    host.copy_(ids, non_blocking=True)
-                    staged[:] = [host]
+        def stage(ids):
+            if host_ids:
+                nbytes = ids.numel() * ids.element_size()
+                host = self._pinned(nbytes)[:nbytes].view(ids.dtype).view(ids.shape)
+                host.copy_(ids, non_blocking=True)
+                staged[:] = [host]
 
-            ids, mask = self.bpe_backend.padded_device(seqs, device=device, min_width=min_width,
-                                                       pad_multiple=pad_multiple, stage_ids=stage)
-            if staged and staged[0].shape[1] == ids.stride(0):      # (not those of a first, too narrow, try)
-                self._staged_host_ids = staged[0][:, :ids.shape[1]]
-            return ids, mask
-        tok, offsets, lengths, t_cap = self.bpe_backend.tokens_device(seqs, device=device, meta_tail=2)
-        return self._pad_bpe_runs(tok, offsets, lengths, t_cap, dtype=dtype, min_width=min_width,
-                                  pad_multiple=pad_multiple, host_ids=host_ids, stats_behind_lengths=True)
+        ids, mask = self.bpe_backend.padded_device(seqs, device=device, min_width=min_width,
+                                                   pad_multiple=pad_multiple, stage_ids=stage,
+                                                   pad_left=left, dtype=dtype)
+        if staged and staged[0].shape[1] == ids.stride(0):      # (not those of a first, too narrow, try)
+            cap, width = staged[0].shape[1], ids.shape[1]
+            self._staged_host_ids = staged[0][:, cap - width:] if left else staged[0][:, :width]
+        return ids, mask
 
     def _pad_bpe_runs(self, tok, offsets, lengths, t_cap: int, *, dtype, min_width: int, pad_multiple: int,
                       host_ids: bool = False, stats_behind_lengths: bool = False):

@@ -65,10 +65,13 @@ class DnatokBpeKernel:
         return self._impl.encoder.encode(data, offsets, max_len, lengths=lengths)
 
     def tokenize_padded_device(self, data: torch.Tensor, offsets: torch.Tensor, max_len: int, stride: int,
-                               pad_id: int, *, remap: Optional[torch.Tensor] = None, out=None):
-        """Device-resident entry with the padding done by the engine: (ids int32 [B, stride], mask
-        uint8 [B, stride], lengths int32 [B], longest int32 [1]); see ``BpeEncoder.encode_padded``."""
-        return self._impl.encoder.encode_padded(data, offsets, max_len, stride, pad_id, remap=remap, out=out)
+                               pad_id: int, *, remap: Optional[torch.Tensor] = None, out=None,
+                               pad_left: bool = False):
+        """Device-resident entry with the padding done by the engine: (ids [B, stride] of the type
+        of ``out``'s ids (int32 without ``out``), mask uint8 [B, stride], lengths int32 [B], longest
+        int32 [1]); see ``BpeEncoder.encode_padded``."""
+        return self._impl.encoder.encode_padded(data, offsets, max_len, stride, pad_id, remap=remap, out=out,
+                                                pad_left=pad_left)
 
     def tokenize_batch(self, texts: Sequence[str], *, clone: bool = False
                        ) -> Tuple[torch.Tensor, torch.Tensor]:

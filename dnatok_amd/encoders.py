@@ -470,9 +470,11 @@ class BpeEncoder:
 
     def encode_padded(self, data: torch.Tensor, offsets: torch.Tensor, max_len: int, stride: int, pad_id: int, *,
                       remap: Optional[torch.Tensor] = None, want_mask: bool = True, want_longest: bool = True,
-                      out=None, tok_tmp: Optional[torch.Tensor] = None):
-        """Engine and padding in one pass: ``ids[B, stride]`` int32 (through ``remap``, ``pad_id``
-        behind a row's tokens), ``mask[B, stride]`` uint8, ``lengths[B]`` (full token counts) and
+                      out=None, tok_tmp: Optional[torch.Tensor] = None, pad_left: bool = False,
+                      dtype: torch.dtype = torch.int32):
+        """Engine and padding in one pass: ``ids[B, stride]`` of ``dtype`` (uint8, int16, int32 or
+        int64; through ``remap``, ``pad_id`` behind a row's tokens -- with ``pad_left`` before them,
+        the tokens ending at the row's last cell), ``mask[B, stride]`` uint8, ``lengths[B]`` (full token counts) and
         ``longest[1]`` (their maximum; None with ``want_longest=False`` or in ``out``: the caller takes it
         from the lengths), all on the device.  A row with more tokens than ``stride``
         keeps its first ``stride``: compare ``longest`` with it.  ``out`` = (ids, mask, lengths,
@@ -485,7 +487,7 @@ class BpeEncoder:
         dev = data.device
         stride = int(stride)
         if out is None:
-            ids = torch.empty((n_rows, stride), dtype=torch.int32, device=dev)
+            ids = torch.empty((n_rows, stride), dtype=dtype, device=dev)
             mask = torch.empty((n_rows, stride), dtype=torch.uint8, device=dev) if want_mask else None
             lengths = torch.empty(n_rows, dtype=torch.int32, device=dev)
             longest = torch.empty(1, dtype=torch.int32, device=dev) if want_longest else None
@@ -493,14 +495,17 @@ class BpeEncoder:
             ids, mask, lengths, longest = out
             if ids.shape != (n_rows, stride) or not ids.is_contiguous():
                 raise ValueError("ids must be a contiguous [n_rows, stride] tensor")
+        if ids.dtype not in (torch.uint8, torch.int16, torch.int32, torch.int64):
+            raise ValueError("ids must be uint8, int16, int32 or int64")
         if int(max_len) > self.padded_direct_max() and tok_tmp is None:
             tok_tmp = torch.empty(max(total, 1), dtype=torch.int32, device=dev)
         scratch = self._get_scratch(n_rows, int(max_len), total, dev)
-        _lib.check(_lib.lib().dnatok_bpe_encode_padded(
+        _lib.check(_lib.lib().dnatok_bpe_encode_padded_as(
             self._h, _ptr(data), _ptr(offsets), n_rows, int(max_len), total, _ptr(scratch), scratch.numel(),
             _ptr(tok_tmp) if tok_tmp is not None else None, _ptr(remap) if remap is not None else None,
-            int(pad_id), stride, _ptr(ids), _ptr(mask) if mask is not None else None, _ptr(lengths), _ptr(longest),
-            _stream()), "dnatok_bpe_encode_padded")
+            int(pad_id), stride, 1 if pad_left else 0, _ptr(ids), ids.element_size(),
+            _ptr(mask) if mask is not None else None, _ptr(lengths), _ptr(longest),
+            _stream()), "dnatok_bpe_encode_padded_as")
         return ids, mask, lengths, longest
 
     def padded_direct_max(self) -> int:

@@ -449,10 +449,12 @@ class GPUTokBPEBackend:
         return tok, offsets, lengths, t_cap
 
     def padded_device(self, seqs: List[str], *, device: object = "cuda", min_width: int = 0,
-                      pad_multiple: int = 1, stage_ids=None) -> Tuple[torch.Tensor, torch.Tensor]:
-        """Strings -> ``(ids int32 [B, T], mask uint8 [B, T])`` on the device, tokenizer ids, padded
-        on the right with ``pad_id`` to the longest row (at least ``min_width``, a multiple of
-        ``pad_multiple``): one engine launch writes the padded rows (``dnatok_bpe_encode_padded``),
+                      pad_multiple: int = 1, stage_ids=None, pad_left: bool = False,
+                      dtype: torch.dtype = torch.int32) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Strings -> ``(ids [B, T] of dtype, mask uint8 [B, T])`` on the device, tokenizer ids, padded
+        with ``pad_id`` (on the right, or with ``pad_left`` on the left) to the longest row (at least
+        ``min_width``, a multiple of ``pad_multiple``): one engine launch writes the padded rows in
+        their final type and on their final side (``dnatok_bpe_encode_padded_as``),
         one copy brings the lengths to the host.  The rows are laid out only as
         far apart as the recent batches of this backend were wide (``encoders.WidthGuess``); a batch
         that needs more room is encoded again with room for the worst case (a token per byte).
@@ -471,10 +473,10 @@ class GPUTokBPEBackend:
         lengths = torch.empty(n, dtype=torch.int32, device=dev)
         while True:
             # (no longest row from the device: the lengths come down anyway, and the launch ends earlier without it)
-            out = (torch.empty((n, cap), dtype=torch.int32, device=dev),
+            out = (torch.empty((n, cap), dtype=dtype, device=dev),
                    torch.empty((n, cap), dtype=torch.uint8, device=dev), lengths, None)
             ids, mask, _, _ = self._dnatok.tokenize_padded_device(data, offsets, t_cap, cap, int(self.pad_id),
-                                                                  remap=self._remap_on(dev), out=out)
+                                                                  remap=self._remap_on(dev), out=out, pad_left=pad_left)
             if stage_ids is not None and cap < worst:
                 stage_ids(ids)
             lengths_h = lengths.cpu().numpy()                            # (the one wait)
@@ -486,12 +488,16 @@ class GPUTokBPEBackend:
             cap = worst                                  # a row was cut: once more, with room for all
         self._widths.update(longest)
         width = min(rounded(max(longest, int(min_width))), cap)
+        if pad_left:                                     # (the rows' tokens end at the stride's last cell)
+            return ids[:, cap - width:], mask[:, cap - width:]
         return ids[:, :width], mask[:, :width]
 
     def encode_batch(self, seqs: List[str], *, device: object = "cuda"
                      ) -> Tuple[torch.Tensor, torch.Tensor]:
-        ids32, mask = self.padded_device(seqs, device=device)
-        return ids32.to(torch.long), mask.contiguous()
+        """(ids int64 [B, L] padded with the tokenizer's pad id, mask uint8 [B, L]), as the reference
+        returns them (src/gputok_bpe_backend.py:489, 581-600); the engine writes int64 itself."""
+        ids, mask = self.padded_device(seqs, device=device, dtype=torch.long)
+        return ids, mask
 
     def encode_batch_ids_only(self, seqs: List[str], *, device: object = "cuda") -> torch.Tensor:
         ids, _ = self.encode_batch(seqs, device=device)

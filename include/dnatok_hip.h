@@ -236,6 +236,21 @@ int dnatok_bpe_encode_padded(const dnatok_bpe_t *t, const uint8_t *bytes, const 
                              int32_t *ids, uint8_t *mask, int32_t *lengths, int32_t *longest,
                              void *stream);
 
+/* The same with the two layout choices DNATok and GPUTokBPEBackend make after the encode, so that
+ * the engine's launch writes the final tensor: ids = [n_rows, stride] of id_bytes-wide integers
+ * (1: uint8, 2: int16, 4: int32, 8: int64 -- the reference's backend returns int64,
+ * src/gputok_bpe_backend.py:581-600; DNATok.encode_batch_with_padding the narrowest type that holds
+ * the vocabulary, src/dna_tokenizer.py:2150-2236), and pad_left = 1 puts a row's tokens at the END
+ * of its `stride` cells with the padding before them (src/dna_tokenizer.py:2072-2078 re-pads the
+ * backend's rows to padding_side): the caller views the last `width` columns.  A row with more tokens
+ * than the stride keeps its first `stride` either way. */
+int dnatok_bpe_encode_padded_as(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets,
+                                int64_t n_rows, int64_t max_len, int64_t total,
+                                void *scratch, size_t scratch_bytes, int32_t *tok_tmp,
+                                const int32_t *remap, int32_t pad_id, int64_t stride, int pad_left,
+                                void *ids, int32_t id_bytes, uint8_t *mask, int32_t *lengths,
+                                int32_t *longest, void *stream);
+
 /* Longest row, in bytes, that dnatok_bpe_encode_padded writes without tok_tmp with this table
  * (the size of an extended chunk, 2048 unless dnatok_bpe_table_set_chunk_geometry changed it;
  * t = NULL: the shipped value). */

@@ -832,6 +832,45 @@ def test_bpe_padded_in_one_pass(bpe):
     check_padded(enc, bo, long_rows, 300, ref=ref)
 
 
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.int16, torch.int32, torch.int64])
+@pytest.mark.parametrize("pad_left", [False, True])
+def test_bpe_padded_in_every_layout(bpe, dtype, pad_left):
+    """dnatok_bpe_encode_padded_as: the engine's launch writes the final tensor -- any id width, the
+    padding on either side -- for rows it takes whole (every team shape, one row per team and a work
+    list) and, through the token buffer, for rows that are cut into chunks.  Expected: the oracle's
+    rows padded by the oracle's pad_rows with the same options (a row with more tokens than the
+    stride keeps its first ones on either side)."""
+    which, enc, bo = bpe
+    say(f"bpe{which} padded as {dtype} left={pad_left}")
+    rng = random.Random(17)
+    rnd = lambda n: "".join(rng.choices("ACGTN", weights=[24, 24, 24, 24, 4], k=n))
+    top = {torch.uint8: 200, torch.int16: 30000, torch.int32: 70000, torch.int64: 70000}[dtype]
+    remap_h = np.random.default_rng(4).integers(0, top, size=70000).astype(np.int32)
+    np_dtype = {torch.uint8: np.uint8, torch.int16: np.int16, torch.int32: np.int32, torch.int64: np.int64}[dtype]
+    pad_id = 7
+    batches = [([rnd(n) for n in (0, 1, 7, 8, 9, 63, 300, 511, 0, 333)], (160, 5)),              # one-wave teams
+               ([rnd(n) for n in (1000, 1024, 0, 3, 700)], (300, 64)),                             # 256-thread teams
+               ([rnd(rng.randint(0, 700)) for _ in range(3000)], (256, 100)),                      # more rows than teams
+               ([rnd(rng.randint(20, 300)) for _ in range(1500)] + [rnd(900), rnd(640)], (256,)),  # split between two launches
+               (wl.config5_ragged(30, seed=13).strings() + ["", rnd(5000), "A" * 9000], (4000, 250))]  # through the token buffer
+    for seqs, strides in batches:
+        b = util.batch_from_strings(seqs)
+        data, off = to_dev(b)
+        max_len = int(b.lengths().max())
+        rows = [remap_h[np.asarray(e, dtype=np.int64)] for e in bo.encode_batch(b.data, b.offsets)]
+        for stride in strides:
+            ids, mask, lengths, longest = enc.encode_padded(data, off, max_len, stride, pad_id,
+                                                            remap=torch.from_numpy(remap_h).to(DEV), pad_left=pad_left,
+                                                            dtype=dtype)
+            torch.cuda.synchronize()
+            assert ids.dtype == dtype and tuple(ids.shape) == (len(seqs), stride)
+            want_ids, want_mask = O.pad_rows(rows, pad_id, stride, pad_left=pad_left, dtype=np_dtype)
+            np.testing.assert_array_equal(lengths.cpu().numpy(), [len(r) for r in rows])
+            assert int(longest.item()) == max(len(r) for r in rows)
+            np.testing.assert_array_equal(ids.cpu().numpy(), want_ids, err_msg=f"{len(seqs)} rows, stride {stride}")
+            np.testing.assert_array_equal(mask.cpu().numpy(), want_mask, err_msg=f"{len(seqs)} rows, stride {stride}")
+
+
 def test_bpe_padded_on_two_streams_and_in_a_graph(bpe):
     """Every stream has its own tree; replays of a captured call give the eager result each time,
     with eager calls (which use the same tree) in between."""
