@@ -852,8 +852,76 @@ def short_reads_kmer(host, off_h, data, off) -> dict:
     same_rows([buf[0][first + r, :ln[first + r]].cpu().numpy() for r in range(512)], want, "short reads, 6-mer")
     _, dm = time_steps(W(), 50, 10)
     by = int(off_h[-1]) + 5 * n_rows * width + 4 * n_rows
-    return {"bases": int(off_h[-1]), "device_us_per_call": dm * 1e3, "mbp_per_s": float(off_h[-1]) / (dm * 1e-3) / 1e6,
-            "hbm_frac": by / (dm * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    out = {"bases": int(off_h[-1]), "device_us_per_call": dm * 1e3, "mbp_per_s": float(off_h[-1]) / (dm * 1e-3) / 1e6,
+           "hbm_frac": by / (dm * 1e-3) / 1e9 / HBM_PEAK_GBS}
+
+    def packed(d, o, o_h, h, what):
+        """The packed layout (tokens back to back, no padding): 1 B read twice per base, 4 B per
+        token, 8 B of offsets and 4 B of length per row."""
+        n = o_h.size - 1
+        pbuf = (torch.empty(int(o_h[-1]), dtype=torch.int32, device="cuda"), torch.empty(n + 1, dtype=torch.int64, device="cuda"),
+                None, torch.empty(n, dtype=torch.int32, device="cuda"), torch.empty(n, dtype=torch.int32, device="cuda"))
+
+        class P:
+            def step(self):
+                enc.encode_packed(d, o, out=pbuf)
+        P().step()
+        torch.cuda.synchronize()
+        oo = pbuf[1].cpu().numpy()
+        flat = pbuf[0].cpu().numpy()
+        rows = np.concatenate([np.arange(n - 256, n), np.argsort(o_h[1:] - o_h[:-1])[-8:]])
+        want = hf_live_rows(hf.build_kmer_tokenizer(6), np.concatenate([h[o_h[r]:o_h[r + 1]] for r in rows]),
+                            np.concatenate([[0], np.cumsum([o_h[r + 1] - o_h[r] for r in rows])]))
+        same_rows([flat[oo[r]:oo[r + 1]] for r in rows], want, what)
+        _, pm = time_steps(P(), 50, 10)
+        pby = 2 * int(o_h[-1]) + 4 * int(oo[-1]) + 12 * n
+        return {"tokens": int(oo[-1]), "device_us_per_call": pm * 1e3, "mbp_per_s": float(o_h[-1]) / (pm * 1e-3) / 1e6,
+                "hbm_frac": pby / (pm * 1e-3) / 1e9 / HBM_PEAK_GBS}
+
+    out["packed"] = packed(data, off, off_h, host, "short reads, 6-mer, packed")
+    # the same reads with 50 rows of 2-20 kbp among them: every row gets its kernel by its own length
+    rng = np.random.Generator(np.random.PCG64(1007))
+    where = np.sort(rng.choice(n_rows, 50, replace=False))
+    parts, lens2, prev = [], [], 0
+    for at in where:
+        parts.append(host[off_h[prev]:off_h[at]])
+        lens2.extend((off_h[prev + 1:at + 1] - off_h[prev:at]).tolist())
+        n_long = int(rng.integers(2000, 20001))
+        parts.append(rng.choice(np.frombuffer(b"ACGT", dtype=np.uint8), n_long))
+        lens2.append(n_long)
+        prev = at
+    parts.append(host[off_h[prev]:])
+    lens2.extend((off_h[prev + 1:] - off_h[prev:-1]).tolist())
+    host2 = np.concatenate(parts)
+    off2_h = np.zeros(len(lens2) + 1, dtype=np.int64)
+    off2_h[1:] = np.cumsum(lens2)
+    data2, off2 = _dev(host2), _dev(off2_h)
+    n2 = off2_h.size - 1
+    cap2 = int(max(lens2)) // 6 + 6
+    cap2 += (-cap2) % 128
+    buf2 = (torch.empty((n2, cap2), dtype=torch.int32, device="cuda"), torch.empty((n2, cap2), dtype=torch.uint8, device="cuda"),
+            torch.empty(n2, dtype=torch.int32, device="cuda"), torch.empty(n2, dtype=torch.int32, device="cuda"),
+            torch.empty(1, dtype=torch.int32, device="cuda"))
+    mixed = {"rows": n2, "bases": int(off2_h[-1]), "rows_apart": cap2}
+    for name, team_rows in (("by_row_class", -1), ("a_wave_per_row", 0)):
+        enc.set_team_rows(team_rows)
+
+        class M:
+            def step(self):
+                enc.encode_padded(data2, off2, cap2, fill_to=0, width_guess=0, out=buf2)
+        M().step()
+        torch.cuda.synchronize()
+        ln2 = buf2[2].cpu().numpy()
+        rows = np.concatenate([np.arange(n2 - 128, n2), np.argsort(lens2)[-8:]])
+        want = hf_live_rows(hf.build_kmer_tokenizer(6), np.concatenate([host2[off2_h[r]:off2_h[r + 1]] for r in rows]),
+                            np.concatenate([[0], np.cumsum([lens2[r] for r in rows])]))
+        same_rows([buf2[0][r, :ln2[r]].cpu().numpy() for r in rows], want, f"mixed rows, 6-mer, {name}")
+        _, mm = time_steps(M(), 30, 5)
+        mixed[name + "_us_per_call"] = mm * 1e3
+    enc.set_team_rows(-1)
+    mixed["packed"] = packed(data2, off2, off2_h, host2, "mixed rows, 6-mer, packed")
+    out["with_50_rows_of_2_to_20_kbp"] = mixed
+    return out
 
 
 def kmer_rows_with_n_extra():
@@ -925,6 +993,52 @@ def kmer_rows_with_n_extra():
     return out
 
 
+def strings_in_extra():
+    """What a caller of DNATok sees: Python strings in, int64 ids back on the host
+    (`DNATok.encode_batch_to_ids`), on the workload of the reference's own CLI example
+    (docs/CLI.md:104-115: 1000 sequences of 4096 bp) at 32 and at 256 sequences per call, for the
+    single-nucleotide, the 6-mer and the BPE-4096 tokenizer.  Every call's ids are compared with the
+    Hugging Face tokenizer's (an untimed pass); the tokenizer itself is timed beside it on this
+    host's threads.  Includes the bus both ways and all of the Python around the kernels."""
+    import random
+    import torch
+    from dnatok_amd import dnatok_cli
+    from tests.support import hf_tokenizers as hf
+    rng = random.Random(42)
+    seqs = ["".join(rng.choices("ACGT", k=4096)) for _ in range(1000)]
+    bases = sum(map(len, seqs))
+    out = {"workload": "1000 sequences x 4096 bp of random ACGT, strings in, int64 ids on the host out",
+           "host_threads": host_threads()}
+    for name, model in (("char", "char"), ("kmer6", "kmer6"), ("bpe4096", hf.bpe_tokenizer_path("4096"))):
+        tok, dn = dnatok_cli._build_dnatok(model, "cuda")
+        row = {"path": dnatok_cli._detect_path(dn)}
+        for chunk in (32, 256):
+            for i in range(0, len(seqs), chunk):                       # untimed: warm-up and the check
+                got = dn.encode_batch_to_ids(seqs[i:i + chunk])
+                want = tok(seqs[i:i + chunk], add_special_tokens=False)["input_ids"]
+                for r, w_ in zip(got.tolist(), want):
+                    assert r[:len(w_)] == list(w_) and all(x == dn.id_pad for x in r[len(w_):]), (name, chunk, i)
+            best = None
+            for _ in range(3):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for i in range(0, len(seqs), chunk):
+                    dn.encode_batch_to_ids(seqs[i:i + chunk])
+                torch.cuda.synchronize()
+                dt = time.perf_counter() - t0
+                best = dt if best is None or dt < best else best
+            t0 = time.perf_counter()
+            for i in range(0, len(seqs), chunk):
+                tok(seqs[i:i + chunk], add_special_tokens=False)
+            t_hf = time.perf_counter() - t0
+            row[f"{chunk}_per_call"] = {"mbp_per_s": bases / best / 1e6, "ms_per_call": best / ((len(seqs) + chunk - 1) // chunk) * 1e3,
+                                        "hf_tokenizers_mbp_per_s": bases / t_hf / 1e6}
+        out[name] = row
+        del dn, tok
+        torch.cuda.empty_cache()
+    return out
+
+
 def merge_table_placement_extra():
     """The BPE merge table of the 4096 vocabulary in global memory (L2; the default) against its compact
     48 KB form kept in LDS by every workgroup (`dnatok_bpe_table_set_placement`), on batches of 1 KB rows:
@@ -980,7 +1094,7 @@ def main() -> None:
     ap.add_argument("--config", default="C2", choices=["C1", "C2", "C3", "C4", "C5"])
     ap.add_argument("--per-call", action="store_true", help="time one exact batch instead of the sustained form")
     ap.add_argument("--no-extras", action="store_true")
-    ap.add_argument("--only-extra", default="", choices=["", "merge_table_placement", "pathological", "kmer_rows_with_n",
+    ap.add_argument("--only-extra", default="", choices=["", "merge_table_placement", "pathological", "kmer_rows_with_n", "strings_in",
                                                          "short_reads"],
                     help="run only this extra after the headline (for profiling it)")
     ap.add_argument("--no-cpu", action="store_true")
@@ -1083,7 +1197,7 @@ def main() -> None:
         result[args.only_extra] = {"merge_table_placement": merge_table_placement_extra,
                                    "pathological": pathological_extra,
                                    "kmer_rows_with_n": kmer_rows_with_n_extra,
-                                   "short_reads": short_reads_extra}[args.only_extra]()
+                                   "short_reads": short_reads_extra, "strings_in": strings_in_extra}[args.only_extra]()
     elif not args.no_extras:
         per_call = {}
         for cfg in ["C1", "C2", "C3", "C4", "C5"]:
@@ -1137,6 +1251,7 @@ def main() -> None:
         result["pathological"] = pathological_extra()
         result["short_reads"] = short_reads_extra()
         result["merge_table_placement"] = merge_table_placement_extra()
+        result["strings_in"] = strings_in_extra()
 
     print(json.dumps(result), flush=True)
 

@@ -20,6 +20,7 @@ EXPORTS = [
     "dnatok_char_embed_packed",
     "dnatok_char_unpack_2bit", "dnatok_host_clean_ascii", "dnatok_host_pack_2bit", "dnatok_host_fasta_scan",
     "dnatok_kmer_table_create", "dnatok_kmer_table_destroy", "dnatok_kmer_table_set_team_rows", "dnatok_kmer_encode_padded",
+    "dnatok_kmer_encode_padded_sized", "dnatok_kmer_encode_packed",
     "dnatok_bpe_table_create", "dnatok_bpe_table_destroy", "dnatok_bpe_scratch_bytes",
     "dnatok_bpe_encode", "dnatok_bpe_encode_with_chars", "dnatok_bpe_encode_padded", "dnatok_bpe_encode_padded_as", "dnatok_bpe_padded_direct_max",
     "dnatok_bpe_static_scratch_bytes", "dnatok_bpe_encode_static",
@@ -93,6 +94,10 @@ def lib() -> ctypes.CDLL:
     L.dnatok_kmer_table_set_team_rows.argtypes = [c_void_p, c_int32]
     L.dnatok_kmer_encode_padded.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    L.dnatok_kmer_encode_padded_sized.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                                                  c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    L.dnatok_kmer_encode_packed.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p,
+                                            c_void_p, c_void_p, c_void_p, c_void_p]
     L.dnatok_bpe_table_create.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32,
                                           c_void_p, POINTER(c_void_p)]
     L.dnatok_bpe_table_destroy.argtypes = [c_void_p]

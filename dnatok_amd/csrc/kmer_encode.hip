@@ -129,6 +129,19 @@ struct MaxRef {
     unsigned long long *tree;      // kTreeWords words of the slot's stream, all zero between calls
 };
 
+// Where a launch puts its rows and which rows it takes.
+struct RowPlace {
+    // packed output: row b's cells are ids[row_at[b] .. row_at[b + 1]) (and the same cells of the
+    // mask), no padding; null: row b's cells start at ids[b * t_cap]
+    const int64_t *row_at;
+    // 0: every row; 1: the rows of at most kGroupsMaxUnits units; 2: the other rows (a batch of
+    // mostly short rows with some long ones is split between kmer_groups_kernel and kmer_rows_kernel)
+    int32_t row_class;
+    // the rows' lengths are all that is written (the first pass of a packed encode)
+    int32_t count_only;
+};
+constexpr int kGroupsMaxUnits = 384;
+
 // Stores the group of 4 cells [e, e + 4) of a row whose cells are addressed from the
 // 16-byte-aligned pointer pair (outA, moutA); only cells inside [lo, hi) are written.
 __device__ __forceinline__ void store_group(int32_t *outA, uint8_t *moutA, int e, int lo, int hi,
@@ -173,12 +186,15 @@ __device__ __forceinline__ void wave_sync()
 // apart (0, 1, 2, 3); v_perm_b32 with those bits as selectors rebuilds the byte they stand for,
 // and a byte that differs from it is not one of the four.  The window code holds character i in
 // bits 2i, 2i + 1 (a.lut4r is indexed that way).
-template <int K, bool LUT4_LDS, bool CHARS, bool HAS_MASK, bool ARITH>
+// PLACED: the launch honours `place` (packed output, a class of rows, counting only); without it the
+// argument is ignored and the rows lie a stride apart, so that the kernel of the padded layout is
+// compiled exactly as it would be without these modes (as run-time choices they cost it 2 %).
+template <int K, bool LUT4_LDS, bool CHARS, bool HAS_MASK, bool ARITH, bool PLACED = false>
 __global__ __launch_bounds__(kRowsThreads) void kmer_rows_kernel(
     KmerArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
     int64_t n_rows, int64_t t_cap, int64_t fill_to, int32_t *__restrict__ ids,
     uint8_t *__restrict__ mask, int32_t *__restrict__ lengths, int32_t *__restrict__ status,
-    int32_t *__restrict__ max_len, MaxRef mref, int publish)
+    int32_t *__restrict__ max_len, MaxRef mref, int publish, RowPlace place)
 {
     constexpr uint32_t POW4 = 1u << (2 * K);
     __shared__ uint32_t s_dig[256];
@@ -206,26 +222,60 @@ __global__ __launch_bounds__(kRowsThreads) void kmer_rows_kernel(
 
     const int lane = threadIdx.x & 63;
     int32_t *const buf = s_stage[__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6))];
-    const int cap = t_cap > INT_MAX - 16 ? INT_MAX - 16 : (int)t_cap;
-    const int fill = fill_to > cap ? cap : (int)fill_to;
+    const int cap_all = t_cap > INT_MAX - 16 ? INT_MAX - 16 : (int)t_cap;
+    const int fill_all = fill_to > cap_all ? cap_all : (int)fill_to;
     int64_t wave_max = 0;
     const unsigned long long slot_gen = mref.slot ? mref.slot[1] : 0ull;
     const int wave_in_wg = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int64_t wave = (int64_t)blockIdx.x * (kRowsThreads / 64) + wave_in_wg;
     const int64_t n_waves = (int64_t)gridDim.x * (kRowsThreads / 64);
 
-    for (int64_t row = wave; row < n_rows; row += n_waves) {
+    // Which rows the wave takes: every n_waves-th row; of a batch that is split by row class, the
+    // long rows of every n_waves-th block of 64 rows -- the lanes look at a row each, so that the
+    // short rows, which are nearly all of such a batch, cost a wave one load per 64 of them.
+    const bool long_rows_only = PLACED && place.row_class == 2;
+    int64_t cursor = long_rows_only ? wave * 64 : wave;
+    uint64_t pending = 0;                                // (long_rows_only) rows of the block at `cursor` still to do
+    auto next_row = [&]() -> int64_t {
+        if (!long_rows_only) {
+            const int64_t r = cursor;
+            cursor += n_waves;
+            return r < n_rows ? r : -1;
+        }
+        while (pending == 0) {
+            if (cursor >= n_rows) return -1;
+            const int64_t r = cursor + lane;
+            bool is_long = false;
+            if (r < n_rows) {
+                const int64_t l = offsets[r + 1] - offsets[r];
+                is_long = l / K + l % K > kGroupsMaxUnits;
+            }
+            pending = __ballot(is_long);
+            if (pending == 0) cursor += n_waves * 64;
+        }
+        const int at = __builtin_ctzll(pending);
+        pending &= pending - 1;
+        const int64_t r = cursor + at;
+        if (pending == 0) cursor += n_waves * 64;
+        return r;
+    };
+    for (int64_t row = next_row(); row >= 0; row = next_row()) {
         const int64_t row_start = offsets[row];
         // positions inside a row are 32-bit: a row is shorter than 2^31 bytes
         const int len = (int)(offsets[row + 1] - row_start);
         const int full = len / K;
         const int n_units = full + (len - full * K);
         const uint8_t *src = bytes + row_start;
-        int32_t *out = ids + row * t_cap;
+        // the row's cells: a stride apart, or (packed) where the rows before it end
+        const int64_t cell0 = PLACED && place.row_at ? place.row_at[row] : row * t_cap;
+        const int cap = !PLACED ? cap_all
+                                : place.count_only ? 0 : place.row_at ? (int)(place.row_at[row + 1] - cell0) : cap_all;
+        const int fill = PLACED && place.row_at ? 0 : fill_all;
+        int32_t *out = ids + cell0;
         // cells are addressed from the 16-byte boundary at or below the row's first cell
         const int mis = (int)((reinterpret_cast<uintptr_t>(out) >> 2) & 3);
         int32_t *outA = out - mis;
-        uint8_t *moutA = HAS_MASK ? mask + row * t_cap - mis : nullptr;
+        uint8_t *moutA = HAS_MASK ? mask + cell0 - mis : nullptr;
         const int lo = mis, hi_cap = mis + cap;
         int running = 0;
         int32_t my_status = 0;
@@ -259,7 +309,7 @@ __global__ __launch_bounds__(kRowsThreads) void kmer_rows_kernel(
         const __amdgpu_buffer_rsrc_t rs_ids =
             __builtin_amdgcn_make_buffer_rsrc(out, (short)0, vec_cap * 4, 0x00020000);
         const __amdgpu_buffer_rsrc_t rs_msk = __builtin_amdgcn_make_buffer_rsrc(
-            HAS_MASK ? mask + row * t_cap : reinterpret_cast<uint8_t *>(out), (short)0, HAS_MASK ? vec_cap : 0,
+            HAS_MASK ? mask + cell0 : reinterpret_cast<uint8_t *>(out), (short)0, HAS_MASK ? vec_cap : 0,
             0x00020000);
         // group of 4 cells starting at row cell r (whole = inside the row and the descriptor)
         auto store_vec = [&](bool whole, int r, const int32_t *v) {
@@ -438,6 +488,10 @@ __global__ __launch_bounds__(kRowsThreads) void kmer_rows_kernel(
 
             const uint32_t inc = wave_inclusive_sum_u32(lane_cnt);
             const uint32_t step_total = __builtin_amdgcn_readlane(inc, 63);
+            if (PLACED && place.count_only) {      // (the step's tokens are counted, not made)
+                running += (int)step_total;
+                continue;
+            }
 
             // what the step's common store (one 4-cell group per lane) will write
             bool sv_whole = false;
@@ -650,7 +704,7 @@ __global__ __launch_bounds__(kRowsThreads) void kmer_rows_kernel(
         int32_t st = 0;
         if (__ballot(my_status & DNATOK_ROW_INVALID_BYTE)) st |= DNATOK_ROW_INVALID_BYTE;
         if (__ballot(my_status & DNATOK_ROW_MISSING_KMER)) st |= DNATOK_ROW_MISSING_KMER;
-        if (running > t_cap) st |= DNATOK_ROW_TRUNCATED;
+        if (PLACED ? running > cap : running > t_cap) st |= DNATOK_ROW_TRUNCATED;
         if (lane == 0) {
             lengths[row] = (int32_t)running;
             if (status) status[row] = st;
@@ -720,7 +774,7 @@ __global__ __launch_bounds__(kGroupThreads) void kmer_groups_kernel(
     KmerArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
     int64_t n_rows, int64_t t_cap, int64_t fill_to, int32_t *__restrict__ ids,
     uint8_t *__restrict__ mask, int32_t *__restrict__ lengths, int32_t *__restrict__ status,
-    int32_t *__restrict__ max_len, MaxRef mref, int publish)
+    int32_t *__restrict__ max_len, MaxRef mref, int publish, RowPlace place)
 {
     constexpr uint32_t POW4 = 1u << (2 * K);
     constexpr int kLaneBytes = kUnitsPerLane * K;                 // bytes of a lane's four windows
@@ -738,8 +792,8 @@ __global__ __launch_bounds__(kGroupThreads) void kmer_groups_kernel(
     __syncthreads();
 
     const int lane = threadIdx.x & 63, gl = lane & 15;
-    const int cap = (int)t_cap;                                   // (at most kGroupsMaxStride)
-    const int fill = fill_to > cap ? cap : (int)fill_to;
+    const int cap_all = t_cap > INT_MAX - 16 ? INT_MAX - 16 : (int)t_cap;
+    const int fill_all = fill_to > cap_all ? cap_all : (int)fill_to;
     const int64_t group = ((int64_t)blockIdx.x * kGroupThreads + threadIdx.x) >> 4;
     const int64_t n_groups = (int64_t)gridDim.x * (kGroupThreads / 16);
     const unsigned long long slot_gen = mref.slot ? mref.slot[1] : 0ull;
@@ -751,13 +805,21 @@ __global__ __launch_bounds__(kGroupThreads) void kmer_groups_kernel(
     const int64_t wave_first = group - (lane >> 4);
     for (int64_t row0 = wave_first; row0 < n_rows; row0 += n_groups) {
         const int64_t row = row0 + (lane >> 4);
-        const bool have = row < n_rows;
+        bool have = row < n_rows;
         const int64_t start = have ? offsets[row] : 0;
-        const int len = have ? (int)(offsets[row + 1] - start) : 0;
+        int len = have ? (int)(offsets[row + 1] - start) : 0;
+        if (place.row_class == 1 && len / K + len % K > kGroupsMaxUnits) {     // (kmer_rows_kernel's row)
+            have = false;
+            len = 0;
+        }
         const int full = len / K, tail = len - full * K;
         const int n_slots = full + (tail ? 1 : 0);                // windows, and one slot for the trailing characters
-        int32_t *out = ids + row * t_cap;
-        uint8_t *mout = HAS_MASK ? mask + row * t_cap : nullptr;
+        // the row's cells: a stride apart, or (packed) where the rows before it end
+        const int64_t cell0 = !have ? 0 : place.row_at ? place.row_at[row] : row * t_cap;
+        const int cap = place.count_only || !have ? 0 : place.row_at ? (int)(place.row_at[row + 1] - cell0) : cap_all;
+        const int fill = place.row_at || !have ? 0 : fill_all;
+        int32_t *out = ids + cell0;
+        uint8_t *mout = HAS_MASK ? mask + cell0 : nullptr;
         int running = 0;
         bool foreign_seen = false;
 
@@ -850,7 +912,7 @@ __global__ __launch_bounds__(kGroupThreads) void kmer_groups_kernel(
 
             auto byte_of = [&](int bi) -> uint32_t { return (w[bi >> 2] >> (8 * (bi & 3))) & 255u; };
             if (lane_cnt == kUnitsPerLane && cnt[0] == 1 && cnt[1] == 1 && cnt[2] == 1 && cnt[3] == 1 &&
-                (t[0] | t[1] | t[2] | t[3]) >= 0 && (s & 3u) == 0 && (int)s + 4 <= cap && ((reinterpret_cast<uintptr_t>(out) & 15) == 0)) {
+                (t[0] | t[1] | t[2] | t[3]) >= 0 && (int)s + 4 <= cap && ((reinterpret_cast<uintptr_t>(out + s) & 15) == 0)) {
                 const int4v x = {t[0], t[1], t[2], t[3]};
                 __builtin_nontemporal_store(x, reinterpret_cast<int4v *>(out + s));
             } else if (lane_cnt) {
@@ -1552,7 +1614,7 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
         if (grid > kTreeRows) grid = kTreeRows;                                                   \
         kmer_groups_kernel<KK, L, M><<<(int)grid, kGroupThreads, 0, s>>>(                         \
             a, bytes, offsets, n_rows, t_cap, tight ? t_cap : fill_to, ids, mask, lengths, status, max_len, mref, \
-            tight ? 1 : 0);                                                                       \
+            tight ? 1 : 0, RowPlace{nullptr, 0, 0});                                              \
     } while (0)
 #define GROUPS(KK, L)                                                                             \
     do {                                                                                          \
@@ -1590,7 +1652,7 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
         padded_in_kernel = tight && grid <= kTreeRows;                                            \
         kmer_rows_kernel<KK, L, C, M, AR><<<(int)grid, kRowsThreads, 0, s>>>(                     \
             a, bytes, offsets, n_rows, t_cap, padded_in_kernel ? t_cap : fill_to, ids, mask,      \
-            lengths, status, max_len, mref, padded_in_kernel ? 1 : 0);                            \
+            lengths, status, max_len, mref, padded_in_kernel ? 1 : 0, RowPlace{nullptr, 0, 0});   \
     } while (0)
 #define LAUNCH2(KK, L, C)                                                                         \
     do {                                                                                          \
@@ -1617,4 +1679,171 @@ extern "C" int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *
     if (to_longest && !padded_in_kernel)
         return launch_pad(ids, mask, lengths, n_rows, t_cap, max_len, t->pad_id, (int32_t)guess, mref, s);
     return DNATOK_OK;
+}
+
+// ---- rows placed by the caller's layout: row classes, packed output ------------------------------
+
+namespace dnatok {
+int launch_scan_lengths(const int32_t *lengths, int64_t n_rows, int64_t *out_offsets, void *scratch,
+                        size_t scratch_bytes, hipStream_t s);   // pack.hip
+}
+
+// One launch of kmer_rows_kernel<..., PLACED> (which = 0) or kmer_groups_kernel (which = 1) with a
+// RowPlace.  The longest row, where asked for, goes to mref.slot / max_len by atomicMax (no tree:
+// two launches may share one call).
+static int launch_placed(const dnatok_kmer_t *t, int which, const uint8_t *bytes, const int64_t *offsets, int64_t n_rows,
+                         int64_t t_cap, int64_t fill_to, int32_t *ids, uint8_t *mask, int32_t *lengths,
+                         int32_t *status, int32_t *max_len, MaxRef mref, RowPlace place, hipStream_t s)
+{
+    KmerArgs a{t->digit, t->single, t->lut4, t->lut4r, t->fold, t->entry, t->flat, t->pad_id, t->missing_id};
+    if (which == 1) {
+#define PG2(KK, L, M)                                                                              \
+    do {                                                                                          \
+        static const int resident = resident_workgroups(kmer_groups_kernel<KK, L, M>, kGroupThreads, 0, 8); \
+        int64_t grid = (n_rows + kGroupThreads / 16 - 1) / (kGroupThreads / 16);                  \
+        if (grid > resident) grid = resident;                                                     \
+        kmer_groups_kernel<KK, L, M><<<(int)grid, kGroupThreads, 0, s>>>(                         \
+            a, bytes, offsets, n_rows, t_cap, fill_to, ids, mask, lengths, status, max_len, mref, 0, place); \
+    } while (0)
+#define PG(KK, L)                                                                                 \
+    do {                                                                                          \
+        if (mask) PG2(KK, L, true); else PG2(KK, L, false);                                       \
+    } while (0)
+        switch (t->k) {
+            case 2: PG(2, true); break;
+            case 3: PG(3, true); break;
+            case 4: PG(4, true); break;
+            case 5: PG(5, true); break;
+            case 6: PG(6, true); break;
+            case 7: PG(7, false); break;
+            default: PG(8, false); break;
+        }
+#undef PG
+#undef PG2
+    } else {
+        const int64_t want = (n_rows + kRowsThreads / 64 - 1) / (kRowsThreads / 64);
+#define PR4(KK, L, C, M, AR)                                                                      \
+    do {                                                                                          \
+        static const int resident = resident_workgroups(kmer_rows_kernel<KK, L, C, M, AR, true>, kRowsThreads, 0, 2); \
+        const int64_t grid = want < resident ? want : resident;                                   \
+        kmer_rows_kernel<KK, L, C, M, AR, true><<<(int)grid, kRowsThreads, 0, s>>>(               \
+            a, bytes, offsets, n_rows, t_cap, fill_to, ids, mask, lengths, status, max_len, mref, 0, place); \
+    } while (0)
+#define PR3(KK, L, C, M)                                                                          \
+    do {                                                                                          \
+        if (t->arith) PR4(KK, L, C, M, true); else PR4(KK, L, C, M, false);                       \
+    } while (0)
+#define PR2(KK, L, C)                                                                             \
+    do {                                                                                          \
+        if (mask) PR3(KK, L, C, true); else PR3(KK, L, C, false);                                 \
+    } while (0)
+#define PR(KK, L)                                                                                 \
+    do {                                                                                          \
+        if (t->chars_mode) PR2(KK, L, true); else PR2(KK, L, false);                              \
+    } while (0)
+        switch (t->k) {
+            case 2: PR(2, true); break;
+            case 3: PR(3, true); break;
+            case 4: PR(4, true); break;
+            case 5: PR(5, true); break;
+            case 6: PR(6, true); break;
+            case 7: PR(7, false); break;
+            default: PR(8, false); break;
+        }
+#undef PR
+#undef PR2
+#undef PR3
+#undef PR4
+    }
+    DNATOK_HIP_TRY(hipGetLastError());
+    return DNATOK_OK;
+}
+
+// A batch of mostly short rows (the mean at most kGroupsMaxUnits units) whose table the 16-lane
+// kernel serves: that kernel takes the rows of at most kGroupsMaxUnits units, a wave per row the
+// others.  (The row's class is read from its length on the device; what the host knows is the mean.)
+static bool split_by_row_class(const dnatok_kmer_t *t, int64_t n_rows, int64_t total)
+{
+    return t->arith && t->chars_mode && n_rows > 0 && total / n_rows <= (int64_t)kGroupsMaxUnits * t->k;
+}
+
+extern "C" int dnatok_kmer_encode_padded_sized(const dnatok_kmer_t *t, const uint8_t *bytes, const int64_t *offsets,
+                                               int64_t n_rows, int64_t total, int64_t t_cap, int64_t fill_to,
+                                               int32_t *ids, uint8_t *mask, int32_t *lengths, int32_t *status,
+                                               int32_t *max_len, void *stream)
+{
+    DNATOK_REQUIRE(t && offsets && ids && lengths, DNATOK_E_INVALID, "dnatok_kmer_encode_padded_sized: null argument");
+    DNATOK_REQUIRE(n_rows >= 0 && total >= 0 && t_cap >= 0 && fill_to <= t_cap, DNATOK_E_INVALID,
+                   "dnatok_kmer_encode_padded_sized: need fill_to <= t_cap and sizes >= 0");
+    DNATOK_REQUIRE(fill_to > 0 || max_len, DNATOK_E_INVALID, "dnatok_kmer_encode_padded_sized: fill_to <= 0 needs max_len");
+    // A stride within the 16-lane kernel's reach says that every row is short; a batch of few rows,
+    // or of rows that are long on average, is as well off with one kernel for all of them.
+    const int team_rows = t->team_rows.load(std::memory_order_relaxed);
+    if (n_rows < 1024 || t_cap <= kGroupsMaxStride || (t_cap & 3) != 0 || team_rows != -1 ||
+        !split_by_row_class(t, n_rows, total))
+        return dnatok_kmer_encode_padded(t, bytes, offsets, n_rows, t_cap, fill_to, ids, mask, lengths, status, max_len,
+                                         stream);
+    const bool to_longest = fill_to <= 0;
+    int64_t guess = to_longest ? -fill_to : 0;
+    if (guess > t_cap) guess = t_cap;
+    if (to_longest) fill_to = guess;
+    hipStream_t s = (hipStream_t)stream;
+    MaxRef mref{nullptr, nullptr};
+    if (to_longest) {
+        std::lock_guard<std::mutex> hold(t->slot_lock);
+        auto it = t->slot_of_stream.find(stream);
+        if (it == t->slot_of_stream.end() && (int)t->slot_of_stream.size() < kMaxSlots)
+            it = t->slot_of_stream.emplace(stream, (int)t->slot_of_stream.size()).first;
+        if (it != t->slot_of_stream.end()) {
+            mref.slot = t->max_slots + (size_t)it->second * kMaxSlotStride;
+            mref.tree = t->max_trees + (size_t)it->second * kTreeWords;
+        }
+        if (!mref.slot) {
+            kmer_init_kernel<<<1, 1, 0, s>>>(max_len);
+            DNATOK_HIP_TRY(hipGetLastError());
+        }
+    }
+    int rc = launch_placed(t, 1, bytes, offsets, n_rows, t_cap, fill_to, ids, mask, lengths, status, max_len, mref,
+                           RowPlace{nullptr, 1, 0}, s);
+    if (rc) return rc;
+    rc = launch_placed(t, 0, bytes, offsets, n_rows, t_cap, fill_to, ids, mask, lengths, status, max_len, mref,
+                       RowPlace{nullptr, 2, 0}, s);
+    if (rc) return rc;
+    if (to_longest) return launch_pad(ids, mask, lengths, n_rows, t_cap, max_len, t->pad_id, (int32_t)guess, mref, s);
+    return DNATOK_OK;
+}
+
+extern "C" int dnatok_kmer_encode_packed(const dnatok_kmer_t *t, const uint8_t *bytes, const int64_t *offsets,
+                                         int64_t n_rows, int64_t total, int32_t *ids_out, int64_t *out_offsets,
+                                         uint8_t *mask_out, int32_t *lengths, int32_t *status, void *stream)
+{
+    DNATOK_REQUIRE(t && offsets && out_offsets && lengths, DNATOK_E_INVALID, "dnatok_kmer_encode_packed: null argument");
+    DNATOK_REQUIRE(n_rows >= 0 && total >= 0, DNATOK_E_INVALID, "dnatok_kmer_encode_packed: negative size");
+    DNATOK_REQUIRE(ids_out || total == 0, DNATOK_E_INVALID, "dnatok_kmer_encode_packed: null ids_out");
+    hipStream_t s = (hipStream_t)stream;
+    const bool split = split_by_row_class(t, n_rows, total);
+    const MaxRef none{nullptr, nullptr};
+    // first pass: every row's token count (nothing else is written), then where every row starts
+    if (n_rows > 0) {
+        int rc;
+        if (split) {
+            rc = launch_placed(t, 1, bytes, offsets, n_rows, 0, 0, nullptr, nullptr, lengths, nullptr, nullptr, none,
+                               RowPlace{nullptr, 1, 1}, s);
+            if (rc) return rc;
+        }
+        rc = launch_placed(t, 0, bytes, offsets, n_rows, 0, 0, nullptr, nullptr, lengths, nullptr, nullptr, none,
+                           RowPlace{nullptr, split ? 2 : 0, 1}, s);
+        if (rc) return rc;
+    }
+    // (ids_out is not written yet: its first bytes, when 8-byte aligned, are the scan's spare room)
+    int rc = launch_scan_lengths(lengths, n_rows, out_offsets, ids_out, (size_t)total * 4, s);
+    if (rc || n_rows == 0) return rc;
+    // second pass: the tokens, each row behind the one before it
+    if (split) {
+        rc = launch_placed(t, 1, bytes, offsets, n_rows, 0, 0, ids_out, mask_out, lengths, status, nullptr, none,
+                           RowPlace{out_offsets, 1, 0}, s);
+        if (rc) return rc;
+    }
+    return launch_placed(t, 0, bytes, offsets, n_rows, 0, 0, ids_out, mask_out, lengths, status, nullptr, none,
+                         RowPlace{out_offsets, split ? 2 : 0, 0}, s);
 }

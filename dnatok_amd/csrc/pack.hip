@@ -7,36 +7,141 @@ namespace dnatok {
 
 constexpr int kScanThreads = 1024;
 
-// out_offsets[b] = sum of max(lengths[0..b), 0); single workgroup, 1024 rows per step.
+// out_offsets[b] = sum of max(lengths[0..b), 0); single workgroup, 4096 rows per step (four
+// consecutive rows per thread), the next step's lengths requested before this step's barrier.
 __global__ __launch_bounds__(kScanThreads) void scan_lengths_kernel(
     const int32_t *__restrict__ lengths, int64_t n_rows, int64_t *__restrict__ out_offsets)
 {
-    __shared__ uint32_t wave_tot[kScanThreads / 64];
-    __shared__ int64_t carry;
-    if (threadIdx.x == 0) carry = 0;
-    __syncthreads();
+    constexpr int kPer = 4;
+    __shared__ uint32_t wave_tot[2][kScanThreads / 64];
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    for (int64_t base = 0; base < n_rows; base += kScanThreads) {
-        const int64_t i = base + threadIdx.x;
-        int32_t v = (i < n_rows) ? lengths[i] : 0;
-        if (v < 0) v = 0;
-        const uint32_t inc = wave_inclusive_sum_u32((uint32_t)v);
-        if (lane == 63) wave_tot[wv] = inc;
-        __syncthreads();
+    auto fetch = [&](int64_t base, int32_t (&v)[kPer]) {
+#pragma unroll
+        for (int q = 0; q < kPer; ++q) {
+            const int64_t i = base + (int64_t)threadIdx.x * kPer + q;
+            const int32_t x = i < n_rows ? lengths[i] : 0;
+            v[q] = x < 0 ? 0 : x;
+        }
+    };
+    int32_t next[kPer];
+    fetch(0, next);
+    int64_t carry = 0;                                   // (every thread keeps the same running total)
+    int par = 0;
+    for (int64_t base = 0; base < n_rows; base += kScanThreads * kPer, par ^= 1) {
+        int32_t v[kPer];
+#pragma unroll
+        for (int q = 0; q < kPer; ++q) v[q] = next[q];
+        fetch(base + kScanThreads * kPer, next);
+        const uint32_t mine = (uint32_t)v[0] + (uint32_t)v[1] + (uint32_t)v[2] + (uint32_t)v[3];
+        const uint32_t inc = wave_inclusive_sum_u32(mine);
+        if (lane == 63) wave_tot[par][wv] = inc;
+        __syncthreads();                                 // (the other half of wave_tot is the previous step's)
         uint32_t before = 0, total = 0;
 #pragma unroll
         for (int w = 0; w < kScanThreads / 64; ++w) {
-            const uint32_t t = wave_tot[w];
+            const uint32_t t = wave_tot[par][w];
             if (w < wv) before += t;
             total += t;
         }
-        const int64_t c = carry;
-        if (i < n_rows) out_offsets[i] = c + before + inc - (uint32_t)v;
-        __syncthreads();
-        if (threadIdx.x == 0) carry = c + total;
-        __syncthreads();
+        int64_t at = carry + before + inc - mine;
+#pragma unroll
+        for (int q = 0; q < kPer; ++q) {
+            const int64_t i = base + (int64_t)threadIdx.x * kPer + q;
+            if (i < n_rows) out_offsets[i] = at;
+            at += v[q];
+        }
+        carry += total;
     }
     if (threadIdx.x == 0) out_offsets[n_rows] = carry;
+}
+
+// The same for very many rows (the packed k-mer encode of 100,000 reads: the one workgroup above
+// walks them 4096 at a time, a trip to memory per step, 58 us), in two launches of a workgroup per
+// tile of 4096 rows: the tiles' sums, then every tile adds up the sums of the tiles before it and
+// scans its own rows.
+constexpr int kScanTile = kScanThreads * 4;
+
+__device__ __forceinline__ void scan_tile_load(const int32_t *__restrict__ lengths, int64_t n_rows, int64_t base,
+                                               uint32_t (&v)[4])
+{
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int64_t i = base + (int64_t)threadIdx.x * 4 + q;
+        const int32_t x = i < n_rows ? lengths[i] : 0;
+        v[q] = x < 0 ? 0u : (uint32_t)x;
+    }
+}
+
+__global__ __launch_bounds__(kScanThreads) void scan_tile_sums_kernel(
+    const int32_t *__restrict__ lengths, int64_t n_rows, unsigned long long *__restrict__ tile_sum)
+{
+    __shared__ uint32_t wave_tot[kScanThreads / 64];
+    uint32_t v[4];
+    scan_tile_load(lengths, n_rows, (int64_t)blockIdx.x * kScanTile, v);
+    const uint32_t inc = wave_inclusive_sum_u32(v[0] + v[1] + v[2] + v[3]);
+    if ((threadIdx.x & 63) == 63) wave_tot[threadIdx.x >> 6] = inc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned long long t = 0;
+        for (int w = 0; w < kScanThreads / 64; ++w) t += wave_tot[w];
+        tile_sum[blockIdx.x] = t;
+    }
+}
+
+__global__ __launch_bounds__(kScanThreads) void scan_tiles_kernel(
+    const int32_t *__restrict__ lengths, int64_t n_rows, const unsigned long long *__restrict__ tile_sum,
+    int64_t *__restrict__ out_offsets)
+{
+    __shared__ uint32_t wave_tot[kScanThreads / 64];
+    __shared__ unsigned long long part[kScanThreads / 64];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    uint32_t v[4];
+    scan_tile_load(lengths, n_rows, (int64_t)blockIdx.x * kScanTile, v);
+    // the tiles before this one
+    unsigned long long mine = 0;
+    for (unsigned j = threadIdx.x; j < blockIdx.x; j += kScanThreads) mine += tile_sum[j];
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) mine += __shfl_xor(mine, d, 64);
+    if (lane == 0) part[wv] = mine;
+    const uint32_t own = v[0] + v[1] + v[2] + v[3];
+    const uint32_t inc = wave_inclusive_sum_u32(own);
+    if (lane == 63) wave_tot[wv] = inc;
+    __syncthreads();
+    unsigned long long before_tiles = 0;
+    uint32_t before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < kScanThreads / 64; ++w) {
+        before_tiles += part[w];
+        const uint32_t t = wave_tot[w];
+        if (w < wv) before += t;
+        total += t;
+    }
+    int64_t at = (int64_t)before_tiles + before + inc - own;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int64_t i = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * 4 + q;
+        if (i < n_rows) out_offsets[i] = at;
+        at += v[q];
+    }
+    if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) out_offsets[n_rows] = (int64_t)before_tiles + total;
+}
+
+// (also used by the packed k-mer encode)  `scratch` (8-byte aligned, NULL allowed) is room the caller
+// can spare until the scan is done; with 8 bytes per 4096 rows of it, very many rows take the two
+// launches above.
+int launch_scan_lengths(const int32_t *lengths, int64_t n_rows, int64_t *out_offsets, void *scratch,
+                        size_t scratch_bytes, hipStream_t s)
+{
+    const int64_t tiles = (n_rows + kScanTile - 1) / kScanTile;
+    if (tiles >= 4 && scratch && ((uintptr_t)scratch & 7) == 0 && scratch_bytes >= (size_t)tiles * 8 && tiles < (1 << 20)) {
+        scan_tile_sums_kernel<<<(int)tiles, kScanThreads, 0, s>>>(lengths, n_rows, (unsigned long long *)scratch);
+        scan_tiles_kernel<<<(int)tiles, kScanThreads, 0, s>>>(lengths, n_rows, (const unsigned long long *)scratch,
+                                                             out_offsets);
+    } else {
+        scan_lengths_kernel<<<1, kScanThreads, 0, s>>>(lengths, n_rows, out_offsets);
+    }
+    DNATOK_HIP_TRY(hipGetLastError());
+    return DNATOK_OK;
 }
 
 constexpr int kPackTile = 4096;          // output cells one workgroup copies
@@ -191,8 +296,10 @@ extern "C" int dnatok_pack_ragged(const int32_t *tok_tmp, const int64_t *in_offs
                    "dnatok_pack_ragged: null argument");
     DNATOK_REQUIRE(n_rows >= 0, DNATOK_E_INVALID, "dnatok_pack_ragged: negative row count");
     hipStream_t s = (hipStream_t)stream;
-    scan_lengths_kernel<<<1, kScanThreads, 0, s>>>(lengths, n_rows, out_offsets);
-    DNATOK_HIP_TRY(hipGetLastError());
+    {
+        const int rc = launch_scan_lengths(lengths, n_rows, out_offsets, nullptr, 0, s);
+        if (rc) return rc;
+    }
     if (n_rows == 0) return DNATOK_OK;
     DNATOK_REQUIRE(tok_tmp && ids_out, DNATOK_E_INVALID, "dnatok_pack_ragged: null buffer");
     // the packed size is only known on the device: a fixed grid strides over its tiles, and

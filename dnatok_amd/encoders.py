@@ -409,12 +409,38 @@ class KmerEncoder:
             max_len = torch.empty(1, dtype=torch.int32, device=dev)
         else:
             ids, mask, lengths, status, max_len = out
-        _lib.check(_lib.lib().dnatok_kmer_encode_padded(
-            self._h, _ptr(data), _ptr(offsets), n_rows, int(t_cap),
+        # (the batch's size tells the call how long its rows are on average: a batch of mostly short
+        # rows with some long ones is split between two kernels, row by row on the device)
+        _lib.check(_lib.lib().dnatok_kmer_encode_padded_sized(
+            self._h, _ptr(data), _ptr(offsets), n_rows, int(data.numel()), int(t_cap),
             int(fill_to) if fill_to > 0 else -min(int(width_guess), int(t_cap)), _ptr(ids),
             _ptr(mask), _ptr(lengths), _ptr(status), _ptr(max_len), _stream()),
-            "dnatok_kmer_encode_padded")
+            "dnatok_kmer_encode_padded_sized")
         return ids, mask, lengths, status, max_len
+
+    def encode_packed(self, data: torch.Tensor, offsets: torch.Tensor, *, want_mask: bool = False, out=None):
+        """Packed layout: ``(ids int32 [total], out_offsets int64 [B + 1], mask uint8 [total] or None,
+        lengths int32 [B], status int32 [B])``; row b's tokens are ``ids[out_offsets[b] :
+        out_offsets[b + 1]]``, nothing is padded.  ``ids`` and ``mask`` have room for one cell per
+        input byte; ``out`` = (ids, out_offsets, mask, lengths, status) reuses caller buffers."""
+        _require_cuda(data, torch.uint8, "data")
+        _require_cuda(offsets, torch.int64, "offsets")
+        n_rows = offsets.numel() - 1
+        total = int(data.numel())
+        dev = data.device
+        if out is None:
+            ids = torch.empty(max(total, 1), dtype=torch.int32, device=dev)
+            out_offsets = torch.empty(n_rows + 1, dtype=torch.int64, device=dev)
+            mask = torch.empty(max(total, 1), dtype=torch.uint8, device=dev) if want_mask else None
+            lengths = torch.empty(n_rows, dtype=torch.int32, device=dev)
+            status = torch.empty(n_rows, dtype=torch.int32, device=dev)
+        else:
+            ids, out_offsets, mask, lengths, status = out
+        _lib.check(_lib.lib().dnatok_kmer_encode_packed(
+            self._h, _ptr(data), _ptr(offsets), n_rows, total, _ptr(ids), _ptr(out_offsets),
+            _ptr(mask) if mask is not None else None, _ptr(lengths), _ptr(status), _stream()),
+            "dnatok_kmer_encode_packed")
+        return ids, out_offsets, mask, lengths, status
 
 
 class BpeEncoder:

@@ -147,8 +147,9 @@ void dnatok_kmer_table_destroy(dnatok_kmer_t *t);
  * Which of the two k-mer kernels the calls with this table use.  A batch of up to max_rows rows is
  * encoded with a workgroup per row (four waves share a row: the latency of a small batch), a
  * larger one with a wave per row (the bandwidth of a large one).  -1 (default): as many rows as
- * workgroups fit the chip at once; 0: always a wave per row.  The setting belongs to the table
- * object; a call reads it once when it starts. */
+ * workgroups fit the chip at once; 0: always a wave per row (and no split by row class in
+ * dnatok_kmer_encode_padded_sized).  The setting belongs to the table object; a call reads it once
+ * when it starts. */
 int dnatok_kmer_table_set_team_rows(dnatok_kmer_t *t, int32_t max_rows);
 
 /* ids int32[n_rows, t_cap], mask uint8[n_rows, t_cap] (NULL allowed): t_cap is the row stride.
@@ -169,6 +170,30 @@ int dnatok_kmer_encode_padded(const dnatok_kmer_t *t, const uint8_t *bytes, cons
                               int64_t n_rows, int64_t t_cap, int64_t fill_to,
                               int32_t *ids, uint8_t *mask, int32_t *lengths, int32_t *status,
                               int32_t *max_len, void *stream);
+
+/* The same for a caller that knows the batch's size in bytes (`total`; the strings' lengths are on
+ * the host anyway), which tells the call how long the rows are on average.  The reference groups the
+ * rows of a batch by length before it encodes them (src/dna_tokenizer.py:1476-1531); here a batch
+ * of mostly short rows with some long ones among them (mean at most 384 windows, stride above 384
+ * cells) is split between two kernels over the one output: the rows of at most 384 units get
+ * sixteen lanes each, the others a wave each, chosen row by row on the device from the offsets.
+ * Any other batch is encoded exactly as by dnatok_kmer_encode_padded.  Results are identical. */
+int dnatok_kmer_encode_padded_sized(const dnatok_kmer_t *t, const uint8_t *bytes, const int64_t *offsets,
+                                    int64_t n_rows, int64_t total, int64_t t_cap, int64_t fill_to,
+                                    int32_t *ids, uint8_t *mask, int32_t *lengths, int32_t *status,
+                                    int32_t *max_len, void *stream);
+
+/* Packed layout, for ragged batches whose padded form would be mostly padding (100,000 reads of
+ * 100-300 bp beside a few rows of 20 kbp): ids_out int32[sum of lengths] holds the rows' tokens
+ * back to back, out_offsets int64[n_rows + 1] their boundaries, mask_out uint8 (NULL allowed) is
+ * one per token, lengths / status as above.  ids_out and mask_out have room for `total` cells (a row
+ * never has more tokens than bytes).  Two passes over the bytes: the rows' token counts, their
+ * prefix sum, then the tokens; no padding is written and nothing returns to the host.  The k-mer
+ * counterpart of dnatok_pack_ragged; the reference has no packed k-mer output (its rows go through
+ * _pad_id_list, src/dna_tokenizer.py:1878-1894). */
+int dnatok_kmer_encode_packed(const dnatok_kmer_t *t, const uint8_t *bytes, const int64_t *offsets,
+                              int64_t n_rows, int64_t total, int32_t *ids_out, int64_t *out_offsets,
+                              uint8_t *mask_out, int32_t *lengths, int32_t *status, void *stream);
 
 /* ---------------------------------------------------------------------------------------
  * BPE merge engine.  Replaces the pybind class DNATokBPE and its kernel

@@ -305,6 +305,76 @@ def test_kmer_steps_with_more_tokens_than_the_staging_area(kmer_kernel_choice, k
         np.testing.assert_array_equal(mask[:, :width].cpu().numpy(), emask)
 
 
+@pytest.mark.parametrize("k", [3, 6, 8])
+def test_kmer_mostly_short_rows_with_some_long_ones(k):
+    """Rows are given their kernel by their own length: in a batch of thousands of short reads with
+    some rows of 2-20 kbp among them the reads get sixteen lanes each and the long rows a wave each,
+    two launches over the one output (the reference groups rows by length,
+    src/dna_tokenizer.py:1476-1531).  Padded (to a fixed width, to the longest with and without a
+    guess) and packed, against the oracle; the packed form also for a table the 16-lane kernel does
+    not serve and for batches of long rows only."""
+    say(f"kmer mixed row lengths k={k}")
+    vocab = hf.kmer_vocab(k)
+    t = kmer_tables.tables_from_vocab(vocab, k, 0)
+    enc = encoders.KmerEncoder(k, t.digit, t.kmer_lut, t.single, pad_id=1, missing_id=0,
+                               exp_off=t.exp_off, exp_len=t.exp_len, exp_flat=t.exp_flat)
+    ot = O.kmer_tables_from_vocab(vocab, k, 0)
+    rng = np.random.default_rng(60 + k)
+    n_short = 6000
+    lens = rng.integers(0, 301, size=n_short)
+    strings = ["".join(rng.choice(list("ACGTN"), p=[.245, .245, .245, .245, .02], size=n)) for n in lens]
+    for at in rng.choice(n_short, size=40, replace=False):              # the long rows, anywhere in the batch
+        strings[at] = "".join(rng.choice(list("ACGTN"), p=[.248, .248, .248, .248, .008], size=int(rng.integers(2000, 20001))))
+    strings[17] = "ACGTx" * 700
+    strings[18] = "N" * (384 * k)                                       # exactly at the border between the classes
+    strings[19] = "A" * (384 * k + 1)
+    b = util.batch_from_strings(strings)
+    data, off = to_dev(b)
+    erows, estatus = O.kmer_encode(ot, b.data, b.offsets)
+    longest = max(r.size for r in erows)
+    cap = longest + (-longest) % 128
+    for fill_to, guess in ((0, 0), (cap, 0), (0, longest + 3), (0, 64)):
+        ids, mask, lengths, status, max_len = enc.encode_padded(data, off, cap, fill_to=fill_to, width_guess=guess)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(lengths.cpu().numpy(), [r.size for r in erows])
+        np.testing.assert_array_equal(status.cpu().numpy() & 7, estatus)
+        width = fill_to if fill_to else longest
+        if not fill_to:
+            assert int(max_len.item()) == longest
+        eids, emask = O.pad_rows(erows, 1, width)
+        np.testing.assert_array_equal(ids[:, :width].cpu().numpy(), eids)
+        np.testing.assert_array_equal(mask[:, :width].cpu().numpy(), emask)
+
+    def check_packed(e, bb, rows_want, status_want):
+        d, o = to_dev(bb)
+        for want_mask in (True, False):
+            ids, out_off, mask, lengths, status = e.encode_packed(d, o, want_mask=want_mask)
+            torch.cuda.synchronize()
+            oo = out_off.cpu().numpy()
+            np.testing.assert_array_equal(lengths.cpu().numpy(), [r.size for r in rows_want])
+            np.testing.assert_array_equal(oo, np.concatenate([[0], np.cumsum([r.size for r in rows_want])]))
+            np.testing.assert_array_equal(status.cpu().numpy() & 7, status_want)
+            flat = ids.cpu().numpy()
+            np.testing.assert_array_equal(flat[:oo[-1]], np.concatenate(rows_want) if oo[-1] else np.zeros(0, np.int32))
+            if want_mask:
+                assert bool((mask[:oo[-1]] == 1).all())
+
+    check_packed(enc, b, erows, estatus)
+    long_only = [s_ for s_ in strings if len(s_) > 384 * k][:20] + ["", "ACG"]
+    bl = util.batch_from_strings(long_only)
+    check_packed(enc, bl, *O.kmer_encode(ot, bl.data, bl.offsets))
+    # a digit table that is not the plain one: a wave per row for every row, also when packed
+    digit = t.digit.copy()
+    digit[ord("U")] = digit[ord("T")]
+    single = t.single.copy()
+    single[ord("U")] = single[ord("T")]
+    enc2 = encoders.KmerEncoder(k, digit, t.kmer_lut, single, pad_id=1, missing_id=0,
+                                exp_off=t.exp_off, exp_len=t.exp_len, exp_flat=t.exp_flat)
+    sub = strings[:300] + [strings[int(i)] for i in np.argsort([-len(s_) for s_ in strings])[:5]]
+    bs = util.batch_from_strings(sub)
+    check_packed(enc2, bs, *O.kmer_encode(ot, bs.data, bs.offsets))
+
+
 @both_kmer_kernels
 def test_kmer_pad_to_longest_with_width_guess(kmer_kernel_choice):
     """fill_to = 0 with a guess of the longest row: a guess below, at or above the true width
