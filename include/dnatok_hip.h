@@ -291,8 +291,11 @@ int64_t dnatok_bpe_padded_direct_max(const dnatok_bpe_t *t);
  * above 2048 bytes, and the longest row) is refused with DNATOK_E_TOO_LARGE; rows that have to be
  * redone whole are then redone fewer at a time before that happens.  All calls on one GPU share
  * the array: two calls whose device work overlaps (different streams, or another thread) race;
- * calls on one stream, and replays of a captured call, are fine.  Inputs, outputs and results as
- * for dnatok_bpe_encode. */
+ * calls on one stream, and replays of a captured call, are fine.  Before a call is captured, one
+ * eager call of the same shape class (row count, longest row, total of the same order) must have
+ * run in the process: the first call of each kernel form asks the runtime for the form's
+ * attributes and residency, which a capture does not allow.  Inputs, outputs and results as for
+ * dnatok_bpe_encode. */
 #define DNATOK_BPE_STATIC_SCRATCH_BYTES (32u << 20)
 size_t dnatok_bpe_static_scratch_bytes(void);
 int dnatok_bpe_encode_static(const dnatok_bpe_t *t, const uint8_t *bytes, const int64_t *offsets,

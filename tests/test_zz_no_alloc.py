@@ -84,3 +84,50 @@ def test_static_entry_point_refuses_what_its_buffer_cannot_hold():
                                     None)
     torch.cuda.synchronize()
     assert rc == -3 and b"built-in buffer" in L.dnatok_last_error()
+
+
+def test_static_entry_point_replayed_from_a_graph():
+    """The callers this entry point is for capture it into a HIP graph.  After one eager call of
+    the same shape class (the first call of a kernel form sets its attributes and asks the runtime
+    how many workgroups fit, which a capture does not allow), the call is captured and replayed
+    with other input in the same buffers; every replay must give what an eager call gives, with
+    eager calls of another shape (they share the one work buffer) between the replays."""
+    L = _lib.lib()
+    cfg = util.tokenizer_json("4096")
+    kv = bpe_vocab.KernelVocab(bpe_vocab.split_merges(cfg["model"]["merges"]))
+    remap = kv.remap_to(cfg["model"]["vocab"], cfg["model"]["vocab"]["[UNK]"])
+    enc = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv), out_remap=remap)
+    bo = util.bpe_oracle("4096")
+    n, length = 96, 3000                                           # rows cut into chunks: work list, seams, gather
+    batches = [wl.config3_bpe4096(n, length, seed=70 + i) for i in range(3)]
+    data = torch.empty(n * length, dtype=torch.uint8, device=DEV)
+    off = torch.from_numpy(batches[0].offsets).to(DEV)
+    tok = torch.empty(n * length, dtype=torch.int32, device=DEV)
+    lengths = torch.empty(n, dtype=torch.int32, device=DEV)
+    side = torch.cuda.Stream()
+
+    def call():
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        _lib.check(L.dnatok_bpe_encode_static(enc._h, _ptr(data), _ptr(off), n, length, n * length, _ptr(tok),
+                                              _ptr(lengths), stream), "dnatok_bpe_encode_static")
+
+    data.copy_(torch.from_numpy(batches[0].data))
+    print(f"dnatok_bpe_encode_static in a graph rows={n} length={length}", flush=True)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        call()                                                     # the eager call of this shape, on the capture's stream
+        torch.cuda.synchronize()
+        with torch.cuda.graph(g, stream=side):
+            call()
+    other = util.batch_from_strings(wl.config5_ragged(50, seed=9).strings())
+    for b in batches:
+        data.copy_(torch.from_numpy(b.data))
+        tok.fill_(-1)
+        lengths.fill_(-1)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        ln, flat = lengths.cpu().numpy(), tok.cpu().numpy()
+        for i, e in enumerate(bo.encode_batch(b.data, b.offsets)):
+            np.testing.assert_array_equal(flat[i * length:i * length + ln[i]], np.asarray(e), err_msg=f"replayed row {i}")
+        _encode_both(enc, other)                                   # eager work on the shared buffer in between
