@@ -50,6 +50,7 @@ struct dnatok_bpe_table {
     int32_t *out_remap;          // [n_symbols] or nullptr
     uint32_t *ltab;              // the compact form of the table that fits LDS (kLdsTabWords words), or nullptr
     uint32_t lmul1, lmul2;       // its two multipliers
+    void *first;                 // dnatok::FirstPairs on the device, or nullptr (more bytes with rules than classes)
     // dnatok_bpe_encode_padded: the tree of atomics that carries a call's longest row
     // (dnatok::publish_max), one per stream that encodes with this table (calls on one stream are
     // ordered, calls on different streams may overlap); a stream beyond the kMaxTreeSlots-th gets
@@ -78,6 +79,7 @@ struct BpeArgs {
     int32_t n_merges;
     const uint32_t *ltab;
     uint32_t lmul1, lmul2;
+    const void *first;           // FirstPairs (global memory) or nullptr
     // single-character ids of the same bytes, written in the same pass (dnatok_bpe_encode_with_chars):
     // char_ids[i] = char_lut[bytes[i]], char_mask[i] = 1 (null: no mask)
     const int32_t *char_lut;
@@ -115,6 +117,18 @@ typedef uint32_t bpe_u32_a1 __attribute__((aligned(1)));
 // symbol the rule produces, and the rule's gate (lowest rank of any rule using that product).
 struct PairInfo {
     uint32_t rank, product, gate;
+};
+
+// The rules between two single-byte symbols, by the bytes themselves: what every position of a row
+// needs first.  A DNA alphabet has a handful of bytes with such rules (A C G T N), so the bytes are
+// put into at most kFirstClasses classes and the rule of a pair of classes is one 8-byte read from
+// a table a workgroup keeps in LDS, where the general table costs two reads from L2 behind two
+// hashes (11 % of a 1 KB row's time went into its first pairs).  A table with more such bytes than
+// classes has no FirstPairs and every lookup goes to the general table.
+constexpr int kFirstClasses = 8;
+struct FirstPairs {
+    uint8_t cls[256];                                   // the byte's class, or 255: no rule pairs it with another byte
+    uint2 rule[kFirstClasses * kFirstClasses];          // [left class * 8 + right class] {rank, product | gate << 16}; rank kNone: no rule
 };
 
 // The merge table is a cuckoo hash: every rule sits in one of the two slots its key hashes to, so
@@ -292,7 +306,8 @@ __device__ __forceinline__ int32_t bpe_row(
     const int32_t *__restrict__ char_lut = nullptr, int32_t *__restrict__ char_ids = nullptr,
     uint8_t *__restrict__ char_mask = nullptr, const int char_lo = 0, const int char_hi = 0,
     const int pad_stride = 0, const int32_t pad_id = 0, uint8_t *__restrict__ pad_mask = nullptr,
-    const int32_t *__restrict__ remap2 = nullptr, const int pad_elem = 4, const int pad_left = 0)
+    const int32_t *__restrict__ remap2 = nullptr, const int pad_elem = 4, const int pad_left = 0,
+    const FirstPairs *first = nullptr)
 {
     static_assert(!CHARS || PER > 0, "the single-character ids are written from the staged bytes");
     constexpr IT NIL = (IT)~(IT)0;
@@ -373,6 +388,23 @@ __device__ __forceinline__ int32_t bpe_row(
         team_sync<NT>();
     }
     auto byte_at = [&](int i) -> uint32_t { return PER > 0 ? stage[head + i] : src[i]; };
+    if (PER > 0 && first) {
+        // the first pairs by byte class: one 8-byte read from the workgroup's own table per position
+        for (int i = tid; i < n0; i += NT) {
+            const uint32_t ba = byte_at(i), bb = i + 1 < n0 ? byte_at(i + 1) : 0u;
+            const uint32_t ca = first->cls[ba], cb = i + 1 < n0 ? first->cls[bb] : 255u;
+            uint2 rule = uint2{kNone, kNone | (kNone << 16)};
+            if ((ca | cb) < (uint32_t)kFirstClasses) rule = first->rule[ca * kFirstClasses + cb];
+            PosRec<IT> x;
+            x.r = (IT)rule.x;
+            x.nx = (i + 1 < n0) ? (IT)(i + 1) : NIL;
+            x.pv = (i > 0) ? (IT)(i - 1) : NIL;
+            x.s = (IT)byte_to_sym[ba];
+            P[i] = x;
+            NS[i] = (uint16_t)(rule.y & 0xFFFFu); MC[i] = (uint16_t)(rule.y >> 16);
+            if (rule.x != kNone) { cmin = umin(cmin, rule.x); cgate = umin(cgate, rule.y >> 16); }
+        }
+    } else
     for (int i0 = tid; i0 < n0; i0 += kProbes * NT) {
         decltype(pair_probe(pt, 0u, 0u)) e[kProbes];
         uint32_t sa[kProbes], sb[kProbes];
@@ -1111,6 +1143,15 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
     const PairTable pt{a.tab, a.shift, a.mul1, a.mul2};
     uint16_t *b2s = reinterpret_cast<uint16_t *>(sp); sp += 512;
     for (int i = threadIdx.x; i < 256; i += NT * TEAMS) b2s[i] = a.byte_to_sym[i];
+    // the rules between single bytes, by byte class (when the table has few enough such bytes)
+    FirstPairs *const first_lds = reinterpret_cast<FirstPairs *>(sp); sp += sizeof(FirstPairs);
+    static_assert(sizeof(FirstPairs) % 16 == 0, "the state arrays behind it stay aligned");
+    if (a.first) {
+        const uint32_t *src = reinterpret_cast<const uint32_t *>(a.first);
+        for (int i = threadIdx.x; i < (int)(sizeof(FirstPairs) / 4); i += NT * TEAMS)
+            reinterpret_cast<uint32_t *>(first_lds)[i] = src[i];
+    }
+    const FirstPairs *const first_pairs = a.first ? first_lds : nullptr;
     const int team = threadIdx.x / NT, tid = threadIdx.x % NT;
     int32_t *next_item = reinterpret_cast<int32_t *>(sp) + team; sp += 16 * sizeof(int32_t);
     uint32_t *red = reinterpret_cast<uint32_t *>(sp) + team * (4 * (NT / 64) + 4); sp += TEAMS * (4 * (NT / 64) + 4) * 4;
@@ -1230,7 +1271,7 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
                     CHARS && a.char_mask ? a.char_mask + start : nullptr, 0, (int)len,
                     padded ? (int)a.pad_stride : 0, a.pad_id,
                     padded && a.pad_mask ? a.pad_mask + (int64_t)row * a.pad_stride : nullptr, a.pad_remap,
-                    padded ? a.pad_elem : 4, padded ? a.pad_left : 0);
+                    padded ? a.pad_elem : 4, padded ? a.pad_left : 0, first_pairs);
                 team_longest = n_tok > team_longest ? n_tok : team_longest;
             }
         } else if (CHUNKS) {
@@ -1249,7 +1290,7 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
                 pt, b2s, a.out_remap, bytes + start + e0, (int)(e1 - e0), P, NS, MC, Q, C, D, red, tid, nullptr,
                 nullptr, raw, (int)(mid_lo - e0), (int)(mid_hi - e0), p.cnt + 4 * (size_t)m, a.char_lut,
                 CHARS ? a.char_ids + start + e0 : nullptr, CHARS && a.char_mask ? a.char_mask + start + e0 : nullptr,
-                (int)((int64_t)k * p.core - e0), (int)(core_hi - e0));
+                (int)((int64_t)k * p.core - e0), (int)(core_hi - e0), 0, 0, nullptr, nullptr, 4, 0, first_pairs);
         }
         team_sync<NT>();
     }
@@ -1579,11 +1620,43 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
         }
     }
 
+    // FirstPairs: the rules whose two symbols both stand for single bytes, by classes of bytes
+    FirstPairs first{};
+    bool have_first = false;
+    {
+        std::vector<int> cls_of_sym(n_symbols, -1);
+        std::vector<uint8_t> byte_sym(n_symbols, 0);
+        for (int v = 0; v < 256; ++v) byte_sym[b2s[v]] = 1;
+        std::vector<uint32_t> members;                        // symbols with a class, in class order
+        auto give_class = [&](uint32_t sym) {
+            if (cls_of_sym[sym] < 0) { cls_of_sym[sym] = (int)members.size(); members.push_back(sym); }
+        };
+        for (int32_t i = 0; i < n_merges; ++i) {
+            const uint32_t pa = (uint32_t)pair_a_h[i], pb = (uint32_t)pair_b_h[i];
+            if (last_entry[(pa << 16) | pb] != i || !byte_sym[pa] || !byte_sym[pb]) continue;
+            give_class(pa);
+            give_class(pb);
+        }
+        if ((int)members.size() <= kFirstClasses) {
+            have_first = true;
+            for (int v = 0; v < 256; ++v) first.cls[v] = cls_of_sym[b2s[v]] < 0 ? 255 : (uint8_t)cls_of_sym[b2s[v]];
+            for (int q = 0; q < kFirstClasses * kFirstClasses; ++q) first.rule[q] = uint2{kNone, kNone | (kNone << 16)};
+            for (size_t ca = 0; ca < members.size(); ++ca)
+                for (size_t cb = 0; cb < members.size(); ++cb) {
+                    const uint32_t key = (members[ca] << 16) | members[cb];
+                    const uint4 &e1 = tab[pair_slot(key, mul1, shift)], &e2 = tab[pair_slot(key, mul2, shift)];
+                    const uint4 *hit = e1.x == key ? &e1 : (e2.x == key ? &e2 : nullptr);
+                    if (hit) first.rule[ca * kFirstClasses + cb] = uint2{hit->y, hit->z};
+                }
+        }
+    }
+
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
     const size_t o_tab = 0;
     const size_t o_b2s = up(o_tab + (size_t)slots * sizeof(uint4));
     const size_t o_remap = up(o_b2s + 512);
-    const size_t o_ltab = up(o_remap + (out_remap_h ? (size_t)n_symbols * 4 : 0));
+    const size_t o_first = up(o_remap + (out_remap_h ? (size_t)n_symbols * 4 : 0));
+    const size_t o_ltab = up(o_first + sizeof(FirstPairs));
     const size_t o_trees = up(o_ltab + ltab.size() * 4);
     const size_t total = up(o_trees + (size_t)kMaxTreeSlots * kTreeWords * 8) + 256;
     std::vector<uint8_t> host(total, 0);             // (the trees start as zeros)
@@ -1591,6 +1664,7 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
     memcpy(&host[o_b2s], b2s.data(), 512);
     if (out_remap_h) memcpy(&host[o_remap], out_remap_h, (size_t)n_symbols * 4);
     if (!ltab.empty()) memcpy(&host[o_ltab], ltab.data(), ltab.size() * 4);
+    memcpy(&host[o_first], &first, sizeof(FirstPairs));
     void *blob = nullptr;
     hipError_t e = hipMalloc(&blob, total);
     if (e == hipSuccess) e = hipMemcpy(blob, host.data(), total, hipMemcpyHostToDevice);
@@ -1608,6 +1682,7 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
     t->out_remap = out_remap_h ? (int32_t *)(b + o_remap) : nullptr;
     t->ltab = ltab.empty() ? nullptr : (uint32_t *)(b + o_ltab);
     t->lmul1 = lmul1; t->lmul2 = lmul2;
+    t->first = have_first ? (void *)(b + o_first) : nullptr;
     t->max_trees = (unsigned long long *)(b + o_trees);
     *out = t;
     return DNATOK_OK;
@@ -1673,7 +1748,8 @@ __global__ __launch_bounds__(1024) void bpe_longest_kernel(const int32_t *__rest
 template <int NT, int TEAMS, int CAP>
 constexpr size_t lds_bytes()
 {
-    return 512 + 64 + (size_t)TEAMS * (4 * (NT / 64) + 4) * 4 + (size_t)TEAMS * CAP * 15 + (size_t)TEAMS * NT + 64;
+    return 512 + sizeof(FirstPairs) + 64 + (size_t)TEAMS * (4 * (NT / 64) + 4) * 4 + (size_t)TEAMS * CAP * 15 +
+           (size_t)TEAMS * NT + 64;
 }
 
 // Teams of the LDS kernel that are resident at once: of the form that works through a list with
@@ -1833,7 +1909,7 @@ static int bpe_encode_launch(const dnatok_bpe_t *t, const uint8_t *bytes, const 
                              uint8_t *char_mask = nullptr, const BpeArgs *padded = nullptr)
 {
     BpeArgs a{t->tab, t->byte_to_sym, t->out_remap, t->shift, t->mul1, t->mul2, t->n_merges, t->ltab, t->lmul1, t->lmul2,
-              char_lut, char_ids, char_mask};
+              t->first, char_lut, char_ids, char_mask};
     a.placement = t->placement.load(std::memory_order_relaxed);
     if (padded) {
         a.pad_ids = padded->pad_ids; a.pad_mask = padded->pad_mask; a.pad_remap = padded->pad_remap;
