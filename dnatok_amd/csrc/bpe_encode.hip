@@ -110,6 +110,24 @@ struct BpeArgs {
     int32_t placement;
 };
 
+// The arguments of the running kernel where they lie in memory.  What a kernel needs once per row
+// and late (where a padded row goes, what pads it) is read from there at that point, after the
+// merges, instead of held in registers all through them: a register more during the merges is a
+// team less per CU at the sizes that count.
+typedef const __attribute__((address_space(4))) BpeArgs *BpeArgsInMemory;
+
+// (the pointer's halves go through an empty asm statement, so that the reads behind it stay where
+// they are written instead of being moved to the kernel's start)
+__device__ __forceinline__ BpeArgsInMemory kernel_args_now()
+{
+    const uintptr_t at = (uintptr_t)__builtin_amdgcn_kernarg_segment_ptr();
+    uint32_t lo = (uint32_t)at, hi = (uint32_t)(at >> 32);
+    asm volatile("" : "+v"(lo), "+v"(hi));
+    lo = __builtin_amdgcn_readfirstlane(lo);
+    hi = __builtin_amdgcn_readfirstlane(hi);
+    return (BpeArgsInMemory)(((uintptr_t)hi << 32) | lo);
+}
+
 typedef int32_t bpe_int4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 typedef uint32_t bpe_u32_a1 __attribute__((aligned(1)));
 
@@ -305,9 +323,7 @@ __device__ __forceinline__ int32_t bpe_row(
     const int mid_lo = 0, const int mid_hi = 0, int32_t *__restrict__ mid_out = nullptr,
     const int32_t *__restrict__ char_lut = nullptr, int32_t *__restrict__ char_ids = nullptr,
     uint8_t *__restrict__ char_mask = nullptr, const int char_lo = 0, const int char_hi = 0,
-    const int pad_stride = 0, const int32_t pad_id = 0, uint8_t *__restrict__ pad_mask = nullptr,
-    const int32_t *__restrict__ remap2 = nullptr, const int pad_elem = 4, const int pad_left = 0,
-    const FirstPairs *first = nullptr)
+    const FirstPairs *first = nullptr, const int32_t pad_row = 0)
 {
     static_assert(!CHARS || PER > 0, "the single-character ids are written from the staged bytes");
     constexpr IT NIL = (IT)~(IT)0;
@@ -771,10 +787,25 @@ __device__ __forceinline__ int32_t bpe_row(
     // consecutive cells.  (A contiguous piece per thread, as before, cost a fifth of a 1 KB row's
     // time: strided LDS reads, two scans and stores scattered over the row.)
     constexpr int NW = NT / 64;
-    constexpr int kBlockPasses = 8;
+    // (a row of at most PER passes never has more in a block: the passes beyond cost registers for nothing)
+    constexpr int kBlockPasses = (PER > 0 && PER < 8) ? PER : 8;
     uint32_t *wave_cnt = reinterpret_cast<uint32_t *>(NS);           // [kBlockPasses][NW]
     const int lane = tid & 63;
     uint32_t done = 0;                                               // tokens of earlier blocks of passes
+    // PAD: where row pad_row of the padded output lies and what pads it, from the kernel's
+    // arguments (the first of them is the BpeArgs), read here and not before the merges
+    int pad_stride = 0, pad_elem = 4, pad_left = 0;
+    int32_t pad_id = 0;
+    uint8_t *pad_mask = nullptr;
+    const int32_t *remap2 = nullptr;
+    if (PAD) {
+        const BpeArgsInMemory ka = kernel_args_now();
+        pad_stride = (int)ka->pad_stride; pad_elem = ka->pad_elem; pad_left = ka->pad_left; pad_id = ka->pad_id;
+        remap2 = ka->pad_remap;
+        out = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(ka->pad_ids) +
+                                          (int64_t)pad_row * ka->pad_stride * pad_elem);
+        if (ka->pad_mask) pad_mask = ka->pad_mask + (int64_t)pad_row * ka->pad_stride;
+    }
     // cell c of a padded row, in the row's own integer width
     auto put_cell = [&](int c, int32_t v) {
         if (!PAD || pad_elem == 4) out[c] = v;
@@ -1132,9 +1163,15 @@ __global__ __launch_bounds__(256) void bpe_expand_kernel(const int64_t *__restri
 // built without the chunk path, whose copy of the engine costs it registers (a workgroup per CU
 // for rows of at most 1 KB).
 // PADDED: a row's ids go straight to its row of a.pad_ids, padded (dnatok_bpe_encode_padded).
+// Waves per SIMD that the compiler has to leave room for.  Teams of four waves over rows of at
+// most 1 KB are limited by registers, not by LDS: 72 registers are seven teams per CU, 73 are six.
+template <int NT, int TEAMS, int CAP, bool CHUNKS>
+constexpr int kBpeWaves = (NT == 256 && TEAMS == 1 && CAP <= 1024 && !CHUNKS) ? 7 : 1;
+
 template <int NT, int TEAMS, int CAP, bool PLANNED, bool LTAB = false, bool CHARS = false, bool CHUNKS = PLANNED,
           bool PADDED = false>
-__global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
+__global__ __launch_bounds__(NT *TEAMS) __attribute__((amdgpu_waves_per_eu(kBpeWaves<NT, TEAMS, CAP, CHUNKS>)))
+void bpe_lds_kernel(
     BpeArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
     BpePlan p, int32_t n_rows, int32_t *__restrict__ tok_tmp, int32_t *__restrict__ lengths)
 {
@@ -1242,13 +1279,18 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
             // too long: left to the whole-row kernel (row_fail is set); empty: no tokens
             if (tid == 0) lengths[row] = len > CAP ? -1 : 0;
             if (padded) {
-                for (int64_t i = tid; i < a.pad_stride; i += NT) {
-                    const int64_t at = (int64_t)row * a.pad_stride + i;
-                    if (a.pad_elem == 4) reinterpret_cast<int32_t *>(a.pad_ids)[at] = a.pad_id;
-                    else if (a.pad_elem == 8) reinterpret_cast<int64_t *>(a.pad_ids)[at] = (int64_t)a.pad_id;
-                    else if (a.pad_elem == 2) reinterpret_cast<int16_t *>(a.pad_ids)[at] = (int16_t)a.pad_id;
-                    else reinterpret_cast<uint8_t *>(a.pad_ids)[at] = (uint8_t)a.pad_id;
-                    if (a.pad_mask) a.pad_mask[at] = 0;
+                const BpeArgsInMemory ka = kernel_args_now();
+                const int64_t stride = ka->pad_stride;
+                const int32_t elem = ka->pad_elem, pad_id = ka->pad_id;
+                void *const ids = ka->pad_ids;
+                uint8_t *const mask = ka->pad_mask;
+                for (int64_t i = tid; i < stride; i += NT) {
+                    const int64_t at = (int64_t)row * stride + i;
+                    if (elem == 4) reinterpret_cast<int32_t *>(ids)[at] = pad_id;
+                    else if (elem == 8) reinterpret_cast<int64_t *>(ids)[at] = (int64_t)pad_id;
+                    else if (elem == 2) reinterpret_cast<int16_t *>(ids)[at] = (int16_t)pad_id;
+                    else reinterpret_cast<uint8_t *>(ids)[at] = (uint8_t)pad_id;
+                    if (mask) mask[at] = 0;
                 }
             }
             if (CHARS) {
@@ -1264,14 +1306,9 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
             else {
                 const int32_t n_tok = bpe_row<NT, uint16_t, (CAP + NT - 1) / NT, CHARS, PADDED>(
                     pt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC, Q, C, D, red, tid,
-                    padded ? reinterpret_cast<int32_t *>(reinterpret_cast<char *>(a.pad_ids) +
-                                                         (int64_t)row * a.pad_stride * a.pad_elem)
-                           : tok_tmp + start,
+                    padded ? nullptr : tok_tmp + start,        // (a padded row finds its own cells)
                     lengths + row, nullptr, 0, 0, nullptr, a.char_lut, CHARS ? a.char_ids + start : nullptr,
-                    CHARS && a.char_mask ? a.char_mask + start : nullptr, 0, (int)len,
-                    padded ? (int)a.pad_stride : 0, a.pad_id,
-                    padded && a.pad_mask ? a.pad_mask + (int64_t)row * a.pad_stride : nullptr, a.pad_remap,
-                    padded ? a.pad_elem : 4, padded ? a.pad_left : 0, first_pairs);
+                    CHARS && a.char_mask ? a.char_mask + start : nullptr, 0, (int)len, first_pairs, row);
                 team_longest = n_tok > team_longest ? n_tok : team_longest;
             }
         } else if (CHUNKS) {
@@ -1290,14 +1327,15 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
                 pt, b2s, a.out_remap, bytes + start + e0, (int)(e1 - e0), P, NS, MC, Q, C, D, red, tid, nullptr,
                 nullptr, raw, (int)(mid_lo - e0), (int)(mid_hi - e0), p.cnt + 4 * (size_t)m, a.char_lut,
                 CHARS ? a.char_ids + start + e0 : nullptr, CHARS && a.char_mask ? a.char_mask + start + e0 : nullptr,
-                (int)((int64_t)k * p.core - e0), (int)(core_hi - e0), 0, 0, nullptr, nullptr, 4, 0, first_pairs);
+                (int)((int64_t)k * p.core - e0), (int)(core_hi - e0), first_pairs);
         }
         team_sync<NT>();
     }
     // (padded) every workgroup reports once, whether it had a row or not
-    if (padded && a.max_tree) {
+    const BpeArgsInMemory ka = kernel_args_now();
+    if (padded && ka->max_tree) {
         if (TEAMS == 1) {
-            if (threadIdx.x == 0) publish_max(a.max_tree, (unsigned)team_longest, a.longest);
+            if (threadIdx.x == 0) publish_max(ka->max_tree, (unsigned)team_longest, ka->longest);
         } else {
             __shared__ int32_t s_longest[TEAMS];
             if (tid == 0) s_longest[team] = team_longest;
@@ -1306,7 +1344,7 @@ __global__ __launch_bounds__(NT *TEAMS) void bpe_lds_kernel(
                 int32_t m = 0;
 #pragma unroll
                 for (int q = 0; q < TEAMS; ++q) m = s_longest[q] > m ? s_longest[q] : m;
-                publish_max(a.max_tree, (unsigned)m, a.longest);
+                publish_max(ka->max_tree, (unsigned)m, ka->longest);
             }
         }
     }
