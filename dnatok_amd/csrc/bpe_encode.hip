@@ -143,11 +143,22 @@ struct PairInfo {
 // a table a workgroup keeps in LDS, where the general table costs two reads from L2 behind two
 // hashes (11 % of a 1 KB row's time went into its first pairs).  A table with more such bytes than
 // classes has no FirstPairs and every lookup goes to the general table.
+// The table takes the place of the byte-to-symbol table in a workgroup's LDS (a class knows its
+// symbol; the symbol of a byte without a class is read from memory): 144 bytes more, not 768.
+// LDS is handed out in pieces of kLdsPiece bytes, 128 per CU, and the forms for 2 KB chunks and for
+// four rows of 512 bytes sit 304 and 256 bytes under a piece boundary: beyond it a CU holds four
+// workgroups instead of five (measured: a batch of 100 kbp rows 13 % slower).
 constexpr int kFirstClasses = 8;
+constexpr uint32_t kNoClass = 15;
 struct FirstPairs {
-    uint8_t cls[256];                                   // the byte's class, or 255: no rule pairs it with another byte
+    uint8_t cls4[128];                                  // the byte's class, 4 bits each (low nibble: even byte); kNoClass: no rule pairs it with another byte
+    uint16_t sym[kFirstClasses];                        // the class's symbol
     uint2 rule[kFirstClasses * kFirstClasses];          // [left class * 8 + right class] {rank, product | gate << 16}; rank kNone: no rule
+    __device__ __forceinline__ uint32_t cls(uint32_t byte) const { return (cls4[byte >> 1] >> ((byte & 1u) * 4u)) & 15u; }
 };
+constexpr int kLdsPiece = 1280, kLdsPieces = 128;
+// what a workgroup keeps of the table's small parts: FirstPairs, or the byte-to-symbol table
+constexpr size_t kLeadBytes = sizeof(FirstPairs) > 512 ? sizeof(FirstPairs) : 512;
 
 // The merge table is a cuckoo hash: every rule sits in one of the two slots its key hashes to, so
 // a lookup is two independent reads issued together and never a chain of dependent ones.  (With
@@ -323,7 +334,8 @@ __device__ __forceinline__ int32_t bpe_row(
     const int mid_lo = 0, const int mid_hi = 0, int32_t *__restrict__ mid_out = nullptr,
     const int32_t *__restrict__ char_lut = nullptr, int32_t *__restrict__ char_ids = nullptr,
     uint8_t *__restrict__ char_mask = nullptr, const int char_lo = 0, const int char_hi = 0,
-    const FirstPairs *first = nullptr, const int32_t pad_row = 0)
+    const FirstPairs *first = nullptr, const int32_t pad_row = 0,
+    const uint16_t *__restrict__ byte_to_sym_far = nullptr)
 {
     static_assert(!CHARS || PER > 0, "the single-character ids are written from the staged bytes");
     constexpr IT NIL = (IT)~(IT)0;
@@ -406,16 +418,17 @@ __device__ __forceinline__ int32_t bpe_row(
     auto byte_at = [&](int i) -> uint32_t { return PER > 0 ? stage[head + i] : src[i]; };
     if (PER > 0 && first) {
         // the first pairs by byte class: one 8-byte read from the workgroup's own table per position
+        // (byte_to_sym is not staged then: byte_to_sym_far is the table in memory)
         for (int i = tid; i < n0; i += NT) {
             const uint32_t ba = byte_at(i), bb = i + 1 < n0 ? byte_at(i + 1) : 0u;
-            const uint32_t ca = first->cls[ba], cb = i + 1 < n0 ? first->cls[bb] : 255u;
+            const uint32_t ca = first->cls(ba), cb = i + 1 < n0 ? first->cls(bb) : kNoClass;
             uint2 rule = uint2{kNone, kNone | (kNone << 16)};
             if ((ca | cb) < (uint32_t)kFirstClasses) rule = first->rule[ca * kFirstClasses + cb];
             PosRec<IT> x;
             x.r = (IT)rule.x;
             x.nx = (i + 1 < n0) ? (IT)(i + 1) : NIL;
             x.pv = (i > 0) ? (IT)(i - 1) : NIL;
-            x.s = (IT)byte_to_sym[ba];
+            x.s = (IT)(ca < (uint32_t)kFirstClasses ? first->sym[ca] : byte_to_sym_far[ba]);
             P[i] = x;
             NS[i] = (uint16_t)(rule.y & 0xFFFFu); MC[i] = (uint16_t)(rule.y >> 16);
             if (rule.x != kNone) { cmin = umin(cmin, rule.x); cgate = umin(cgate, rule.y >> 16); }
@@ -1178,15 +1191,17 @@ void bpe_lds_kernel(
     extern __shared__ __align__(16) uint8_t smem[];
     uint8_t *sp = smem;
     const PairTable pt{a.tab, a.shift, a.mul1, a.mul2};
-    uint16_t *b2s = reinterpret_cast<uint16_t *>(sp); sp += 512;
-    for (int i = threadIdx.x; i < 256; i += NT * TEAMS) b2s[i] = a.byte_to_sym[i];
-    // the rules between single bytes, by byte class (when the table has few enough such bytes)
-    FirstPairs *const first_lds = reinterpret_cast<FirstPairs *>(sp); sp += sizeof(FirstPairs);
-    static_assert(sizeof(FirstPairs) % 16 == 0, "the state arrays behind it stay aligned");
+    // the rules between single bytes by byte class, when the table has few enough such bytes, or
+    // else the byte-to-symbol table, in the same place
+    uint16_t *b2s = reinterpret_cast<uint16_t *>(sp);
+    FirstPairs *const first_lds = reinterpret_cast<FirstPairs *>(sp); sp += kLeadBytes;
+    static_assert(kLeadBytes % 16 == 0, "the state arrays behind it stay aligned");
     if (a.first) {
         const uint32_t *src = reinterpret_cast<const uint32_t *>(a.first);
         for (int i = threadIdx.x; i < (int)(sizeof(FirstPairs) / 4); i += NT * TEAMS)
             reinterpret_cast<uint32_t *>(first_lds)[i] = src[i];
+    } else {
+        for (int i = threadIdx.x; i < 256; i += NT * TEAMS) b2s[i] = a.byte_to_sym[i];
     }
     const FirstPairs *const first_pairs = a.first ? first_lds : nullptr;
     const int team = threadIdx.x / NT, tid = threadIdx.x % NT;
@@ -1302,13 +1317,15 @@ void bpe_lds_kernel(
         } else if (!CHUNKS || nc == 1) {
             if (LTAB)
                 bpe_row<NT, uint16_t, (CAP + NT - 1) / NT>(lpt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC,
-                                      Q, C, D, red, tid, tok_tmp + start, lengths + row);
+                                      Q, C, D, red, tid, tok_tmp + start, lengths + row, nullptr, 0, 0, nullptr,
+                                      nullptr, nullptr, nullptr, 0, 0, first_pairs, 0, a.byte_to_sym);
             else {
                 const int32_t n_tok = bpe_row<NT, uint16_t, (CAP + NT - 1) / NT, CHARS, PADDED>(
                     pt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC, Q, C, D, red, tid,
                     padded ? nullptr : tok_tmp + start,        // (a padded row finds its own cells)
                     lengths + row, nullptr, 0, 0, nullptr, a.char_lut, CHARS ? a.char_ids + start : nullptr,
-                    CHARS && a.char_mask ? a.char_mask + start : nullptr, 0, (int)len, first_pairs, row);
+                    CHARS && a.char_mask ? a.char_mask + start : nullptr, 0, (int)len, first_pairs, row,
+                    a.byte_to_sym);
                 team_longest = n_tok > team_longest ? n_tok : team_longest;
             }
         } else if (CHUNKS) {
@@ -1327,7 +1344,7 @@ void bpe_lds_kernel(
                 pt, b2s, a.out_remap, bytes + start + e0, (int)(e1 - e0), P, NS, MC, Q, C, D, red, tid, nullptr,
                 nullptr, raw, (int)(mid_lo - e0), (int)(mid_hi - e0), p.cnt + 4 * (size_t)m, a.char_lut,
                 CHARS ? a.char_ids + start + e0 : nullptr, CHARS && a.char_mask ? a.char_mask + start + e0 : nullptr,
-                (int)((int64_t)k * p.core - e0), (int)(core_hi - e0), first_pairs);
+                (int)((int64_t)k * p.core - e0), (int)(core_hi - e0), first_pairs, 0, a.byte_to_sym);
         }
         team_sync<NT>();
     }
@@ -1677,7 +1694,11 @@ extern "C" int dnatok_bpe_table_create(const int32_t *byte_to_id_h, const int32_
         }
         if ((int)members.size() <= kFirstClasses) {
             have_first = true;
-            for (int v = 0; v < 256; ++v) first.cls[v] = cls_of_sym[b2s[v]] < 0 ? 255 : (uint8_t)cls_of_sym[b2s[v]];
+            for (int v = 0; v < 256; ++v) {
+                const uint32_t c = cls_of_sym[b2s[v]] < 0 ? kNoClass : (uint32_t)cls_of_sym[b2s[v]];
+                first.cls4[v >> 1] |= (uint8_t)(c << ((v & 1) * 4));
+            }
+            for (size_t c = 0; c < members.size(); ++c) first.sym[c] = (uint16_t)members[c];
             for (int q = 0; q < kFirstClasses * kFirstClasses; ++q) first.rule[q] = uint2{kNone, kNone | (kNone << 16)};
             for (size_t ca = 0; ca < members.size(); ++ca)
                 for (size_t cb = 0; cb < members.size(); ++cb) {
@@ -1786,9 +1807,18 @@ __global__ __launch_bounds__(1024) void bpe_longest_kernel(const int32_t *__rest
 template <int NT, int TEAMS, int CAP>
 constexpr size_t lds_bytes()
 {
-    return 512 + sizeof(FirstPairs) + 64 + (size_t)TEAMS * (4 * (NT / 64) + 4) * 4 + (size_t)TEAMS * CAP * 15 +
+    return kLeadBytes + 64 + (size_t)TEAMS * (4 * (NT / 64) + 4) * 4 + (size_t)TEAMS * CAP * 15 +
            (size_t)TEAMS * NT + 64;
 }
+// workgroups of a form that a CU's LDS holds
+template <int NT, int TEAMS, int CAP>
+constexpr int lds_workgroups_per_cu()
+{
+    return kLdsPieces / (int)((lds_bytes<NT, TEAMS, CAP>() + kLdsPiece - 1) / kLdsPiece);
+}
+static_assert(lds_workgroups_per_cu<256, 1, 2048>() == 5 && lds_workgroups_per_cu<64, 4, 512>() == 5 &&
+              lds_workgroups_per_cu<256, 1, 1408>() == 7 && lds_workgroups_per_cu<256, 1, 1536>() == 6,
+              "a form grew over a piece boundary of the LDS");
 
 // Teams of the LDS kernel that are resident at once: of the form that works through a list with
 // chunks, which holds the most registers (a batch of more rows than that gets a list).
