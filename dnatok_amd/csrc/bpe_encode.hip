@@ -340,10 +340,11 @@ __device__ __forceinline__ int32_t bpe_row(
     static_assert(!CHARS || PER > 0, "the single-character ids are written from the staged bytes");
     constexpr IT NIL = (IT)~(IT)0;
     constexpr IT DEAD = (IT)kNone;
-    // pairs of table reads in flight per thread.  (Four cost 20 registers and a wave per SIMD; four
-    // for the first pairs only, or all bytes of a thread's positions requested before the first
-    // table read, gained nothing.)
-    constexpr int kProbes = 2;
+    // pairs of table reads in flight per thread.  (Two cost eight registers, the difference between
+    // seven and eight waves per SIMD for rows up to 1 KB: 16 batches of 1024 x 1 KB 272 -> 253 us, one
+    // batch 33.5 -> 32.7 us.  Four cost 20; four for the first pairs only, or all bytes of a thread's
+    // positions requested before the first table read, gained nothing.)
+    constexpr int kProbes = 1;
     const int wv = (NT == 64) ? 0 : (tid >> 6);
     uint32_t *qn = red + 4 * (NT / 64);        // number of merges queued in the current round
     uint32_t *cn = qn + 1;                     // number of candidates queued in the current round
@@ -1176,10 +1177,34 @@ __global__ __launch_bounds__(256) void bpe_expand_kernel(const int64_t *__restri
 // built without the chunk path, whose copy of the engine costs it registers (a workgroup per CU
 // for rows of at most 1 KB).
 // PADDED: a row's ids go straight to its row of a.pad_ids, padded (dnatok_bpe_encode_padded).
-// Waves per SIMD that the compiler has to leave room for.  Teams of four waves over rows of at
-// most 1 KB are limited by registers, not by LDS: 72 registers are seven teams per CU, 73 are six.
+// LDS of a workgroup of the engine kernel: the small tables, the work item, the reduction cells
+// and 15 bytes of state per position and team.
+template <int NT, int TEAMS, int CAP>
+constexpr size_t lds_bytes()
+{
+    return kLeadBytes + 64 + (size_t)TEAMS * (4 * (NT / 64) + 4) * 4 + (size_t)TEAMS * CAP * 15 +
+           (size_t)TEAMS * NT + 64;
+}
+// workgroups of a form that a CU's LDS holds
+template <int NT, int TEAMS, int CAP>
+constexpr int lds_workgroups_per_cu()
+{
+    return kLdsPieces / (int)((lds_bytes<NT, TEAMS, CAP>() + kLdsPiece - 1) / kLdsPiece);
+}
+static_assert(lds_workgroups_per_cu<256, 1, 2048>() == 5 && lds_workgroups_per_cu<64, 4, 512>() == 5 &&
+              lds_workgroups_per_cu<256, 1, 1408>() == 7 && lds_workgroups_per_cu<256, 1, 1536>() == 6,
+              "a form grew over a piece boundary of the LDS");
+
+// Waves per SIMD that the compiler has to leave room for: as many as the LDS lets a CU hold (a
+// workgroup is a wave on every SIMD).  Teams of four waves over rows of at most 1 KB are limited by
+// registers, not by LDS (17 KB a team): 64 registers are eight teams per CU, 65 are seven, 73 six,
+// and left to itself the compiler takes 72 to 85, depending on the form.  The forms that also cut
+// rows into chunks hold a second copy of the engine and are left alone below 2 KB (test geometries);
+// the forms with a wave per row stop at seven (the eighth wave costs them spills to memory).
 template <int NT, int TEAMS, int CAP, bool CHUNKS>
-constexpr int kBpeWaves = (NT == 256 && TEAMS == 1 && CAP <= 1024 && !CHUNKS) ? 7 : 1;
+constexpr int kBpeWaves = (CHUNKS && CAP < 2048) ? 1
+                          : lds_workgroups_per_cu<NT, TEAMS, CAP>() < (NT == 256 ? 8 : 7)
+                                ? lds_workgroups_per_cu<NT, TEAMS, CAP>() : (NT == 256 ? 8 : 7);
 
 template <int NT, int TEAMS, int CAP, bool PLANNED, bool LTAB = false, bool CHARS = false, bool CHUNKS = PLANNED,
           bool PADDED = false>
@@ -1804,21 +1829,6 @@ __global__ __launch_bounds__(1024) void bpe_longest_kernel(const int32_t *__rest
     }
 }
 
-template <int NT, int TEAMS, int CAP>
-constexpr size_t lds_bytes()
-{
-    return kLeadBytes + 64 + (size_t)TEAMS * (4 * (NT / 64) + 4) * 4 + (size_t)TEAMS * CAP * 15 +
-           (size_t)TEAMS * NT + 64;
-}
-// workgroups of a form that a CU's LDS holds
-template <int NT, int TEAMS, int CAP>
-constexpr int lds_workgroups_per_cu()
-{
-    return kLdsPieces / (int)((lds_bytes<NT, TEAMS, CAP>() + kLdsPiece - 1) / kLdsPiece);
-}
-static_assert(lds_workgroups_per_cu<256, 1, 2048>() == 5 && lds_workgroups_per_cu<64, 4, 512>() == 5 &&
-              lds_workgroups_per_cu<256, 1, 1408>() == 7 && lds_workgroups_per_cu<256, 1, 1536>() == 6,
-              "a form grew over a piece boundary of the LDS");
 
 // Teams of the LDS kernel that are resident at once: of the form that works through a list with
 // chunks, which holds the most registers (a batch of more rows than that gets a list).
