@@ -1039,6 +1039,42 @@ def strings_in_extra():
     return out
 
 
+PHASE_NAMES = ["initial_pairs", "round_minimum", "collect_candidates", "decide", "late_walks_or_scan", "apply",
+               "re_rank", "refresh", "output"]
+
+
+def bpe_phase_cycles_extra():
+    """Where the teams of the BPE engine spend their cycles, phase by phase, on the three BPE
+    configurations: from the build of the library with the phase clocks compiled in
+    (libdnatok_hip_phases.so, which this process loads in place of the product library: run with
+    --only-extra bpe_phase_cycles, nothing else in the line is then the product's).  The shares are
+    what thread 0 of each team saw, barriers counted with the phase they end."""
+    import ctypes
+    import torch
+    from dnatok_amd import _lib
+    L = _lib.lib()
+    if not hasattr(L, "dnatok_bpe_phase_cycles"):
+        raise RuntimeError("the loaded library has no phase clocks (python -m dnatok_amd.build makes libdnatok_hip_phases.so)")
+    cells = (ctypes.c_ulonglong * 16)()
+    out = {}
+    for cfg, sustained in (("C3", False), ("C3", True), ("C4", False), ("C5", False)):
+        w = make_workload(cfg, sustained)
+        w.check()
+        _lib.check(L.dnatok_bpe_phase_cycles(cells, 1), "dnatok_bpe_phase_cycles")
+        _, dm = time_steps(w, 20, 0)
+        _lib.check(L.dnatok_bpe_phase_cycles(cells, 1), "dnatok_bpe_phase_cycles")
+        total = float(sum(cells[:9])) or 1.0
+        items, positions = int(cells[15]) or 1, int(cells[14]) or 1
+        out[cfg + ("_sustained" if sustained else "_per_call")] = {
+            "workload": w.name, "device_ms_per_call_instrumented": dm,
+            "share": {n: round(cells[q] / total, 4) for q, n in enumerate(PHASE_NAMES)},
+            "cycles_per_position": round(total / positions, 2), "rounds_per_item": round(cells[12] / items, 2),
+            "merges_per_item": round(cells[13] / items, 1), "positions_per_item": round(positions / items, 1)}
+        del w
+        torch.cuda.empty_cache()
+    return out
+
+
 def merge_table_placement_extra():
     """The BPE merge table of the 4096 vocabulary in global memory (L2; the default) against its compact
     48 KB form kept in LDS by every workgroup (`dnatok_bpe_table_set_placement`), on batches of 1 KB rows:
@@ -1095,7 +1131,7 @@ def main() -> None:
     ap.add_argument("--per-call", action="store_true", help="time one exact batch instead of the sustained form")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--only-extra", default="", choices=["", "merge_table_placement", "pathological", "kmer_rows_with_n", "strings_in",
-                                                         "short_reads"],
+                                                         "short_reads", "bpe_phase_cycles"],
                     help="run only this extra after the headline (for profiling it)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -1106,6 +1142,10 @@ def main() -> None:
         print("bench.py: this backend and this benchmark are single-GPU (rows are independent: several "
               "GPUs would each take a share of the rows, with no exchange). Run with --gpus 1.", file=sys.stderr)
         raise SystemExit(2)
+    if args.only_extra == "bpe_phase_cycles":
+        # the build with the phase clocks in place of the product library, for this whole process
+        from dnatok_amd import _lib, build as _build
+        _lib.LIB_PATH = _build.PHASES_LIB_PATH
 
     import torch
     from dnatok_amd import _lib
@@ -1197,7 +1237,8 @@ def main() -> None:
         result[args.only_extra] = {"merge_table_placement": merge_table_placement_extra,
                                    "pathological": pathological_extra,
                                    "kmer_rows_with_n": kmer_rows_with_n_extra,
-                                   "short_reads": short_reads_extra, "strings_in": strings_in_extra}[args.only_extra]()
+                                   "short_reads": short_reads_extra, "strings_in": strings_in_extra,
+                                   "bpe_phase_cycles": bpe_phase_cycles_extra}[args.only_extra]()
     elif not args.no_extras:
         per_call = {}
         for cfg in ["C1", "C2", "C3", "C4", "C5"]:

@@ -12,6 +12,9 @@ SOURCES = ["errors.hip", "char_encode.hip", "kmer_encode.hip", "bpe_encode.hip",
 # bench.py's memory-only kernels: a library of their own (include/dnatok_diag.h), not part of the product
 DIAG_LIB_PATH = os.path.join(_HERE, "libdnatok_diag.so")
 DIAG_SOURCES = ["diag.hip", "errors.hip"]
+# the BPE engine with its per-phase cycle counters compiled in (-DDNATOK_BPE_PHASE_CYCLES): a whole
+# library beside the product's, for bench.py --only-extra bpe_phase_cycles
+PHASES_LIB_PATH = os.path.join(_HERE, "libdnatok_hip_phases.so")
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # packed-FP32 instruction forms are kept out of all device code
@@ -56,6 +59,11 @@ def build_extension(verbose: bool = False) -> str:
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
         if src in SOURCES:
             objs.append(obj)
+    phases_obj = os.path.join(CSRC, "bpe_encode_phases.o")
+    cmd = [hipcc(), *HIPCC_FLAGS, "-DDNATOK_BPE_PHASE_CYCLES", "-c", os.path.join(CSRC, "bpe_encode.hip"), "-o", phases_obj]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    procs.append(("bpe_encode.hip (phase cycles)", subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
     failed = False
     for src, p in procs:
         out, _ = p.communicate()
@@ -73,6 +81,8 @@ def build_extension(verbose: bool = False) -> str:
     subprocess.check_call(cmd)
     diag_objs = [os.path.join(CSRC, x.replace(".hip", ".o")) for x in DIAG_SOURCES]
     subprocess.check_call([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", DIAG_LIB_PATH, *diag_objs])
+    phases_objs = [phases_obj if o.endswith("bpe_encode.o") else o for o in objs]
+    subprocess.check_call([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PHASES_LIB_PATH, *phases_objs])
     build_hostpack(verbose)
     return LIB_PATH
 

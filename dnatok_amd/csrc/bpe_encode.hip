@@ -306,6 +306,51 @@ __device__ __forceinline__ uint32_t team_exclusive_sum(uint32_t v, uint32_t *red
     return carry + inc - v;
 }
 
+// Where a team's time goes, phase by phase: a build option (-DDNATOK_BPE_PHASE_CYCLES: the library
+// libdnatok_hip_phases.so, never the product library, whose PhaseClock is empty and costs nothing).
+// Thread 0 of every team reads the shader clock at the end of each phase of bpe_row and adds the
+// cycles since the last reading to the phase's cell; a barrier at the end of a phase counts for
+// that phase.  The cells of a workgroup (kPhaseCells each, workgroups modulo kPhaseGroups) are read
+// and cleared by dnatok_bpe_phase_cycles.  The instrumented kernels hold more registers than the
+// shipped ones (fewer teams per CU): the shares of the phases are what the numbers are for.
+enum BpePhase {
+    kPhInitial = 0, kPhMinimum, kPhCollect, kPhDecide, kPhLate, kPhApply, kPhRerank, kPhRefresh, kPhOutput,
+    kPhRounds = 12, kPhMerges = 13, kPhPositions = 14, kPhItems = 15, kPhaseCells = 16
+};
+#ifdef DNATOK_BPE_PHASE_CYCLES
+constexpr int kPhaseGroups = 4096;
+__device__ unsigned long long g_phase_cycles[kPhaseGroups * kPhaseCells];
+struct PhaseClock {
+    long long t, cell[kPhaseCells];
+    __device__ __forceinline__ PhaseClock() : t(clock64())
+    {
+#pragma unroll
+        for (int q = 0; q < kPhaseCells; ++q) cell[q] = 0;
+    }
+    __device__ __forceinline__ void lap(const int phase)
+    {
+        const long long now = clock64();
+        cell[phase] += now - t;
+        t = now;
+    }
+    __device__ __forceinline__ void count(const int what, const long long n) { cell[what] += n; }
+    __device__ __forceinline__ void flush(const int tid)
+    {
+        if (tid != 0) return;
+        unsigned long long *g = g_phase_cycles + (size_t)(blockIdx.x % kPhaseGroups) * kPhaseCells;
+#pragma unroll
+        for (int q = 0; q < kPhaseCells; ++q)
+            if (cell[q]) atomicAdd(&g[q], (unsigned long long)cell[q]);
+    }
+};
+#else
+struct PhaseClock {
+    __device__ __forceinline__ void lap(int) {}
+    __device__ __forceinline__ void count(int, long long) {}
+    __device__ __forceinline__ void flush(int) {}
+};
+#endif
+
 // What the engine keeps per position, in one record so that a step along a chain of candidates
 // is one read: rank of the pair the position starts (kNone = no rule / dead), right and left
 // live neighbour, symbol.  8 bytes with 16-bit links (LDS kernels), 16 bytes with 32-bit links
@@ -361,6 +406,7 @@ __device__ __forceinline__ int32_t bpe_row(
     // position i belongs to thread i % NT: in every pass the lanes of a wave touch consecutive
     // positions, so the LDS state arrays are read and written without bank conflicts
 
+    PhaseClock clk;
     // symbols, links and the initial pair of every position, kProbes pairs of table reads in flight at a time
     uint32_t cmin = kEmptyKey, cgate = kEmptyKey;
     D[tid] = 0;
@@ -475,6 +521,7 @@ __device__ __forceinline__ int32_t bpe_row(
         }
     }
 
+    clk.lap(kPhInitial);
     int flip = 0;
     int budget = n0 + 8;                       // every round merges at least one pair
     bool stuck = false;
@@ -483,7 +530,9 @@ __device__ __forceinline__ int32_t bpe_row(
         uint32_t rmin, gate;
         team_min2<NT>(cmin, cgate, red + flip * (NT / 64) * 2, wv, rmin, gate);   // (syncs the team)
         flip ^= 1;
+        clk.lap(kPhMinimum);
         if (rmin >= kNone) break;
+        clk.count(kPhRounds, 1);
         const bool single = gate <= rmin;          // non-monotone table: one merge this round
         uint32_t leftmost = 0;
         if (single) {
@@ -553,6 +602,7 @@ __device__ __forceinline__ int32_t bpe_row(
                 }
             }
             team_sync<NT>();
+            clk.lap(kPhCollect);
             ncand = (int)*cn;
             for (int c0 = 0; c0 < ncand; c0 += NT) {      // the same trip count for every lane
                 const int c = c0 + tid;
@@ -596,6 +646,7 @@ __device__ __forceinline__ int32_t bpe_row(
             }
         }
         team_sync<NT>();
+        clk.lap(kPhDecide);
         const uint32_t late = single ? 0u : *capf;
         const bool by_scan = late > kLateMax || ncand + (int)late > n0;
         if (late != 0 && !by_scan) {
@@ -704,6 +755,8 @@ __device__ __forceinline__ int32_t bpe_row(
             team_sync<NT>();
         }
         const int nm = (int)*qn;                   // merges of this round (they do not overlap)
+        clk.lap(kPhLate);
+        clk.count(kPhMerges, nm);
 
         // apply: position i absorbs its right neighbour j; one merge per thread and pass
         for (int m = tid; m < nm; m += NT) {
@@ -718,6 +771,7 @@ __device__ __forceinline__ int32_t bpe_row(
             D[(int)(j % NT)] = 1;             // j's owner must refresh its cached minimum
         }
         team_sync<NT>();
+        clk.lap(kPhApply);
 
         // re-rank the two pairs around every new symbol: probe 2m is the pair (new, right
         // neighbour), probe 2m + 1 the pair (left neighbour, new).  The probes are dealt evenly to
@@ -755,6 +809,7 @@ __device__ __forceinline__ int32_t bpe_row(
             }
         }
         team_sync<NT>();
+        clk.lap(kPhRerank);
         if (tid == 0) { *qn = 0; *cn = 0; *capf = 0; }   // seen by the next round's decide (a sync lies between)
 
         if (D[tid]) {
@@ -776,7 +831,10 @@ __device__ __forceinline__ int32_t bpe_row(
                 }
             }
         }
+        clk.lap(kPhRefresh);
     }
+    clk.count(kPhPositions, n0);
+    clk.count(kPhItems, 1);
 
     if (raw_out) {
         // chunk of a long row: hand back the symbol at every start position (kNone elsewhere) and
@@ -792,6 +850,8 @@ __device__ __forceinline__ int32_t bpe_row(
         team_sync<NT>();                         // red may still be read by the last round's minimum
         (void)team_exclusive_sum<NT>(live, red, wv, total);
         if (tid == 0) *mid_out = (int32_t)total;
+        clk.lap(kPhOutput);
+        clk.flush(tid);
         return 0;
     }
     // Compact the live symbols to the output, in position order.  Position i = pass * NT + tid, so a
@@ -874,6 +934,8 @@ __device__ __forceinline__ int32_t bpe_row(
         if (pad_mask)
             for (int i = tid; i < pad_stride; i += NT) pad_mask[i] = (i >= pad_from && i < pad_to) ? 0 : 1;
     }
+    clk.lap(kPhOutput);
+    clk.flush(tid);
     return (int32_t)done;
 }
 
@@ -1201,10 +1263,15 @@ static_assert(lds_workgroups_per_cu<256, 1, 2048>() == 5 && lds_workgroups_per_c
 // and left to itself the compiler takes 72 to 85, depending on the form.  The forms that also cut
 // rows into chunks hold a second copy of the engine and are left alone below 2 KB (test geometries);
 // the forms with a wave per row stop at seven (the eighth wave costs them spills to memory).
+#ifdef DNATOK_BPE_PHASE_CYCLES
+template <int NT, int TEAMS, int CAP, bool CHUNKS>
+constexpr int kBpeWaves = 1;              // (the phase clock's cells take registers: no limit in that build)
+#else
 template <int NT, int TEAMS, int CAP, bool CHUNKS>
 constexpr int kBpeWaves = (CHUNKS && CAP < 2048) ? 1
                           : lds_workgroups_per_cu<NT, TEAMS, CAP>() < (NT == 256 ? 8 : 7)
                                 ? lds_workgroups_per_cu<NT, TEAMS, CAP>() : (NT == 256 ? 8 : 7);
+#endif
 
 template <int NT, int TEAMS, int CAP, bool PLANNED, bool LTAB = false, bool CHARS = false, bool CHUNKS = PLANNED,
           bool PADDED = false>
@@ -2234,3 +2301,24 @@ extern "C" int dnatok_bpe_encode_static(const dnatok_bpe_t *t, const uint8_t *by
     const BpePlan p = make_plan(t, base, n_rows, max_len, total, slabs);
     return bpe_encode_launch(t, bytes, offsets, n_rows, max_len, total, p, tok_tmp, lengths, (hipStream_t)stream);
 }
+
+#ifdef DNATOK_BPE_PHASE_CYCLES
+// (measurement build only) The cells of all workgroups added up: cycles[0 .. 15], see BpePhase;
+// reset != 0 clears them afterwards.  Synchronises the device.
+extern "C" int dnatok_bpe_phase_cycles(unsigned long long *cycles, int reset)
+{
+    DNATOK_REQUIRE(cycles, DNATOK_E_INVALID, "dnatok_bpe_phase_cycles: null argument");
+    std::vector<unsigned long long> all((size_t)kPhaseGroups * kPhaseCells);
+    DNATOK_HIP_TRY(hipDeviceSynchronize());
+    DNATOK_HIP_TRY(hipMemcpyFromSymbol(all.data(), HIP_SYMBOL(g_phase_cycles), all.size() * sizeof(unsigned long long)));
+    for (int q = 0; q < kPhaseCells; ++q) cycles[q] = 0;
+    for (size_t g = 0; g < (size_t)kPhaseGroups; ++g)
+        for (int q = 0; q < kPhaseCells; ++q) cycles[q] += all[g * kPhaseCells + q];
+    if (reset) {
+        void *at = nullptr;
+        DNATOK_HIP_TRY(hipGetSymbolAddress(&at, HIP_SYMBOL(g_phase_cycles)));
+        DNATOK_HIP_TRY(hipMemset(at, 0, all.size() * sizeof(unsigned long long)));
+    }
+    return DNATOK_OK;
+}
+#endif

@@ -27,6 +27,15 @@ int dnatok_diag_copy_tiles(const void *src, void *dst, size_t bytes, void *strea
 int dnatok_diag_kmer_shape(const uint8_t *bytes, const int64_t *offsets, int64_t n_rows,
                            int64_t t_cap, int64_t fill_to, int32_t *ids, uint8_t *mask, void *stream);
 
+/* libdnatok_hip_phases.so only (the whole product library compiled with -DDNATOK_BPE_PHASE_CYCLES;
+ * same entry points as include/dnatok_hip.h, plus this one): where the teams of the BPE engine spent
+ * their shader-clock cycles since the last reset, summed over all teams, as thread 0 of each team saw
+ * them.  cycles[0..8] = initial pairs, round minimum, collect candidates, decide, late walks / scan,
+ * apply, re-rank, refresh, output; cycles[12..15] = rounds, merges, positions, items (rows and chunks).
+ * reset != 0 clears the cells afterwards.  Synchronises the device.  The instrumented kernels hold
+ * more registers than the shipped ones: read the shares, not the totals. */
+int dnatok_bpe_phase_cycles(unsigned long long *cycles, int reset);
+
 #ifdef __cplusplus
 }
 #endif

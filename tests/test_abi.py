@@ -57,3 +57,17 @@ def test_measurement_library_is_separate():
     assert D.dnatok_diag_kmer_shape(None, None, 1, 8, 8, None, None, None) == -1
     P = ctypes.CDLL(_lib.LIB_PATH)
     assert not hasattr(P, "dnatok_diag_copy_tiles") and not hasattr(P, "dnatok_diag_kmer_shape")
+
+
+def test_phase_cycle_counters_are_a_build_of_their_own():
+    """The engine's per-phase cycle counters are compiled into libdnatok_hip_phases.so only
+    (-DDNATOK_BPE_PHASE_CYCLES); that library carries the whole C ABI besides."""
+    from dnatok_amd import build
+    assert os.path.exists(build.PHASES_LIB_PATH), "build with: python -m dnatok_amd.build"
+    Q = ctypes.CDLL(build.PHASES_LIB_PATH)
+    assert hasattr(Q, "dnatok_bpe_phase_cycles")
+    Q.dnatok_last_error.restype = ctypes.c_char_p
+    assert Q.dnatok_bpe_phase_cycles(None, 0) == -1 and b"null" in Q.dnatok_last_error()
+    for name in _lib.EXPORTS:
+        assert hasattr(Q, name), name
+    assert not hasattr(ctypes.CDLL(_lib.LIB_PATH), "dnatok_bpe_phase_cycles")
