@@ -1197,6 +1197,50 @@ def test_bpe_nonmonotone_random_tables():
             np.testing.assert_array_equal(r, e, err_msg=f"trial {trial} {s} {merges}")
 
 
+@pytest.mark.parametrize("letters, ruled", [(12, 12), (9, 6), (8, 8), (20, 3)])
+def test_bpe_tables_over_larger_alphabets(letters, ruled):
+    """The first pair of a position comes from a table by byte class when at most 8 bytes take part in
+    rules between single bytes, and from the general table otherwise; bytes that take part in no such
+    rule have no class.  Alphabets of `letters` bytes of which `ruled` occur in rules between single
+    bytes: more than 8 (no class table), exactly 8, and fewer with classless bytes among the input;
+    rows up to 5,000 bytes, so that whole rows, chunks and one-wave teams all meet them."""
+    say(f"bpe alphabets: {letters} letters, {ruled} in rules between single bytes")
+    rng = random.Random(100 * letters + ruled)
+    alpha = "ACGTNRYKMSWBDHVacgt"[:letters] if letters <= 19 else "ACGTNRYKMSWBDHVacgtn"
+    for trial in range(6):
+        base = list(alpha[:ruled])
+        toks, merges, seen = list(base), [], set()
+        while len(merges) < rng.randint(20, 120):
+            a, b2 = rng.choice(toks), rng.choice(toks)
+            if (a, b2) in seen or len(a + b2) > 8:
+                continue
+            seen.add((a, b2))
+            merges.append((a, b2))
+            if a + b2 not in toks:
+                toks.append(a + b2)
+        # rules of a longer token with a letter that pairs with no single byte: the letter has a symbol, no class
+        for c in alpha[ruled:]:
+            long_toks = [t for t in toks if len(t) > 1]
+            if long_toks:
+                t = rng.choice(long_toks)
+                if (t, c) not in seen and len(t + c) <= 9:
+                    seen.add((t, c))
+                    merges.append((t, c))
+        # monotone: a rule's product is only used by later rules (rows may then be cut into chunks)
+        kv = bpe_vocab.KernelVocab(merges)
+        enc = encoders.BpeEncoder(kv.pair_a, kv.pair_b, kv.new_id, len(kv))
+        bo = O.BpeOracle(merges)
+        seqs = ["".join(rng.choice(alpha) for _ in range(rng.choice([1, 2, 63, 200, 400, 900, 1024, 1500, 2048, 3000, 5000])))
+                for _ in range(40)]
+        seqs += ["".join(rng.choice(alpha[:max(ruled, 1)]) for _ in range(700)), alpha * 30]
+        b = util.batch_from_strings(seqs)
+        for s2, r, e in zip(seqs, bpe_rows(enc, b), bo.encode_batch(b.data, b.offsets, remap=False)):
+            np.testing.assert_array_equal(r, e, err_msg=f"trial {trial} {s2[:40]}")
+        short = util.batch_from_strings([q[:300] for q in seqs] * 40)          # teams of one wave
+        for s2, r, e in zip(seqs * 40, bpe_rows(enc, short), bo.encode_batch(short.data, short.offsets, remap=False)):
+            np.testing.assert_array_equal(r, e, err_msg=f"short, trial {trial} {s2[:40]}")
+
+
 def test_bpe_nonmonotone_tables_with_rows_above_the_lds_capacity():
     """Tables with two rules for one string are not chunked: rows above 2048 bytes go to the whole-row
     kernel (state in global memory), including its rounds that merge a single pair."""
