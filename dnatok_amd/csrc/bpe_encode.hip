@@ -1459,25 +1459,37 @@ void bpe_lds_kernel(
     }
 }
 
-// One workgroup per chunk of a multi-chunk row: the seam with the chunk to its right.  The two
-// runs over the shared stretch (at most 2 x overlap positions) are staged in LDS first: the search
-// walks from token start to token start, a chain of dependent reads that is several times
-// shorter there than in L2.  (One wave per chunk instead of one workgroup was measured for this
-// kernel and the two after it: twice as slow, the per-lane loops over the chunk get too long.)
-constexpr int kSeamStage = 1024;          // positions of the shared stretch held in LDS
+// The seam between a chunk of a multi-chunk row and the chunk to its right, by a team of NT threads
+// (256 / NT teams to a workgroup).  The two runs over the shared stretch (2 x overlap positions) are
+// staged in the team's part of LDS first: the search walks from token start to token start, a chain
+// of dependent reads that is several times shorter there than in L2.  A seam is two dependent trips
+// to memory and a few hundred instructions.  With few seams (all of them resident at once as
+// workgroups: one batch of 32 rows of 100 kbp) the 256-thread team is faster (the call 160 against
+// 165 us: the per-lane loops are a quarter as long).  With many, what counts is the number of seams in
+// flight, and a wave per seam holds four times as many, with no workgroup barrier (8 such batches per
+// call: 56 -> 38 us, 8 ragged batches of 12 Mbp: 97 -> 56 us).
+constexpr int kSeamStage = 1024;          // positions of the shared stretch a team holds in LDS
+constexpr int kSeamWaveFrom = 2048;       // from this many chunk slots on: a wave per seam
 
+template <int NT>
 __global__ __launch_bounds__(256) void bpe_seam_kernel(const int64_t *__restrict__ offsets, BpePlan p)
 {
-    __shared__ uint32_t best[4], red[8];
-    __shared__ uint16_t sa_s[kSeamStage], sb_s[kSeamStage];
+    constexpr int TEAMS = 256 / NT;
+    __shared__ uint16_t stage_s[TEAMS][2 * kSeamStage];
+    __shared__ uint32_t red_s[TEAMS][4 * (NT / 64) + 4];
+    const int team = threadIdx.x / NT, tid = threadIdx.x % NT;
+    const int wv = (NT == 64) ? 0 : (tid >> 6);
+    uint16_t *const sa_s = stage_s[team], *const sb_s = stage_s[team] + kSeamStage;
+    uint32_t *const red = red_s[team];
     // (the first record is requested beside the count, not behind it; the slot exists either way)
+    const int32_t m0 = (int32_t)blockIdx.x * TEAMS + team;
     int4 rc_first = make_int4(0, 0, 0, 0);
-    if ((int64_t)blockIdx.x < p.max_mc) rc_first = p.rec[blockIdx.x];
+    if ((int64_t)m0 < p.max_mc) rc_first = p.rec[m0];
     const int32_t n_mc = p.counts[1];
-    for (int32_t m = blockIdx.x; m < n_mc; m += gridDim.x) {
-        const int4 rc = m == (int32_t)blockIdx.x ? rc_first : p.rec[m];
+    for (int32_t m = m0; m < n_mc; m += (int32_t)gridDim.x * TEAMS) {
+        const int4 rc = m == m0 ? rc_first : p.rec[m];
         const int32_t row = rc.x, k = rc.y, nc = rc.z;
-        if (k + 1 >= nc) continue;                                   // last chunk: no seam to the right
+        if (k + 1 >= nc) continue;                                   // last chunk: no seam to the right (the same for the whole team)
         const int64_t len = rc.w;
         const int64_t ea0 = (int64_t)k * p.core - p.overlap < 0 ? 0 : (int64_t)k * p.core - p.overlap;
         int64_t ea1 = (int64_t)(k + 1) * p.core + p.overlap;
@@ -1486,26 +1498,25 @@ __global__ __launch_bounds__(256) void bpe_seam_kernel(const int64_t *__restrict
         const uint16_t *A = p.chunk_sym + (size_t)m * p.ext;         // A[i - ea0]
         const uint16_t *B = p.chunk_sym + (size_t)(m + 1) * p.ext;   // B[i - eb0]
         const int n = (int)(ea1 - eb0);                              // shared positions eb0 .. ea1
-        const bool staged = n <= kSeamStage;                         // (the same for the whole workgroup)
+        const bool staged = n <= kSeamStage;                         // (the same for the whole team)
+        team_sync<NT>();                                             // the team's last seam is read no more
         if (staged) {
-            for (int j = threadIdx.x; j < n; j += 256) { sa_s[j] = A[eb0 - ea0 + j]; sb_s[j] = B[j]; }
-            __syncthreads();
+            for (int j = tid; j < n; j += NT) { sa_s[j] = A[eb0 - ea0 + j]; sb_s[j] = B[j]; }
+            team_sync<NT>();
         }
         auto a_at = [&](int j) -> uint32_t { return staged ? sa_s[j] : A[eb0 - ea0 + j]; };
         auto b_at = [&](int j) -> uint32_t { return staged ? sb_s[j] : B[j]; };
         uint32_t mine = 0xFFFFFFFFu;
-        for (int i = threadIdx.x; i < n; i += 256) {
+        for (int i = tid; i < n; i += NT) {
             const uint32_t sa = a_at(i);
             if (sa == kNone || sa != b_at(i)) continue;
             int j = i + 1;                                           // next token start in A
             while (j < n && a_at(j) == kNone) ++j;
             if (j < n && a_at(j) == b_at(j)) { mine = (uint32_t)(eb0 + j); break; }
         }
-        mine = wave_min_u32(mine);
-        if ((threadIdx.x & 63) == 0) best[threadIdx.x >> 6] = mine;
-        __syncthreads();
-        const uint32_t b = umin(umin(best[0], best[1]), umin(best[2], best[3]));
-        if (threadIdx.x == 0) {
+        uint32_t b, unused;
+        team_min2<NT>(mine, kEmptyKey, red, wv, b, unused);
+        if (tid == 0) {
             if (b == 0xFFFFFFFFu) {
                 p.seam[m] = -1;
                 if (atomicExch(&p.row_fail[row], 1) == 0) atomicAdd(&p.counts[3], 1);
@@ -1518,18 +1529,18 @@ __global__ __launch_bounds__(256) void bpe_seam_kernel(const int64_t *__restrict
         uint32_t tail = 0, head = 0;
         if (b != 0xFFFFFFFFu) {
             const int cut = (int)((int64_t)b - eb0);
-            for (int i = threadIdx.x; i < n; i += 256) {
+            for (int i = tid; i < n; i += NT) {
                 if (i < cut) tail += a_at(i) != kNone;
                 else head += b_at(i) != kNone;
             }
         }
+        team_sync<NT>();                                 // (red is still being read for the minimum)
         uint32_t both;                                   // (each count is below 2^16: one sum for the two)
-        (void)team_exclusive_sum<256>(tail | (head << 16), red, threadIdx.x >> 6, both);
-        if (threadIdx.x == 0) {
+        (void)team_exclusive_sum<NT>(tail | (head << 16), red, wv, both);
+        if (tid == 0) {
             p.cnt[4 * (size_t)m + 2] = (int32_t)(both & 0xFFFFu);
             p.cnt[4 * (size_t)(m + 1) + 1] = (int32_t)(both >> 16);
         }
-        __syncthreads();
     }
 }
 
@@ -2099,7 +2110,12 @@ static int bpe_encode_launch(const dnatok_bpe_t *t, const uint8_t *bytes, const 
     if (long_rows) {
         if (chunking) {
             int64_t g = p.max_mc < 4096 ? p.max_mc : 4096;
-            bpe_seam_kernel<<<(int)(g < 1 ? 1 : g), 256, 0, s>>>(offsets, p);
+            if (p.max_mc >= kSeamWaveFrom) {                               // a wave per seam, up to two rounds of workgroups
+                int64_t gs = (p.max_mc + 3) / 4;
+                bpe_seam_kernel<64><<<(int)(gs > 4096 ? 4096 : gs), 256, 0, s>>>(offsets, p);
+            } else {
+                bpe_seam_kernel<256><<<(int)(g < 1 ? 1 : g), 256, 0, s>>>(offsets, p);
+            }
             DNATOK_HIP_TRY(hipGetLastError());
             bpe_gather_kernel<<<(int)(g < 1 ? 1 : g), 256, 0, s>>>(a, offsets, p, tok_tmp, lengths);
             DNATOK_HIP_TRY(hipGetLastError());
