@@ -1562,43 +1562,50 @@ __device__ __forceinline__ ChunkSpan chunk_span(const BpePlan &p, int32_t m)
     return c;
 }
 
-// One workgroup per chunk: its tokens, compacted, behind those of the row's earlier chunks.
-// Positions are taken 256 at a time: a ballot per wave places every live symbol among its wave's,
-// the waves' counts go through LDS, all symbols (and their remapped ids) of a block of passes are
-// loaded before the first store, and a wave's stores go to consecutive cells.  (A contiguous piece
-// per thread with load, remap and store in one loop ran as a chain of dependent loads: the
-// stores may alias what the next iteration reads.)
+// A team of NT threads per chunk (256 / NT teams to a workgroup): its tokens, compacted, behind those
+// of the row's earlier chunks.  Positions are taken NT at a time: a ballot per wave places every live
+// symbol among its wave's, the waves' counts go through LDS, all symbols (and their remapped ids) of a
+// block of passes are loaded before the first store, and a wave's stores go to consecutive cells.  (A
+// contiguous piece per thread with load, remap and store in one loop ran as a chain of dependent
+// loads: the stores may alias what the next iteration reads.)  As with the seams: a 256-thread team
+// when all chunks are resident at once anyway, a wave per chunk (four times as many in flight) when
+// there are many.
+template <int NT>
 __global__ __launch_bounds__(256) void bpe_gather_kernel(
     BpeArgs a, const int64_t *__restrict__ offsets, BpePlan p, int32_t *__restrict__ tok_tmp,
     int32_t *__restrict__ lengths)
 {
     constexpr int kPasses = 8;
-    __shared__ uint32_t red[8];
-    __shared__ uint32_t wave_cnt[kPasses][4];
-    const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    constexpr int TEAMS = 256 / NT, NW = NT / 64;
+    __shared__ uint32_t red_s[TEAMS][4 * NW + 4];
+    __shared__ uint32_t wave_cnt_s[TEAMS][kPasses][NW];
+    const int team = threadIdx.x / NT, tid = threadIdx.x % NT;
+    const int wv = (NT == 64) ? 0 : (tid >> 6), lane = tid & 63;
+    uint32_t *const red = red_s[team];
+    uint32_t (*const wave_cnt)[NW] = wave_cnt_s[team];
     const int32_t n_mc = p.counts[1];
-    for (int32_t m = blockIdx.x; m < n_mc; m += gridDim.x) {
+    for (int32_t m = (int32_t)blockIdx.x * TEAMS + team; m < n_mc; m += (int32_t)gridDim.x * TEAMS) {
         const ChunkSpan c = chunk_span(p, m);
-        if (p.row_fail[c.row]) continue;
+        if (p.row_fail[c.row]) continue;                 // (the same for the whole team)
         // tokens of the row's chunks before this one.  (Summing them behind the first block's
         // loads instead of in front of them made the kernel 10 % slower; requesting the chunk's
         // record beside the chunk count, and both seams beside the record, 5 %.)
         uint32_t before = 0;
-        for (int32_t j = threadIdx.x; j < c.k; j += 256) {
+        for (int32_t j = tid; j < c.k; j += NT) {
             const int32_t *part = p.cnt + 4 * (size_t)(m - c.k + j);       // {unshared, after left seam, before right seam}
             before += (uint32_t)(part[0] + (j > 0 ? part[1] : 0) + part[2]);
         }
         uint32_t base;
-        (void)team_exclusive_sum<256>(before, red, wv, base);
+        (void)team_exclusive_sum<NT>(before, red, wv, base);
         const uint16_t *sym = p.chunk_sym + (size_t)m * p.ext;
         int32_t *out = tok_tmp + offsets[c.row];
         uint32_t done = base;
-        for (int64_t i0 = c.lo; i0 < c.hi; i0 += kPasses * 256) {
+        for (int64_t i0 = c.lo; i0 < c.hi; i0 += kPasses * NT) {
             uint32_t sy[kPasses], ahead[kPasses];
             int32_t val[kPasses];
 #pragma unroll
             for (int k = 0; k < kPasses; ++k) {
-                const int64_t i = i0 + k * 256 + threadIdx.x;
+                const int64_t i = i0 + k * NT + tid;
                 sy[k] = i < c.hi ? (uint32_t)sym[i - c.e0] : kNone;
             }
 #pragma unroll
@@ -1608,13 +1615,13 @@ __global__ __launch_bounds__(256) void bpe_gather_kernel(
                 ahead[k] = (uint32_t)__builtin_popcountll(live & ((1ull << lane) - 1ull));
                 if (lane == 0) wave_cnt[k][wv] = (uint32_t)__builtin_popcountll(live);
             }
-            __syncthreads();
+            team_sync<NT>();
             uint32_t at = done;
 #pragma unroll
             for (int k = 0; k < kPasses; ++k) {
                 uint32_t mine = at;
 #pragma unroll
-                for (int w = 0; w < 4; ++w) {
+                for (int w = 0; w < NW; ++w) {
                     const uint32_t n = wave_cnt[k][w];
                     if (w < wv) mine += n;
                     at += n;
@@ -1622,9 +1629,9 @@ __global__ __launch_bounds__(256) void bpe_gather_kernel(
                 if (sy[k] != kNone) out[mine + ahead[k]] = val[k];
             }
             done = at;
-            __syncthreads();                                 // wave_cnt is rewritten by the next block
+            team_sync<NT>();                                 // wave_cnt is rewritten by the next block
         }
-        if (threadIdx.x == 0 && c.k + 1 == c.nc) lengths[c.row] = (int32_t)done;
+        if (tid == 0 && c.k + 1 == c.nc) lengths[c.row] = (int32_t)done;
     }
 }
 
@@ -2117,7 +2124,12 @@ static int bpe_encode_launch(const dnatok_bpe_t *t, const uint8_t *bytes, const 
                 bpe_seam_kernel<256><<<(int)(g < 1 ? 1 : g), 256, 0, s>>>(offsets, p);
             }
             DNATOK_HIP_TRY(hipGetLastError());
-            bpe_gather_kernel<<<(int)(g < 1 ? 1 : g), 256, 0, s>>>(a, offsets, p, tok_tmp, lengths);
+            if (p.max_mc >= kSeamWaveFrom) {
+                int64_t gs = (p.max_mc + 3) / 4;
+                bpe_gather_kernel<64><<<(int)(gs > 4096 ? 4096 : gs), 256, 0, s>>>(a, offsets, p, tok_tmp, lengths);
+            } else {
+                bpe_gather_kernel<256><<<(int)(g < 1 ? 1 : g), 256, 0, s>>>(a, offsets, p, tok_tmp, lengths);
+            }
             DNATOK_HIP_TRY(hipGetLastError());
         }
         bpe_long_kernel<kLongThreads><<<p.n_slabs, kLongThreads, 0, s>>>(a, bytes, offsets, n_rows, max_len, p,
