@@ -987,6 +987,7 @@ struct BpePlan {                          // device arrays inside the scratch bu
     int32_t *cnt;         // [max_mc][4] tokens of a chunk: in the stretch it shares with no other chunk, from the
                           // seam on its left to that stretch, from that stretch to the seam on its right
     int32_t *row_fail;    // [n_rows] 1 = redo the row with the whole-row kernel
+    int32_t *tile_sums;   // [n_rows / 4096 + 1][8] what the rows of a tile add to the work list's scans, and its failed rows
     uint16_t *chunk_sym;  // [max_mc][ext]
     uint8_t *slabs;       // whole-row fallback state
     size_t slab_bytes, total_bytes;
@@ -1046,6 +1047,7 @@ static BpePlan make_plan(const dnatok_bpe_t *t, uint8_t *base, int64_t n_rows, i
     const size_t o_seam = take(4 * (size_t)p.max_mc);
     const size_t o_cnt = take(16 * (size_t)p.max_mc);
     const size_t o_fail = take(4 * (size_t)n_rows);
+    const size_t o_tiles = take(4 * 8 * (size_t)(n_rows / 4096 + 1));
     const size_t o_sym = take(2 * (size_t)p.ext * (size_t)p.max_mc);
     p.slab_bytes = chunks ? long_slab_bytes(max_len) : 0;
     const int64_t slabs = n_rows < max_slabs ? n_rows : max_slabs;
@@ -1061,6 +1063,7 @@ static BpePlan make_plan(const dnatok_bpe_t *t, uint8_t *base, int64_t n_rows, i
         p.seam = (int32_t *)(base + o_seam);
         p.cnt = (int32_t *)(base + o_cnt);
         p.row_fail = (int32_t *)(base + o_fail);
+        p.tile_sums = (int32_t *)(base + o_tiles);
         p.chunk_sym = (uint16_t *)(base + o_sym);
         p.slabs = base + o_slabs;
     }
@@ -1068,26 +1071,57 @@ static BpePlan make_plan(const dnatok_bpe_t *t, uint8_t *base, int64_t n_rows, i
 }
 
 // Work list: ceil(len / core) chunk slots per long row, one entry in its length class per other
-// row.  Single workgroup; a thread takes four consecutive rows per step, so that 4096 rows are one
-// round of loads and one scan (the kernel is a chain of load latencies and barriers, not work).
+// row.  A thread takes four consecutive rows per step, so that a tile of 4096 rows is one round of
+// loads and one scan (the kernel is a chain of load latencies and barriers, not work).
+// PASS 0: the whole list by one workgroup, tile after tile (up to kPlanTiledFrom rows: one launch).
+// More rows take two launches with a workgroup per tile (32,768 rows: 38 us by one workgroup, while
+// nothing else runs, against about 10 us for the two): PASS 1 adds up what each tile contributes (and marks the
+// rows left to the whole-row kernel), PASS 2 places every tile behind the tiles before it; its
+// last workgroup, which sees all the sums, writes the counters.
 constexpr int kPlanRows = 4;
+constexpr int kPlanTile = 1024 * kPlanRows;
+constexpr int64_t kPlanTiledFrom = 2 * kPlanTile + 1;
 constexpr int kPlanScans = 1 + kSingleClasses;
 constexpr int kPlanInlineRows = 4096;      // the plan kernel writes the chunk entries itself up to this
 constexpr int kPlanInlineChunks = 8192;    // many rows and this many chunks (a bound known on the host)
 
+template <int PASS>
 __global__ __launch_bounds__(1024) void bpe_plan_kernel(
     const int64_t *__restrict__ offsets, int64_t n_rows, int chunking, int expand_here, BpePlan p)
 {
-    __shared__ uint32_t wt[kPlanScans][16];
+    __shared__ uint32_t wt[kPlanScans + 1][16];
     __shared__ int32_t carry[kPlanScans];
     __shared__ int32_t fail_s;
-    __shared__ int32_t s_mc[kPlanInlineRows], s_len[kPlanInlineRows];   // first chunk and length of every row (expand_here)
+    __shared__ int32_t s_mc[PASS == 0 ? kPlanInlineRows : 1], s_len[PASS == 0 ? kPlanInlineRows : 1];   // first chunk and length of every row (expand_here)
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     if (threadIdx.x < kPlanScans) carry[threadIdx.x] = 0;
     if (threadIdx.x == 0) fail_s = 0;
     __syncthreads();
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    if (PASS == 2) {
+        // what the tiles before this one add up to (the last workgroup: all but its own), and their failed rows
+        int32_t part[kPlanScans + 1];
+#pragma unroll
+        for (int q = 0; q <= kPlanScans; ++q) part[q] = 0;
+        for (int64_t t = threadIdx.x; t < (int64_t)blockIdx.x; t += 1024)
+#pragma unroll
+            for (int q = 0; q <= kPlanScans; ++q) part[q] += p.tile_sums[8 * t + q];
+#pragma unroll
+        for (int q = 0; q <= kPlanScans; ++q) {
+            const uint32_t inc = wave_inclusive_sum_u32((uint32_t)part[q]);
+            if (lane == 63) wt[q][wv] = inc;
+        }
+        __syncthreads();
+        if (threadIdx.x <= kPlanScans) {
+            uint32_t t = 0;
+            for (int w = 0; w < 16; ++w) t += wt[threadIdx.x][w];
+            if (threadIdx.x < kPlanScans) carry[threadIdx.x] = (int32_t)t; else fail_s = (int32_t)t;
+        }
+        __syncthreads();
+    }
     int32_t n_fail = 0;
-    for (int64_t base = 0; base < n_rows; base += 1024 * kPlanRows) {
+    const int64_t first_row = PASS == 0 ? 0 : (int64_t)blockIdx.x * kPlanTile;
+    const int64_t end_row = PASS == 0 ? n_rows : (first_row + kPlanTile < n_rows ? first_row + kPlanTile : n_rows);
+    for (int64_t base = first_row; base < end_row; base += kPlanTile) {
         const int64_t row0 = base + (int64_t)threadIdx.x * kPlanRows;
         int64_t off[kPlanRows + 1];
 #pragma unroll
@@ -1110,8 +1144,7 @@ __global__ __launch_bounds__(1024) void bpe_plan_kernel(
                     for (int q = 0; q < kSingleClasses; ++q) add[r][1 + q] = q == c ? 1u : 0u;
                 }
                 const int fail = (len > p.ext && !chunking) ? 1 : 0;
-                p.row_fail[row0 + r] = fail;
-                n_fail += fail;
+                if (PASS != 2) { p.row_fail[row0 + r] = fail; n_fail += fail; }
             }
 #pragma unroll
             for (int q = 0; q < kPlanScans; ++q) sum[q] += add[r][q];
@@ -1135,6 +1168,12 @@ __global__ __launch_bounds__(1024) void bpe_plan_kernel(
             at[q] = carry[q] + (int32_t)(b + inc[q] - sum[q]);
             tot[q] = carry[q] + (int32_t)t;
         }
+        if (PASS == 1) {                                 // (one tile: the sums are all this pass is for)
+            if (threadIdx.x < kPlanScans)
+#pragma unroll
+                for (int q = 0; q < kPlanScans; ++q) if ((int)threadIdx.x == q) p.tile_sums[8 * (size_t)blockIdx.x + q] = tot[q];
+            break;
+        }
 #pragma unroll
         for (int r = 0; r < kPlanRows; ++r) {
             if (row0 + r >= n_rows) continue;
@@ -1143,7 +1182,7 @@ __global__ __launch_bounds__(1024) void bpe_plan_kernel(
             // the entries of the chunks are written by bpe_expand_kernel (a single workgroup
             // writing tens of thousands of scattered words is bound by its one CU's store path),
             // except for a batch of few chunks, whose entries are written below (a launch less)
-            if (expand_here) { s_mc[row] = at[0]; s_len[row] = (int32_t)(off[r + 1] - off[r]); }
+            if (PASS == 0 && expand_here) { s_mc[row] = at[0]; s_len[row] = (int32_t)(off[r + 1] - off[r]); }
 #pragma unroll
             for (int q = 0; q < kSingleClasses; ++q)
                 if (add[r][1 + q]) p.single[q][at[1 + q]] = row;
@@ -1159,7 +1198,16 @@ __global__ __launch_bounds__(1024) void bpe_plan_kernel(
     }
     if (n_fail) atomicAdd(&fail_s, n_fail);
     __syncthreads();
-    if (expand_here) {
+    if (PASS == 1) {
+        if (threadIdx.x == 0) p.tile_sums[8 * (size_t)blockIdx.x + kPlanScans] = fail_s;
+        return;
+    }
+    if (PASS == 2) {
+        if (blockIdx.x + 1 != gridDim.x) return;         // the last tile's workgroup has the totals
+        if (threadIdx.x == 0) fail_s += p.tile_sums[8 * (size_t)blockIdx.x + kPlanScans];
+        __syncthreads();
+    }
+    if (PASS == 0 && expand_here) {
         // chunk c belongs to the last row whose first chunk is at or before c
         const int32_t total = carry[0];
         for (int32_t c = threadIdx.x; c < total; c += 1024) {
@@ -2023,7 +2071,14 @@ int run_lds_part(bool long_rows, int chunking, bool force_plan, const BpeArgs &a
             DNATOK_HIP_TRY(hipGetLastError());
         } else {
             const int expand_here = chunking >> 1;
-            bpe_plan_kernel<<<1, 1024, 0, s>>>(offsets, n_rows, chunking & 1, expand_here, p);
+            if (n_rows >= kPlanTiledFrom) {
+                const int tiles = (int)((n_rows + kPlanTile - 1) / kPlanTile);
+                bpe_plan_kernel<1><<<tiles, 1024, 0, s>>>(offsets, n_rows, chunking & 1, 0, p);
+                DNATOK_HIP_TRY(hipGetLastError());
+                bpe_plan_kernel<2><<<tiles, 1024, 0, s>>>(offsets, n_rows, chunking & 1, 0, p);
+            } else {
+                bpe_plan_kernel<0><<<1, 1024, 0, s>>>(offsets, n_rows, chunking & 1, expand_here, p);
+            }
             DNATOK_HIP_TRY(hipGetLastError());
             if ((chunking & 1) && !expand_here) {
                 bpe_expand_kernel<<<(int)((n_rows + 255) / 256), 256, 0, s>>>(offsets, n_rows, p);

@@ -1059,6 +1059,24 @@ def test_bpe_mostly_short_rows_with_some_long_ones(bpe, long_ones):
         np.testing.assert_array_equal(tok[b.offsets[i]:b.offsets[i] + lengths[i]], e, err_msg=f"row {i}")
 
 
+def test_bpe_work_list_of_many_rows_built_tile_by_tile(bpe):
+    """Above 8,192 rows the work list is built by two launches with a workgroup per tile of 4,096
+    rows (sums, then placement) instead of by one workgroup: 21,000 ragged rows of all classes,
+    long rows that are cut into chunks (one of them a homopolymer), empty rows, a last tile that is
+    not full."""
+    which, enc, bo = bpe
+    say(f"bpe{which} work list of 21,000 rows")
+    rng = random.Random(91)
+    rnd = lambda n: "".join(rng.choices("ACGTN", weights=[24, 24, 24, 24, 4], k=n))
+    seqs = [rnd(rng.choice([0, 1, 40, 200, 300, 520, 700, 1030, 1500, 2048])) for _ in range(21_000)]
+    for e in [rnd(2049), rnd(5000), rnd(20_001), "A" * 7000, rnd(3000)] + [rnd(rng.randint(2049, 9000)) for _ in range(25)]:
+        seqs.insert(rng.randint(0, len(seqs)), e)
+    b = util.batch_from_strings(seqs)
+    ref = bo.encode_batch(b.data, b.offsets)
+    for i, (r, e) in enumerate(zip(bpe_rows(enc, b), ref)):
+        np.testing.assert_array_equal(r, e, err_msg=f"row {i} of {len(seqs[i])} bytes")
+
+
 def test_bpe_rows_without_a_seam_fall_back_to_the_whole_row_kernel(bpe):
     """Tandem repeats far longer than the chunk overlap: neighbouring chunk runs can stay out
     of phase, no seam is accepted, and the row is redone by the whole-row kernel."""
