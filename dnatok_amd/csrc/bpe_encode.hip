@@ -1325,7 +1325,8 @@ template <int NT, int TEAMS, int CAP, bool PLANNED, bool LTAB = false, bool CHAR
           bool PADDED = false>
 __global__ __launch_bounds__(NT *TEAMS) __attribute__((amdgpu_waves_per_eu(kBpeWaves<NT, TEAMS, CAP, CHUNKS>)))
 void bpe_lds_kernel(
-    BpeArgs a, const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
+    BpeArgs a /* stays the first parameter: kernel_args_now() reads it from the start of the argument segment */,
+    const uint8_t *__restrict__ bytes, const int64_t *__restrict__ offsets,
     BpePlan p, int32_t n_rows, int32_t *__restrict__ tok_tmp, int32_t *__restrict__ lengths)
 {
     extern __shared__ __align__(16) uint8_t smem[];
