@@ -418,29 +418,45 @@ __device__ __forceinline__ int32_t bpe_row(
     uint8_t *stage = reinterpret_cast<uint8_t *>(C);
     int head = 0;
     if (PER > 0) {
-        const uintptr_t a0 = reinterpret_cast<uintptr_t>(src) & ~(uintptr_t)7;
-        head = (int)(reinterpret_cast<uintptr_t>(src) - a0);
+        head = (int)(reinterpret_cast<uintptr_t>(src) & (uintptr_t)7);
+        // (derived from src by pointer arithmetic, so that the loads stay loads from global memory:
+        // through an address rebuilt from an integer they become flat loads, which count as LDS
+        // accesses too)
+        const uint2 *const words = reinterpret_cast<const uint2 *>(src - head);
         const int n_words = (head + n0 + 7) >> 3;
         for (int wd = tid; wd < n_words; wd += NT) {
             const int first = 8 * wd - head;                  // row position of the word's first byte
             uint2 v;
             if (first >= 0 && first + 8 <= n0) {
-                v = *reinterpret_cast<const uint2 *>(a0 + 8 * (uintptr_t)wd);
+                v = words[wd];
             } else {
+                // (all eight bytes requested together, from positions clamped into the row: a load
+                // behind a condition each is a chain of eight trips to the cache, which a row that
+                // does not start on an 8-byte boundary pays in its first and its last word while the
+                // whole team waits)
+                uint32_t b[8];
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    const int pos = first + q;
+                    b[q] = src[pos < 0 ? 0 : (pos < n0 ? pos : n0 - 1)];
+                }
                 uint32_t lo = 0, hi = 0;
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    if (first + q >= 0 && first + q < n0) lo |= (uint32_t)src[first + q] << (8 * q);
-                    if (first + 4 + q >= 0 && first + 4 + q < n0) hi |= (uint32_t)src[first + 4 + q] << (8 * q);
+                    if (first + q >= 0 && first + q < n0) lo |= b[q] << (8 * q);
+                    if (first + 4 + q >= 0 && first + 4 + q < n0) hi |= b[4 + q] << (8 * q);
                 }
                 v = uint2{lo, hi};
             }
             *reinterpret_cast<uint2 *>(stage + 8 * wd) = v;
-            if (CHARS) {
-                if (first >= char_lo && first + 8 <= char_hi) {
-                    int32_t c[8];
+            if (CHARS && first + 8 > char_lo && first < char_hi) {
+                // (the eight ids are requested together whether the word lies wholly inside the
+                // range or not: a load, a wait and a store per byte made the two words at the
+                // range's ends a chain of eight trips to the cache, for which the whole team waited)
+                int32_t c[8];
 #pragma unroll
-                    for (int q = 0; q < 8; ++q) c[q] = char_lut[((q < 4 ? v.x : v.y) >> (8 * (q & 3))) & 255u];
+                for (int q = 0; q < 8; ++q) c[q] = char_lut[((q < 4 ? v.x : v.y) >> (8 * (q & 3))) & 255u];
+                if (first >= char_lo && first + 8 <= char_hi) {
                     const bpe_int4_a4 x0 = {c[0], c[1], c[2], c[3]}, x1 = {c[4], c[5], c[6], c[7]};
                     __builtin_nontemporal_store(x0, reinterpret_cast<bpe_int4_a4 *>(char_ids + first));
                     __builtin_nontemporal_store(x1, reinterpret_cast<bpe_int4_a4 *>(char_ids + first + 4));
@@ -453,7 +469,7 @@ __device__ __forceinline__ int32_t bpe_row(
                     for (int q = 0; q < 8; ++q) {
                         const int pos = first + q;
                         if (pos >= char_lo && pos < char_hi) {
-                            char_ids[pos] = char_lut[((q < 4 ? v.x : v.y) >> (8 * (q & 3))) & 255u];
+                            char_ids[pos] = c[q];
                             if (char_mask) char_mask[pos] = 1;
                         }
                     }
@@ -475,7 +491,14 @@ __device__ __forceinline__ int32_t bpe_row(
             x.r = (IT)rule.x;
             x.nx = (i + 1 < n0) ? (IT)(i + 1) : NIL;
             x.pv = (i > 0) ? (IT)(i - 1) : NIL;
-            x.s = (IT)(ca < (uint32_t)kFirstClasses ? first->sym[ca] : byte_to_sym_far[ba]);
+            // (the class's symbol is read from LDS whatever the class, and the table in memory only
+            // behind a branch.  Left to the compiler, the two reads become one flat load from a
+            // selected address, which counts as an access to memory: every position then waits for
+            // all stores that are still under way.  The empty asm keeps the LDS read where it is.)
+            uint32_t sym_a = first->sym[ca & (uint32_t)(kFirstClasses - 1)];
+            asm volatile("" : "+v"(sym_a));
+            if (ca >= (uint32_t)kFirstClasses) sym_a = byte_to_sym_far[ba];
+            x.s = (IT)sym_a;
             P[i] = x;
             NS[i] = (uint16_t)(rule.y & 0xFFFFu); MC[i] = (uint16_t)(rule.y >> 16);
             if (rule.x != kNone) { cmin = umin(cmin, rule.x); cgate = umin(cgate, rule.y >> 16); }
@@ -1553,8 +1576,9 @@ __global__ __launch_bounds__(256) void bpe_seam_kernel(const int64_t *__restrict
             for (int j = tid; j < n; j += NT) { sa_s[j] = A[eb0 - ea0 + j]; sb_s[j] = B[j]; }
             team_sync<NT>();
         }
-        auto a_at = [&](int j) -> uint32_t { return staged ? sa_s[j] : A[eb0 - ea0 + j]; };
-        auto b_at = [&](int j) -> uint32_t { return staged ? sb_s[j] : B[j]; };
+        // (two instances, one reading LDS and one reading memory: a choice per read would be a
+        // flat load from a selected address)
+        auto search = [&](auto a_at, auto b_at) {
         uint32_t mine = 0xFFFFFFFFu;
         for (int i = tid; i < n; i += NT) {
             const uint32_t sa = a_at(i);
@@ -1590,6 +1614,11 @@ __global__ __launch_bounds__(256) void bpe_seam_kernel(const int64_t *__restrict
             p.cnt[4 * (size_t)m + 2] = (int32_t)(both & 0xFFFFu);
             p.cnt[4 * (size_t)(m + 1) + 1] = (int32_t)(both >> 16);
         }
+        };
+        if (staged)
+            search([&](int j) -> uint32_t { return sa_s[j]; }, [&](int j) -> uint32_t { return sb_s[j]; });
+        else
+            search([&](int j) -> uint32_t { return A[eb0 - ea0 + j]; }, [&](int j) -> uint32_t { return B[j]; });
     }
 }
 
