@@ -920,13 +920,27 @@ __device__ __forceinline__ int32_t bpe_row(
     }
     for (int i0 = 0; i0 < n0; i0 += kBlockPasses * NT) {
         uint32_t sy[kBlockPasses], before[kBlockPasses];
+        int32_t id[kBlockPasses];
 #pragma unroll
         for (int k = 0; k < kBlockPasses; ++k) {
             const int i = i0 + k * NT + tid;
             sy[k] = i < n0 ? (uint32_t)P[i].s : kNone;
+        }
+        // the ids of all symbols of the block are requested before the first of them is stored (a
+        // load behind a store waits for the store as well: one trip to the cache per pass otherwise)
+#pragma unroll
+        for (int k = 0; k < kBlockPasses; ++k)
+            id[k] = (sy[k] != kNone && out_remap) ? out_remap[sy[k]] : (int32_t)sy[k];
+#pragma unroll
+        for (int k = 0; k < kBlockPasses; ++k) {
             const uint64_t live = __ballot(sy[k] != kNone);
             before[k] = (uint32_t)__builtin_popcountll(live & ((1ull << lane) - 1ull));
             if (lane == 0) wave_cnt[k * NW + wv] = (uint32_t)__builtin_popcountll(live);
+        }
+        if (PAD && remap2) {
+#pragma unroll
+            for (int k = 0; k < kBlockPasses; ++k)
+                if (sy[k] != kNone) id[k] = remap2[id[k]];
         }
         team_sync<NT>();
         uint32_t at = done;
@@ -940,11 +954,7 @@ __device__ __forceinline__ int32_t bpe_row(
                 at += c;
             }
             const uint32_t cell = mine + before[k];
-            if (sy[k] != kNone && (!PAD || cell < (uint32_t)pad_stride)) {
-                int32_t id = out_remap ? out_remap[sy[k]] : (int32_t)sy[k];
-                if (PAD && remap2) id = remap2[id];
-                put_cell(shift + (int)cell, id);
-            }
+            if (sy[k] != kNone && (!PAD || cell < (uint32_t)pad_stride)) put_cell(shift + (int)cell, id[k]);
         }
         done = at;
         team_sync<NT>();                                             // wave_cnt is rewritten by the next block
