@@ -797,6 +797,91 @@ def test_bpe_long_rows(bpe):
         np.testing.assert_array_equal(r, e)
 
 
+BPE_LENGTH_MIXES = [
+    [(1.0, 1, 300)],
+    [(0.1, 0, 0), (0.5, 1, 40), (0.4, 100, 520)],
+    [(1.0, 900, 1100)],
+    [(0.6, 1, 600), (0.3, 600, 2100), (0.1, 2100, 9000)],
+    [(0.5, 2040, 2060), (0.5, 1, 30)],
+    [(0.9, 1, 3000), (0.1, 20000, 40000)],
+]
+
+
+@pytest.mark.parametrize("mix", range(len(BPE_LENGTH_MIXES)))
+def test_bpe_random_batches_in_buffers_that_start_anywhere(bpe, mix):
+    """Rows of mixed lengths (every form of the engine in one batch or another) made of corpus
+    pieces, random bases, short tandem repeats and stretches with N, in a device buffer that starts
+    1-7 bytes off an 8-byte boundary: the engine brings a row in by aligned 8-byte words, and the
+    words at a row's two ends take a path of their own.  Token runs, the single-character ids of
+    the same pass and the rows padded by the engine, against the oracle."""
+    which, enc, bo = bpe
+    rng = np.random.default_rng(4200 + mix)
+    kinds = BPE_LENGTH_MIXES[mix]
+    n_rows = [300, 400, 120, 150, 160, 24][mix]
+    lens = np.array([int(rng.integers(kinds[j][1], kinds[j][2] + 1))
+                     for j in rng.choice(len(kinds), size=n_rows, p=[k[0] for k in kinds])], dtype=np.int64)
+    total = int(lens.sum())
+    corpus = wl.bpe_corpus("4096", 1 << 18).reshape(-1)
+    letters = np.frombuffer(b"ACGT", dtype=np.uint8)
+    data = np.empty(total, dtype=np.uint8)
+    pos = 0
+    while pos < total:
+        n = int(min(total - pos, rng.integers(1, 4000)))
+        kind = int(rng.integers(0, 4))
+        if kind == 0:
+            at = int(rng.integers(0, corpus.size - n))
+            data[pos:pos + n] = corpus[at:at + n]
+        elif kind == 1:
+            data[pos:pos + n] = letters[rng.integers(0, 4, n)]
+        elif kind == 2:
+            data[pos:pos + n] = np.resize(letters[rng.integers(0, 4, int(rng.integers(1, 7)))], n)
+        else:
+            piece = letters[rng.integers(0, 4, n)]
+            piece[rng.random(n) < 0.01] = ord("N")
+            data[pos:pos + n] = piece
+        pos += n
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    shift = 1 + mix % 7
+    say(f"bpe{which} random batch {mix}: {n_rows} rows, {total} bytes, buffer {shift} bytes off")
+    buf = torch.empty(total + 16, dtype=torch.uint8, device="cuda")
+    assert buf.data_ptr() % 8 == 0
+    d = buf[shift:shift + total]
+    d.copy_(torch.from_numpy(data))
+    o = torch.from_numpy(off).cuda()
+    max_len = int(lens.max())
+    want = bo.encode_batch(data, off)
+    lut = np.zeros(256, dtype=np.int32)
+    for i, ch in enumerate("ACGTN"):
+        lut[ord(ch)] = 5 + i
+    tok, lengths, cids, cmask = enc.encode_with_chars(d, o, max_len, torch.from_numpy(lut).cuda())
+    tok2, lengths2 = enc.encode(d, o, max_len)
+    torch.cuda.synchronize()
+    assert torch.equal(lengths, lengths2)
+    lh = lengths.cpu().numpy()
+    for t in (tok.cpu().numpy(), tok2.cpu().numpy()):
+        for i in range(n_rows):
+            np.testing.assert_array_equal(t[off[i]:off[i] + lh[i]], want[i], err_msg=f"row {i}")
+    np.testing.assert_array_equal(cids.cpu().numpy()[:total], lut[data])
+    assert bool((cmask[:total] == 1).all())
+    longest = max(1, int(lh.max()))
+    for pad_left in (False, True):
+        stride = longest + 5
+        ids, mask, pl, plong = enc.encode_padded(d, o, max_len, stride, -3, pad_left=pad_left, dtype=torch.int64)
+        torch.cuda.synchronize()
+        assert int(plong.item()) == int(lh.max()) and torch.equal(pl, lengths)
+        ih, mh = ids.cpu().numpy(), mask.cpu().numpy()
+        for i in range(n_rows):
+            n = int(lh[i])
+            row = np.full(stride, -3, dtype=np.int64)
+            m = np.zeros(stride, dtype=np.uint8)
+            if pad_left:
+                row[stride - n:] = want[i]; m[stride - n:] = 1
+            else:
+                row[:n] = want[i]; m[:n] = 1
+            np.testing.assert_array_equal(ih[i], row, err_msg=f"row {i} pad_left={pad_left}")
+            np.testing.assert_array_equal(mh[i], m, err_msg=f"mask of row {i} pad_left={pad_left}")
+
+
 def test_bpe_with_single_character_ids_from_the_same_pass(bpe):
     """dnatok_bpe_encode_with_chars: the tokens are those of dnatok_bpe_encode and the character ids
     are lut[byte] for every byte, on every route a row can take: short rows one per team, more rows
