@@ -417,7 +417,42 @@ __device__ __forceinline__ int32_t bpe_row(
     // together from single bytes, so that nothing outside the row is read.
     uint8_t *stage = reinterpret_cast<uint8_t *>(C);
     int head = 0;
+    // The single-character ids of a word's eight bytes, stored where the word lies inside
+    // [char_lo, char_hi).  The eight ids are requested together whether the word lies wholly inside
+    // the range or not (a load, a wait and a store per byte made the two words at the range's ends a
+    // chain of eight trips to the cache, for which the whole team waited).
+    auto chars_of_word = [&](const int first, const uint2 v, auto id_of) {
+        int32_t c[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) c[q] = id_of(((q < 4 ? v.x : v.y) >> (8 * (q & 3))) & 255u);
+        if (first >= char_lo && first + 8 <= char_hi) {
+            const bpe_int4_a4 x0 = {c[0], c[1], c[2], c[3]}, x1 = {c[4], c[5], c[6], c[7]};
+            __builtin_nontemporal_store(x0, reinterpret_cast<bpe_int4_a4 *>(char_ids + first));
+            __builtin_nontemporal_store(x1, reinterpret_cast<bpe_int4_a4 *>(char_ids + first + 4));
+            if (char_mask) {
+                __builtin_nontemporal_store((bpe_u32_a1)0x01010101u, reinterpret_cast<bpe_u32_a1 *>(char_mask + first));
+                __builtin_nontemporal_store((bpe_u32_a1)0x01010101u, reinterpret_cast<bpe_u32_a1 *>(char_mask + first + 4));
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const int pos = first + q;
+                if (pos >= char_lo && pos < char_hi) {
+                    char_ids[pos] = c[q];
+                    if (char_mask) char_mask[pos] = 1;
+                }
+            }
+        }
+    };
+    // Teams of 256 threads (pieces of at least 1 KB: the merge queue holds 1 KB or more and is free
+    // until the first round decides) bring the table of the 256 ids into LDS beside the row's
+    // bytes, one entry per thread in the same trip to memory, and look the ids up there once the
+    // bytes are staged: looked up in memory, the ids were a second trip behind the bytes.
+    constexpr bool kIdsFromLds = CHARS && PER > 0 && NT == 256;
+    int32_t *const ids_s = reinterpret_cast<int32_t *>(Q);
     if (PER > 0) {
+        int32_t id_mine = 0;
+        if (kIdsFromLds) id_mine = char_lut[tid];
         head = (int)(reinterpret_cast<uintptr_t>(src) & (uintptr_t)7);
         // (derived from src by pointer arithmetic, so that the loads stay loads from global memory:
         // through an address rebuilt from an integer they become flat loads, which count as LDS
@@ -449,34 +484,19 @@ __device__ __forceinline__ int32_t bpe_row(
                 v = uint2{lo, hi};
             }
             *reinterpret_cast<uint2 *>(stage + 8 * wd) = v;
-            if (CHARS && first + 8 > char_lo && first < char_hi) {
-                // (the eight ids are requested together whether the word lies wholly inside the
-                // range or not: a load, a wait and a store per byte made the two words at the
-                // range's ends a chain of eight trips to the cache, for which the whole team waited)
-                int32_t c[8];
-#pragma unroll
-                for (int q = 0; q < 8; ++q) c[q] = char_lut[((q < 4 ? v.x : v.y) >> (8 * (q & 3))) & 255u];
-                if (first >= char_lo && first + 8 <= char_hi) {
-                    const bpe_int4_a4 x0 = {c[0], c[1], c[2], c[3]}, x1 = {c[4], c[5], c[6], c[7]};
-                    __builtin_nontemporal_store(x0, reinterpret_cast<bpe_int4_a4 *>(char_ids + first));
-                    __builtin_nontemporal_store(x1, reinterpret_cast<bpe_int4_a4 *>(char_ids + first + 4));
-                    if (char_mask) {
-                        __builtin_nontemporal_store((bpe_u32_a1)0x01010101u, reinterpret_cast<bpe_u32_a1 *>(char_mask + first));
-                        __builtin_nontemporal_store((bpe_u32_a1)0x01010101u, reinterpret_cast<bpe_u32_a1 *>(char_mask + first + 4));
-                    }
-                } else {
-#pragma unroll
-                    for (int q = 0; q < 8; ++q) {
-                        const int pos = first + q;
-                        if (pos >= char_lo && pos < char_hi) {
-                            char_ids[pos] = c[q];
-                            if (char_mask) char_mask[pos] = 1;
-                        }
-                    }
-                }
+            if (CHARS && !kIdsFromLds && first + 8 > char_lo && first < char_hi)
+                chars_of_word(first, v, [&](uint32_t byte) -> int32_t { return char_lut[byte]; });
+        }
+        if (kIdsFromLds) ids_s[tid] = id_mine;
+        team_sync<NT>();
+        if (kIdsFromLds) {
+            for (int wd = tid; wd < n_words; wd += NT) {
+                const int first = 8 * wd - head;
+                if (first + 8 > char_lo && first < char_hi)
+                    chars_of_word(first, *reinterpret_cast<const uint2 *>(stage + 8 * wd),
+                                  [&](uint32_t byte) -> int32_t { return ids_s[byte]; });
             }
         }
-        team_sync<NT>();
     }
     auto byte_at = [&](int i) -> uint32_t { return PER > 0 ? stage[head + i] : src[i]; };
     if (PER > 0 && first) {
@@ -1404,6 +1424,7 @@ void bpe_lds_kernel(
                             : (a.part == 2 ? n_shortest : p.counts[0] - (a.part == 1 ? n_shortest : 0));
     int32_t *const deal = PLANNED ? p.deal + (a.part == 2 ? kDealers * kDealerStride : 0) : nullptr;
     static_assert(PLANNED || !CHUNKS, "chunks come from the work list");
+    static_assert(!(CHARS && NT == 256) || CAP >= 1024, "the merge queue holds the table of single-character ids (1 KB)");
     static_assert(!PADDED || (!CHUNKS && !LTAB), "padded rows: whole rows");
     const int32_t n_mc = CHUNKS ? p.counts[1] : 0;
     const int32_t n_single0 = PLANNED ? p.counts[4] : 0, n_single1 = PLANNED ? p.counts[5] : 0;
