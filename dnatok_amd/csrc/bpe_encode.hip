@@ -286,6 +286,43 @@ __device__ __forceinline__ void team_min2(uint32_t a, uint32_t b, uint32_t *red,
     ra = x; rb = y;
 }
 
+// The same for two values below 2^16 (ranks, gates and positions of pieces that fit LDS; anything
+// above counts as 0xFFFF): both ride in one register, and one packed 16-bit minimum per step
+// reduces them together.  Half the vector instructions of the two separate reductions, in a
+// kernel that is bound by their number.
+typedef unsigned short bpe_u16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pk_min_u16(uint32_t a, uint32_t b)
+{
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(bpe_u16x2, a),
+                                                                  __builtin_bit_cast(bpe_u16x2, b)));
+}
+
+template <int NT>
+__device__ __forceinline__ void team_min2_u16(uint32_t a, uint32_t b, uint32_t *red, int wv,
+                                              uint32_t &ra, uint32_t &rb)
+{
+    uint32_t v = umin(a, 0xFFFFu) | (umin(b, 0xFFFFu) << 16);
+    v = pk_min_u16(v, dpp_u32<0xB1>(v));    // quad_perm [1,0,3,2]
+    v = pk_min_u16(v, dpp_u32<0x4E>(v));    // quad_perm [2,3,0,1]
+    v = pk_min_u16(v, dpp_u32<0x141>(v));   // row_half_mirror
+    v = pk_min_u16(v, dpp_u32<0x140>(v));   // row_mirror
+    const uint32_t r0 = __builtin_amdgcn_readlane(v, 0), r1 = __builtin_amdgcn_readlane(v, 16);
+    const uint32_t r2 = __builtin_amdgcn_readlane(v, 32), r3 = __builtin_amdgcn_readlane(v, 48);
+    v = pk_min_u16(pk_min_u16(r0, r1), pk_min_u16(r2, r3));
+    if (NT == 64) {
+        team_sync<NT>();
+    } else {
+        constexpr int NW = NT / 64;
+        if ((threadIdx.x & 63) == 0) red[wv] = v;
+        __syncthreads();
+        v = red[0];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) v = pk_min_u16(v, red[w]);
+    }
+    ra = v & 0xFFFFu; rb = v >> 16;
+}
+
 // Exclusive prefix sum over the team (one value per thread) and the team total.
 template <int NT>
 __device__ __forceinline__ uint32_t team_exclusive_sum(uint32_t v, uint32_t *red, int wv, uint32_t &total)
@@ -571,7 +608,8 @@ __device__ __forceinline__ int32_t bpe_row(
     for (;;) {
         if (--budget < 0) { stuck = true; break; }   // cannot happen; keeps the loop bounded
         uint32_t rmin, gate;
-        team_min2<NT>(cmin, cgate, red + flip * (NT / 64) * 2, wv, rmin, gate);   // (syncs the team)
+        if (sizeof(IT) == 2) team_min2_u16<NT>(cmin, cgate, red + flip * (NT / 64) * 2, wv, rmin, gate);   // (syncs the team)
+        else team_min2<NT>(cmin, cgate, red + flip * (NT / 64) * 2, wv, rmin, gate);
         flip ^= 1;
         clk.lap(kPhMinimum);
         if (rmin >= kNone) break;
@@ -584,7 +622,8 @@ __device__ __forceinline__ int32_t bpe_row(
                 for (int i = tid; i < n0; i += NT)
                     if (P[i].r == rmin) { mypos = (uint32_t)i; break; }
             uint32_t dummy;
-            team_min2<NT>(mypos, mypos, red + flip * (NT / 64) * 2, wv, leftmost, dummy);
+            if (sizeof(IT) == 2) team_min2_u16<NT>(mypos, mypos, red + flip * (NT / 64) * 2, wv, leftmost, dummy);
+            else team_min2<NT>(mypos, mypos, red + flip * (NT / 64) * 2, wv, leftmost, dummy);
             flip ^= 1;
         }
         const uint32_t limit = single ? rmin + 1 : gate;
