@@ -323,6 +323,13 @@ __device__ __forceinline__ void team_min2_u16(uint32_t a, uint32_t b, uint32_t *
     ra = v & 0xFFFFu; rb = v >> 16;
 }
 
+// Number of set bits of a ballot below the calling lane (two instructions; written as a popcount
+// of the ballot under a mask of the lower lanes it is four, and the engine is bound by their number).
+__device__ __forceinline__ uint32_t lanes_below(uint64_t ballot)
+{
+    return __builtin_amdgcn_mbcnt_hi((uint32_t)(ballot >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ballot, 0u));
+}
+
 // Exclusive prefix sum over the team (one value per thread) and the team total.
 template <int NT>
 __device__ __forceinline__ uint32_t team_exclusive_sum(uint32_t v, uint32_t *red, int wv, uint32_t &total)
@@ -654,8 +661,8 @@ __device__ __forceinline__ int32_t bpe_row(
                     at = (uint32_t)__builtin_amdgcn_readfirstlane((int)at);
 #pragma unroll
                     for (int k = 0; k < PER; ++k) {
-                        if (bal[k] >> lane & 1ull)
-                            C[at + (uint32_t)__builtin_popcountll(bal[k] & ((1ull << lane) - 1ull))] =
+                        if (myr[k] < limit)                       // (the lane's own bit of the ballot)
+                            C[at + lanes_below(bal[k])] =
                                 (IT)(tid + k * NT);
                         at += (uint32_t)__builtin_popcountll(bal[k]);
                     }
@@ -677,7 +684,7 @@ __device__ __forceinline__ int32_t bpe_row(
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
                         if (bal[k] >> lane & 1ull)
-                            C[at + (uint32_t)__builtin_popcountll(bal[k] & ((1ull << lane) - 1ull))] =
+                            C[at + lanes_below(bal[k])] =
                                 (IT)(b0 + k * NT + tid);
                         at += (uint32_t)__builtin_popcountll(bal[k]);
                     }
@@ -723,7 +730,7 @@ __device__ __forceinline__ int32_t bpe_row(
                     uint32_t at = 0;
                     if (lane == 0) at = atomicAdd(qn, (uint32_t)__builtin_popcountll(bal));
                     at = (uint32_t)__builtin_amdgcn_readfirstlane((int)at);
-                    if (merges) Q[at + (uint32_t)__builtin_popcountll(bal & ((1ull << lane) - 1ull))] = (IT)i;
+                    if (merges) Q[at + lanes_below(bal)] = (IT)i;
                 }
             }
         }
@@ -760,7 +767,7 @@ __device__ __forceinline__ int32_t bpe_row(
                 uint32_t at = 0;
                 if (lane == 0) at = atomicAdd(qn, (uint32_t)__builtin_popcountll(bal));
                 at = (uint32_t)__builtin_amdgcn_readfirstlane((int)at);
-                if (merges) Q[at + (uint32_t)__builtin_popcountll(bal & ((1ull << lane) - 1ull))] = (IT)i;
+                if (merges) Q[at + lanes_below(bal)] = (IT)i;
             }
             team_sync<NT>();
         }
@@ -831,7 +838,7 @@ __device__ __forceinline__ int32_t bpe_row(
                     uint32_t at = 0;
                     if (lane == 0) at = atomicAdd(qn, (uint32_t)__builtin_popcountll(bal));
                     at = (uint32_t)__builtin_amdgcn_readfirstlane((int)at);
-                    if (merges) Q[at + (uint32_t)__builtin_popcountll(bal & ((1ull << lane) - 1ull))] = (IT)i;
+                    if (merges) Q[at + lanes_below(bal)] = (IT)i;
                 }
             }
             team_sync<NT>();
@@ -993,7 +1000,7 @@ __device__ __forceinline__ int32_t bpe_row(
 #pragma unroll
         for (int k = 0; k < kBlockPasses; ++k) {
             const uint64_t live = __ballot(sy[k] != kNone);
-            before[k] = (uint32_t)__builtin_popcountll(live & ((1ull << lane) - 1ull));
+            before[k] = lanes_below(live);
             if (lane == 0) wave_cnt[k * NW + wv] = (uint32_t)__builtin_popcountll(live);
         }
         if (PAD && remap2) {
@@ -1760,7 +1767,7 @@ __global__ __launch_bounds__(256) void bpe_gather_kernel(
             for (int k = 0; k < kPasses; ++k) {
                 val[k] = (sy[k] != kNone && a.out_remap) ? a.out_remap[sy[k]] : (int32_t)sy[k];
                 const uint64_t live = __ballot(sy[k] != kNone);
-                ahead[k] = (uint32_t)__builtin_popcountll(live & ((1ull << lane) - 1ull));
+                ahead[k] = lanes_below(live);
                 if (lane == 0) wave_cnt[k][wv] = (uint32_t)__builtin_popcountll(live);
             }
             team_sync<NT>();
