@@ -134,8 +134,9 @@ typedef uint32_t bpe_u32_a1 __attribute__((aligned(1)));
 // What a position keeps about the pair it starts: the rule's rank (kNone = no rule), the
 // symbol the rule produces, and the rule's gate (lowest rank of any rule using that product).
 struct PairInfo {
-    uint32_t rank, product, gate;
+    uint32_t rank, pg;           // pg: the rule's product | its gate << 16, as the tables and the state hold them
 };
+constexpr uint32_t kNoPg = kNone | (kNone << 16);
 
 // The rules between two single-byte symbols, by the bytes themselves: what every position of a row
 // needs first.  A DNA alphabet has a handful of bytes with such rules (A C G T N), so the bytes are
@@ -198,8 +199,8 @@ __device__ __forceinline__ PairInfo pair_finish(uint32_t a, uint32_t b, const Pa
     const uint32_t key = (a << 16) | b;
     const bool first = pr.e1.x == key;
     const uint32_t y = first ? pr.e1.y : pr.e2.y, z = first ? pr.e1.z : pr.e2.z;
-    if (!first && pr.e2.x != key) return PairInfo{kNone, kNone, kNone};
-    return PairInfo{y, z & 0xFFFFu, z >> 16};
+    if (!first && pr.e2.x != key) return PairInfo{kNone, kNoPg};
+    return PairInfo{y, z};
 }
 
 // The compact form of the merge table, for tables of at most 8192 symbols and 4095 rules: small
@@ -243,10 +244,9 @@ __device__ __forceinline__ LdsPairProbe pair_probe(const LdsPairTable &t, uint32
 __device__ __forceinline__ PairInfo pair_finish(const LdsPairTable &t, uint32_t, uint32_t, const LdsPairProbe &pr)
 {
     const bool first = (pr.e1 & 0x7FFFu) == pr.want1;
-    if (!first && (pr.e2 & 0x7FFFu) != pr.want2) return PairInfo{kNone, kNone, kNone};
+    if (!first && (pr.e2 & 0x7FFFu) != pr.want2) return PairInfo{kNone, kNoPg};
     const uint32_t rank = (first ? pr.e1 : pr.e2) >> 15;
-    const uint32_t pg = t.pg[rank];
-    return PairInfo{rank, pg & 0xFFFFu, pg >> 16};
+    return PairInfo{rank, t.pg[rank]};
 }
 
 __device__ __forceinline__ PairInfo pair_finish(const PairTable &, uint32_t a, uint32_t b, const PairProbe &pr)
@@ -404,7 +404,8 @@ struct alignas(4 * sizeof(IT)) PosRec {
     IT r, nx, pv, s;
 };
 
-// One row.  tid = index in the team; P/NS/MC hold n0 entries, Q (the merges of the current round)
+// One row.  tid = index in the team; P and PG (product and gate of the pair a position starts) hold
+// n0 entries, Q (the merges of the current round)
 // n0 / 2, C (its candidates) n0; D holds NT bytes; PER > 0 says that n0 <= PER * NT, and every thread
 // then keeps the ranks of its own positions in registers as well; red holds 4 * (NT / 64) + 4 words.  Tokens go to out[0 .. *out_len).
 // CHARS: while the piece's bytes pass through the registers on their way into LDS, the
@@ -418,7 +419,7 @@ template <int NT, typename IT, int PER, bool CHARS = false, bool PAD = false, ty
 __device__ __forceinline__ int32_t bpe_row(
     const PT pt, const uint16_t *byte_to_sym,
     const int32_t *out_remap, const uint8_t *__restrict__ src, const int n0, PosRec<IT> *P,
-    uint16_t *NS, uint16_t *MC, IT *Q, IT *C, uint8_t *D, uint32_t *red, const int tid,
+    uint32_t *PG, IT *Q, IT *C, uint8_t *D, uint32_t *red, const int tid,
     int32_t *__restrict__ out, int32_t *__restrict__ out_len, uint16_t *__restrict__ raw_out = nullptr,
     const int mid_lo = 0, const int mid_hi = 0, int32_t *__restrict__ mid_out = nullptr,
     const int32_t *__restrict__ char_lut = nullptr, int32_t *__restrict__ char_ids = nullptr,
@@ -451,6 +452,8 @@ __device__ __forceinline__ int32_t bpe_row(
     // positions, so the LDS state arrays are read and written without bank conflicts
 
     PhaseClock clk;
+    // a position's product and gate as 16-bit halves of its word of PG
+    const uint16_t *const product_of = reinterpret_cast<const uint16_t *>(PG), *const gate_of = product_of + 1;
     // symbols, links and the initial pair of every position, kProbes pairs of table reads in flight at a time
     uint32_t cmin = kEmptyKey, cgate = kEmptyKey;
     D[tid] = 0;
@@ -564,7 +567,7 @@ __device__ __forceinline__ int32_t bpe_row(
             if (ca >= (uint32_t)kFirstClasses) sym_a = byte_to_sym_far[ba];
             x.s = (IT)sym_a;
             P[i] = x;
-            NS[i] = (uint16_t)(rule.y & 0xFFFFu); MC[i] = (uint16_t)(rule.y >> 16);
+            PG[i] = rule.y;
             if (rule.x != kNone) { cmin = umin(cmin, rule.x); cgate = umin(cgate, rule.y >> 16); }
         }
     } else
@@ -583,7 +586,7 @@ __device__ __forceinline__ int32_t bpe_row(
         for (int j = 0; j < kProbes; ++j) {
             const int i = i0 + j * NT;
             if (i >= n0) continue;
-            PairInfo pi{kNone, kNone, kNone};
+            PairInfo pi{kNone, kNoPg};
             if (i + 1 < n0) pi = pair_finish(pt, sa[j], sb[j], e[j]);
             PosRec<IT> x;
             x.r = (IT)pi.rank;
@@ -591,8 +594,8 @@ __device__ __forceinline__ int32_t bpe_row(
             x.pv = (i > 0) ? (IT)(i - 1) : NIL;
             x.s = (IT)sa[j];
             P[i] = x;
-            NS[i] = (uint16_t)pi.product; MC[i] = (uint16_t)pi.gate;
-            if (pi.rank != kNone) { cmin = umin(cmin, pi.rank); cgate = umin(cgate, pi.gate); }
+            PG[i] = pi.pg;
+            if (pi.rank != kNone) { cmin = umin(cmin, pi.rank); cgate = umin(cgate, pi.pg >> 16); }
         }
     }
 
@@ -852,7 +855,7 @@ __device__ __forceinline__ int32_t bpe_row(
             const IT i = Q[m];
             const IT j = P[i].nx;
             const IT k = P[j].nx;
-            P[i].s = (IT)NS[i];
+            P[i].s = (IT)product_of[2 * (int)i];
             P[i].nx = k;
             P[j].s = DEAD;
             P[j].r = DEAD;
@@ -890,10 +893,10 @@ __device__ __forceinline__ int32_t bpe_row(
 #pragma unroll
             for (int j = 0; j < kProbes; ++j) {
                 if (target[j] == NIL) continue;       // no probe, or no left neighbour
-                PairInfo pi{kNone, kNone, kNone};
+                PairInfo pi{kNone, kNoPg};
                 if (valid[j]) pi = pair_finish(pt, sa[j], sb[j], e[j]);
                 const int q = (int)target[j];
-                P[q].r = (IT)pi.rank; NS[q] = (uint16_t)pi.product; MC[q] = (uint16_t)pi.gate;
+                P[q].r = (IT)pi.rank; PG[q] = pi.pg;
                 D[q % NT] = 1;
             }
         }
@@ -909,14 +912,14 @@ __device__ __forceinline__ int32_t bpe_row(
                 for (int k = 0; k < PER; ++k) {
                     const int i = tid + k * NT;
                     const uint32_t r = i < n0 ? (uint32_t)P[i].r : kNone;
-                    const uint32_t g = MC[i < n0 ? i : tid];      // read beside the rank, not after it
+                    const uint32_t g = gate_of[2 * (i < n0 ? i : tid)];      // read beside the rank, not after it
                     myr[k] = r;
                     if (r != kNone) { cmin = umin(cmin, r); cgate = umin(cgate, g); }
                 }
             } else {
                 for (int i = tid; i < n0; i += NT) {
                     const uint32_t r = P[i].r;
-                    if (r != kNone) { cmin = umin(cmin, r); cgate = umin(cgate, MC[i]); }
+                    if (r != kNone) { cmin = umin(cmin, r); cgate = umin(cgate, gate_of[2 * i]); }
                 }
             }
         }
@@ -945,14 +948,14 @@ __device__ __forceinline__ int32_t bpe_row(
     }
     // Compact the live symbols to the output, in position order.  Position i = pass * NT + tid, so a
     // pass is NT consecutive positions: a ballot per wave gives every lane its place among the
-    // wave's live symbols, the waves' counts of a block of passes go through LDS (NS is free by
+    // wave's live symbols, the waves' counts of a block of passes go through LDS (PG is free by
     // now: every thread left the loop behind the same barrier), and the stores of a wave go to
     // consecutive cells.  (A contiguous piece per thread, as before, cost a fifth of a 1 KB row's
     // time: strided LDS reads, two scans and stores scattered over the row.)
     constexpr int NW = NT / 64;
     // (a row of at most PER passes never has more in a block: the passes beyond cost registers for nothing)
     constexpr int kBlockPasses = (PER > 0 && PER < 8) ? PER : 8;
-    uint32_t *wave_cnt = reinterpret_cast<uint32_t *>(NS);           // [kBlockPasses][NW]
+    uint32_t *wave_cnt = PG;                                         // [kBlockPasses][NW]
     const int lane = tid & 63;
     uint32_t done = 0;                                               // tokens of earlier blocks of passes
     // PAD: where row pad_row of the padded output lies and what pads it, from the kernel's
@@ -1448,8 +1451,7 @@ void bpe_lds_kernel(
     int32_t *next_item = reinterpret_cast<int32_t *>(sp) + team; sp += 16 * sizeof(int32_t);
     uint32_t *red = reinterpret_cast<uint32_t *>(sp) + team * (4 * (NT / 64) + 4); sp += TEAMS * (4 * (NT / 64) + 4) * 4;
     PosRec<uint16_t> *P = reinterpret_cast<PosRec<uint16_t> *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 8;
-    uint16_t *NS = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
-    uint16_t *MC = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
+    uint32_t *PG = reinterpret_cast<uint32_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 4;   // product | gate << 16
     uint16_t *Q = reinterpret_cast<uint16_t *>(sp) + (size_t)team * (CAP / 2); sp += (size_t)TEAMS * CAP;
     uint16_t *C = reinterpret_cast<uint16_t *>(sp) + (size_t)team * CAP; sp += (size_t)TEAMS * CAP * 2;
     uint8_t *D = sp + (size_t)team * NT; sp += (size_t)TEAMS * NT;
@@ -1557,12 +1559,12 @@ void bpe_lds_kernel(
             }
         } else if (!CHUNKS || nc == 1) {
             if (LTAB)
-                bpe_row<NT, uint16_t, (CAP + NT - 1) / NT>(lpt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC,
+                bpe_row<NT, uint16_t, (CAP + NT - 1) / NT>(lpt, b2s, a.out_remap, bytes + start, (int)len, P, PG,
                                       Q, C, D, red, tid, tok_tmp + start, lengths + row, nullptr, 0, 0, nullptr,
                                       nullptr, nullptr, nullptr, 0, 0, first_pairs, 0, a.byte_to_sym);
             else {
                 const int32_t n_tok = bpe_row<NT, uint16_t, (CAP + NT - 1) / NT, CHARS, PADDED>(
-                    pt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC, Q, C, D, red, tid,
+                    pt, b2s, a.out_remap, bytes + start, (int)len, P, PG, Q, C, D, red, tid,
                     padded ? nullptr : tok_tmp + start,        // (a padded row finds its own cells)
                     lengths + row, nullptr, 0, 0, nullptr, a.char_lut, CHARS ? a.char_ids + start : nullptr,
                     CHARS && a.char_mask ? a.char_mask + start : nullptr, 0, (int)len, first_pairs, row,
@@ -1582,7 +1584,7 @@ void bpe_lds_kernel(
             // the single-character ids of a long row are written chunk by chunk: every chunk those of its core
             const int64_t core_hi = (int64_t)(k + 1) * p.core < len ? (int64_t)(k + 1) * p.core : len;
             bpe_row<NT, uint16_t, (CAP + NT - 1) / NT, CHARS>(
-                pt, b2s, a.out_remap, bytes + start + e0, (int)(e1 - e0), P, NS, MC, Q, C, D, red, tid, nullptr,
+                pt, b2s, a.out_remap, bytes + start + e0, (int)(e1 - e0), P, PG, Q, C, D, red, tid, nullptr,
                 nullptr, raw, (int)(mid_lo - e0), (int)(mid_hi - e0), p.cnt + 4 * (size_t)m, a.char_lut,
                 CHARS ? a.char_ids + start + e0 : nullptr, CHARS && a.char_mask ? a.char_mask + start + e0 : nullptr,
                 (int)((int64_t)k * p.core - e0), (int)(core_hi - e0), first_pairs, 0, a.byte_to_sym);
@@ -1898,11 +1900,10 @@ __global__ __launch_bounds__(NT) void bpe_long_kernel(
         }
         const size_t n = ((size_t)len + 7) & ~(size_t)7;
         PosRec<uint32_t> *P = reinterpret_cast<PosRec<uint32_t> *>(slab);
-        uint16_t *NS = reinterpret_cast<uint16_t *>(P + n);
-        uint16_t *MC = NS + n;
-        uint32_t *Q = reinterpret_cast<uint32_t *>(MC + n);      // n / 2 entries
+        uint32_t *PG = reinterpret_cast<uint32_t *>(P + n);      // product | gate << 16
+        uint32_t *Q = PG + n;                                    // n / 2 entries
         uint32_t *C = Q + n / 2;                                 // n entries
-        bpe_row<NT, uint32_t, 0>(pt, b2s, a.out_remap, bytes + start, (int)len, P, NS, MC,
+        bpe_row<NT, uint32_t, 0>(pt, b2s, a.out_remap, bytes + start, (int)len, P, PG,
                               Q, C, D, red, threadIdx.x, tok_tmp + start, lengths + row);
         __syncthreads();
     }
