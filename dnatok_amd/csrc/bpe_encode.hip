@@ -866,8 +866,8 @@ __device__ __forceinline__ int32_t bpe_row(
         team_sync<NT>();
         clk.lap(kPhApply);
 
-        // re-rank the two pairs around every new symbol: probe 2m is the pair (new, right
-        // neighbour), probe 2m + 1 the pair (left neighbour, new).  The probes are dealt evenly to
+        // re-rank the two pairs around every new symbol: probe m is the pair (new, right
+        // neighbour), probe nm + m the pair (left neighbour, new).  The probes are dealt evenly to
         // the threads, kProbes pairs of table reads in flight per thread.
         for (int p0 = tid; p0 < 2 * nm; p0 += kProbes * NT) {
             decltype(pair_probe(pt, 0u, 0u)) e[kProbes];
@@ -879,9 +879,12 @@ __device__ __forceinline__ int32_t bpe_row(
                 const int p = p0 + j * NT;
                 sa[j] = 0; sb[j] = 0; target[j] = NIL; valid[j] = false;
                 if (p < 2 * nm) {
-                    const IT i = Q[p >> 1];
+                    // (probes 0 .. nm - 1 are the pairs to the right, nm .. 2 nm - 1 those to the left:
+                    // with the two kinds alternating lane by lane every wave ran both branches)
+                    const bool to_the_left = p >= nm;
+                    const IT i = Q[to_the_left ? p - nm : p];
                     const PosRec<IT> x = P[i];
-                    if (p & 1) {
+                    if (to_the_left) {
                         target[j] = x.pv;
                         if (x.pv != NIL) { sa[j] = P[x.pv].s; sb[j] = x.s; valid[j] = true; }
                     } else {
