@@ -434,7 +434,8 @@ __device__ __forceinline__ int32_t bpe_row(
     // seven and eight waves per SIMD for rows up to 1 KB: 16 batches of 1024 x 1 KB 272 -> 253 us, one
     // batch 33.5 -> 32.7 us.  Four cost 20; four for the first pairs only, or all bytes of a thread's
     // positions requested before the first table read, gained nothing.  Two for the 2 KB forms alone,
-    // which have the registers: 8 batches of 32 x 100 kbp 705 -> 730 us.)
+    // which have the registers: 8 batches of 32 x 100 kbp 705 -> 730 us; two only in passes in which every
+    // thread has two probes, one in the others: 700 -> 715 us.)
     constexpr int kProbes = 1;
     const int wv = (NT == 64) ? 0 : (tid >> 6);
     uint32_t *qn = red + 4 * (NT / 64);        // number of merges queued in the current round
