@@ -1706,6 +1706,83 @@ __global__ __launch_bounds__(256) void bpe_seam_kernel(const int64_t *__restrict
     }
 }
 
+// The same search for shared stretches of at most kSeamMaskSpan positions (twice the shipped
+// overlap), a wave per seam, with no walk from token start to token start and no staging: position
+// 64 q + lane of the stretch is lane's in pass q, a ballot per pass gives the token starts of A, those
+// of B, and the starts of A whose token is the same in B, as 64-bit masks that every lane holds.
+// A seam is a start j of A that matches and whose previous start of A matches too: the previous
+// start is the highest set bit below j in the mask of its pass, or the last start of the passes
+// before (a running value that is the same in all lanes).  The counts the gather needs are popcounts
+// of the masks on either side of the seam.  A seam is then one trip to memory behind its record and
+// some hundred instructions; the walks were chains of dependent LDS reads, a token long each.
+constexpr int kSeamMaskSpan = 256;
+
+__global__ __launch_bounds__(256) void bpe_seam_mask_kernel(BpePlan p)
+{
+    constexpr int kPasses = kSeamMaskSpan / 64;
+    const int team = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int32_t n_mc = p.counts[1];
+    for (int64_t m64 = (int64_t)blockIdx.x * 4 + team; m64 < n_mc; m64 += (int64_t)gridDim.x * 4) {
+        const int32_t m = (int32_t)m64;
+        const int4 rc = p.rec[m];
+        const int32_t row = rc.x, k = rc.y, nc = rc.z;
+        if (k + 1 >= nc) continue;                                   // last chunk: no seam to the right (the same for the whole wave)
+        const int64_t len = rc.w;
+        const int64_t ea0 = (int64_t)k * p.core - p.overlap < 0 ? 0 : (int64_t)k * p.core - p.overlap;
+        int64_t ea1 = (int64_t)(k + 1) * p.core + p.overlap;
+        if (ea1 > len) ea1 = len;
+        const int64_t eb0 = (int64_t)(k + 1) * p.core - p.overlap;
+        const uint16_t *A = p.chunk_sym + (size_t)m * p.ext + (eb0 - ea0);       // A[i], B[i]: position eb0 + i
+        const uint16_t *B = p.chunk_sym + (size_t)(m + 1) * p.ext;
+        const int n = (int)(ea1 - eb0);                              // shared positions, at most kSeamMaskSpan
+        uint32_t sa[kPasses], sb[kPasses];
+#pragma unroll
+        for (int q = 0; q < kPasses; ++q) {
+            const int i = 64 * q + lane;
+            sa[q] = i < n ? (uint32_t)A[i] : kNone;
+            sb[q] = i < n ? (uint32_t)B[i] : kNone;
+        }
+        uint64_t starts_a[kPasses], starts_b[kPasses];
+        int seam = -1;                                               // position within the stretch
+        bool last_start_matches = false;                             // the last start of A in the passes so far: is it one of B's, same token?
+#pragma unroll
+        for (int q = 0; q < kPasses; ++q) {
+            const uint64_t s_a = __ballot(sa[q] != kNone);
+            const uint64_t same = __ballot(sa[q] != kNone && sa[q] == sb[q]);
+            starts_a[q] = s_a;
+            starts_b[q] = __ballot(sb[q] != kNone);
+            // the previous start of A before this lane's position
+            const uint64_t below = s_a & ((1ull << lane) - 1ull);
+            const bool prev_matches = below ? (same >> (63 - __builtin_clzll(below)) & 1ull) != 0 : last_start_matches;
+            const uint64_t ok = __ballot(sa[q] != kNone && sa[q] == sb[q] && prev_matches);
+            if (seam < 0 && ok) seam = 64 * q + __builtin_ctzll(ok);
+            if (s_a) last_start_matches = (same >> (63 - __builtin_clzll(s_a)) & 1ull) != 0;
+        }
+        // (a matched first start of the stretch with no start before it is no seam: the walk began at
+        // a matched start and took the next one)
+        uint32_t tail = 0, head = 0;                                 // tokens of A left of the seam, of B from the seam on
+        if (seam >= 0) {
+#pragma unroll
+            for (int q = 0; q < kPasses; ++q) {
+                const int lo = seam - 64 * q;                        // bits below lo belong to A's side
+                const uint64_t left = lo <= 0 ? 0ull : (lo >= 64 ? ~0ull : ((1ull << lo) - 1ull));
+                tail += (uint32_t)__builtin_popcountll(starts_a[q] & left);
+                head += (uint32_t)__builtin_popcountll(starts_b[q] & ~left);
+            }
+        }
+        if (lane == 0) {
+            if (seam < 0) {
+                p.seam[m] = -1;
+                if (atomicExch(&p.row_fail[row], 1) == 0) atomicAdd(&p.counts[3], 1);
+            } else {
+                p.seam[m] = (int32_t)(eb0 + seam);
+            }
+            p.cnt[4 * (size_t)m + 2] = (int32_t)tail;
+            p.cnt[4 * (size_t)(m + 1) + 1] = (int32_t)head;
+        }
+    }
+}
+
 // The part of a row that chunk k contributes: from the seam on its left to the seam on its right.
 struct ChunkSpan {
     int32_t row, k, nc;
@@ -2366,7 +2443,10 @@ static int bpe_encode_launch(const dnatok_bpe_t *t, const uint8_t *bytes, const 
     if (long_rows) {
         if (chunking) {
             int64_t g = p.max_mc < 4096 ? p.max_mc : 4096;
-            if (p.max_mc >= kSeamWaveFrom) {                               // a wave per seam, up to two rounds of workgroups
+            if (2 * p.overlap <= kSeamMaskSpan) {                          // a wave per seam, the search on ballots
+                int64_t gs = (p.max_mc + 3) / 4;
+                bpe_seam_mask_kernel<<<(int)(gs > 4096 ? 4096 : gs), 256, 0, s>>>(p);
+            } else if (p.max_mc >= kSeamWaveFrom) {                        // a wave per seam, up to two rounds of workgroups
                 int64_t gs = (p.max_mc + 3) / 4;
                 bpe_seam_kernel<64><<<(int)(gs > 4096 ? 4096 : gs), 256, 0, s>>>(offsets, p);
             } else {

@@ -1192,14 +1192,15 @@ def test_bpe_long_runs_of_equal_pairs(bpe):
         np.testing.assert_array_equal(r, e, err_msg=f"{s[:24]}... ({len(s)} bp)")
 
 
-@pytest.mark.parametrize("core,overlap", [(256, 32), (512, 96), (300, 35)])
+@pytest.mark.parametrize("core,overlap", [(256, 32), (512, 96), (300, 35), (700, 160)])
 def test_bpe_small_chunks_many_seams_and_fallbacks(bpe, core, overlap):
     """The chunk / seam / gather / whole-row-fallback machinery with chunks far smaller than the
     shipped ones: a few thousand ragged, random and tandem-repeat rows per vocabulary go through tens
     of thousands of seams, many of which find no position and send their row to the whole-row
     kernel.  Every row is compared with the oracle.  (300, 35): a chunk of 370 symbols is no whole
     number of 16-byte loads, which takes the gather's general form instead of the one that holds
-    a whole chunk per wave.)"""
+    a whole chunk per wave; (700, 160): a shared stretch of more than 256 positions, which takes the
+    seam search that walks from token start to token start instead of the one on ballots.)"""
     which, enc, bo = bpe
     say(f"bpe{which} chunks of {core} + 2 x {overlap}")
     ext = core + 2 * overlap
