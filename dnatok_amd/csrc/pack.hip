@@ -155,7 +155,11 @@ int launch_scan_lengths(const int32_t *lengths, int64_t n_rows, int64_t *out_off
     return DNATOK_OK;
 }
 
-constexpr int kPackTile = 4096;          // output cells one workgroup copies
+// output cells one workgroup copies (the grid is 4,096 workgroups whatever the batch, its size being
+// known on the device only: with 4,096 cells a batch of 4,096 ragged reads was 1.1 tiles per
+// workgroup, i.e. the time of two; 2,048: the call 258.2 -> 255.0 us, eight such batches 1,782 -> 1,786 us;
+// 1,024: 256.0 and 1,798 us)
+constexpr int kPackTile = 2048;
 
 // Packed layout.  A workgroup takes kPackTile consecutive cells of the packed output, finds the
 // first row that reaches into them (binary search in out_offsets) and copies row piece after
